@@ -1,0 +1,65 @@
+"""Engine tuning knobs and per-request sampling options.
+
+Names and meanings follow the reference: ``EngineConfig`` (block_size,
+num_blocks, max_batch_size; src/minigpt_infer/config.py:21-29) and
+``SamplingParams`` (src/minigpt_infer/config.py:32-41).  The token budget, the
+prefill portion size and the mixed-batch switch have no counterpart there: the
+reference never cuts a prompt and never mixes prompt work with decoding
+(src/minigpt_infer/engine/scheduler.py:9-12).
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Optional
+
+
+@dataclass
+class EngineConfig:
+    block_size: int = 16             # tokens per KV page (the reference's "KV block")
+    num_blocks: int = 2048           # pages in the fixed pool, per cache group
+    max_batch_size: int = 256        # most requests running at once (= state slots)
+    max_num_batched_tokens: int = 4096   # token budget of one step
+    prefill_chunk: int = 0           # largest prompt portion per request and step; 0 = no limit
+    mixed_batches: bool = True       # False: a step with admissions runs prompts only,
+                                     # as the reference does (scheduler.py:52-56)
+    dtype: str = "bfloat16"          # "bfloat16" (serving) or "float32" (true 32-bit path)
+    use_graph: bool = True           # replay decode-only steps from a captured HIP graph
+    seed: int = 0                    # engine-wide sampler seed
+    real_vocab_size: Optional[int] = None  # ids at or above it are never sampled
+                                           # (src/minigpt_infer/tokenizer.py:37-46)
+
+    def __post_init__(self) -> None:
+        if self.block_size <= 0 or self.num_blocks <= 0 or self.max_batch_size <= 0:
+            raise ValueError("block_size, num_blocks and max_batch_size must be positive")
+        if self.max_num_batched_tokens <= 0:
+            raise ValueError("max_num_batched_tokens must be positive")
+        if self.prefill_chunk < 0:
+            raise ValueError("prefill_chunk must be >= 0")
+        if self.dtype in ("bf16",):
+            self.dtype = "bfloat16"
+        if self.dtype in ("fp32",):
+            self.dtype = "float32"
+        if self.dtype not in ("bfloat16", "float32"):
+            raise ValueError(f"dtype must be bfloat16 or float32, got {self.dtype!r}")
+
+
+@dataclass
+class SamplingParams:
+    max_tokens: int = 128
+    temperature: float = 1.0         # 0.0 => greedy (src/minigpt_infer/sampling.py:120)
+    top_k: Optional[int] = None
+    top_p: Optional[float] = None
+    seed: Optional[int] = None       # per-request sampler stream; None = derived from the request's arrival order
+    n: int = 1
+
+    def __post_init__(self) -> None:
+        if self.n != 1:
+            # src/minigpt_infer/engine/engine.py:70
+            raise ValueError("n>1 completions per request are not supported")
+        if self.max_tokens <= 0:
+            raise ValueError("max_tokens must be positive")
+        if self.top_k is not None and self.top_k <= 0:
+            raise ValueError("top_k must be positive")
+        if self.top_p is not None and not (0.0 < self.top_p <= 1.0):
+            raise ValueError("top_p must lie in (0, 1]")

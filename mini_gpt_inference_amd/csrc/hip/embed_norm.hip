@@ -1,0 +1,93 @@
+// Token embedding (+ learned position rows) into the 32-bit residual stream,
+// and LayerNorm with 32-bit statistics.
+//
+// embedding: x0[t] = tok_emb[id_t] + pos_emb[pos_t]   (reference: src/minigpt_infer/model.py:183)
+// LayerNorm: y = (x - mean) / sqrt(var_biased + eps) * w (+ b) over the last dim
+//            (reference: nn.LayerNorm at src/minigpt_infer/model.py:107,109,127)
+#include "common.h"
+
+template <typename WT>
+__global__ void embed_kernel(const int* __restrict__ ids, const int* __restrict__ pos,
+                             const WT* __restrict__ tok, const WT* __restrict__ postab,
+                             float* __restrict__ x, int n_tokens, int width) {
+  int n = blockIdx.x;
+  if (n >= n_tokens) return;
+  long id = ids[n];
+  const WT* trow = tok + id * (long)width;
+  const WT* prow = postab ? postab + (long)pos[n] * width : nullptr;
+  float* xr = x + (long)n * width;
+  for (int c = threadIdx.x; c < width; c += blockDim.x) {
+    float v = to_float<WT>(trow[c]);
+    if (prow) v += to_float<WT>(prow[c]);
+    xr[c] = v;
+  }
+}
+
+extern "C" int mgpt_embed(const int* ids, const int* pos, const void* tok, const void* postab,
+                          float* x, int n_tokens, int width, int table_dtype, hipStream_t stream) {
+  if (n_tokens == 0) return MGPT_OK;
+  if (!ids || !tok || !x || (postab && !pos)) return MGPT_ERR_NULL;
+  if (n_tokens < 0 || width <= 0) return MGPT_ERR_BAD_SHAPE;
+  int threads = width >= 256 ? 256 : 64;
+  if (table_dtype == MGPT_F32) {
+    hipLaunchKernelGGL(embed_kernel<float>, dim3(n_tokens), dim3(threads), 0, stream, ids, pos,
+                       (const float*)tok, (const float*)postab, x, n_tokens, width);
+  } else if (table_dtype == MGPT_BF16) {
+    hipLaunchKernelGGL(embed_kernel<bf16_t>, dim3(n_tokens), dim3(threads), 0, stream, ids, pos,
+                       (const bf16_t*)tok, (const bf16_t*)postab, x, n_tokens, width);
+  } else {
+    return MGPT_ERR_BAD_DTYPE;
+  }
+  return mgpt_last_error();
+}
+
+// One wave per row; four rows per workgroup.  Mean, then centred variance, then
+// the normalised row: three passes over a row that stays in cache, so any width
+// works and the variance is never a difference of large numbers.
+template <typename OT>
+__global__ void layernorm_kernel(const float* __restrict__ x, const float* __restrict__ w,
+                                 const float* __restrict__ b, OT* __restrict__ out,
+                                 const int* __restrict__ rows, int n_rows, int width, float eps) {
+  int lane = threadIdx.x & (MGPT_WAVE - 1);
+  int row = blockIdx.x * (blockDim.x / MGPT_WAVE) + (threadIdx.x / MGPT_WAVE);
+  if (row >= n_rows) return;
+  long src = rows ? rows[row] : row;
+  const float* xr = x + src * (long)width;
+  float s = 0.f;
+  for (int c = lane; c < width; c += MGPT_WAVE) s += xr[c];
+  float mean = wave_sum(s) / (float)width;
+  float v = 0.f;
+  for (int c = lane; c < width; c += MGPT_WAVE) {
+    float d = xr[c] - mean;
+    v += d * d;
+  }
+  float var = wave_sum(v) / (float)width;
+  float rstd = 1.0f / sqrtf(var + eps);
+  OT* orow = out + (long)row * width;
+  for (int c = lane; c < width; c += MGPT_WAVE) {
+    float y = (xr[c] - mean) * rstd * w[c];
+    if (b) y += b[c];
+    orow[c] = from_float<OT>(y);
+  }
+}
+
+// rows: optional gather list (n_rows entries) of source rows of x; out row i <- x row rows[i].
+extern "C" int mgpt_layernorm(const float* x, const float* w, const float* b, void* out,
+                              const int* rows, int n_rows, int width, float eps, int out_dtype,
+                              hipStream_t stream) {
+  if (n_rows == 0) return MGPT_OK;
+  if (!x || !w || !out) return MGPT_ERR_NULL;
+  if (n_rows < 0 || width <= 0) return MGPT_ERR_BAD_SHAPE;
+  const int rows_per_block = 4;
+  dim3 grid((n_rows + rows_per_block - 1) / rows_per_block), block(rows_per_block * MGPT_WAVE);
+  if (out_dtype == MGPT_F32) {
+    hipLaunchKernelGGL(layernorm_kernel<float>, grid, block, 0, stream, x, w, b, (float*)out, rows,
+                       n_rows, width, eps);
+  } else if (out_dtype == MGPT_BF16) {
+    hipLaunchKernelGGL(layernorm_kernel<bf16_t>, grid, block, 0, stream, x, w, b, (bf16_t*)out,
+                       rows, n_rows, width, eps);
+  } else {
+    return MGPT_ERR_BAD_DTYPE;
+  }
+  return mgpt_last_error();
+}

@@ -1,0 +1,131 @@
+// Plain tiled matrix product with 32-bit FMA accumulation, for every storage
+// type pair.  out[n, o] = sum_k A[n, k] * W[o, k] (+ bias[o]) with an optional
+// GELU-tanh or residual-add epilogue: y = x W^T + b as nn.Linear
+// (reference: src/minigpt_infer/model.py:43-44,96-101).
+//
+// This is the kernel of the true 32-bit path: k runs 0..K-1 in order for every
+// output element, so a row's result does not depend on which other rows share
+// the launch.  The bfloat16 serving path uses it only for shapes the MFMA
+// kernels refuse.
+#include "common.h"
+
+#define EPI_NONE 0
+#define EPI_GELU 1
+#define EPI_RESIDUAL 2  // out (float) += result
+
+#define TILE 64
+#define BK 16
+#define PAD 4
+
+template <typename AT, typename WT, typename OT, int EPI>
+__global__ __launch_bounds__(256) void linear_generic_kernel(
+    const AT* __restrict__ A, long lda, const WT* __restrict__ W, const float* __restrict__ bias,
+    OT* __restrict__ out, long ldo, int n_rows, int n_out, int k_dim) {
+  __shared__ float As[BK][TILE + PAD];
+  __shared__ float Ws[BK][TILE + PAD];
+  const int tid = threadIdx.x;
+  const int tx = tid & 15, ty = tid >> 4;
+  const int row0 = blockIdx.y * TILE, col0 = blockIdx.x * TILE;
+  const int lrow = tid >> 2, lk = (tid & 3) * 4;
+
+  float acc[4][4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) acc[i][j] = 0.f;
+
+  const int arow = row0 + lrow, wrow = col0 + lrow;
+  const bool a_ok = arow < n_rows, w_ok = wrow < n_out;
+  const AT* ap = A + (long)arow * lda + lk;
+  const WT* wp = W + (long)wrow * k_dim + lk;
+
+  for (int k0 = 0; k0 < k_dim; k0 += BK) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      As[lk + i][lrow] = a_ok ? to_float<AT>(ap[k0 + i]) : 0.f;
+      Ws[lk + i][lrow] = w_ok ? to_float<WT>(wp[k0 + i]) : 0.f;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int kk = 0; kk < BK; ++kk) {
+      float a[4], w[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) a[i] = As[kk][ty * 4 + i];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) w[j] = Ws[kk][tx * 4 + j];
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] = fmaf(a[i], w[j], acc[i][j]);
+    }
+    __syncthreads();
+  }
+
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    int r = row0 + ty * 4 + i;
+    if (r >= n_rows) continue;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      int c = col0 + tx * 4 + j;
+      if (c >= n_out) continue;
+      float v = acc[i][j];
+      if (bias) v += bias[c];
+      if (EPI == EPI_GELU) v = gelu_tanh(v);
+      OT* dst = out + (long)r * ldo + c;
+      if (EPI == EPI_RESIDUAL) {
+        *dst = from_float<OT>(to_float<OT>(*dst) + v);
+      } else {
+        *dst = from_float<OT>(v);
+      }
+    }
+  }
+}
+
+template <typename AT, typename WT, typename OT>
+static int launch_epi(const void* A, long lda, const void* W, const float* bias, void* out, long ldo,
+                      int n_rows, int n_out, int k_dim, int epi, hipStream_t stream) {
+  dim3 grid((n_out + TILE - 1) / TILE, (n_rows + TILE - 1) / TILE), block(256);
+#define LAUNCH(E)                                                                               \
+  hipLaunchKernelGGL((linear_generic_kernel<AT, WT, OT, E>), grid, block, 0, stream, (const AT*)A, \
+                     lda, (const WT*)W, bias, (OT*)out, ldo, n_rows, n_out, k_dim)
+  if (epi == EPI_NONE) LAUNCH(EPI_NONE);
+  else if (epi == EPI_GELU) LAUNCH(EPI_GELU);
+  else if (epi == EPI_RESIDUAL) LAUNCH(EPI_RESIDUAL);
+  else return MGPT_ERR_BAD_SHAPE;
+#undef LAUNCH
+  return mgpt_last_error();
+}
+
+template <typename AT, typename WT>
+static int launch_out(const void* A, long lda, const void* W, const float* bias, void* out, long ldo,
+                      int n_rows, int n_out, int k_dim, int epi, int out_dtype, hipStream_t stream) {
+  if (out_dtype == MGPT_F32)
+    return launch_epi<AT, WT, float>(A, lda, W, bias, out, ldo, n_rows, n_out, k_dim, epi, stream);
+  if (out_dtype == MGPT_BF16) {
+    if (epi == EPI_RESIDUAL) return MGPT_ERR_BAD_DTYPE;  // the residual stream is 32-bit
+    return launch_epi<AT, WT, bf16_t>(A, lda, W, bias, out, ldo, n_rows, n_out, k_dim, epi, stream);
+  }
+  return MGPT_ERR_BAD_DTYPE;
+}
+
+// A: [n_rows, k_dim] with row stride lda; W: [n_out, k_dim] dense; out: [n_rows, n_out] with row
+// stride ldo.  k_dim must be a multiple of 16.
+extern "C" int mgpt_linear_generic(const void* A, int a_dtype, long lda, const void* W, int w_dtype,
+                                   const float* bias, void* out, int out_dtype, long ldo, int n_rows,
+                                   int n_out, int k_dim, int epilogue, hipStream_t stream) {
+  if (n_rows == 0 || n_out == 0) return MGPT_OK;
+  if (!A || !W || !out) return MGPT_ERR_NULL;
+  if (n_rows < 0 || n_out < 0 || k_dim <= 0 || (k_dim % BK) != 0 || lda < k_dim || ldo < n_out)
+    return MGPT_ERR_BAD_SHAPE;
+  if ((n_rows + TILE - 1) / TILE > 65535) return MGPT_ERR_TOO_LARGE;
+  if (a_dtype == MGPT_F32 && w_dtype == MGPT_F32)
+    return launch_out<float, float>(A, lda, W, bias, out, ldo, n_rows, n_out, k_dim, epilogue, out_dtype, stream);
+  if (a_dtype == MGPT_BF16 && w_dtype == MGPT_BF16)
+    return launch_out<bf16_t, bf16_t>(A, lda, W, bias, out, ldo, n_rows, n_out, k_dim, epilogue, out_dtype, stream);
+  if (a_dtype == MGPT_BF16 && w_dtype == MGPT_F32)
+    return launch_out<bf16_t, float>(A, lda, W, bias, out, ldo, n_rows, n_out, k_dim, epilogue, out_dtype, stream);
+  if (a_dtype == MGPT_F32 && w_dtype == MGPT_BF16)
+    return launch_out<float, bf16_t>(A, lda, W, bias, out, ldo, n_rows, n_out, k_dim, epilogue, out_dtype, stream);
+  return MGPT_ERR_BAD_DTYPE;
+}

@@ -1,0 +1,228 @@
+// Next-token choice from 32-bit logits: one workgroup per row.
+//
+// Order of operations as the reference (src/minigpt_infer/sampling.py:97-137,
+// src/minigpt_infer/engine/engine.py:154-159): ids at or above real_vocab are
+// never chosen; temperature <= 0 takes the argmax of the unscaled logits (the
+// lowest index among equals); otherwise s = logits / max(T, 1e-6); top-k keeps
+// the values >= the k-th largest (ties pass, sampling.py:39-52); top-p keeps a
+// token iff the probability mass of the strictly larger ones is <= p, so the
+// largest always stays (sampling.py:55-76); then a softmax over what is left.
+//
+// Where the reference draws with torch.multinomial from one shared generator,
+// this draws by inverse CDF in vocabulary order with a uniform number that is a
+// pure function of (engine seed, request seed, index of the output token), so a
+// request's tokens do not depend on batching or preemption.
+#include "common.h"
+
+#define SAMPLE_THREADS 1024
+#define SAMPLE_WAVES (SAMPLE_THREADS / MGPT_WAVE)
+
+__device__ __forceinline__ unsigned int float_key(float f) {
+  unsigned int u = __float_as_uint(f);
+  return (u & 0x80000000u) ? ~u : (u | 0x80000000u);  // monotone: larger float -> larger key
+}
+
+__device__ __forceinline__ uint64_t mix64(uint64_t z) {
+  z ^= z >> 30; z *= 0xBF58476D1CE4E5B9ull;
+  z ^= z >> 27; z *= 0x94D049BB133111EBull;
+  z ^= z >> 31;
+  return z;
+}
+
+// uniform in [0, 1) with 24 bits
+__device__ __forceinline__ float sample_uniform(uint64_t engine_seed, uint64_t request_seed,
+                                                uint64_t index) {
+  uint64_t z = engine_seed * 0x9E3779B97F4A7C15ull + request_seed * 0xD1B54A32D192ED03ull +
+               index * 0x8CB92BA72F3D8DD7ull + 0x2545F4914F6CDD1Dull;
+  z = mix64(mix64(z));
+  return (float)(z >> 40) * (1.0f / 16777216.0f);
+}
+
+__device__ float block_sum(float v, float* red) {
+  v = wave_sum(v);
+  __syncthreads();
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
+  __syncthreads();
+  float t = 0.f;
+  for (int i = 0; i < SAMPLE_WAVES; ++i) t += red[i];  // fixed order
+  return t;
+}
+
+__device__ int block_sum_int(int v, int* red) {
+  v = wave_sum_int(v);
+  __syncthreads();
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
+  __syncthreads();
+  int t = 0;
+  for (int i = 0; i < SAMPLE_WAVES; ++i) t += red[i];
+  return t;
+}
+
+__device__ float block_max(float v, float* red) {
+  v = wave_max(v);
+  __syncthreads();
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
+  __syncthreads();
+  float t = -INFINITY;
+  for (int i = 0; i < SAMPLE_WAVES; ++i) t = fmaxf(t, red[i]);
+  return t;
+}
+
+__global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
+    const float* __restrict__ logits, long ld, int vocab, int real_vocab,
+    const float* __restrict__ temperature, const int* __restrict__ top_k,
+    const float* __restrict__ top_p, const uint64_t* __restrict__ request_seed,
+    const int* __restrict__ out_index, uint64_t engine_seed, int* __restrict__ out_tokens) {
+  __shared__ float red_f[SAMPLE_WAVES];
+  __shared__ int red_i[SAMPLE_WAVES];
+  __shared__ float part[SAMPLE_THREADS];
+  __shared__ float wave_off[SAMPLE_WAVES + 1];
+  __shared__ int chosen;
+
+  const int row = blockIdx.x, tid = threadIdx.x;
+  const float* lg = logits + (long)row * ld;
+  const int nv = real_vocab < vocab ? real_vocab : vocab;
+  const float temp = temperature[row];
+
+  if (temp <= 0.f) {
+    float best = -INFINITY;
+    int best_i = 0x7fffffff;
+    for (int i = tid; i < nv; i += SAMPLE_THREADS) {
+      float v = lg[i];
+      if (v > best || (v == best && i < best_i)) { best = v; best_i = i; }
+    }
+    // NaN-free rows always have a candidate; a row of -inf falls back to index 0
+    for (int off = 32; off > 0; off >>= 1) {
+      float ov = __shfl_xor(best, off, MGPT_WAVE);
+      int oi = __shfl_xor(best_i, off, MGPT_WAVE);
+      if (ov > best || (ov == best && oi < best_i)) { best = ov; best_i = oi; }
+    }
+    if ((tid & 63) == 0) { red_f[tid >> 6] = best; red_i[tid >> 6] = best_i; }
+    __syncthreads();
+    if (tid == 0) {
+      for (int i = 1; i < SAMPLE_WAVES; ++i)
+        if (red_f[i] > best || (red_f[i] == best && red_i[i] < best_i)) { best = red_f[i]; best_i = red_i[i]; }
+      out_tokens[row] = best_i == 0x7fffffff ? 0 : best_i;
+    }
+    return;
+  }
+
+  const float t_safe = fmaxf(temp, 1e-6f);
+  // largest scaled logit
+  float mx = -INFINITY;
+  for (int i = tid; i < nv; i += SAMPLE_THREADS) mx = fmaxf(mx, lg[i] / t_safe);
+  mx = block_max(mx, red_f);
+
+  // top-k: key of the k-th largest value, by bisection on the ordered bit pattern
+  unsigned int key_floor = 0u;  // keep keys >= key_floor
+  const int k = top_k ? top_k[row] : 0;
+  if (k > 0 && k < nv) {
+    unsigned int lo = 0u, hi = 0xffffffffu;  // invariant: count(key >= lo) >= k
+    while (lo < hi) {
+      unsigned int mid = lo + (unsigned int)(((uint64_t)hi - lo + 1) >> 1);
+      int cnt = 0;
+      for (int i = tid; i < nv; i += SAMPLE_THREADS) cnt += float_key(lg[i] / t_safe) >= mid;
+      cnt = block_sum_int(cnt, red_i);
+      if (cnt >= k) lo = mid; else hi = mid - 1;
+    }
+    key_floor = lo;
+  }
+
+  // top-p: smallest key kappa with mass(key > kappa) <= p * Z
+  const float p = top_p ? top_p[row] : 1.0f;
+  if (p < 1.0f) {
+    float z = 0.f;
+    for (int i = tid; i < nv; i += SAMPLE_THREADS) {
+      float s = lg[i] / t_safe;
+      if (float_key(s) >= key_floor) z += expf(s - mx);
+    }
+    z = block_sum(z, red_f);
+    const float budget = p * z;
+    unsigned int lo = key_floor, hi = float_key(mx);  // G(hi) = 0 <= budget always
+    while (lo < hi) {
+      unsigned int mid = lo + ((hi - lo) >> 1);
+      float g = 0.f;
+      for (int i = tid; i < nv; i += SAMPLE_THREADS) {
+        float s = lg[i] / t_safe;
+        unsigned int key = float_key(s);
+        if (key > mid && key >= key_floor) g += expf(s - mx);
+      }
+      g = block_sum(g, red_f);
+      if (g <= budget) hi = mid; else lo = mid + 1;
+    }
+    key_floor = lo;
+  }
+
+  // inverse CDF in vocabulary order over what is kept
+  const int per = (nv + SAMPLE_THREADS - 1) / SAMPLE_THREADS;
+  const int i0 = tid * per, i1 = (i0 + per < nv) ? i0 + per : nv;
+  float mine = 0.f;
+  int last_kept = -1;
+  for (int i = i0; i < i1; ++i) {
+    float s = lg[i] / t_safe;
+    if (float_key(s) >= key_floor) { mine += expf(s - mx); last_kept = i; }
+  }
+  part[tid] = mine;
+  if (tid == 0) chosen = 0x7fffffff;
+  __syncthreads();
+  // serial scans keep the prefix sums monotone
+  if ((tid & 63) == 0) {
+    float run = 0.f;
+    for (int i = 0; i < MGPT_WAVE; ++i) { run += part[tid + i]; part[tid + i] = run; }
+  }
+  __syncthreads();
+  if (tid == 0) {
+    float run = 0.f;
+    wave_off[0] = 0.f;
+    for (int w = 0; w < SAMPLE_WAVES; ++w) { run += part[w * MGPT_WAVE + MGPT_WAVE - 1]; wave_off[w + 1] = run; }
+  }
+  __syncthreads();
+  const float total = wave_off[SAMPLE_WAVES];
+  const float u = sample_uniform(engine_seed, request_seed ? request_seed[row] : 0ull,
+                                 (uint64_t)(out_index ? out_index[row] : 0));
+  const float target = u * total;
+  const int w = tid >> 6;
+  const float incl = wave_off[w] + part[tid];
+  const float excl = (tid & 63) ? wave_off[w] + part[tid - 1] : wave_off[w];
+  if (mine > 0.f && excl <= target && target < incl) {
+    float run = excl;
+    int pick = last_kept;
+    for (int i = i0; i < i1; ++i) {
+      float s = lg[i] / t_safe;
+      if (float_key(s) >= key_floor) {
+        run += expf(s - mx);
+        if (run > target) { pick = i; break; }
+      }
+    }
+    atomicMin(&chosen, pick);
+  }
+  // rounding can leave target >= total: then the last kept id stands
+  int lk = last_kept;
+  for (int off = 32; off > 0; off >>= 1) lk = max(lk, __shfl_xor(lk, off, MGPT_WAVE));
+  __syncthreads();
+  if ((tid & 63) == 0) red_i[tid >> 6] = lk;
+  __syncthreads();
+  if (tid == 0) {
+    int c = chosen;
+    if (c == 0x7fffffff) {
+      c = 0;
+      for (int i = 0; i < SAMPLE_WAVES; ++i) c = max(c, red_i[i]);
+    }
+    out_tokens[row] = c;
+  }
+}
+
+// logits: [n_rows, vocab] floats with row stride ld.  top_k (0 = off), top_p (1 = off),
+// request_seed and out_index may be null.
+extern "C" int mgpt_sample(const float* logits, long ld, int n_rows, int vocab, int real_vocab,
+                           const float* temperature, const int* top_k, const float* top_p,
+                           const uint64_t* request_seed, const int* out_index, uint64_t engine_seed,
+                           int* out_tokens, hipStream_t stream) {
+  if (n_rows == 0) return MGPT_OK;
+  if (!logits || !temperature || !out_tokens) return MGPT_ERR_NULL;
+  if (n_rows < 0 || vocab <= 0 || real_vocab <= 0 || ld < vocab) return MGPT_ERR_BAD_SHAPE;
+  hipLaunchKernelGGL(sample_kernel, dim3(n_rows), dim3(SAMPLE_THREADS), 0, stream, logits, ld, vocab,
+                     real_vocab, temperature, top_k, top_p, request_seed, out_index, engine_seed,
+                     out_tokens);
+  return mgpt_last_error();
+}

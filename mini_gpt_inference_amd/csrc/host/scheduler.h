@@ -1,0 +1,121 @@
+// Continuous-batching scheduler: admits requests, cuts prompts into portions
+// under a token budget, decodes, finishes and frees.
+//
+// Queues, first-come admission with head-of-line blocking, newest-first
+// preempt-by-recompute and free-on-finish follow the reference
+// (src/minigpt_infer/engine/scheduler.py:23-117).  Prompt portions and steps
+// that mix prompt work with decoding are not in the reference
+// (scheduler.py:9-12); with mixed = false and prefill_chunk = 0 the policy is
+// the reference's: a step that has prompt work runs prompts only.
+//
+// One rule covers prompts, portions, recompute and decoding: a request's context
+// is prompt + outputs; a step feeds context[num_computed : num_computed + q]
+// with 1 <= q <= remaining; only when num_computed reaches the context's length
+// is a logit row produced and one token sampled (src/minigpt_infer/engine/engine.py:243-244,
+// 281-282; src/minigpt_infer/engine/request.py:59-63).
+#pragma once
+
+#include <cstdint>
+#include <deque>
+#include <memory>
+#include <vector>
+
+#include "cache_manager.h"
+
+namespace mgpt {
+
+enum RequestStatus { WAITING = 0, RUNNING = 1, FINISHED = 2 };
+enum FinishReason { NOT_FINISHED = 0, FINISH_EOT = 1, FINISH_LENGTH = 2, FINISH_CANCELLED = 3 };
+
+struct SchedulerConfig {
+  int max_batch_size;          // most requests running at once
+  int max_num_batched_tokens;  // token budget of one step
+  int prefill_chunk;           // largest prompt portion per request and step; 0 = no limit
+  bool mixed;                  // prompt portions beside decode tokens in one step
+  int max_positions;           // prompt + max_tokens may not exceed it (engine.py:83-88)
+};
+
+struct Request {
+  int id = -1;
+  std::vector<int> prompt;
+  std::vector<int> output;
+  int max_tokens = 0;
+  int eot = -1;  // -1: none
+  float temperature = 1.0f;
+  int top_k = 0;       // 0: off
+  float top_p = 1.0f;  // 1: off
+  uint64_t seed = 0;
+  int num_computed = 0;  // tokens whose keys and values are in the cache
+  int slot = -1;
+  RequestStatus status = WAITING;
+  FinishReason finish_reason = NOT_FINISHED;
+  int num_tokens() const { return (int)(prompt.size() + output.size()); }
+  int token_at(int i) const { return i < (int)prompt.size() ? prompt[i] : output[i - prompt.size()]; }
+};
+
+struct StepEntry {
+  int id;       // request id
+  int ctx;      // tokens already cached = position of the first new token
+  int q_len;    // tokens fed in this step
+  bool sample;  // the context is complete after this step: a logit row and one new token
+};
+
+struct StepOutput {
+  int id;
+  int token;
+  int finished;  // 0/1
+  int reason;    // FinishReason
+};
+
+class Scheduler {
+ public:
+  // add_request errors
+  static constexpr int ERR_EMPTY_PROMPT = -1;
+  static constexpr int ERR_TOO_LONG = -2;      // prompt + max_tokens > max_positions
+  static constexpr int ERR_NEVER_FITS = -3;    // more pages than the whole pool holds
+  static constexpr int ERR_BAD_PARAMS = -4;
+
+  Scheduler(CacheManager* cache, const SchedulerConfig& cfg);
+
+  int add_request(const int* prompt, int n_prompt, int max_tokens, int eot, float temperature,
+                  int top_k, float top_p, uint64_t seed, bool has_seed);
+  bool has_work() const { return !waiting_.empty() || !running_.empty(); }
+  bool cancel(int id);
+
+  // Decides the next step.  The entries stay valid until the next call.
+  const std::vector<StepEntry>& schedule();
+  // Takes the tokens sampled for the entries with sample = true, in entry order.
+  const std::vector<StepOutput>& commit(const int* tokens, int n_tokens);
+
+  const Request* request(int id) const;
+  const std::deque<int>& waiting() const { return waiting_; }
+  const std::vector<int>& running() const { return running_; }
+  const std::vector<StepEntry>& entries() const { return entries_; }
+
+  long num_preemptions = 0;
+  long num_steps = 0;
+  long num_prompt_tokens = 0;  // scheduled as part of a portion of more than one token or an unfinished prompt
+  long num_decode_tokens = 0;
+
+  // drops the records of finished requests (their ids are not reused)
+  void forget_finished();
+
+ private:
+  Request* get(int id);
+  void preempt(Request& r);
+  void finish(Request& r, FinishReason why);
+  void ensure_capacity_for_decode();
+  void schedule_decodes(int& budget);
+  void schedule_prompts(int& budget, bool allow_admission);
+
+  CacheManager* cache_;
+  SchedulerConfig cfg_;
+  std::vector<std::unique_ptr<Request>> requests_;  // index = id
+  std::deque<int> waiting_;
+  std::vector<int> running_;  // admission order
+  std::vector<StepEntry> entries_;
+  std::vector<StepOutput> outputs_;
+  bool preempted_this_step_ = false;
+};
+
+}  // namespace mgpt

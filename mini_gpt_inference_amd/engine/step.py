@@ -1,0 +1,184 @@
+"""The step function: one batch of (request, its next tokens) through the model.
+
+A step is described by flat int32 arrays (one entry per token, per request, per wanted logit
+row).  They are written into one pinned host arena, uploaded with one copy into a device arena
+of the same layout, and every kernel reads them there; no mask tensor exists, masking is
+key position <= query position inside the attention kernels.  The reference builds a
+rectangular (B, T) ForwardBatch with a mask instead and never mixes prompts with decoding
+(src/minigpt_infer/batch.py:19-65, src/minigpt_infer/engine/engine.py:210-283).
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Dict, List, Optional, Sequence, Tuple
+
+import numpy as np
+import torch
+
+from ..cache.kv_store import KVStore
+from ..cache.manager import CacheManager
+from ..parts.base import GroupView, StepContext, Workspace
+from ..parts.model import DecoderModel
+
+
+def _round_up(n: int, m: int) -> int:
+    return (n + m - 1) // m * m
+
+
+def _bucket(n: int) -> int:
+    """Capacities grow in powers of two so that few arenas are ever made."""
+    b = 1
+    while b < n:
+        b *= 2
+    return b
+
+
+class StepArena:
+    """Pinned host arrays and their device mirror for steps of up to (n_cap tokens, r_cap requests,
+    m_cap logit rows)."""
+
+    def __init__(self, n_cap: int, r_cap: int, m_cap: int, n_groups: int, max_blocks: int,
+                 device: torch.device) -> None:
+        self.n_cap, self.r_cap, self.m_cap, self.n_groups, self.max_blocks = n_cap, r_cap, m_cap, n_groups, max_blocks
+        fields: List[Tuple[str, int, type]] = [
+            ("seeds", 2 * m_cap, np.int32),   # 64-bit, first so that it is 8-byte aligned
+            ("token_ids", n_cap, np.int32), ("positions", n_cap, np.int32), ("q_req", n_cap, np.int32),
+            ("cu_q", r_cap + 1, np.int32), ("seq_lens", r_cap, np.int32), ("state_slots", r_cap, np.int32),
+            ("logit_rows", m_cap, np.int32), ("slot_mapping", n_groups * n_cap, np.int32),
+            ("block_tables", n_groups * r_cap * max_blocks, np.int32),
+            ("temperature", m_cap, np.float32), ("top_k", m_cap, np.int32), ("top_p", m_cap, np.float32),
+            ("out_index", m_cap, np.int32),
+        ]
+        total = sum(_round_up(n, 4) for _, n, _ in fields)
+        self.host_t = torch.zeros(total, dtype=torch.int32, pin_memory=device.type == "cuda")
+        self.dev_t = torch.zeros(total, dtype=torch.int32, device=device)
+        host_np = self.host_t.numpy()
+        self.h: Dict[str, np.ndarray] = {}
+        self.d: Dict[str, torch.Tensor] = {}
+        off = 0
+        for name, n, typ in fields:
+            self.h[name] = host_np[off:off + n].view(typ)
+            dv = self.dev_t[off:off + n]
+            self.d[name] = dv.view(torch.float32) if typ is np.float32 else dv
+            off += _round_up(n, 4)
+        self.h["seeds"] = self.h["seeds"].view(np.uint64)
+        self.d["seeds"] = self.d["seeds"].view(torch.int64)
+        self.tokens_out = torch.zeros(m_cap, dtype=torch.int32, device=device)
+        self.tokens_host = torch.zeros(m_cap, dtype=torch.int32, pin_memory=device.type == "cuda")
+
+    def upload(self) -> None:
+        self.dev_t.copy_(self.host_t, non_blocking=True)
+
+
+@dataclass
+class StepShape:
+    n_tokens: int
+    n_req: int
+    n_logits: int
+    max_q_len: int
+    max_seq_len: int
+    q_lens: List[int]
+    ctx_lens: List[int]
+    slots: List[int]
+
+
+class ModelRunner:
+    """Owns the device side of stepping: arenas, workspace, the cache's pools, the model."""
+
+    def __init__(self, model: DecoderModel, cache: CacheManager, store: KVStore, dtype: torch.dtype,
+                 device: torch.device, max_positions: Optional[int]) -> None:
+        self.model, self.cache, self.store = model, cache, store
+        self.dtype, self.device = dtype, device
+        self.exact = dtype == torch.float32
+        self.max_positions = max_positions
+        self.vocab_size = model.spec.vocab_size
+        self.workspace = Workspace(device)
+        self._arenas: Dict[Tuple[int, int, int], StepArena] = {}
+        self.n_groups = len(cache.groups)
+        # enough block-table columns for the longest sequence this model can hold
+        if max_positions is not None:
+            self.max_blocks = max(1, max(-(-max_positions // g.page_size) for g in cache.groups))
+        else:
+            self.max_blocks = max(g.num_pages for g in cache.groups)
+
+    # ------------------------------------------------------------------ arenas
+    def arena(self, n_tokens: int, n_req: int, n_logits: int) -> StepArena:
+        key = (_bucket(max(n_tokens, 1)), _bucket(max(n_req, 1)), _bucket(max(n_logits, 1)))
+        a = self._arenas.get(key)
+        if a is None:
+            a = StepArena(*key, self.n_groups, self.max_blocks, self.device)
+            self._arenas[key] = a
+        return a
+
+    # ------------------------------------------------------------------ describing a step
+    def describe(self, arena: StepArena, slots: Sequence[int], ctx_lens: Sequence[int], q_lens: Sequence[int],
+                 tokens: Sequence[int], logit_rows: Sequence[int]) -> StepShape:
+        """Fills the arena for requests given by their cache slots: request i brings q_lens[i] tokens
+        (its part of the flat `tokens`) on top of ctx_lens[i] cached ones.  logit_rows index `tokens`."""
+        h = arena.h
+        n = self.cache.build_step(slots, ctx_lens, q_lens, arena.n_cap, arena.r_cap, arena.max_blocks,
+                                  h["positions"], h["q_req"], h["cu_q"], h["seq_lens"], h["slot_mapping"],
+                                  h["block_tables"])
+        if n != len(tokens):
+            raise ValueError(f"the step's requests bring {n} tokens, but {len(tokens)} token ids were given")
+        h["token_ids"][:n] = np.asarray(tokens, dtype=np.int32)
+        h["token_ids"][n:] = 0
+        r, m = len(slots), len(logit_rows)
+        h["state_slots"][:r] = np.asarray(slots, dtype=np.int32)
+        h["state_slots"][r:] = -1
+        rows = np.asarray(logit_rows, dtype=np.int32)
+        if m and (rows.min() < 0 or rows.max() >= n):
+            raise ValueError("a wanted logit row lies outside the step's tokens")
+        h["logit_rows"][:m] = rows
+        h["logit_rows"][m:] = 0
+        return self.shape_of(arena, n, r, m, list(q_lens), list(ctx_lens), list(slots))
+
+    def shape_of(self, arena: StepArena, n: int, r: int, m: int, q_lens: List[int], ctx_lens: List[int],
+                 slots: List[int]) -> StepShape:
+        h = arena.h
+        ids = h["token_ids"][:n]
+        if n and (ids.min() < 0 or ids.max() >= self.vocab_size):
+            raise ValueError(f"token id outside 0..{self.vocab_size - 1}")
+        max_seq = max((c + q for c, q in zip(ctx_lens, q_lens)), default=0)
+        if self.max_positions is not None and max_seq > self.max_positions:
+            # src/minigpt_infer/model.py:177-182
+            raise ValueError(f"position {max_seq - 1} >= block_size={self.max_positions}: "
+                             "the position table has no such row")
+        return StepShape(n, r, m, max(q_lens, default=0), max_seq, q_lens, ctx_lens, slots)
+
+    # ------------------------------------------------------------------ running
+    def context(self, arena: StepArena, shape: StepShape, padded: bool, workspace: Optional[Workspace] = None
+                ) -> StepContext:
+        d = arena.d
+        groups = []
+        for g, geo in enumerate(self.cache.groups):
+            groups.append(GroupView(
+                page_size=geo.page_size, window=geo.window,
+                slot_mapping=d["slot_mapping"][g * arena.n_cap:(g + 1) * arena.n_cap],
+                block_tables=d["block_tables"][g * arena.r_cap * arena.max_blocks:
+                                               (g + 1) * arena.r_cap * arena.max_blocks]
+                .view(arena.r_cap, arena.max_blocks),
+                k_pools=self.store.k_pools(g), v_pools=self.store.v_pools(g)))
+        return StepContext(
+            n_tokens=shape.n_tokens, n_rows=arena.n_cap if padded else shape.n_tokens,
+            n_req=shape.n_req, n_logits=shape.n_logits, m_rows=arena.m_cap if padded else shape.n_logits,
+            token_ids=d["token_ids"], positions=d["positions"], q_req=d["q_req"], cu_q=d["cu_q"],
+            seq_lens=d["seq_lens"], state_slots=d["state_slots"], logit_rows=d["logit_rows"],
+            groups=groups, state_pools=self.store.state_pools, dtype=self.dtype,
+            workspace=workspace or self.workspace, max_q_len=shape.max_q_len, max_seq_len=shape.max_seq_len,
+            decode_only=shape.max_q_len <= 1, host_q_lens=shape.q_lens, host_ctx_lens=shape.ctx_lens,
+            host_state_slots=shape.slots, exact=self.exact)
+
+    def run(self, arena: StepArena, shape: StepShape) -> torch.Tensor:
+        """Uploads the arena and runs the model eagerly.  Returns float32 logits [n_logits, vocab]."""
+        arena.upload()
+        ctx = self.context(arena, shape, padded=False)
+        return self.model.forward(ctx)
+
+    def step(self, slots: Sequence[int], ctx_lens: Sequence[int], q_lens: Sequence[int], tokens: Sequence[int],
+             logit_rows: Sequence[int]) -> torch.Tensor:
+        """The step function for callers that hold cache slots themselves (trace replay, tests)."""
+        arena = self.arena(len(tokens), len(slots), len(logit_rows))
+        shape = self.describe(arena, slots, ctx_lens, q_lens, tokens, logit_rows)
+        return self.run(arena, shape)

@@ -1,0 +1,216 @@
+"""Typed Python entry points of the HIP kernels.
+
+Each function checks on the host that operand shapes, strides, dtypes and
+devices are what the kernel and its grid assume, then launches on the current
+HIP stream.  Tensors are torch tensors used as plain device buffers; no torch
+operator computes anything here.
+"""
+
+from __future__ import annotations
+
+import ctypes
+from typing import Optional
+
+import torch
+
+from . import library
+
+F32, BF16 = 0, 1
+EPI_NONE, EPI_GELU, EPI_RESIDUAL = 0, 1, 2
+
+_ERRORS = {
+    -1: "unsupported dtype combination",
+    -2: "unsupported shape",
+    -3: "size beyond what the launch grid can hold",
+    -4: "null pointer",
+}
+
+
+class KernelError(RuntimeError):
+    pass
+
+
+def _dtype_code(t: torch.Tensor) -> int:
+    if t.dtype == torch.float32:
+        return F32
+    if t.dtype == torch.bfloat16:
+        return BF16
+    raise KernelError(f"kernels take float32 or bfloat16 buffers, got {t.dtype}")
+
+
+def _ptr(t: Optional[torch.Tensor]) -> ctypes.c_void_p:
+    return ctypes.c_void_p(0 if t is None else t.data_ptr())
+
+
+def _stream() -> ctypes.c_void_p:
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _check(rc: int, what: str) -> None:
+    if rc == 0:
+        return
+    if rc < 0:
+        raise KernelError(f"{what}: refused, {_ERRORS.get(rc, rc)}")
+    raise KernelError(f"{what}: HIP error {rc}")
+
+
+def _need(cond: bool, msg: str) -> None:
+    if not cond:
+        raise KernelError(msg)
+
+
+def _need_cuda(*tensors: Optional[torch.Tensor]) -> None:
+    for t in tensors:
+        if t is not None and not t.is_cuda:
+            raise KernelError("kernel operands must live on the GPU; there is no CPU path")
+
+
+def _need_i32(name: str, t: torch.Tensor, n: int) -> None:
+    _need(t.dtype == torch.int32 and t.is_contiguous() and t.numel() >= n,
+          f"{name} must be a contiguous int32 buffer of at least {n} entries")
+
+
+def embed(ids: torch.Tensor, positions: Optional[torch.Tensor], table: torch.Tensor,
+          pos_table: Optional[torch.Tensor], x: torch.Tensor, n_tokens: int) -> None:
+    """x[t] = table[ids[t]] (+ pos_table[positions[t]]), into the float32 residual stream."""
+    _need_cuda(ids, positions, table, pos_table, x)
+    width = table.shape[1]
+    _need(table.dim() == 2 and table.is_contiguous(), "embedding table must be dense [vocab, width]")
+    _need(x.dtype == torch.float32 and x.is_contiguous() and x.shape[1] == width and x.shape[0] >= n_tokens,
+          "residual stream must be dense float32 [>=n_tokens, width]")
+    _need_i32("ids", ids, n_tokens)
+    if pos_table is not None:
+        _need(pos_table.dtype == table.dtype and pos_table.is_contiguous() and pos_table.shape[1] == width,
+              "position table must match the token table's dtype and width")
+        _need(positions is not None, "positions are needed with a position table")
+        _need_i32("positions", positions, n_tokens)
+    rc = library.kernels().mgpt_embed(_ptr(ids), _ptr(positions), _ptr(table), _ptr(pos_table), _ptr(x),
+                                      n_tokens, width, _dtype_code(table), _stream())
+    _check(rc, "embed")
+
+
+def layer_norm(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor,
+               n_rows: int, eps: float, rows: Optional[torch.Tensor] = None) -> None:
+    """out[i] = LayerNorm(x[rows[i]] or x[i]); statistics in float32."""
+    _need_cuda(x, weight, bias, out, rows)
+    width = x.shape[1]
+    _need(x.dtype == torch.float32 and x.is_contiguous(), "LayerNorm input must be dense float32")
+    _need(weight.dtype == torch.float32 and weight.numel() == width, "LayerNorm weight must be float32 [width]")
+    _need(bias is None or (bias.dtype == torch.float32 and bias.numel() == width),
+          "LayerNorm bias must be float32 [width]")
+    _need(out.is_contiguous() and out.shape[1] == width and out.shape[0] >= n_rows, "LayerNorm output too small")
+    if rows is None:
+        _need(x.shape[0] >= n_rows, "LayerNorm input has fewer rows than asked for")
+    else:
+        _need_i32("rows", rows, n_rows)
+    rc = library.kernels().mgpt_layernorm(_ptr(x), _ptr(weight), _ptr(bias), _ptr(out), _ptr(rows), n_rows,
+                                          width, float(eps), _dtype_code(out), _stream())
+    _check(rc, "layer_norm")
+
+
+def linear_generic(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor,
+                   n_rows: int, epilogue: int = EPI_NONE) -> None:
+    """out[:n_rows] = a[:n_rows] @ w.T (+ bias), optional GELU, or added into a float32 out."""
+    _need_cuda(a, w, bias, out)
+    n_out, k_dim = w.shape
+    _need(w.is_contiguous(), "weight must be dense [out, in]")
+    _need(a.dim() == 2 and a.stride(1) == 1 and a.shape[1] == k_dim and a.shape[0] >= n_rows,
+          f"activation must be [>=n_rows, {k_dim}] with unit inner stride")
+    _need(out.dim() == 2 and out.stride(1) == 1 and out.shape[1] == n_out and out.shape[0] >= n_rows,
+          f"output must be [>=n_rows, {n_out}] with unit inner stride")
+    _need(k_dim % 16 == 0, f"inner size {k_dim} is not a multiple of 16")
+    _need(bias is None or (bias.dtype == torch.float32 and bias.numel() == n_out), "bias must be float32 [out]")
+    rc = library.kernels().mgpt_linear_generic(
+        _ptr(a), _dtype_code(a), a.stride(0), _ptr(w), _dtype_code(w), _ptr(bias), _ptr(out), _dtype_code(out),
+        out.stride(0), n_rows, n_out, k_dim, epilogue, _stream())
+    _check(rc, "linear_generic")
+
+
+def kv_write(qkv: torch.Tensor, k_off: int, v_off: int, k_pool: torch.Tensor, v_pool: torch.Tensor,
+             slot_mapping: torch.Tensor, n_tokens: int) -> None:
+    """Stores the new keys and values of n_tokens rows of qkv into their pages.
+
+    Pools are [num_pages, n_kv_head, page_size, head_dim]."""
+    _need_cuda(qkv, k_pool, v_pool, slot_mapping)
+    _need(k_pool.shape == v_pool.shape and k_pool.dim() == 4 and k_pool.is_contiguous() and v_pool.is_contiguous(),
+          "key and value pools must be dense [pages, kv_heads, page_size, head_dim]")
+    _, n_kv_head, page_size, head_dim = k_pool.shape
+    _need(qkv.dtype == k_pool.dtype == v_pool.dtype, "pools must have the activations' dtype")
+    _need(qkv.stride(1) == 1 and qkv.shape[0] >= n_tokens, "qkv rows must have unit inner stride")
+    width = n_kv_head * head_dim
+    _need(0 <= k_off and k_off + width <= qkv.shape[1] and 0 <= v_off and v_off + width <= qkv.shape[1],
+          "key/value columns lie outside the qkv buffer")
+    _need_i32("slot_mapping", slot_mapping, n_tokens)
+    rc = library.kernels().mgpt_kv_write(_ptr(qkv), _dtype_code(qkv), qkv.stride(0), k_off, v_off, _ptr(k_pool),
+                                         _ptr(v_pool), _ptr(slot_mapping), n_tokens, n_kv_head, head_dim,
+                                         page_size, _stream())
+    _check(rc, "kv_write")
+
+
+def _check_attention_args(q, out, k_pool, v_pool, block_tables, cu_q, seq_lens, q_req, n_tokens, n_req, n_head):
+    _need_cuda(q, out, k_pool, v_pool, block_tables, cu_q, seq_lens, q_req)
+    _need(k_pool.shape == v_pool.shape and k_pool.dim() == 4 and k_pool.is_contiguous() and v_pool.is_contiguous(),
+          "key and value pools must be dense [pages, kv_heads, page_size, head_dim]")
+    _, n_kv_head, page_size, head_dim = k_pool.shape
+    _need(q.dtype == out.dtype == k_pool.dtype == v_pool.dtype, "queries, output and pools must share a dtype")
+    _need(q.stride(1) == 1 and out.stride(1) == 1, "query and output rows must have unit inner stride")
+    _need(q.shape[0] >= n_tokens and out.shape[0] >= n_tokens, "query/output buffers have too few rows")
+    _need(q.shape[1] >= n_head * head_dim and out.shape[1] >= n_head * head_dim,
+          "query/output rows are narrower than n_head * head_dim")
+    _need(n_head % n_kv_head == 0, "n_head must be a multiple of the number of key/value heads")
+    _need(block_tables.dim() == 2 and block_tables.dtype == torch.int32 and block_tables.is_contiguous()
+          and block_tables.shape[0] >= n_req, "block_tables must be dense int32 [>=requests, max_blocks]")
+    _need_i32("cu_q", cu_q, n_req + 1)
+    _need_i32("seq_lens", seq_lens, n_req)
+    _need_i32("q_req", q_req, n_tokens)
+    return n_kv_head, page_size, head_dim
+
+
+def paged_attention_generic(q: torch.Tensor, out: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor,
+                            block_tables: torch.Tensor, cu_q: torch.Tensor, seq_lens: torch.Tensor,
+                            q_req: torch.Tensor, n_tokens: int, n_req: int, n_head: int, scale: float,
+                            window: int = 0, fast_exp: bool = False) -> None:
+    """Causal attention of the step's tokens over their requests' pages (any q_len, any dtype)."""
+    n_kv_head, page_size, head_dim = _check_attention_args(
+        q, out, k_pool, v_pool, block_tables, cu_q, seq_lens, q_req, n_tokens, n_req, n_head)
+    _need(head_dim <= 256, f"head size {head_dim} exceeds the kernel's limit of 256")
+    rc = library.kernels().mgpt_paged_attention_generic(
+        _ptr(q), q.stride(0), _ptr(out), out.stride(0), _ptr(k_pool), _ptr(v_pool), _ptr(block_tables),
+        block_tables.shape[1], _ptr(cu_q), _ptr(seq_lens), _ptr(q_req), n_tokens, n_head, n_kv_head, head_dim,
+        page_size, float(scale), int(window), _dtype_code(q), int(fast_exp), _stream())
+    _check(rc, "paged_attention_generic")
+
+
+def sample(logits: torch.Tensor, n_rows: int, real_vocab: int, temperature: torch.Tensor,
+           top_k: Optional[torch.Tensor], top_p: Optional[torch.Tensor], request_seed: Optional[torch.Tensor],
+           out_index: Optional[torch.Tensor], engine_seed: int, out_tokens: torch.Tensor) -> None:
+    """One token per row of float32 logits: argmax where temperature <= 0, else seeded sampling."""
+    _need_cuda(logits, temperature, top_k, top_p, request_seed, out_index, out_tokens)
+    _need(logits.dtype == torch.float32 and logits.dim() == 2 and logits.stride(1) == 1 and logits.shape[0] >= n_rows,
+          "logits must be float32 [>=n_rows, vocab] with unit inner stride")
+    vocab = logits.shape[1]
+    _need(0 < real_vocab <= vocab, "real_vocab must lie in 1..vocab")
+    _need(temperature.dtype == torch.float32 and temperature.numel() >= n_rows, "temperature must be float32 [rows]")
+    _need(top_k is None or (top_k.dtype == torch.int32 and top_k.numel() >= n_rows), "top_k must be int32 [rows]")
+    _need(top_p is None or (top_p.dtype == torch.float32 and top_p.numel() >= n_rows), "top_p must be float32 [rows]")
+    _need(request_seed is None or (request_seed.dtype in (torch.int64, torch.uint64) and request_seed.numel() >= n_rows),
+          "request_seed must be 64-bit [rows]")
+    _need(out_index is None or (out_index.dtype == torch.int32 and out_index.numel() >= n_rows),
+          "out_index must be int32 [rows]")
+    _need_i32("out_tokens", out_tokens, n_rows)
+    rc = library.kernels().mgpt_sample(_ptr(logits), logits.stride(0), n_rows, vocab, real_vocab,
+                                       _ptr(temperature), _ptr(top_k), _ptr(top_p), _ptr(request_seed),
+                                       _ptr(out_index), ctypes.c_ulonglong(engine_seed & (2**64 - 1)),
+                                       _ptr(out_tokens), _stream())
+    _check(rc, "sample")
+
+
+def linear_bf16(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor,
+                n_rows: int, epilogue: int) -> bool:
+    """bfloat16 MFMA matrix product.  Returns False when no MFMA kernel takes the shape."""
+    return False
+
+
+def attention_bf16(ctx, q, out, k_pool, v_pool, group, n_head: int, scale: float, window: int) -> bool:
+    """bfloat16 attention fast paths.  Returns False when none takes the case."""
+    return False

@@ -1,0 +1,83 @@
+"""Sequence mixers.  A mixer adds its output into the residual stream."""
+
+from __future__ import annotations
+
+from typing import Dict, Optional, Union
+
+import torch
+
+from ..ops import attention as attention_ops
+from ..ops import kernels
+from ..ops.linear import linear
+from .base import (CacheBinding, KVNeed, MATRIX, Part, StateNeed, StepContext, VECTOR, WeightRequest,
+                   register_mixer)
+from .positions import PositionEncoding
+
+
+class Mixer(Part):
+    category = "mixer"
+
+    def cache_need(self) -> Union[KVNeed, StateNeed, None]:
+        return None
+
+    def forward_add(self, ctx: StepContext, h: torch.Tensor, x: torch.Tensor, binding: CacheBinding,
+                    position: PositionEncoding) -> None:
+        """x[:n_rows] += mixer(h[:n_rows]); h is the normed input in the compute dtype, x the
+        float32 residual stream."""
+        raise NotImplementedError
+
+
+@register_mixer("paged_causal_attention")
+class PagedCausalAttention(Mixer):
+    """Multi-head causal self-attention over the paged cache.
+
+    qkv = h Wqkv^T (+ b); q = columns [0, H*D), k = the next Hkv*D, v = the last Hkv*D, head i of
+    each = columns i*D..(i+1)*D (reference: src/minigpt_infer/model.py:43,49-53).  New keys and
+    values are stored unscaled before attention reads everything up to and including them
+    (model.py:55-59).  S = q k^T * scale with scale = 1/sqrt(D) unless given (SDPA's default,
+    model.py:87); a query sees the keys of its own request at positions <= its own (and, with a
+    window, only the last `window` of them); softmax in float32; y = P v; heads concatenated
+    head-major; out = y Wproj^T (+ b) (model.py:89-90), added into the residual (model.py:113)."""
+
+    def __init__(self, width: int, n_head: int, head_dim: int, bias: bool, n_kv_head: Optional[int] = None,
+                 scale: Optional[float] = None, window: int = 0) -> None:
+        self.width, self.n_head, self.head_dim = int(width), int(n_head), int(head_dim)
+        self.n_kv_head = int(n_kv_head) if n_kv_head is not None else self.n_head
+        self.has_bias = bool(bias)
+        self.scale = float(scale) if scale is not None else self.head_dim ** -0.5
+        self.window = int(window)
+        if self.head_dim % 16 != 0 or self.head_dim > 256:
+            raise ValueError(f"head size {self.head_dim}: the kernels take multiples of 16 up to 256")
+        if self.n_head % self.n_kv_head != 0:
+            raise ValueError("n_head must be a multiple of n_kv_head")
+        self.q_width = self.n_head * self.head_dim
+        self.kv_width = self.n_kv_head * self.head_dim
+        self.qkv_weight = self.qkv_bias = self.proj_weight = self.proj_bias = None
+
+    def weight_requests(self) -> Dict[str, WeightRequest]:
+        total = self.q_width + 2 * self.kv_width
+        req = {"qkv_weight": WeightRequest((total, self.width), MATRIX),
+               "proj_weight": WeightRequest((self.width, self.q_width), MATRIX)}
+        if self.has_bias:
+            req["qkv_bias"] = WeightRequest((total,), VECTOR)
+            req["proj_bias"] = WeightRequest((self.width,), VECTOR)
+        return req
+
+    def cache_need(self) -> KVNeed:
+        return KVNeed(self.n_kv_head, self.head_dim, self.window)
+
+    def forward_add(self, ctx: StepContext, h: torch.Tensor, x: torch.Tensor, binding: CacheBinding,
+                    position: PositionEncoding) -> None:
+        n = ctx.n_rows
+        total = self.q_width + 2 * self.kv_width
+        qkv = ctx.workspace.get("qkv", n, total, ctx.dtype)
+        linear(ctx, h, self.qkv_weight, self.qkv_bias, qkv, n)
+        position.rotate(ctx, qkv[:, :self.q_width], qkv[:, self.q_width:self.q_width + self.kv_width], n)
+        group = ctx.groups[binding.group]
+        k_pool, v_pool = group.k_pools[binding.index], group.v_pools[binding.index]
+        if binding.writes:
+            kernels.kv_write(qkv, self.q_width, self.q_width + self.kv_width, k_pool, v_pool,
+                             group.slot_mapping, n)
+        y = ctx.workspace.get("attn_out", n, self.q_width, ctx.dtype)
+        attention_ops.paged_attention(ctx, qkv, y, k_pool, v_pool, group, self.n_head, self.scale, self.window)
+        linear(ctx, y, self.proj_weight, self.proj_bias, x, n, kernels.EPI_RESIDUAL)

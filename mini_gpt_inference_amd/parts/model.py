@@ -1,0 +1,174 @@
+"""A decoder as data (ModelSpec) and the object that runs it (DecoderModel).
+
+The specification lists the distinct layers and, separately, the order in which
+they run.  The order is a list of runs; a run names a layer and says where its
+mixer keeps its cache: in a cache of its own, or in the one an earlier run of
+the same step writes (then it only reads).  A layer may appear in several runs.
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Dict, List, Optional, Tuple
+
+import torch
+
+from . import block as _block  # noqa: F401  (registers the parts)
+from . import embedding as _embedding  # noqa: F401
+from . import feedforward as _feedforward  # noqa: F401
+from . import mixers as _mixers  # noqa: F401
+from . import norms as _norms  # noqa: F401
+from . import positions as _positions  # noqa: F401
+from .base import (ARRANGEMENTS, CacheBinding, EMBEDDINGS, FEED_FORWARDS, HEADS, KVNeed, MIXERS, NORMS,
+                   POSITIONS, Part, PartSpec, StateNeed, StepContext, WeightRequest)
+
+
+@dataclass(frozen=True)
+class LayerSpec:
+    arrangement: PartSpec
+    norm1: PartSpec
+    mixer: PartSpec
+    norm2: PartSpec
+    feed_forward: PartSpec
+
+
+@dataclass(frozen=True)
+class LayerRun:
+    layer: int                        # index into ModelSpec.layers
+    reads_cache_of: Optional[int] = None   # index of an earlier run whose cache this run reads instead of its own
+
+
+@dataclass(frozen=True)
+class ModelSpec:
+    width: int
+    vocab_size: int
+    embedding: PartSpec
+    position: PartSpec
+    layers: Tuple[LayerSpec, ...]
+    order: Tuple[LayerRun, ...]
+    final_norm: PartSpec
+    head: PartSpec
+    max_positions: Optional[int] = None
+
+
+@dataclass(frozen=True)
+class CacheGroupSpec:
+    """Runs whose mixers keep the same kind of pages share a page table and a pool geometry."""
+    n_kv_head: int
+    head_dim: int
+    window: int
+    n_pools: int       # caches (one per writing run) in the group
+
+
+@dataclass
+class CacheLayout:
+    groups: List[CacheGroupSpec]
+    state_numels: List[int]            # one entry per run that keeps per-request state
+    bindings: List[CacheBinding]       # one per run
+
+
+@dataclass
+class _Layer:
+    arrangement: Part
+    norm1: Part
+    mixer: Part
+    norm2: Part
+    feed_forward: Part
+
+
+class DecoderModel:
+    def __init__(self, spec: ModelSpec) -> None:
+        self.spec = spec
+        self.embedding = EMBEDDINGS.build(spec.embedding)
+        self.position = POSITIONS.build(spec.position)
+        self.layers: List[_Layer] = [
+            _Layer(ARRANGEMENTS.build(ls.arrangement), NORMS.build(ls.norm1), MIXERS.build(ls.mixer),
+                   NORMS.build(ls.norm2), FEED_FORWARDS.build(ls.feed_forward))
+            for ls in spec.layers
+        ]
+        self.final_norm = NORMS.build(spec.final_norm)
+        self.head = HEADS.build(spec.head)
+        for i, run in enumerate(spec.order):
+            if not (0 <= run.layer < len(self.layers)):
+                raise ValueError(f"run {i} names layer {run.layer}, but there are {len(self.layers)} layers")
+            if run.reads_cache_of is not None and not (0 <= run.reads_cache_of < i):
+                raise ValueError(f"run {i} can only read the cache of an earlier run, not {run.reads_cache_of}")
+        self.cache_layout = self._plan_cache()
+
+    # ------------------------------------------------------------------ weights
+    def _named_parts(self) -> List[Tuple[Part, PartSpec]]:
+        pairs = [(self.embedding, self.spec.embedding), (self.position, self.spec.position)]
+        for layer, ls in zip(self.layers, self.spec.layers):
+            pairs += [(layer.norm1, ls.norm1), (layer.mixer, ls.mixer), (layer.norm2, ls.norm2),
+                      (layer.feed_forward, ls.feed_forward)]
+        pairs += [(self.final_norm, self.spec.final_norm), (self.head, self.spec.head)]
+        return pairs
+
+    def weight_requests(self) -> Dict[str, WeightRequest]:
+        """Checkpoint tensor name -> shape and role, over all parts.  Two parts may name the same
+        tensor (a tied head); then shape and role must agree."""
+        wanted: Dict[str, WeightRequest] = {}
+        for part, spec in self._named_parts():
+            for local, req in part.weight_requests().items():
+                if local not in spec.weights:
+                    raise KeyError(f"{spec.kind}: no checkpoint name given for parameter {local!r}")
+                name = spec.weights[local]
+                if name in wanted and (wanted[name].shape != req.shape):
+                    raise ValueError(f"tensor {name} is asked for with shapes {wanted[name].shape} and {req.shape}")
+                if name not in wanted or req.role == "table":
+                    wanted[name] = req
+        return wanted
+
+    def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
+        for part, spec in self._named_parts():
+            part.bind({local: tensors[spec.weights[local]] for local in part.weight_requests()})
+
+    # ------------------------------------------------------------------ cache
+    def _plan_cache(self) -> CacheLayout:
+        groups: List[CacheGroupSpec] = []
+        keys: List[Tuple[int, int, int]] = []
+        state_numels: List[int] = []
+        bindings: List[CacheBinding] = []
+        for i, run in enumerate(self.spec.order):
+            need = self.layers[run.layer].mixer.cache_need()
+            if run.reads_cache_of is not None:
+                src = bindings[run.reads_cache_of]
+                src_need = self.layers[self.spec.order[run.reads_cache_of].layer].mixer.cache_need()
+                if need != src_need or src.kind != "kv":
+                    raise ValueError(f"run {i} cannot read the cache of run {run.reads_cache_of}: different needs")
+                bindings.append(CacheBinding("kv", src.group, src.index, writes=False))
+            elif isinstance(need, KVNeed):
+                key = (need.n_kv_head, need.head_dim, need.window)
+                if key not in keys:
+                    keys.append(key)
+                    groups.append(CacheGroupSpec(need.n_kv_head, need.head_dim, need.window, 0))
+                g = keys.index(key)
+                bindings.append(CacheBinding("kv", g, groups[g].n_pools, writes=True))
+                groups[g] = CacheGroupSpec(*key, groups[g].n_pools + 1)
+            elif isinstance(need, StateNeed):
+                bindings.append(CacheBinding("state", -1, len(state_numels), writes=True))
+                state_numels.append(int(need.numel))
+            else:
+                bindings.append(CacheBinding("none"))
+        return CacheLayout(groups, state_numels, bindings)
+
+    # ------------------------------------------------------------------ forward
+    def forward(self, ctx: StepContext) -> torch.Tensor:
+        """Runs the step's tokens through every run of the order and returns float32 logits
+        [m_rows, vocab] at ctx.logit_rows (reference: src/minigpt_infer/model.py:183-187, there for
+        the last position only)."""
+        n = ctx.n_rows
+        ws = ctx.workspace
+        x = ws.get("residual", n, self.spec.width, torch.float32)
+        self.embedding.forward(ctx, self.position, x)
+        for run, binding in zip(self.spec.order, self.cache_layout.bindings):
+            layer = self.layers[run.layer]
+            layer.arrangement.run(ctx, x, layer.norm1, layer.mixer, layer.norm2, layer.feed_forward, binding,
+                                  self.position)
+        m = ctx.m_rows
+        logits = ws.get("logits", m, self.spec.vocab_size, torch.float32)
+        if m:
+            hf = ws.get("final_normed", m, self.spec.width, ctx.dtype)
+            self.final_norm.forward(ctx, x, hf, m, rows=ctx.logit_rows)
+            self.head.forward(ctx, hf, logits, m)
+        return logits[:m]
