@@ -1,0 +1,202 @@
+"""LLMEngine: scheduler + cache + step function + sampler behind the reference's entry points
+(add_request / step / has_unfinished_requests / cancel_request,
+src/minigpt_infer/engine/engine.py:42-118), plus generate() and constructors from a model folder
+or from a configuration and a seed.
+"""
+
+from __future__ import annotations
+
+import shutil
+import tempfile
+from typing import Dict, List, Optional, Sequence, Union
+
+import numpy as np
+import torch
+
+from ..cache.kv_store import KVStore
+from ..cache.manager import CacheManager, GroupGeometry
+from ..config.engine_config import EngineConfig, SamplingParams
+from ..parts.base import Workspace
+from ..sampling.sampler import Sampler
+from ..weights.loader import load_model
+from ..weights.random_init import write_random_model
+from .request import Request, RequestOutput
+from .scheduler import Scheduler
+from .step import ModelRunner, StepArena, StepShape, _bucket
+
+_TORCH_DTYPES = {"bfloat16": torch.bfloat16, "float32": torch.float32}
+
+
+class _GraphedDecode:
+    """One captured HIP graph: a decode-only step (model + sampling) for up to `cap` requests.
+    The arena and the workspace are its own, so their addresses never change."""
+
+    def __init__(self, runner: ModelRunner, sampler: Sampler, cap: int) -> None:
+        self.runner, self.sampler, self.cap = runner, sampler, cap
+        self.arena = StepArena(cap, cap, cap, runner.n_groups, runner.max_blocks, runner.device)
+        self.workspace = Workspace(runner.device)
+        self.graph: Optional[torch.cuda.CUDAGraph] = None
+
+    def _launch(self, shape: StepShape) -> None:
+        ctx = self.runner.context(self.arena, shape, padded=True, workspace=self.workspace)
+        # launch geometry must not depend on this step's lengths: size it for the longest sequence
+        ctx.max_seq_len = self.runner.max_positions or ctx.max_seq_len
+        logits = self.runner.model.forward(ctx)
+        self.sampler.sample(logits, self.arena, self.cap)
+
+    def run(self, shape: StepShape) -> None:
+        self.arena.upload()
+        if self.graph is None:
+            # once eagerly, so that every workspace buffer exists before capture
+            self._launch(shape)
+            torch.cuda.synchronize()
+            self.workspace.frozen = True
+            graph = torch.cuda.CUDAGraph()
+            side = torch.cuda.Stream()
+            side.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(side):
+                graph.capture_begin()
+                self._launch(shape)
+                graph.capture_end()
+            torch.cuda.current_stream().wait_stream(side)
+            self.graph = graph
+            # the eager launch above already did this step's work (and wrote its keys and values);
+            # replaying it writes the same values again
+        self.graph.replay()
+
+
+class LLMEngine:
+    def __init__(self, model, config, engine_config: EngineConfig, device: str = "cuda") -> None:
+        self.model, self.config, self.engine_config = model, config, engine_config
+        self.device = torch.device(device)
+        self.dtype = _TORCH_DTYPES[engine_config.dtype]
+        layout = model.cache_layout
+        geometry = [GroupGeometry(engine_config.block_size, engine_config.num_blocks, g.window)
+                    for g in layout.groups]
+        self.cache = CacheManager(geometry, engine_config.max_batch_size)
+        self.store = KVStore(layout, geometry, engine_config.max_batch_size, self.dtype, self.device)
+        max_positions = model.spec.max_positions
+        self.runner = ModelRunner(model, self.cache, self.store, self.dtype, self.device, max_positions)
+        self.scheduler = Scheduler(
+            self.cache, engine_config.max_batch_size,
+            max(engine_config.max_num_batched_tokens, engine_config.max_batch_size),
+            engine_config.prefill_chunk, engine_config.mixed_batches,
+            max_positions if max_positions is not None else 2 ** 30)
+        self.sampler = Sampler(model.spec.vocab_size, engine_config.real_vocab_size, engine_config.seed)
+        self._ids: Dict[int, str] = {}        # scheduler id -> caller's request id
+        self._rids: Dict[str, int] = {}
+        self._graphs: Dict[int, _GraphedDecode] = {}
+        self._tmpdir: Optional[str] = None
+        self.num_graph_steps = 0
+        self.num_eager_steps = 0
+
+    # ------------------------------------------------------------------ constructors
+    @classmethod
+    def from_folder(cls, model_dir: str, engine_config: Optional[EngineConfig] = None,
+                    device: str = "cuda") -> "LLMEngine":
+        engine_config = engine_config or EngineConfig()
+        model, config, _ = load_model(model_dir, engine_config.dtype, device)
+        return cls(model, config, engine_config, device)
+
+    @classmethod
+    def from_random(cls, config, seed: int, engine_config: Optional[EngineConfig] = None,
+                    device: str = "cuda", std_scale: float = 1.0) -> "LLMEngine":
+        """Random weights: writes a model folder from (config, seed), then loads it like any other."""
+        tmp = tempfile.mkdtemp(prefix="mgpt_random_")
+        try:
+            write_random_model(tmp, config, seed, std_scale=std_scale)
+            return cls.from_folder(tmp, engine_config, device)
+        finally:
+            shutil.rmtree(tmp, ignore_errors=True)
+
+    # ------------------------------------------------------------------ requests
+    def add_request(self, request: Request) -> None:
+        if request.request_id in self._rids:
+            raise ValueError(f"request id {request.request_id!r} is already in use")
+        sp = request.sampling_params
+        vocab = self.model.spec.vocab_size
+        if any((t < 0 or t >= vocab) for t in request.prompt_token_ids):
+            raise ValueError(f"prompt token id outside 0..{vocab - 1}")
+        sid = self.scheduler.add_request(request.prompt_token_ids, sp.max_tokens, request.eot_token_id,
+                                         sp.temperature, sp.top_k, sp.top_p, sp.seed)
+        self._ids[sid] = request.request_id
+        self._rids[request.request_id] = sid
+
+    def has_unfinished_requests(self) -> bool:
+        return self.scheduler.has_work()
+
+    def cancel_request(self, request_id: str) -> bool:
+        sid = self._rids.get(request_id)
+        return False if sid is None else self.scheduler.cancel(sid)
+
+    # ------------------------------------------------------------------ stepping
+    def step(self) -> List[RequestOutput]:
+        n, r, m = self.scheduler.schedule()
+        if r == 0:
+            return []
+        decode_only = n == r
+        use_graph = decode_only and self.engine_config.use_graph and m == r
+        if use_graph:
+            cap = _bucket(r)
+            graphed = self._graphs.get(cap)
+            if graphed is None:
+                graphed = self._graphs[cap] = _GraphedDecode(self.runner, self.sampler, cap)
+            arena = graphed.arena
+        else:
+            arena = self.runner.arena(n, r, m)
+        self.scheduler.fill(arena)
+        _, ctx_lens, q_lens, _ = self.scheduler.entry_arrays()
+        slots = arena.h["state_slots"][:r]
+        shape = self.runner.shape_of(arena, n, r, m, q_lens.tolist(), ctx_lens.tolist(), slots.tolist())
+        if use_graph:
+            graphed.run(shape)
+            self.num_graph_steps += 1
+        else:
+            logits = self.runner.run(arena, shape)
+            if m:
+                self.sampler.sample(logits, arena, m)
+            self.num_eager_steps += 1
+        if m:
+            arena.tokens_host.copy_(arena.tokens_out, non_blocking=True)
+        torch.cuda.current_stream().synchronize()
+        tokens = arena.tokens_host.numpy()[:m]
+        outs = []
+        for sid, token, finished, reason in self.scheduler.commit(tokens):
+            rid = self._ids[sid]
+            outs.append(RequestOutput(rid, [token], finished, reason))
+        return outs
+
+    def generate(self, prompts: Sequence[Sequence[int]],
+                 sampling_params: Union[SamplingParams, Sequence[SamplingParams], None] = None,
+                 eot_token_id: Optional[int] = None) -> List[List[int]]:
+        """Runs the prompts to completion and returns the new token ids of each, in order."""
+        if sampling_params is None:
+            sampling_params = SamplingParams()
+        params = (list(sampling_params) if isinstance(sampling_params, (list, tuple))
+                  else [sampling_params] * len(prompts))
+        if len(params) != len(prompts):
+            raise ValueError("one SamplingParams per prompt, or one for all")
+        base = len(self._rids)
+        names = [f"generate-{base + i}" for i in range(len(prompts))]
+        got: Dict[str, List[int]] = {name: [] for name in names}
+        for name, prompt, sp in zip(names, prompts, params):
+            self.add_request(Request(name, list(prompt), sp, eot_token_id))
+        while self.has_unfinished_requests():
+            outs = self.step()
+            for out in outs:
+                if out.request_id in got:
+                    got[out.request_id].extend(out.new_token_ids)
+            if not outs and not self.scheduler.running:
+                raise RuntimeError("the scheduler cannot make progress: the waiting request does not fit")
+        return [got[name] for name in names]
+
+    # ------------------------------------------------------------------ counters
+    def stats(self) -> Dict[str, int]:
+        s = self.scheduler
+        return {
+            "num_preemptions": s.num_preemptions, "num_steps": s.num_steps,
+            "num_prompt_tokens": s.num_prompt_tokens, "num_decode_tokens": s.num_decode_tokens,
+            "free_blocks": self.cache.num_free_pages(0),
+            "allocated_blocks": self.cache.groups[0].num_pages - self.cache.num_free_pages(0),
+            "graph_steps": self.num_graph_steps, "eager_steps": self.num_eager_steps,
+        }

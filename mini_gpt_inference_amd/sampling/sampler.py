@@ -1,0 +1,25 @@
+"""Next-token choice on the device (csrc/hip/sampling.hip): greedy where temperature <= 0,
+otherwise temperature, top-k, top-p and a seeded draw."""
+
+from __future__ import annotations
+
+import torch
+
+from ..ops import kernels
+
+
+class Sampler:
+    def __init__(self, vocab_size: int, real_vocab_size=None, engine_seed: int = 0) -> None:
+        self.vocab_size = vocab_size
+        self.real_vocab = vocab_size if real_vocab_size is None else int(real_vocab_size)
+        if not (0 < self.real_vocab <= vocab_size):
+            raise ValueError("real_vocab_size must lie in 1..vocab_size")
+        self.engine_seed = int(engine_seed)
+
+    def sample(self, logits: torch.Tensor, arena, n_rows: int) -> torch.Tensor:
+        """Writes one token per logits row into arena.tokens_out, using the arena's per-row sampling
+        arrays.  Returns arena.tokens_out."""
+        d = arena.d
+        kernels.sample(logits, n_rows, self.real_vocab, d["temperature"], d["top_k"], d["top_p"], d["seeds"],
+                       d["out_index"], self.engine_seed, arena.tokens_out)
+        return arena.tokens_out
