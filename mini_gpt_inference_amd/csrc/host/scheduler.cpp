@@ -32,8 +32,9 @@ int Scheduler::add_request(const int* prompt, int n_prompt, int max_tokens, int 
   if (max_tokens <= 0 || top_k < 0 || !(top_p > 0.0f && top_p <= 1.0f)) return ERR_BAD_PARAMS;
   // src/minigpt_infer/engine/engine.py:73-88
   if (n_prompt + max_tokens > cfg_.max_positions) return ERR_TOO_LONG;
+  // the last sampled token is never fed back, so prompt + max_tokens - 1 tokens are cached at most
   for (int g = 0; g < cache_->num_groups(); ++g)
-    if (cache_->pages_needed(g, n_prompt + max_tokens) > cache_->group(g).num_pages)
+    if (cache_->pages_needed(g, n_prompt + max_tokens - 1) > cache_->group(g).num_pages)
       return ERR_NEVER_FITS;
   auto r = std::make_unique<Request>();
   r->id = (int)requests_.size();
@@ -94,20 +95,13 @@ void Scheduler::ensure_capacity_for_decode() {
     if (r.status != RUNNING) continue;  // preempted earlier in this pass
     if (r.num_tokens() - r.num_computed != 1) continue;  // still in its prompt: pages are held
     while (!cache_->reserve(r.slot, r.num_computed + 1)) {
-      Request* victim = nullptr;
-      for (auto it = running_.rbegin(); it != running_.rend(); ++it) {
-        if (*it != id) {
-          victim = get(*it);
-          break;
-        }
-      }
-      if (!victim) {
-        // Alone and still no room.  add_request refuses requests that the whole pool cannot
-        // hold, so this is unreachable with one group; with several it is a stall, not a loop.
-        preempt(r);
-        break;
-      }
-      preempt(*victim);
+      // Evict the newest running request.  The reference never evicts the one that asks
+      // (scheduler.py:78-82 picks the newest other one), which lets a newcomer push out an older
+      // request; here the asker itself goes when it is the newest.
+      Request& victim = *get(running_.back());
+      const bool self = victim.id == id;
+      preempt(victim);
+      if (self) break;
     }
   }
 }

@@ -1,0 +1,225 @@
+"""The scheduler's decisions (no GPU, no model): what the reference's tests pin
+(tests/test_scheduler.py:121-243, tests/test_paged.py:107-143) and what is new here: prompt
+portions under a token budget, mixed steps, and what happens when pages run out."""
+
+import random
+
+import numpy as np
+import pytest
+
+from mini_gpt_inference_amd.cache.manager import CacheManager, GroupGeometry
+from mini_gpt_inference_amd.engine.scheduler import FINISHED, RUNNING, WAITING, Scheduler, SchedulerError
+
+
+def make(num_pages, page_size, max_batch, budget=64, chunk=0, mixed=True, max_positions=1024):
+    cm = CacheManager([GroupGeometry(page_size, num_pages, 0)], max_batch)
+    return cm, Scheduler(cm, max_batch, budget, chunk, mixed, max_positions)
+
+
+def step(sched, token=lambda rid, idx: 100 + idx):
+    """Schedules one step and commits made-up tokens.  Returns (entries, outputs)."""
+    sched.schedule()
+    entries = sched.entries()
+    toks = [token(e.request, sched.info(e.request).output_len) for e in entries if e.sample]
+    outs = sched.commit(np.array(toks, dtype=np.int32))
+    return entries, outs
+
+
+def test_admits_up_to_max_batch_size():
+    cm, s = make(100, 4, max_batch=2, mixed=False)
+    for _ in range(3):
+        s.add_request(list(range(4)), 10)
+    n, r, m = s.schedule()
+    assert (n, r, m) == (8, 2, 2) and len(s.waiting) == 1 and len(s.running) == 2
+
+
+def test_decodes_when_nothing_is_admitted_and_prompts_go_first():
+    cm, s = make(100, 4, max_batch=2, mixed=False)
+    r0 = s.add_request(list(range(4)), 10)
+    ents, _ = step(s)
+    assert [(e.request, e.ctx, e.q_len, e.sample) for e in ents] == [(r0, 0, 4, True)]
+    ents, _ = step(s)
+    assert [(e.request, e.ctx, e.q_len) for e in ents] == [(r0, 4, 1)]
+    # a new arrival's prompt beats decoding of the running set (reference: prefill priority)
+    r1 = s.add_request(list(range(4)), 10)
+    ents, _ = step(s)
+    assert [e.request for e in ents] == [r1]
+
+
+def test_mixed_step_holds_decode_tokens_beside_a_prompt():
+    cm, s = make(100, 4, max_batch=4, mixed=True)
+    r0 = s.add_request(list(range(4)), 10)
+    step(s)
+    r1 = s.add_request(list(range(6)), 10)
+    ents, _ = step(s)
+    assert [(e.request, e.ctx, e.q_len, e.sample) for e in ents] == [(r0, 4, 1, True), (r1, 0, 6, True)]
+    assert s.num_decode_tokens == 1 and s.num_prompt_tokens == 10
+
+
+def test_head_of_line_blocking():
+    # reference tests/test_scheduler.py:159-168, with a head that fits the pool but not right now
+    cm, s = make(3, 4, max_batch=10, mixed=False)
+    first = s.add_request(list(range(8)), 2)   # 2 pages
+    step(s)
+    blocked = s.add_request(list(range(8)), 2)    # needs 2 pages, 1 free: waits
+    behind = s.add_request([1, 2], 2)             # would fit, but is behind it
+    ents, _ = step(s)
+    assert [e.request for e in ents] == [first]   # nothing admitted: the running request decodes
+    assert s.waiting == [blocked, behind]
+    # nothing running and the head does not fit: an empty step, as the reference's ([], False)
+    cm, s = make(3, 4, max_batch=10, mixed=False)
+    a = s.add_request(list(range(8)), 2)
+    slot = cm.acquire_slot()
+    cm.reserve(slot, 8)                           # someone else holds 2 of the 3 pages
+    assert s.schedule() == (0, 0, 0) and s.waiting == [a]
+
+
+def test_nothing_to_do_returns_an_empty_step():
+    cm, s = make(1, 4, max_batch=2, mixed=False, max_positions=16)
+    a = s.add_request(list(range(4)), 1)
+    step(s)
+    assert not s.has_work()
+    assert s.schedule() == (0, 0, 0)
+
+
+def test_prompt_portions_under_a_budget_and_a_chunk():
+    cm, s = make(100, 4, max_batch=4, budget=16, chunk=6, mixed=True)
+    a = s.add_request(list(range(20)), 3)
+    b = s.add_request(list(range(9)), 3)
+    ents, outs = step(s)
+    # a takes a chunk of 6, b a chunk of 6; neither is complete, nothing is sampled
+    assert [(e.request, e.ctx, e.q_len, e.sample) for e in ents] == [(a, 0, 6, False), (b, 0, 6, False)]
+    assert outs == [] and s.info(a).num_computed == 6
+    ents, outs = step(s)
+    assert [(e.request, e.ctx, e.q_len, e.sample) for e in ents] == [(a, 6, 6, False), (b, 6, 3, True)]
+    assert [o[0] for o in outs] == [b]
+    ents, _ = step(s)     # b decodes (1 token), a continues with a chunk
+    assert [(e.request, e.ctx, e.q_len, e.sample) for e in ents] == [(b, 9, 1, True), (a, 12, 6, False)]
+    ents, _ = step(s)
+    assert [(e.request, e.ctx, e.q_len, e.sample) for e in ents] == [(b, 10, 1, True), (a, 18, 2, True)]
+    # the budget cuts a portion short: 16 tokens a step
+    cm, s = make(100, 4, max_batch=4, budget=16, chunk=0, mixed=True)
+    a = s.add_request(list(range(20)), 2)
+    ents, _ = step(s)
+    assert [(e.ctx, e.q_len, e.sample) for e in ents] == [(0, 16, False)]
+    ents, _ = step(s)
+    assert [(e.ctx, e.q_len, e.sample) for e in ents] == [(16, 4, True)]
+
+
+def test_finish_on_length_and_on_eot_frees_in_the_same_step():
+    cm, s = make(10, 4, max_batch=4)
+    a = s.add_request([1, 2, 3], 2)
+    b = s.add_request([1, 2, 3], 30, eot=7)
+    _, outs = step(s, token=lambda rid, idx: 7 if rid == b and idx == 1 else 5)
+    assert outs == [(a, 5, False, None), (b, 5, False, None)]
+    _, outs = step(s, token=lambda rid, idx: 7 if rid == b and idx == 1 else 5)
+    # the eot token is appended and returned (reference engine.py:164,177-183)
+    assert outs == [(a, 5, True, "length"), (b, 7, True, "eot")]
+    assert s.output(b) == [5, 7] and s.info(a).status == FINISHED
+    assert cm.num_free_pages() == 10 and cm.num_free_slots == 4 and not s.has_work()
+
+
+def test_pages_run_out_newest_is_evicted_to_the_front_and_recomputed():
+    # reference tests/test_paged.py:107-143: page size 2, 4 pages, prompts of 2, 4 new tokens each
+    cm, s = make(4, 2, max_batch=2, mixed=True, max_positions=32)
+    a = s.add_request([1, 2], 4)
+    b = s.add_request([4, 5], 4)
+    log = []
+    seen = {}
+    for _ in range(40):
+        if not s.has_work():
+            break
+        ents, outs = step(s, token=lambda rid, idx: 10 * (rid + 1) + idx)
+        log.append([(e.request, e.ctx, e.q_len) for e in ents])
+        for rid, tok, fin, why in outs:
+            seen.setdefault(rid, []).append(tok)
+        assert cm.check() == 0
+    assert not s.has_work()
+    assert s.num_preemptions == 1
+    # each output index was sampled exactly once, also for the evicted request
+    assert seen[a] == [10, 11, 12, 13] and seen[b] == [20, 21, 22, 23]
+    assert cm.num_free_pages() == 4
+    # both prompts, then two decode steps for both (positions 2 and 3 share each one's second page)...
+    assert log[0] == [(a, 0, 2), (b, 0, 2)]
+    assert log[1] == [(a, 2, 1), (b, 2, 1)] and log[2] == [(a, 3, 1), (b, 3, 1)]
+    # ...then both need a third page (position 4): a (older) keeps going, b (newest) is evicted
+    evicted_at = next(i for i, ents in enumerate(log) if [e[0] for e in ents] == [a])
+    assert log[evicted_at] == [(a, 4, 1)]
+    # when a is done, b comes back as one portion of prompt + outputs, from position 0
+    back = next(ents for ents in log[evicted_at:] if ents and ents[0][0] == b)
+    assert back == [(b, 0, 2 + 3)]       # its prompt and the three tokens it had sampled
+
+
+def test_evicted_request_goes_to_the_front_of_waiting():
+    # after reference tests/test_scheduler.py:185-207 (there: 2 pages, which a single request of
+    # this length could never finish in; such a request is refused here)
+    cm, s = make(3, 4, max_batch=2, mixed=False, max_positions=64)
+    old = s.add_request(list(range(4)), 5)
+    new = s.add_request(list(range(4)), 5)
+    later = s.add_request(list(range(4)), 5)     # not admitted: both places are taken
+    step(s)                                       # both prompts (one page each)
+    assert s.running == [old, new] and cm.num_free_pages() == 1
+    ents, _ = step(s)                             # both at position 4: a second page each, one is free
+    assert [e.request for e in ents] == [old]
+    assert s.running == [old] and s.waiting == [new, later] and s.num_preemptions == 1
+    assert len(cm.table(s.info(old).slot)) == 2   # the survivor got the freed page
+    assert s.info(new).num_computed == 0 and s.info(new).output_len == 1 and s.info(new).status == WAITING
+
+
+def test_requests_that_can_never_run_are_refused():
+    cm, s = make(4, 4, max_batch=2, max_positions=32)
+    with pytest.raises(SchedulerError, match="empty"):
+        s.add_request([], 4)
+    with pytest.raises(SchedulerError, match="block_size"):       # reference engine.py:83-88
+        s.add_request(list(range(30)), 3)
+    with pytest.raises(SchedulerError, match="whole pool"):
+        s.add_request(list(range(10)), 8)                          # 17 cached tokens > 4 pages of 4
+    assert s.add_request(list(range(10)), 7) >= 0                  # 16 cached tokens: exactly the pool
+
+
+def test_cancel():
+    cm, s = make(10, 4, max_batch=1)
+    r0 = s.add_request(list(range(4)), 5)
+    r1 = s.add_request(list(range(4)), 5)
+    step(s)
+    assert s.running == [r0] and s.waiting == [r1] and cm.num_free_pages() == 9
+    assert s.cancel(r1) and s.waiting == [] and cm.num_free_pages() == 9
+    assert s.cancel(r0) and s.running == [] and cm.num_free_pages() == 10
+    assert s.info(r0).finish_reason == "cancelled" and s.info(r0).status == FINISHED
+    assert not s.cancel(r0) and not s.cancel(12345)
+
+
+@pytest.mark.parametrize("mixed,chunk", [(True, 0), (True, 5), (False, 0), (False, 7)])
+def test_random_load_keeps_every_invariant(mixed, chunk):
+    rng = random.Random(1234 + chunk)
+    cm, s = make(24, 4, max_batch=5, budget=32, chunk=chunk, mixed=mixed, max_positions=64)
+    want, got, arrivals = {}, {}, 0
+    for it in range(2000):
+        if arrivals < 40 and rng.random() < 0.3:
+            prompt = [rng.randrange(50) for _ in range(rng.randint(1, 30))]
+            rid = s.add_request(prompt, rng.randint(1, 12))
+            want[rid] = None
+            got[rid] = []
+            arrivals += 1
+        if not s.has_work():
+            if arrivals >= 40:
+                break
+            continue
+        n, r, m = s.schedule()
+        ents = s.entries()
+        assert n <= 32 and r <= 5 and len({e.request for e in ents}) == len(ents)
+        for e in ents:
+            info = s.info(e.request)
+            assert info.status == RUNNING
+            assert e.ctx == info.num_computed                       # next position == tokens cached
+            total = info.prompt_len + info.output_len
+            assert 1 <= e.q_len <= total - e.ctx and e.sample == (e.ctx + e.q_len == total)
+            assert len(cm.table(info.slot)) * 4 >= e.ctx + e.q_len   # pages are there before the step
+        outs = s.commit(np.array([len(got[e.request]) for e in ents if e.sample], dtype=np.int32))
+        for rid, tok, fin, why in outs:
+            assert tok == len(got[rid])          # each output index exactly once, in order
+            got[rid].append(tok)
+        assert cm.check() == 0
+    assert not s.has_work() and arrivals == 40
+    assert all(s.info(rid).status == FINISHED and s.info(rid).finish_reason == "length" for rid in want)
+    assert cm.num_free_pages() == 24 and cm.num_free_slots == 5
