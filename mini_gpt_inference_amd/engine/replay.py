@@ -58,6 +58,7 @@ class TraceReplayer:
                     raise TraceError(f"step {step}: more live requests than the {self.cache.max_requests} slots")
                 self.live[rid] = [slot, 0]
             slot, cached = self.live[rid]
+            self.runner.check_positions([cached], [len(toks)])
             if not self.cache.reserve(slot, cached + len(toks)):
                 raise TraceError(f"step {step}: request {rid!r} needs cache for {cached + len(toks)} tokens, "
                                  f"but the pool of {self.num_pages} pages of {self.page_size} tokens is used up")

@@ -117,6 +117,7 @@ class ModelRunner:
         """Fills the arena for requests given by their cache slots: request i brings q_lens[i] tokens
         (its part of the flat `tokens`) on top of ctx_lens[i] cached ones.  logit_rows index `tokens`."""
         h = arena.h
+        self.check_positions(ctx_lens, q_lens)
         n = self.cache.build_step(slots, ctx_lens, q_lens, arena.n_cap, arena.r_cap, arena.max_blocks,
                                   h["positions"], h["q_req"], h["cu_q"], h["seq_lens"], h["slot_mapping"],
                                   h["block_tables"])
@@ -134,17 +135,22 @@ class ModelRunner:
         h["logit_rows"][m:] = 0
         return self.shape_of(arena, n, r, m, list(q_lens), list(ctx_lens), list(slots))
 
+    def check_positions(self, ctx_lens: Sequence[int], q_lens: Sequence[int]) -> int:
+        """The longest sequence after the step; refuses positions the model does not have
+        (reference: src/minigpt_infer/model.py:177-182)."""
+        max_seq = max((c + q for c, q in zip(ctx_lens, q_lens)), default=0)
+        if self.max_positions is not None and max_seq > self.max_positions:
+            raise ValueError(f"position {max_seq - 1} >= block_size={self.max_positions}: "
+                             "the position table has no such row")
+        return max_seq
+
     def shape_of(self, arena: StepArena, n: int, r: int, m: int, q_lens: List[int], ctx_lens: List[int],
                  slots: List[int]) -> StepShape:
         h = arena.h
         ids = h["token_ids"][:n]
         if n and (ids.min() < 0 or ids.max() >= self.vocab_size):
             raise ValueError(f"token id outside 0..{self.vocab_size - 1}")
-        max_seq = max((c + q for c, q in zip(ctx_lens, q_lens)), default=0)
-        if self.max_positions is not None and max_seq > self.max_positions:
-            # src/minigpt_infer/model.py:177-182
-            raise ValueError(f"position {max_seq - 1} >= block_size={self.max_positions}: "
-                             "the position table has no such row")
+        max_seq = self.check_positions(ctx_lens, q_lens)
         return StepShape(n, r, m, max(q_lens, default=0), max_seq, q_lens, ctx_lens, slots)
 
     # ------------------------------------------------------------------ running

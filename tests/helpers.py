@@ -59,3 +59,123 @@ def assert_close(got, want, dtype: str, what: str = "") -> None:
 
 def random_ids(rng: np.random.Generator, vocab: int, n: int):
     return rng.integers(0, vocab, n).tolist()
+
+
+# ----------------------------------------------------------------------------- trace plans
+class TracePlan:
+    """Steps of a trace in bin/trace_run's JSON form, plus the bookkeeping to put the logits that
+    come back into one [length, vocab] array per request."""
+
+    def __init__(self) -> None:
+        self.steps = []        # JSON records
+        self.wanted = {}       # step -> [(request, position)] in file order
+        self._fed = {}         # request -> tokens fed so far
+        self._live = {}        # request -> final length (for the pool size)
+        self.max_tokens = 64
+        self._live_history = []   # per step: final lengths of the requests live during it
+
+    def add_step(self, entries, end=()):
+        """entries: [(request id, tokens, final length of the request)]; every position is wanted."""
+        step = len(self.steps)
+        rec = {"step": step, "entries": [], "end": list(end)}
+        rows = []
+        for rid, toks, final_len in entries:
+            start = self._fed.get(rid, 0)
+            self._live[rid] = final_len
+            rec["entries"].append({"id": rid, "tokens": list(toks), "want": list(range(len(toks)))})
+            rows += [(rid, start + i) for i in range(len(toks))]
+            self._fed[rid] = start + len(toks)
+        self.max_tokens = max(self.max_tokens, sum(-(-n // 64) * 64 for n in self._live.values()))
+        self._live_history.append(list(self._live.values()))
+        for rid in end:
+            self._live.pop(rid, None)
+        self.steps.append(rec)
+        self.wanted[step] = rows
+
+    def tight_tokens(self, page_size):
+        """The smallest pool, in tokens, that holds the live requests of every step."""
+        return max(sum(-(-n // page_size) * page_size for n in lens) for lens in self._live_history)
+
+    def assemble(self, outputs, lengths, vocab):
+        """outputs: step -> array [wanted, vocab].  Returns request -> [length, vocab]."""
+        res = {rid: np.full((n, vocab), np.nan, dtype=np.float64) for rid, n in lengths.items()}
+        for step, rows in self.wanted.items():
+            out = np.asarray(outputs[step], dtype=np.float64).reshape(len(rows), vocab)
+            for (rid, pos), row in zip(rows, out):
+                res[rid][pos] = row
+        return res
+
+
+def plan_whole(reqs):
+    """Each request alone and whole, in one step."""
+    plan = TracePlan()
+    for rid, ids in reqs.items():
+        plan.add_step([(rid, ids, len(ids))], end=[rid])
+    return plan
+
+
+def plan_tail(reqs, tail=32):
+    """Most of it in one step, the last `tail` tokens one by one."""
+    plan = TracePlan()
+    for rid, ids in reqs.items():
+        head = max(len(ids) - tail, 0)
+        if head:
+            plan.add_step([(rid, ids[:head], len(ids))])
+        for i in range(head, len(ids)):
+            plan.add_step([(rid, ids[i:i + 1], len(ids))], end=[rid] if i == len(ids) - 1 else [])
+    return plan
+
+
+def plan_portions(reqs, rng):
+    """Portions of changing size, down to two tokens."""
+    plan = TracePlan()
+    sizes = [2, 7, 3, 16, 2, 5, 17, 33, 4]
+    k = 0
+    for rid, ids in reqs.items():
+        pos = 0
+        while pos < len(ids):
+            q = min(sizes[k % len(sizes)], len(ids) - pos)
+            k += 1
+            plan.add_step([(rid, ids[pos:pos + q], len(ids))], end=[rid] if pos + q == len(ids) else [])
+            pos += q
+    return plan
+
+
+def plan_mixed(reqs, rng, max_live=4, tail=32):
+    """Up to max_live live requests: portions of some beside single decoded tokens of others; a
+    request is now and then left out of a step; finished ones give their pages to later ones."""
+    plan = TracePlan()
+    queue = list(reqs.items())
+    live = {}     # rid -> position
+    while queue or live:
+        while queue and len(live) < max_live:
+            rid, _ = queue.pop(0)
+            live[rid] = 0
+        entries, end = [], []
+        for rid in list(live):
+            ids, pos = reqs[rid], live[rid]
+            if len(live) > 1 and rng.random() < 0.2:
+                continue       # left out of this step
+            remaining = len(ids) - pos
+            q = 1 if remaining <= tail else int(min(remaining - tail, rng.integers(2, 14)))
+            entries.append((rid, ids[pos:pos + q], len(ids)))
+            live[rid] = pos + q
+            if live[rid] == len(ids):
+                end.append(rid)
+                del live[rid]
+        if entries:
+            plan.add_step(entries, end)
+    return plan
+
+
+PLANS = {"whole": lambda reqs, rng: plan_whole(reqs), "tail": lambda reqs, rng: plan_tail(reqs),
+         "portions": plan_portions, "mixed": plan_mixed}
+
+
+def run_plan_in_process(replayer, plan):
+    outputs = {}
+    for rec in plan.steps:
+        logits = replayer.run_step(rec)
+        if logits is not None:
+            outputs[rec["step"]] = logits.cpu().numpy()
+    return outputs

@@ -1,0 +1,210 @@
+"""Trace replay against the plain implementation: the same requests whole, with the last 32
+tokens one by one, in portions of changing size, and mixed with page reuse; in 32-bit and in
+bfloat16; through the replay class and through bin/trace_run itself."""
+
+import json
+import os
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+import helpers
+import plain_gpt as P
+from mini_gpt_inference_amd.engine.replay import TraceError, TraceReplayer
+
+pytestmark = pytest.mark.gpu
+
+LENGTHS = {"A": [5, 17, 30, 64, 41, 23], "B": [1, 9, 33, 64, 100, 128]}
+
+
+def _requests(name, rng):
+    cfg = helpers.CONFIGS[name]
+    return {f"r{i}": helpers.random_ids(rng, cfg.vocab_size, n) for i, n in enumerate(LENGTHS[name])}
+
+
+_plain_cache = {}
+
+
+def _plain_logits(folder, name, reqs):
+    key = (name, tuple(map(tuple, reqs.values())))
+    if key not in _plain_cache:
+        cfg, w = P.read_model_folder(folder)
+        _plain_cache[key] = {rid: P.plain_forward(w, cfg, ids).numpy() for rid, ids in reqs.items()}
+    return _plain_cache[key]
+
+
+@pytest.mark.parametrize("page_size", [16, 4])
+@pytest.mark.parametrize("way", ["whole", "tail", "portions", "mixed"])
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_every_way_of_cutting_matches_the_plain_implementation(model_folders, name, dtype, way, page_size):
+    rng = np.random.default_rng(11)
+    reqs = _requests(name, rng)
+    want = _plain_logits(model_folders[name], name, reqs)
+    plan = helpers.PLANS[way](reqs, np.random.default_rng(5))
+    # the pool holds just what the live requests need, so freed pages are used again;
+    # it starts as NaN, so a read of a slot nobody wrote shows
+    replayer = TraceReplayer(model_folders[name], dtype, plan.tight_tokens(page_size), page_size=page_size,
+                             poison=True)
+    got = plan.assemble(helpers.run_plan_in_process(replayer, plan), {r: len(t) for r, t in reqs.items()},
+                        helpers.CONFIGS[name].vocab_size)
+    for rid in reqs:
+        helpers.assert_close(got[rid], want[rid], dtype, f"{name} {dtype} {way} {rid}")
+    assert replayer.cache.check() == 0
+    assert replayer.cache.num_free_pages() == replayer.num_pages and not replayer.live
+    if way == "mixed":
+        total = sum(-(-len(t) // page_size) for t in reqs.values())
+        assert total > replayer.num_pages, "the pool is so large that no page was used twice"
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_cuts_agree_with_each_other_bit_for_bit_in_32_bit(model_folders, dtype):
+    """On the 32-bit path the order of every sum depends only on a token's position, so all ways of
+    cutting give identical logits, not merely close ones."""
+    rng = np.random.default_rng(3)
+    reqs = _requests("A", rng)
+    results = []
+    for way in ("whole", "tail", "portions", "mixed"):
+        plan = helpers.PLANS[way](reqs, np.random.default_rng(9))
+        replayer = TraceReplayer(model_folders["A"], dtype, plan.max_tokens, poison=True)
+        results.append(plan.assemble(helpers.run_plan_in_process(replayer, plan),
+                                     {r: len(t) for r, t in reqs.items()}, helpers.CONFIGS["A"].vocab_size))
+    for other in results[1:]:
+        for rid in reqs:
+            if dtype == "float32":
+                assert np.array_equal(results[0][rid], other[rid])
+            else:
+                helpers.assert_close(other[rid], results[0][rid], dtype, rid)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_trace_run_program(model_folders, tmp_path, dtype):
+    """bin/trace_run itself: all four ways in one session, files and `done` lines as specified."""
+    name = "B"
+    rng = np.random.default_rng(21)
+    cfg = helpers.CONFIGS[name]
+    reqs = {f"q{i}": helpers.random_ids(rng, cfg.vocab_size, n) for i, n in enumerate([3, 40, 77, 128, 65])}
+    want = _plain_logits(model_folders[name], name, reqs)
+    plans = [helpers.PLANS[w](reqs, np.random.default_rng(2)) for w in ("whole", "tail", "portions", "mixed")]
+    lines, offsets, base = [], [], 0
+    for plan in plans:
+        offsets.append(base)
+        for rec in plan.steps:
+            rec = dict(rec, step=rec["step"] + base)
+            lines.append(json.dumps(rec))
+        base += len(plan.steps)
+    out = tmp_path / "out"
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    proc = subprocess.run([os.path.join(root, "bin", "trace_run"), "--model", model_folders[name], "--dtype", dtype,
+                           "--out", str(out), "--max-tokens", str(max(p.max_tokens for p in plans))],
+                          input="\n".join(lines) + "\n", text=True, capture_output=True, timeout=300)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    assert proc.stdout.split("\n")[:3] == ["done 0", "done 1", "done 2"]
+    assert proc.stdout.count("done ") == base
+    for plan, off in zip(plans, offsets):
+        outputs = {}
+        for step in plan.wanted:
+            raw = np.fromfile(out / f"{step + off}.f32", dtype="<f4")
+            assert raw.size == len(plan.wanted[step]) * cfg.vocab_size
+            outputs[step] = raw
+        got = plan.assemble(outputs, {r: len(t) for r, t in reqs.items()}, cfg.vocab_size)
+        for rid in reqs:
+            helpers.assert_close(got[rid], want[rid], dtype, f"trace_run {dtype} {rid}")
+
+
+def test_trace_run_reports_a_pool_that_is_too_small(model_folders, tmp_path):
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    rec = {"step": 0, "entries": [{"id": "a", "tokens": list(range(1, 60)), "want": []},
+                                  {"id": "b", "tokens": list(range(1, 60)), "want": []}], "end": []}
+    proc = subprocess.run([os.path.join(root, "bin", "trace_run"), "--model", model_folders["A"], "--dtype", "float32",
+                           "--out", str(tmp_path / "o"), "--max-tokens", "64"],
+                          input=json.dumps(rec) + "\n", text=True, capture_output=True, timeout=300)
+    assert proc.returncode == 1 and "used up" in proc.stderr and "done 0" not in proc.stdout
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_want_may_be_empty_or_partial_and_steps_without_logits_write_no_file(model_folders, dtype):
+    cfg = helpers.CONFIGS["A"]
+    ids = helpers.random_ids(np.random.default_rng(0), cfg.vocab_size, 40)
+    pcfg, w = P.read_model_folder(model_folders["A"])
+    want = P.plain_forward(w, pcfg, ids).numpy()
+    rep = TraceReplayer(model_folders["A"], dtype, 64, poison=True)
+    assert rep.run_step({"step": 0, "entries": [{"id": "x", "tokens": ids[:25], "want": []}], "end": []}) is None
+    got = rep.run_step({"step": 1, "entries": [{"id": "x", "tokens": ids[25:], "want": [14, 0]}], "end": ["x"]})
+    helpers.assert_close(got, want[[39, 25]], dtype, "partial want")
+    with pytest.raises(TraceError, match="outside"):
+        rep.run_step({"step": 2, "entries": [{"id": "y", "tokens": [1, 2], "want": [2]}], "end": []})
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_long_decoding_and_first_tokens(model_folders, dtype):
+    """One token at a time from the very first token to the last position the model has."""
+    cfg = helpers.CONFIGS["B"]
+    ids = helpers.random_ids(np.random.default_rng(8), cfg.vocab_size, cfg.block_size)
+    pcfg, w = P.read_model_folder(model_folders["B"])
+    want = P.plain_forward(w, pcfg, ids).numpy()
+    rep = TraceReplayer(model_folders["B"], dtype, cfg.block_size + 8, page_size=8, poison=True)
+    rows = [rep.run_step({"step": i, "entries": [{"id": "x", "tokens": [t], "want": [0]}], "end": []}).cpu().numpy()[0]
+            for i, t in enumerate(ids)]
+    helpers.assert_close(np.stack(rows), want, dtype, "token by token")
+    with pytest.raises(ValueError, match="block_size"):       # reference tests/test_cache.py:147-158
+        rep.run_step({"step": 999, "entries": [{"id": "x", "tokens": [1], "want": [0]}], "end": []})
+
+
+def _far_key_edit(tensors):
+    """Makes the last query of the LONG model look mostly at one far key whose value is the
+    opposite of its own.  Queries and keys share one enlarged projection that reads the first 40
+    channels, values read the last 8 (enlarged too); token 59's embedding is token 60's with the
+    last 8 channels negated, which leaves LayerNorm's statistics almost alone.  So 60's query
+    scores as high with 59's key as with its own, among hundreds of others, and 59's value
+    cancels 60's.  Positions are made faint so that a token looks alike wherever it stands."""
+    c, cut = 48, 40
+    qkv = tensors["blocks.0.attn.qkv.weight"].float()
+    qkv[:c] *= 2.5
+    qkv[:c, cut:] = 0
+    qkv[c:2 * c] = qkv[:c]
+    qkv[2 * c:, :cut] = 0
+    qkv[2 * c:] *= 4.0
+    tensors["blocks.0.attn.qkv.weight"] = qkv.to(torch.bfloat16)
+    bias = tensors["blocks.0.attn.qkv.bias"].float()
+    bias[c:2 * c] = bias[:c]
+    tensors["blocks.0.attn.qkv.bias"] = bias.to(torch.bfloat16)
+    emb = tensors["tok_emb.weight"].float()
+    emb[59] = emb[60]
+    emb[59, cut:] = -emb[60, cut:]
+    tensors["tok_emb.weight"] = emb.to(torch.bfloat16)
+    tensors["pos_emb.weight"] = (tensors["pos_emb.weight"].float() * 0.05).to(torch.bfloat16)
+
+
+@pytest.mark.parametrize("far", [3, 15, 16, 255, 256, 447])
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_far_key_among_hundreds_decides_the_result(tmp_path, dtype, far):
+    folder = helpers.write_model(str(tmp_path / "long"), "LONG", edit=_far_key_edit)
+    cfg = helpers.CONFIGS["LONG"]
+    rng = np.random.default_rng(far)
+    n = 600
+    ids = rng.integers(0, 59, n).tolist()     # tokens 59 and 60 appear only where they are put
+    ids[far] = 59
+    ids[-1] = 60
+    pcfg, w = P.read_model_folder(folder)
+    # the construction works: in the plain implementation the last query puts most weight on `far`
+    x = P.plain_embed(torch.tensor(ids), w["tok_emb.weight"], w["pos_emb.weight"])
+    h = P.plain_layer_norm(x, w["blocks.0.ln1.weight"], w["blocks.0.ln1.bias"], cfg.layer_norm_eps)
+    q, k, v = P.plain_split_heads(P.plain_linear(h, w["blocks.0.attn.qkv.weight"], w["blocks.0.attn.qkv.bias"]), 1)
+    probs = torch.softmax((q[0, -1] @ k[0].t()) / 48 ** 0.5, -1)
+    assert probs[far] > 0.2 and probs[far] > probs[-1], (probs[far].item(), probs[-1].item())
+    want = P.plain_forward(w, pcfg, ids).numpy()
+    rep = TraceReplayer(folder, dtype, 640, poison=True)
+    rep.run_step({"step": 0, "entries": [{"id": "x", "tokens": ids[:-40], "want": []}], "end": []})
+    got = rep.run_step({"step": 1, "entries": [{"id": "x", "tokens": ids[-40:-1], "want": list(range(39))}], "end": []})
+    helpers.assert_close(got, want[-40:-1], dtype, "portion over a long cache")
+    got = rep.run_step({"step": 2, "entries": [{"id": "x", "tokens": ids[-1:], "want": [0]}], "end": ["x"]})
+    helpers.assert_close(got, want[-1:], dtype, f"decode with the deciding key at {far}")
+    # and the far key really decides: with another token there the logits move a lot
+    other = list(ids)
+    other[far] = 7
+    moved = np.abs(P.plain_forward(w, pcfg, other).numpy()[-1] - want[-1]).max()
+    assert moved > 10 * helpers.TOL[dtype] * max(1.0, np.abs(want[-1]).max())
