@@ -1,0 +1,167 @@
+"""Decode and prefill throughput of the engine on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+A step is one decode step of the engine (scheduler, one step of the model from the cache,
+sampling, tokens back on the host).  The default run has the layer sizes of the reference's
+50.9M model (n_layer 8, n_embd 512, n_head 8, vocabulary 50304, 1024 positions, biases) with
+random weights in bfloat16, a batch of 8 requests with 128-token random prompts, KV pages of 16
+tokens.  It prints one JSON line; `value` is decoded tokens per second.  Beside it: the
+prefill of 2,048 tokens (2 prompts of 1,024) as one step, the decode step's bytes against the
+HBM peak, and decode throughput at batch 1 and 64.
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import sys
+import time
+
+HBM_PEAK_GBS = 8000.0                      # MI355X HBM3E
+MFMA_PEAK = {"bfloat16": 2.5e15, "float32": 157.3e12}   # dense, per second
+REFERENCE_DECODE_B8 = 1671.8               # tok/s, the reference's own figure (Tesla T4, fp16, batch 8)
+
+
+def build_engine(args, batch, dtype):
+    from mini_gpt_inference_amd import EngineConfig, GPTConfig
+    from mini_gpt_inference_amd.engine.llm_engine import LLMEngine
+
+    cfg = GPTConfig("gpt2-mini", n_layer=args.layers, n_embd=args.width, n_head=args.heads,
+                    vocab_size=args.vocab, block_size=args.positions, bias=True, layer_norm_eps=1e-5)
+    pages = batch * (-(-args.positions // args.kv_block)) + 8
+    ecfg = EngineConfig(block_size=args.kv_block, num_blocks=pages, max_batch_size=max(batch, 2),
+                        max_num_batched_tokens=max(4096, batch * args.prompt), dtype=dtype,
+                        use_graph=not args.no_graph)
+    return LLMEngine.from_random(cfg, seed=0, engine_config=ecfg), cfg
+
+
+def decode_run(args, batch, steps, warmup, dtype):
+    """Returns (seconds for `steps` decode steps, mean context length during them, engine, cfg)."""
+    import numpy as np
+    import torch
+
+    from mini_gpt_inference_amd import Request, SamplingParams
+
+    engine, cfg = build_engine(args, batch, dtype)
+    rng = np.random.default_rng(0)
+    budget = steps + warmup + 2
+    assert args.prompt + budget <= cfg.block_size, "prompt + decode steps exceed the model's positions"
+    for i in range(batch):
+        engine.add_request(Request(f"b{i}", rng.integers(0, cfg.vocab_size, args.prompt).tolist(),
+                                   SamplingParams(max_tokens=budget, temperature=0.0)))
+    while engine.scheduler.num_decode_tokens == 0:      # prompts, untimed
+        engine.step()
+    for _ in range(warmup):
+        engine.step()
+    torch.cuda.synchronize()
+    start_ctx = args.prompt + 1 + warmup
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        outs = engine.step()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    assert len(outs) == batch, "a request dropped out of the timed decode steps"
+    mean_ctx = start_ctx + (steps - 1) / 2.0 + 1     # keys read per request and step, own token included
+    return elapsed, mean_ctx, engine, cfg
+
+
+def decode_bytes(cfg, batch, mean_ctx, itemsize):
+    """Bytes one decode step has to read: every weight it uses once (the position table is not
+    among them), and the keys and values of the live requests."""
+    c, f, L = cfg.n_embd, 4 * cfg.n_embd, cfg.n_layer
+    per_layer = (3 * c * c + c * c + 2 * f * c) * itemsize + (3 * c + c + f + c + 4 * c) * 4
+    weights = L * per_layer + cfg.vocab_size * c * itemsize + 2 * c * 4
+    kv = batch * mean_ctx * 2 * L * c * itemsize
+    return weights + kv
+
+
+def prefill_run(args, dtype, reps=5):
+    import numpy as np
+    import torch
+
+    engine, cfg = build_engine(args, 2, dtype)
+    runner, cache = engine.runner, engine.cache
+    t_len = min(1024, cfg.block_size)
+    rng = np.random.default_rng(1)
+    tokens = rng.integers(0, cfg.vocab_size, 2 * t_len).tolist()
+    times = []
+    for rep in range(reps + 2):
+        slots = [cache.acquire_slot(), cache.acquire_slot()]
+        for s in slots:
+            assert cache.reserve(s, t_len)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        runner.step(slots, [0, 0], [t_len, t_len], tokens, [t_len - 1, 2 * t_len - 1])
+        torch.cuda.synchronize()
+        times.append(time.perf_counter() - t0)
+        for s in slots:
+            cache.free_slot(s)
+    best = sorted(times[2:])[len(times[2:]) // 2]
+    n = 2 * t_len
+    c, L = cfg.n_embd, cfg.n_layer
+    flops = n * 24 * c * c * L + 2 * (2 * t_len * t_len * c) * L + 2 * 2 * c * cfg.vocab_size
+    return {"value": round(n / best, 1), "tokens": n, "ms": round(best * 1e3, 4),
+            "frac": round(flops / best / MFMA_PEAK[dtype], 5)}
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=256)
+    ap.add_argument("--warmup", type=int, default=16)
+    ap.add_argument("--batch", type=int, default=8)
+    ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
+    ap.add_argument("--layers", type=int, default=8)
+    ap.add_argument("--width", type=int, default=512)
+    ap.add_argument("--heads", type=int, default=8)
+    ap.add_argument("--vocab", type=int, default=50304)
+    ap.add_argument("--positions", type=int, default=1024)
+    ap.add_argument("--prompt", type=int, default=128)
+    ap.add_argument("--kv-block", type=int, default=16)
+    ap.add_argument("--no-graph", action="store_true")
+    ap.add_argument("--no-extras", action="store_true", help="skip prefill and the batch 1 / 64 points")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
+        return 2
+
+    elapsed, mean_ctx, engine, cfg = decode_run(args, args.batch, args.steps, args.warmup, args.dtype)
+    itemsize = 2 if args.dtype == "bfloat16" else 4
+    step_s = elapsed / args.steps
+    value = args.batch * args.steps / elapsed
+    achieved = decode_bytes(cfg, args.batch, mean_ctx, itemsize) / step_s / 1e9
+    stats = engine.stats()
+    record = {
+        "metric": "decode tokens/s (50.9M GPT-2-style, batch 8, 128-token prompts)",
+        "value": round(value, 1), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(step_s * 1e3, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": round(value / REFERENCE_DECODE_B8, 2) if args.batch == 8 else None,
+        "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "data": "synthetic",
+        "config": {
+            "model": "gpt2-mini-50.9M", "n_layer": cfg.n_layer, "n_layer_full": 8, "n_embd": cfg.n_embd,
+            "n_head": cfg.n_head, "head_dim": cfg.head_dim, "mlp_hidden": 4 * cfg.n_embd,
+            "vocab_size": cfg.vocab_size, "block_size": cfg.block_size, "bias": True,
+            "global_batch": args.batch, "seq_len": cfg.block_size, "prompt_len": args.prompt,
+            "mean_context": round(mean_ctx, 1), "kv_block": args.kv_block, "weights": "random",
+            "hip_graph": bool(stats["graph_steps"]), "parallelism": "single-gpu",
+        },
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK_GBS, 5)},
+    }
+    del engine
+    if not args.no_extras:
+        record["prefill"] = prefill_run(args, args.dtype)
+        points = {}
+        for b in (1, 64):
+            k = min(args.steps, 128)
+            el, _, eng, _ = decode_run(args, b, k, min(args.warmup, 8), args.dtype)
+            points[f"decode_b{b}"] = round(b * k / el, 1)
+            del eng
+        record["points"] = points
+    print(json.dumps(record))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -41,9 +41,10 @@ extern "C" int mgpt_embed(const int* ids, const int* pos, const void* tok, const
   return mgpt_last_error();
 }
 
-// One wave per row; four rows per workgroup.  Mean, then centred variance, then
-// the normalised row: three passes over a row that stays in cache, so any width
-// works and the variance is never a difference of large numbers.
+// One wave per row; four rows per workgroup.  Mean (with one correction pass),
+// then centred variance, then the normalised row: passes over a row that stays
+// in cache, so any width works and the variance is never a difference of large
+// numbers.
 template <typename OT>
 __global__ void layernorm_kernel(const float* __restrict__ x, const float* __restrict__ w,
                                  const float* __restrict__ b, OT* __restrict__ out,
@@ -55,17 +56,22 @@ __global__ void layernorm_kernel(const float* __restrict__ x, const float* __res
   const float* xr = x + src * (long)width;
   float s = 0.f;
   for (int c = lane; c < width; c += MGPT_WAVE) s += xr[c];
-  float mean = wave_sum(s) / (float)width;
+  const float mean = wave_sum(s) / (float)width;
+  // The mean as a sum of two floats: what the first pass lost to rounding is kept apart, so that
+  // x - mean stays exact for a row whose values are close together and far from zero.
+  float e = 0.f;
+  for (int c = lane; c < width; c += MGPT_WAVE) e += xr[c] - mean;
+  const float corr = wave_sum(e) / (float)width;
   float v = 0.f;
   for (int c = lane; c < width; c += MGPT_WAVE) {
-    float d = xr[c] - mean;
+    float d = (xr[c] - mean) - corr;
     v += d * d;
   }
   float var = wave_sum(v) / (float)width;
   float rstd = 1.0f / sqrtf(var + eps);
   OT* orow = out + (long)row * width;
   for (int c = lane; c < width; c += MGPT_WAVE) {
-    float y = (xr[c] - mean) * rstd * w[c];
+    float y = ((xr[c] - mean) - corr) * rstd * w[c];
     if (b) y += b[c];
     orow[c] = from_float<OT>(y);
   }

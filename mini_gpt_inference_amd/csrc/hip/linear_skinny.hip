@@ -1,0 +1,262 @@
+// Matrix product for few rows (a decode step: 1..64 tokens) in bfloat16 on the MFMA units.
+//
+// out[n, o] = sum_k act[n, k] * W[o, k] (+ bias[o]), nn.Linear as in
+// src/minigpt_infer/model.py:43-44,96-101 of the reference.  With so few rows the
+// work is streaming W once from HBM, so the kernel is laid out around that: a
+// workgroup of four waves owns a strip of output columns, its waves split the
+// strip and/or the k range, every lane keeps several 16-byte loads of W in
+// flight, and one v_mfma_f32_16x16x32_bf16 per 32 k turns a 16-column tile of W
+// and 16 rows of activations into float32 sums.  Waves that split k add their
+// sums through LDS in a fixed order, so results do not depend on timing.
+//
+// Prologue (optional): LayerNorm of the float32 residual rows, statistics in
+// float32, result in bfloat16 in LDS (src/minigpt_infer/model.py:113-114: every
+// linear that reads the residual stream reads it through a LayerNorm), with an
+// optional gather of rows (the logit rows of the output head).
+// Epilogues: plain store (bfloat16 or float32), GELU-tanh, add into the float32
+// residual stream, or store plus scatter of the key and value columns into
+// their cache pages by slot_mapping (src/minigpt_infer/cache/paged.py:125-137).
+#include "common.h"
+
+typedef __attribute__((__vector_size__(8 * sizeof(short)))) short bf16x8_t;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4_t;
+
+#define SK_EPI_NONE 0
+#define SK_EPI_GELU 1
+#define SK_EPI_RESIDUAL 2
+#define SK_EPI_QKV 3
+
+#define SK_WAVES 4
+#define SK_PAD 8  // bfloat16 elements of padding per LDS row: keeps the 16 rows a MFMA reads on distinct banks
+
+struct SkinnyArgs {
+  const bf16_t* act;  // [n_rows, k_dim] bfloat16, row stride lda (no prologue)
+  long lda;
+  const float* x;     // residual stream, float32, row stride k_dim (LayerNorm prologue)
+  const int* rows;    // optional gather of residual rows
+  const float* ln_w;
+  const float* ln_b;
+  float eps;
+  const bf16_t* w;    // [n_out, k_dim]
+  const float* bias;  // [n_out] or null
+  void* out;          // [n_rows, n_out], row stride ldo
+  long ldo;
+  int n_rows, n_out, k_dim;
+  int ksplit;         // waves of a workgroup that share a column tile: 1, 2 or 4
+  // key/value scatter (SK_EPI_QKV)
+  bf16_t* kpool;
+  bf16_t* vpool;
+  const int* slot_mapping;
+  int q_width, kv_width, head_dim, n_kv_head, page_size;
+};
+
+__device__ __forceinline__ bf16x8_t load8(const bf16_t* p) {
+  return *reinterpret_cast<const bf16x8_t*>(p);
+}
+
+template <int NT, bool LN, int EPI, typename OT>
+__global__ __launch_bounds__(256) void linear_skinny_kernel(SkinnyArgs a) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int ks = a.ksplit, cw_per_wg = SK_WAVES / ks;
+  const int cw = wave / ks, kw = wave - cw * ks;
+  const int o0 = (blockIdx.x * cw_per_wg + cw) * 16;
+  const int K = a.k_dim;
+  const int ldh = K + SK_PAD;
+  bf16_t* hs = reinterpret_cast<bf16_t*>(smem);                       // [NT*16][ldh] when LN
+  float* red = reinterpret_cast<float*>(smem + (LN ? (size_t)NT * 16 * ldh * sizeof(bf16_t) : 0));
+
+  if (LN) {
+    // LayerNorm of up to NT*16 rows: one wave per row, rows round-robin over the waves
+    for (int r = wave; r < NT * 16; r += SK_WAVES) {
+      bf16_t* hr = hs + (long)r * ldh;
+      if (r < a.n_rows) {
+        const float* xr = a.x + (long)(a.rows ? a.rows[r] : r) * K;
+        float s = 0.f;
+        for (int c = lane; c < K; c += 64) s += xr[c];
+        const float mean = wave_sum(s) / (float)K;
+        float e = 0.f;
+        for (int c = lane; c < K; c += 64) e += xr[c] - mean;
+        const float corr = wave_sum(e) / (float)K;  // what the first sum lost to rounding, kept apart
+        float v = 0.f;
+        for (int c = lane; c < K; c += 64) {
+          float d = (xr[c] - mean) - corr;
+          v += d * d;
+        }
+        const float rstd = 1.0f / sqrtf(wave_sum(v) / (float)K + a.eps);
+        for (int c = lane; c < K; c += 64) {
+          float y = ((xr[c] - mean) - corr) * rstd * a.ln_w[c];
+          if (a.ln_b) y += a.ln_b[c];
+          hr[c] = float_to_bf16(y);
+        }
+      } else {
+        for (int c = lane; c < K; c += 64) hr[c] = 0;
+      }
+    }
+    __syncthreads();
+  }
+
+  // this wave's k range, in steps of 32
+  const int k_per = ((K / ks + 31) / 32) * 32;
+  const int k_begin = kw * k_per;
+  const int k_end = (k_begin + k_per < K) ? k_begin + k_per : K;
+  const int lrow = lane & 15, lk = (lane >> 4) * 8;
+
+  f32x4_t acc[NT];
+#pragma unroll
+  for (int t = 0; t < NT; ++t) acc[t] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+
+  const int wo = o0 + lrow;
+  const bool w_ok = wo < a.n_out;
+  const bf16_t* wp = a.w + (long)(w_ok ? wo : 0) * K + lk;
+  const bf16x8_t zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+
+  if (o0 < a.n_out) {
+#pragma unroll 4
+    for (int k0 = k_begin; k0 < k_end; k0 += 32) {
+      const bool k_ok = k0 + lk + 8 <= k_end;
+      bf16x8_t wv = (w_ok && k_ok) ? load8(wp + k0) : zero8;
+#pragma unroll
+      for (int t = 0; t < NT; ++t) {
+        bf16x8_t av;
+        const int n = t * 16 + lrow;
+        if (LN) {
+          av = k_ok ? load8(hs + (long)n * ldh + k0 + lk) : zero8;
+        } else {
+          av = (k_ok && n < a.n_rows) ? load8(a.act + (long)n * a.lda + k0 + lk) : zero8;
+        }
+        acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wv, av, acc[t], 0, 0, 0);
+      }
+    }
+  }
+
+  // waves that split k hand their sums to the first of them, which adds in wave order
+  if (ks > 1) {
+    if (kw > 0) {
+#pragma unroll
+      for (int t = 0; t < NT; ++t)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) red[((wave * NT + t) * 4 + i) * 64 + lane] = acc[t][i];
+    }
+    __syncthreads();
+    if (kw == 0) {
+      for (int s = 1; s < ks; ++s)
+#pragma unroll
+        for (int t = 0; t < NT; ++t)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) acc[t][i] += red[(((wave + s) * NT + t) * 4 + i) * 64 + lane];
+    }
+  }
+  if (kw != 0 || o0 >= a.n_out) return;
+
+  // lane holds out[n = t*16 + (lane & 15)][o0 + (lane >> 4) * 4 + i], i = 0..3
+  const int oc = o0 + (lane >> 4) * 4;
+#pragma unroll
+  for (int t = 0; t < NT; ++t) {
+    const int n = t * 16 + lrow;
+    if (n >= a.n_rows) continue;
+    float v[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      v[i] = acc[t][i];
+      if (a.bias && oc + i < a.n_out) v[i] += a.bias[oc + i];
+      if (EPI == SK_EPI_GELU) v[i] = gelu_tanh(v[i]);
+    }
+    OT* orow = reinterpret_cast<OT*>(a.out) + (long)n * a.ldo;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      if (oc + i >= a.n_out) continue;
+      if (EPI == SK_EPI_RESIDUAL) {
+        orow[oc + i] = from_float<OT>(to_float<OT>(orow[oc + i]) + v[i]);
+      } else {
+        orow[oc + i] = from_float<OT>(v[i]);
+      }
+    }
+    if (EPI == SK_EPI_QKV) {
+      const int slot = a.slot_mapping[n];
+      if (slot >= 0 && oc >= a.q_width) {
+        const long page = slot / a.page_size;
+        const int off = slot - (int)page * a.page_size;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int c = oc + i - a.q_width;  // column among keys then values
+          if (oc + i >= a.n_out) continue;
+          const bool is_v = c >= a.kv_width;
+          const int cc = is_v ? c - a.kv_width : c;
+          const int h = cc / a.head_dim, d = cc - h * a.head_dim;
+          const long dst = ((page * a.n_kv_head + h) * a.page_size + off) * (long)a.head_dim + d;
+          (is_v ? a.vpool : a.kpool)[dst] = float_to_bf16(v[i]);
+        }
+      }
+    }
+  }
+}
+
+template <int NT, bool LN>
+static int launch_nt(const SkinnyArgs& a, int epi, int out_dtype, dim3 grid, size_t smem, hipStream_t s) {
+#define SK_LAUNCH(E, OT) \
+  hipLaunchKernelGGL((linear_skinny_kernel<NT, LN, E, OT>), grid, dim3(256), smem, s, a)
+  if (epi == SK_EPI_NONE && out_dtype == MGPT_BF16) SK_LAUNCH(SK_EPI_NONE, bf16_t);
+  else if (epi == SK_EPI_NONE && out_dtype == MGPT_F32) SK_LAUNCH(SK_EPI_NONE, float);
+  else if (epi == SK_EPI_GELU && out_dtype == MGPT_BF16) SK_LAUNCH(SK_EPI_GELU, bf16_t);
+  else if (epi == SK_EPI_RESIDUAL && out_dtype == MGPT_F32) SK_LAUNCH(SK_EPI_RESIDUAL, float);
+  else if (epi == SK_EPI_QKV && out_dtype == MGPT_BF16) SK_LAUNCH(SK_EPI_QKV, bf16_t);
+  else return MGPT_ERR_BAD_DTYPE;
+#undef SK_LAUNCH
+  return mgpt_last_error();
+}
+
+// LayerNorm prologue when x is given (then act is ignored), plain bfloat16 activations otherwise.
+// Refuses (MGPT_ERR_BAD_SHAPE) more than 64 rows, k_dim that is no multiple of 16, and a LayerNorm
+// prologue whose rows do not fit 64 KB of LDS; the caller then takes the general kernels.
+extern "C" int mgpt_linear_skinny(const void* act, long lda, const float* x, const int* rows,
+                                  const float* ln_w, const float* ln_b, float eps, const void* w,
+                                  const float* bias, void* out, int out_dtype, long ldo, int n_rows,
+                                  int n_out, int k_dim, int epilogue, void* kpool, void* vpool,
+                                  const int* slot_mapping, int q_width, int kv_width, int head_dim,
+                                  int n_kv_head, int page_size, hipStream_t stream) {
+  if (n_rows == 0 || n_out == 0) return MGPT_OK;
+  if (!w || !out || (!act && !x)) return MGPT_ERR_NULL;
+  if (n_rows < 0 || n_rows > 64 || n_out < 0 || k_dim <= 0 || (k_dim % 16) != 0 || ldo < n_out)
+    return MGPT_ERR_BAD_SHAPE;
+  const bool ln = x != nullptr;
+  if (ln && !ln_w) return MGPT_ERR_NULL;
+  if (!ln && (lda < k_dim || (lda % 8) != 0)) return MGPT_ERR_BAD_SHAPE;
+  if (epilogue == SK_EPI_QKV) {
+    if (!kpool || !vpool || !slot_mapping) return MGPT_ERR_NULL;
+    if (head_dim <= 0 || (head_dim % 4) != 0 || (q_width % 4) != 0 || q_width + 2 * kv_width != n_out ||
+        kv_width != n_kv_head * head_dim || page_size <= 0)
+      return MGPT_ERR_BAD_SHAPE;
+  }
+  const int nt = (n_rows + 15) / 16;
+  // waves sharing a column tile: as many as keep every wave at least 64 k wide and the grid large
+  int ks = 1;
+  const int tiles = (n_out + 15) / 16;
+  while (ks < 4 && (k_dim % (64 * ks)) == 0 && k_dim / (ks * 2) >= 64 && tiles / (SK_WAVES / ks) < 1024) ks *= 2;
+  const size_t hs_bytes = ln ? (size_t)nt * 16 * (k_dim + SK_PAD) * sizeof(bf16_t) : 0;
+  size_t red_bytes = ks > 1 ? (size_t)SK_WAVES * nt * 4 * 64 * sizeof(float) : 0;
+  if (hs_bytes + red_bytes > 64 * 1024) {  // give up the k split before giving up the kernel
+    ks = 1;
+    red_bytes = 0;
+  }
+  if (hs_bytes + red_bytes > 64 * 1024) return MGPT_ERR_BAD_SHAPE;
+  SkinnyArgs a;
+  a.act = (const bf16_t*)act; a.lda = lda; a.x = x; a.rows = rows; a.ln_w = ln_w; a.ln_b = ln_b; a.eps = eps;
+  a.w = (const bf16_t*)w; a.bias = bias; a.out = out; a.ldo = ldo; a.n_rows = n_rows; a.n_out = n_out;
+  a.k_dim = k_dim; a.ksplit = ks; a.kpool = (bf16_t*)kpool; a.vpool = (bf16_t*)vpool;
+  a.slot_mapping = slot_mapping; a.q_width = q_width; a.kv_width = kv_width; a.head_dim = head_dim;
+  a.n_kv_head = n_kv_head; a.page_size = page_size;
+  const int cw_per_wg = SK_WAVES / ks;
+  dim3 grid((tiles + cw_per_wg - 1) / cw_per_wg);
+  const size_t smem = hs_bytes + red_bytes;
+#define SK_NT(N)                                                                         \
+  (ln ? launch_nt<N, true>(a, epilogue, out_dtype, grid, smem, stream)                   \
+      : launch_nt<N, false>(a, epilogue, out_dtype, grid, smem, stream))
+  switch (nt) {
+    case 1: return SK_NT(1);
+    case 2: return SK_NT(2);
+    case 3: return SK_NT(3);
+    default: return SK_NT(4);
+  }
+#undef SK_NT
+}

@@ -11,12 +11,16 @@ def paged_attention(ctx, q: torch.Tensor, out: torch.Tensor, k_pool: torch.Tenso
                     group, n_head: int, scale: float, window: int) -> None:
     """Attention of the step's tokens (rows of q) over their requests' pages.
 
-    On the bfloat16 path decode-only steps use the split-over-keys kernel and steps with prompt
-    portions the MFMA tile kernel; the 32-bit path and every shape those refuse use the general
-    kernel, whose order of sums depends only on a query's position."""
+    On the bfloat16 path steps with prompt portions use the MFMA tile kernel and the rest the
+    kernel that splits a query's keys over four waves; the 32-bit path and every shape those
+    refuse use the general kernel, whose order of sums depends only on a query's position."""
     n, r = ctx.n_rows, ctx.cu_q.numel() - 1
     if q.dtype == torch.bfloat16 and not ctx.exact:
-        if kernels.attention_bf16(ctx, q, out, k_pool, v_pool, group, n_head, scale, window):
+        if not ctx.decode_only and kernels.prefill_attention_bf16(ctx, q, out, k_pool, v_pool, group, n_head,
+                                                                  scale, window):
+            return
+        if kernels.paged_attention_split_bf16(q, out, k_pool, v_pool, group.block_tables, ctx.cu_q, ctx.seq_lens,
+                                              ctx.q_req, n, r, n_head, scale, window):
             return
     kernels.paged_attention_generic(q, out, k_pool, v_pool, group.block_tables, ctx.cu_q, ctx.seq_lens,
                                     ctx.q_req, n, r, n_head, scale, window, fast_exp=not ctx.exact)

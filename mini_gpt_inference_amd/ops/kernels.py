@@ -205,12 +205,98 @@ def sample(logits: torch.Tensor, n_rows: int, real_vocab: int, temperature: torc
     _check(rc, "sample")
 
 
-def linear_bf16(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor,
+SK_EPI_QKV = 3
+_SKINNY_MAX_ROWS = 64
+
+
+def linear_skinny(a: Optional[torch.Tensor], w: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor,
+                  n_rows: int, epilogue: int = EPI_NONE, *, ln_x: Optional[torch.Tensor] = None,
+                  ln_weight: Optional[torch.Tensor] = None, ln_bias: Optional[torch.Tensor] = None,
+                  ln_eps: float = 0.0, ln_rows: Optional[torch.Tensor] = None, scatter=None) -> bool:
+    """bfloat16 MFMA product for at most 64 rows, with an optional LayerNorm prologue (ln_x is the
+    float32 residual stream, ln_rows an optional gather) and an optional key/value scatter
+    (scatter = (k_pool, v_pool, slot_mapping, q_width, kv_width)).  Returns False, having launched
+    nothing, when the kernel does not take the shape."""
+    if n_rows > _SKINNY_MAX_ROWS or w.dtype != torch.bfloat16:
+        return False
+    n_out, k_dim = w.shape
+    if k_dim % 16 != 0:
+        return False
+    _need_cuda(a, w, bias, out, ln_x, ln_weight, ln_bias, ln_rows)
+    _need(w.is_contiguous(), "weight must be dense [out, in]")
+    _need(out.dim() == 2 and out.stride(1) == 1 and out.shape[1] >= n_out and out.shape[0] >= n_rows,
+          "output must be [>=n_rows, >=out] with unit inner stride")
+    _need(bias is None or (bias.dtype == torch.float32 and bias.numel() == n_out), "bias must be float32 [out]")
+    if epilogue == EPI_RESIDUAL:
+        _need(out.dtype == torch.float32, "the residual stream is float32")
+    elif epilogue in (EPI_GELU, SK_EPI_QKV):
+        _need(out.dtype == torch.bfloat16, "this epilogue writes bfloat16")
+    lda = 0
+    if ln_x is not None:
+        _need(ln_x.dtype == torch.float32 and ln_x.is_contiguous() and ln_x.shape[1] == k_dim,
+              "LayerNorm prologue reads dense float32 rows of the inner size")
+        _need(ln_weight is not None and ln_weight.dtype == torch.float32 and ln_weight.numel() == k_dim,
+              "LayerNorm weight must be float32 [inner]")
+        _need(ln_bias is None or (ln_bias.dtype == torch.float32 and ln_bias.numel() == k_dim),
+              "LayerNorm bias must be float32 [inner]")
+        if ln_rows is None:
+            _need(ln_x.shape[0] >= n_rows, "too few residual rows")
+        else:
+            _need_i32("ln_rows", ln_rows, n_rows)
+    else:
+        if a is None or a.dtype != torch.bfloat16:
+            return False
+        _need(a.dim() == 2 and a.stride(1) == 1 and a.shape[1] == k_dim and a.shape[0] >= n_rows,
+              "activation must be [>=n_rows, inner] with unit inner stride")
+        if a.stride(0) % 8 != 0 or a.data_ptr() % 16 != 0:
+            return False
+        lda = a.stride(0)
+    kp = vp = sm = None
+    q_width = kv_width = head_dim = n_kv_head = page_size = 0
+    if epilogue == SK_EPI_QKV:
+        kp, vp, sm, q_width, kv_width = scatter
+        _need(kp.shape == vp.shape and kp.dim() == 4 and kp.is_contiguous() and vp.is_contiguous()
+              and kp.dtype == torch.bfloat16 and vp.dtype == torch.bfloat16,
+              "key and value pools must be dense bfloat16 [pages, kv_heads, page_size, head_dim]")
+        _, n_kv_head, page_size, head_dim = kp.shape
+        _need_i32("slot_mapping", sm, n_rows)
+    rc = library.kernels().mgpt_linear_skinny(
+        _ptr(a if ln_x is None else None), lda, _ptr(ln_x), _ptr(ln_rows), _ptr(ln_weight), _ptr(ln_bias),
+        float(ln_eps), _ptr(w), _ptr(bias), _ptr(out), _dtype_code(out), out.stride(0), n_rows, n_out, k_dim,
+        epilogue, _ptr(kp), _ptr(vp), _ptr(sm), q_width, kv_width, head_dim, n_kv_head, page_size, _stream())
+    if rc == -2:
+        return False
+    _check(rc, "linear_skinny")
+    return True
+
+
+def paged_attention_split_bf16(q: torch.Tensor, out: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor,
+                               block_tables: torch.Tensor, cu_q: torch.Tensor, seq_lens: torch.Tensor,
+                               q_req: torch.Tensor, n_tokens: int, n_req: int, n_head: int, scale: float,
+                               window: int = 0) -> bool:
+    """bfloat16 attention with each (token, head)'s keys split over four waves.  False if refused."""
+    if q.dtype != torch.bfloat16:
+        return False
+    n_kv_head, page_size, head_dim = _check_attention_args(
+        q, out, k_pool, v_pool, block_tables, cu_q, seq_lens, q_req, n_tokens, n_req, n_head)
+    if head_dim % 8 != 0 or head_dim > 256 or k_pool.data_ptr() % 16 != 0:
+        return False
+    rc = library.kernels().mgpt_paged_attention_split_bf16(
+        _ptr(q), q.stride(0), _ptr(out), out.stride(0), _ptr(k_pool), _ptr(v_pool), _ptr(block_tables),
+        block_tables.shape[1], _ptr(cu_q), _ptr(seq_lens), _ptr(q_req), n_tokens, n_head, n_kv_head, head_dim,
+        page_size, float(scale), int(window), _stream())
+    if rc == -2:
+        return False
+    _check(rc, "paged_attention_split_bf16")
+    return True
+
+
+def linear_mfma(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor,
                 n_rows: int, epilogue: int) -> bool:
-    """bfloat16 MFMA matrix product.  Returns False when no MFMA kernel takes the shape."""
+    """Tiled bfloat16 MFMA product for many rows.  False when it does not take the shape."""
     return False
 
 
-def attention_bf16(ctx, q, out, k_pool, v_pool, group, n_head: int, scale: float, window: int) -> bool:
-    """bfloat16 attention fast paths.  Returns False when none takes the case."""
+def prefill_attention_bf16(ctx, q, out, k_pool, v_pool, group, n_head: int, scale: float, window: int) -> bool:
+    """MFMA tile attention for steps with prompt portions.  False when it does not take the case."""
     return False

@@ -52,10 +52,10 @@ def _declare_optional(lib: ctypes.CDLL) -> None:
     """Signatures of the bfloat16 fast kernels."""
     P, I, L, F = c_void_p, c_int, c_long, c_float
     table = {
-        "mgpt_linear_bf16_mfma": [P, L, P, P, P, I, L, I, I, I, I, P],
-        "mgpt_linear_bf16_skinny": [P, L, P, P, P, I, L, I, I, I, I, P],
+        "mgpt_linear_skinny": [P, L, P, P, P, P, F, P, P, P, I, L, I, I, I, I, P, P, P, I, I, I, I, I, P],
+        "mgpt_paged_attention_split_bf16": [P, L, P, L, P, P, P, I, P, P, P, I, I, I, I, I, F, I, P],
+        "mgpt_linear_mfma": [P, L, P, P, P, I, L, I, I, I, I, P],
         "mgpt_prefill_attention_bf16": [P, L, P, L, P, P, P, I, P, P, P, I, I, I, I, I, I, F, I, P],
-        "mgpt_decode_attention_bf16": [P, L, P, L, P, P, P, I, P, P, P, I, I, I, I, I, F, I, P, I, P],
     }
     for name, argtypes in table.items():
         fn = getattr(lib, name, None)

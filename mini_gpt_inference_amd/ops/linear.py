@@ -1,23 +1,58 @@
-"""Chooses the matrix-product kernel for a linear layer."""
+"""Chooses the matrix-product kernel for a linear layer, and carries a LayerNorm that has not
+been computed yet to the kernel that can compute it in its prologue."""
 
 from __future__ import annotations
 
-from typing import Optional
+from typing import Optional, Union
 
 import torch
 
 from . import kernels
 
 
-def linear(ctx, a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor,
-           n_rows: int, epilogue: int = kernels.EPI_NONE) -> None:
+class LazyNorm:
+    """The normed residual stream, not yet computed: norm(x[rows]) (or norm(x)).  A linear layer
+    that reads it may compute the norm in its own prologue; anyone else calls tensor()."""
+
+    def __init__(self, norm, x: torch.Tensor, n_rows: int, rows: Optional[torch.Tensor] = None,
+                 buffer: str = "normed") -> None:
+        self.norm, self.x, self.n_rows, self.rows, self.buffer = norm, x, n_rows, rows, buffer
+        self._tensor: Optional[torch.Tensor] = None
+
+    def tensor(self, ctx) -> torch.Tensor:
+        if self._tensor is None:
+            h = ctx.workspace.get(self.buffer, self.n_rows, self.x.shape[1], ctx.dtype)
+            self.norm.forward(ctx, self.x, h, self.n_rows, rows=self.rows)
+            self._tensor = h
+        return self._tensor
+
+
+def as_tensor(ctx, a: Union[torch.Tensor, LazyNorm]) -> torch.Tensor:
+    return a.tensor(ctx) if isinstance(a, LazyNorm) else a
+
+
+def linear(ctx, a: Union[torch.Tensor, LazyNorm], w: torch.Tensor, bias: Optional[torch.Tensor],
+           out: torch.Tensor, n_rows: int, epilogue: int = kernels.EPI_NONE, scatter=None) -> bool:
     """out[:n_rows] = a[:n_rows] @ w.T (+ bias) with the epilogue.
 
-    bfloat16 activations with a bfloat16 matrix go to the MFMA kernels (skinny for few rows);
-    everything else, and every shape those refuse, goes to the 32-bit FMA kernel."""
+    On the bfloat16 path few rows go to the skinny MFMA kernel (with the LayerNorm in its prologue
+    when `a` is a LazyNorm of a fusable norm) and many rows to the tiled MFMA kernel; the 32-bit
+    path, and every shape those refuse, go to the 32-bit FMA kernel.  `scatter` = (k_pool, v_pool,
+    slot_mapping, q_width, kv_width) asks for the new keys and values to be stored into their
+    pages by the same kernel; the return value says whether that was done."""
     if n_rows == 0:
-        return
-    if a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and not ctx.exact:
-        if kernels.linear_bf16(a, w, bias, out, n_rows, epilogue):
-            return
+        return scatter is not None
+    fast = w.dtype == torch.bfloat16 and not ctx.exact and ctx.dtype == torch.bfloat16
+    if fast and n_rows <= 64:
+        epi = kernels.SK_EPI_QKV if scatter is not None else epilogue
+        if isinstance(a, LazyNorm) and getattr(a.norm, "fusable_layer_norm", False) and a._tensor is None:
+            if kernels.linear_skinny(None, w, bias, out, n_rows, epi, ln_x=a.x, ln_weight=a.norm.weight,
+                                     ln_bias=a.norm.bias, ln_eps=a.norm.eps, ln_rows=a.rows, scatter=scatter):
+                return scatter is not None
+        if kernels.linear_skinny(as_tensor(ctx, a), w, bias, out, n_rows, epi, scatter=scatter):
+            return scatter is not None
+    a = as_tensor(ctx, a)
+    if fast and kernels.linear_mfma(a, w, bias, out, n_rows, epilogue):
+        return False
     kernels.linear_generic(a, w, bias, out, n_rows, epilogue)
+    return False

@@ -4,6 +4,7 @@ from __future__ import annotations
 
 import torch
 
+from ..ops.linear import LazyNorm
 from .base import CacheBinding, Part, StepContext, register_arrangement
 from .feedforward import FeedForward
 from .mixers import Mixer
@@ -26,9 +27,8 @@ class PreNorm(Arrangement):
         self.width = int(width)
 
     def run(self, ctx, x, norm1, mixer, norm2, feed_forward, binding, position) -> None:
+        # the norms are handed on uncomputed: a linear layer that can normalise in its prologue
+        # does, everything else calls .tensor(ctx) and gets the normed rows
         n = ctx.n_rows
-        h = ctx.workspace.get("normed", n, self.width, ctx.dtype)
-        norm1.forward(ctx, x, h, n)
-        mixer.forward_add(ctx, h, x, binding, position)
-        norm2.forward(ctx, x, h, n)
-        feed_forward.forward_add(ctx, h, x)
+        mixer.forward_add(ctx, LazyNorm(norm1, x, n), x, binding, position)
+        feed_forward.forward_add(ctx, LazyNorm(norm2, x, n), x)

@@ -17,7 +17,7 @@ class FeedForward(Part):
     category = "feed_forward"
 
     def forward_add(self, ctx: StepContext, h: torch.Tensor, x: torch.Tensor) -> None:
-        """x[:n_rows] += ff(h[:n_rows])."""
+        """x[:n_rows] += ff(h[:n_rows]); h is a tensor or an ops.linear.LazyNorm (see Mixer.forward_add)."""
         raise NotImplementedError
 
 

@@ -22,8 +22,9 @@ class Mixer(Part):
 
     def forward_add(self, ctx: StepContext, h: torch.Tensor, x: torch.Tensor, binding: CacheBinding,
                     position: PositionEncoding) -> None:
-        """x[:n_rows] += mixer(h[:n_rows]); h is the normed input in the compute dtype, x the
-        float32 residual stream."""
+        """x[:n_rows] += mixer(h[:n_rows]).  x is the float32 residual stream; h is the normed input,
+        either a tensor in the compute dtype or an ops.linear.LazyNorm, which linear() takes as it
+        is and as_tensor(ctx, h) turns into a tensor."""
         raise NotImplementedError
 
 
@@ -71,11 +72,16 @@ class PagedCausalAttention(Mixer):
         n = ctx.n_rows
         total = self.q_width + 2 * self.kv_width
         qkv = ctx.workspace.get("qkv", n, total, ctx.dtype)
-        linear(ctx, h, self.qkv_weight, self.qkv_bias, qkv, n)
-        position.rotate(ctx, qkv[:, :self.q_width], qkv[:, self.q_width:self.q_width + self.kv_width], n)
         group = ctx.groups[binding.group]
         k_pool, v_pool = group.k_pools[binding.index], group.v_pools[binding.index]
-        if binding.writes:
+        # a position encoding that rotates queries and keys must act before the keys are stored;
+        # only without one may the projection kernel store them itself
+        scatter = None
+        if binding.writes and not position.rotates:
+            scatter = (k_pool, v_pool, group.slot_mapping, self.q_width, self.kv_width)
+        stored = linear(ctx, h, self.qkv_weight, self.qkv_bias, qkv, n, scatter=scatter)
+        position.rotate(ctx, qkv[:, :self.q_width], qkv[:, self.q_width:self.q_width + self.kv_width], n)
+        if binding.writes and not stored:
             kernels.kv_write(qkv, self.q_width, self.q_width + self.kv_width, k_pool, v_pool,
                              group.slot_mapping, n)
         y = ctx.workspace.get("attn_out", n, self.q_width, ctx.dtype)

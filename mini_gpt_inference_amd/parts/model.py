@@ -13,6 +13,7 @@ from typing import Dict, List, Optional, Tuple
 
 import torch
 
+from ..ops.linear import LazyNorm
 from . import block as _block  # noqa: F401  (registers the parts)
 from . import embedding as _embedding  # noqa: F401
 from . import feedforward as _feedforward  # noqa: F401
@@ -168,7 +169,6 @@ class DecoderModel:
         m = ctx.m_rows
         logits = ws.get("logits", m, self.spec.vocab_size, torch.float32)
         if m:
-            hf = ws.get("final_normed", m, self.spec.width, ctx.dtype)
-            self.final_norm.forward(ctx, x, hf, m, rows=ctx.logit_rows)
-            self.head.forward(ctx, hf, logits, m)
+            self.head.forward(ctx, LazyNorm(self.final_norm, x, m, rows=ctx.logit_rows, buffer="final_normed"),
+                              logits, m)
         return logits[:m]

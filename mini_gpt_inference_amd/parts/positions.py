@@ -17,6 +17,7 @@ from .base import Part, StepContext, TABLE, WeightRequest, register_position
 class PositionEncoding(Part):
     category = "position"
     max_positions: Optional[int] = None   # hard bound on positions, None = unbounded
+    rotates = False                       # True if rotate() changes queries and keys
 
     def embedding_table(self) -> Optional[torch.Tensor]:
         """A [max_positions, width] table whose row pos[t] is added to token t's embedding."""

@@ -48,8 +48,9 @@ def write_model(path: str, name: str, edit: Optional[Callable[[Dict[str, torch.T
 
 def assert_close(got, want, dtype: str, what: str = "") -> None:
     """max |got - want| <= TOL[dtype] * max(1, max |want|)."""
-    got = torch.as_tensor(np.asarray(got.detach().cpu() if isinstance(got, torch.Tensor) else got)).double()
-    want = torch.as_tensor(np.asarray(want.detach().cpu() if isinstance(want, torch.Tensor) else want)).double()
+    got = got.detach().cpu().double() if isinstance(got, torch.Tensor) else torch.as_tensor(np.asarray(got)).double()
+    want = (want.detach().cpu().double() if isinstance(want, torch.Tensor)
+            else torch.as_tensor(np.asarray(want)).double())
     assert got.shape == want.shape, f"{what}: shape {tuple(got.shape)} vs {tuple(want.shape)}"
     assert torch.isfinite(got).all(), f"{what}: non-finite values in the engine's result"
     scale = max(1.0, float(want.abs().max()))

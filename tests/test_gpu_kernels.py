@@ -1,0 +1,321 @@
+"""Each kernel alone against its plain reference, at sizes other than the engine's: widths and
+vocabularies that are no power of two, head sizes in steps of 16, key/value groups, windows."""
+
+import math
+
+import numpy as np
+import pytest
+import torch
+
+import helpers
+import plain_gpt as P
+from mini_gpt_inference_amd.ops import kernels
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+TDT = {"float32": torch.float32, "bfloat16": torch.bfloat16}
+
+
+def rnd(gen, *shape, dtype="float32", scale=1.0):
+    t = torch.randn(*shape, generator=gen, dtype=torch.float32) * scale
+    return t.to(TDT[dtype])
+
+
+def i32(values):
+    return torch.tensor(list(values), dtype=torch.int32, device=DEV)
+
+
+# ----------------------------------------------------------------------------- embedding, norm
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("with_pos", [True, False])
+def test_embed(dtype, with_pos):
+    g = torch.Generator().manual_seed(0)
+    tok, pos = rnd(g, 37, 80, dtype=dtype), rnd(g, 19, 80, dtype=dtype)
+    ids, positions = [5, 36, 0, 5, 12, 7, 30], [0, 18, 3, 4, 4, 9, 1]
+    x = torch.full((7, 80), float("nan"), device=DEV)
+    kernels.embed(i32(ids), i32(positions), tok.to(DEV), pos.to(DEV) if with_pos else None, x, 7)
+    want = tok.double()[ids] + (pos.double()[positions] if with_pos else 0)
+    helpers.assert_close(x, want, "float32", "embed")     # the sum itself is float32 in both cases
+
+
+@pytest.mark.parametrize("out_dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("width,bias,eps", [(80, True, 1e-5), (1000, False, 1e-2), (48, True, 1e-6)])
+def test_layer_norm(out_dtype, width, bias, eps):
+    g = torch.Generator().manual_seed(1)
+    x = rnd(g, 9, width, scale=3.0) + 2.0
+    x[3] = 5.0 + 1e-3 * torch.randn(width, generator=g)     # an almost constant row: eps decides
+    w, b = 1 + 0.1 * rnd(g, width), rnd(g, width) if bias else None
+    out = torch.empty(9, width, dtype=TDT[out_dtype], device=DEV)
+    kernels.layer_norm(x.to(DEV), w.to(DEV), b.to(DEV) if bias else None, out, 9, eps)
+    want = P.plain_layer_norm(x.double(), w.double(), b.double() if bias else None, eps)
+    helpers.assert_close(out, want, out_dtype, "layer_norm")
+    rows = [8, 0, 3]
+    out2 = torch.empty(3, width, dtype=TDT[out_dtype], device=DEV)
+    kernels.layer_norm(x.to(DEV), w.to(DEV), b.to(DEV) if bias else None, out2, 3, eps, rows=i32(rows))
+    helpers.assert_close(out2, want[rows], out_dtype, "layer_norm gather")
+
+
+# ----------------------------------------------------------------------------- linear
+def _linear_want(a, w, bias, epi, prev):
+    y = P.plain_linear(a.double(), w.double(), None if bias is None else bias.double())
+    if epi == kernels.EPI_GELU:
+        y = P.plain_gelu_tanh(y)
+    if epi == kernels.EPI_RESIDUAL:
+        y = prev.double() + y
+    return y
+
+
+@pytest.mark.parametrize("epi", [kernels.EPI_NONE, kernels.EPI_GELU, kernels.EPI_RESIDUAL])
+@pytest.mark.parametrize("a_dt,w_dt,o_dt", [("float32", "float32", "float32"), ("bfloat16", "bfloat16", "bfloat16"),
+                                            ("bfloat16", "bfloat16", "float32"), ("bfloat16", "float32", "bfloat16")])
+def test_linear_generic(a_dt, w_dt, o_dt, epi):
+    if epi == kernels.EPI_RESIDUAL and o_dt != "float32":
+        pytest.skip("the residual stream is float32")
+    g = torch.Generator().manual_seed(2)
+    n, k, o = 70, 48, 203
+    a, w, bias = rnd(g, n, k, dtype=a_dt), rnd(g, o, k, dtype=w_dt, scale=0.3), rnd(g, o)
+    prev = rnd(g, n, o, dtype=o_dt)
+    out = prev.clone().to(DEV)
+    kernels.linear_generic(a.to(DEV), w.to(DEV), bias.to(DEV), out, n, epi)
+    tol = "float32" if (a_dt, w_dt, o_dt) == ("float32",) * 3 else "bfloat16"
+    helpers.assert_close(out, _linear_want(a, w, bias, epi, prev), tol, "linear_generic")
+
+
+def test_linear_generic_refuses_bad_inner_size():
+    a, w = torch.zeros(4, 40, device=DEV), torch.zeros(8, 40, device=DEV)
+    with pytest.raises(kernels.KernelError, match="multiple of 16"):
+        kernels.linear_generic(a, w, None, torch.zeros(4, 8, device=DEV), 4)
+    with pytest.raises(kernels.KernelError, match="GPU"):
+        kernels.linear_generic(a.cpu(), w, None, torch.zeros(4, 8, device=DEV), 4)
+
+
+@pytest.mark.parametrize("n,k,o", [(1, 64, 257), (8, 512, 1536), (17, 96, 503), (33, 80, 48), (64, 2048, 512),
+                                   (5, 48, 16)])
+@pytest.mark.parametrize("epi,o_dt", [(kernels.EPI_NONE, "bfloat16"), (kernels.EPI_NONE, "float32"),
+                                      (kernels.EPI_GELU, "bfloat16"), (kernels.EPI_RESIDUAL, "float32")])
+def test_linear_skinny(n, k, o, epi, o_dt):
+    g = torch.Generator().manual_seed(3)
+    a, w, bias = rnd(g, n, k, dtype="bfloat16"), rnd(g, o, k, dtype="bfloat16", scale=k ** -0.5), rnd(g, o)
+    prev = rnd(g, n, o, dtype=o_dt)
+    out = prev.clone().to(DEV)
+    assert kernels.linear_skinny(a.to(DEV), w.to(DEV), bias.to(DEV), out, n, epi)
+    helpers.assert_close(out, _linear_want(a, w, bias, epi, prev), "bfloat16", f"skinny {n}x{k}x{o}")
+    out2 = prev.clone().to(DEV)
+    assert kernels.linear_skinny(a.to(DEV), w.to(DEV), None, out2, n, epi)
+    helpers.assert_close(out2, _linear_want(a, w, None, epi, prev), "bfloat16", "skinny without bias")
+
+
+@pytest.mark.parametrize("n,k,o,ln_bias,gather", [(8, 512, 1536, True, False), (3, 96, 503, False, True),
+                                                  (40, 80, 257, True, True), (64, 448, 64, False, False)])
+def test_linear_skinny_with_layer_norm_prologue(n, k, o, ln_bias, gather):
+    g = torch.Generator().manual_seed(4)
+    x = rnd(g, 70, k, scale=2.0) + 0.5
+    lw, lb = 1 + 0.1 * rnd(g, k), rnd(g, k) if ln_bias else None
+    w, bias = rnd(g, o, k, dtype="bfloat16", scale=k ** -0.5), rnd(g, o)
+    rows = torch.randperm(70, generator=g)[:n].tolist() if gather else list(range(n))
+    out = torch.empty(n, o, dtype=torch.float32, device=DEV)
+    assert kernels.linear_skinny(None, w.to(DEV), bias.to(DEV), out, n, kernels.EPI_NONE, ln_x=x.to(DEV),
+                                 ln_weight=lw.to(DEV), ln_bias=lb.to(DEV) if ln_bias else None, ln_eps=1e-5,
+                                 ln_rows=i32(rows) if gather else None)
+    h = P.plain_layer_norm(x.double()[rows], lw.double(), lb.double() if ln_bias else None, 1e-5)
+    helpers.assert_close(out, P.plain_linear(h, w.double(), bias.double()), "bfloat16", "LN + skinny")
+
+
+def test_linear_skinny_stores_keys_and_values():
+    g = torch.Generator().manual_seed(5)
+    n, k, h, hk, d, page, pages = 6, 64, 4, 2, 16, 4, 9
+    qw, kvw = h * d, hk * d
+    a, w, bias = rnd(g, n, k, dtype="bfloat16"), rnd(g, qw + 2 * kvw, k, dtype="bfloat16", scale=0.2), rnd(g, qw + 2 * kvw)
+    kp = torch.full((pages, hk, page, d), float("nan"), dtype=torch.bfloat16, device=DEV)
+    vp = kp.clone()
+    slots = [4 * 8 + 3, 0, 7, -1, 4 * 2 + 1, 4 * 8 + 0]
+    out = torch.empty(n, qw + 2 * kvw, dtype=torch.bfloat16, device=DEV)
+    assert kernels.linear_skinny(a.to(DEV), w.to(DEV), bias.to(DEV), out, n, kernels.SK_EPI_QKV,
+                                 scatter=(kp, vp, i32(slots), qw, kvw))
+    want = P.plain_linear(a.double(), w.double(), bias.double())
+    helpers.assert_close(out, want, "bfloat16", "qkv")
+    written = torch.zeros(pages * page, dtype=torch.bool)
+    for t, slot in enumerate(slots):
+        if slot < 0:
+            continue
+        written[slot] = True
+        for head in range(hk):
+            helpers.assert_close(kp[slot // page, head, slot % page], want[t, qw + head * d:qw + (head + 1) * d],
+                                 "bfloat16", "stored key")
+            helpers.assert_close(vp[slot // page, head, slot % page],
+                                 want[t, qw + kvw + head * d:qw + kvw + (head + 1) * d], "bfloat16", "stored value")
+    untouched = kp.float().cpu().permute(0, 2, 1, 3).reshape(pages * page, -1)[~written]
+    assert torch.isnan(untouched).all(), "a slot that no token owns was written"
+
+
+def test_linear_skinny_refuses_what_it_cannot_do():
+    w = torch.zeros(32, 64, dtype=torch.bfloat16, device=DEV)
+    a = torch.zeros(65, 64, dtype=torch.bfloat16, device=DEV)
+    assert not kernels.linear_skinny(a, w, None, torch.zeros(65, 32, dtype=torch.bfloat16, device=DEV), 65)
+    assert not kernels.linear_skinny(a.float(), w, None, torch.zeros(65, 32, dtype=torch.bfloat16, device=DEV), 4)
+    big = torch.zeros(64, 2048, device=DEV)      # 64 normed rows of 2048 do not fit the prologue's LDS
+    wbig = torch.zeros(32, 2048, dtype=torch.bfloat16, device=DEV)
+    assert not kernels.linear_skinny(None, wbig, None, torch.zeros(64, 32, dtype=torch.bfloat16, device=DEV), 64,
+                                     ln_x=big, ln_weight=torch.ones(2048, device=DEV), ln_eps=1e-5)
+
+
+# ----------------------------------------------------------------------------- cache write and attention
+class PagedCase:
+    """Random requests with part of their tokens already cached, laid out in scattered pages."""
+
+    def __init__(self, seq_lens, q_lens, h, hk, d, page, dtype, seed=0, poison=True):
+        g = torch.Generator().manual_seed(seed)
+        self.h, self.hk, self.d, self.page = h, hk, d, page
+        self.seq_lens, self.q_lens = seq_lens, q_lens
+        n_pages = sum(-(-s // page) for s in seq_lens) + 3
+        order = torch.randperm(n_pages, generator=g).tolist()
+        self.k = [rnd(g, s, hk, d, dtype=dtype) for s in seq_lens]
+        self.v = [rnd(g, s, hk, d, dtype=dtype) for s in seq_lens]
+        self.q = [rnd(g, ql, h, d, dtype=dtype) for ql in q_lens]
+        fill = float("nan") if poison else 0.0
+        kp = torch.full((n_pages, hk, page, d), fill, dtype=TDT[dtype])
+        vp = kp.clone()
+        mb = max(-(-s // page) for s in seq_lens) + 1
+        bt = torch.full((len(seq_lens), mb), -1, dtype=torch.int32)
+        self.slots = []
+        for r, s in enumerate(seq_lens):
+            for b in range(-(-s // page)):
+                bt[r, b] = order.pop()
+            for t in range(s):
+                pg, off = bt[r, t // page].item(), t % page
+                kp[pg, :, off] = self.k[r][t]
+                vp[pg, :, off] = self.v[r][t]
+            self.slots += [bt[r, t // page].item() * page + t % page for t in range(s - q_lens[r], s)]
+        self.kp, self.vp, self.bt = kp.to(DEV), vp.to(DEV), bt.to(DEV)
+        self.n = sum(q_lens)
+        self.cu = i32(np.concatenate([[0], np.cumsum(q_lens)]))
+        self.sl = i32(seq_lens)
+        self.q_req = i32([r for r, ql in enumerate(q_lens) for _ in range(ql)])
+        self.q_flat = torch.cat([q.reshape(-1, h * d) for q in self.q]).to(DEV)
+
+    def want(self, scale, window):
+        outs = []
+        for r, (s, ql) in enumerate(zip(self.seq_lens, self.q_lens)):
+            # the plain attention over the whole sequence; the step's queries are its last q_len rows
+            qfull = torch.zeros(self.h, s, self.d, dtype=P.DT)
+            qfull[:, s - ql:] = self.q[r].double().transpose(0, 1)
+            o = P.plain_causal_attention(qfull, self.k[r].double().transpose(0, 1),
+                                         self.v[r].double().transpose(0, 1), scale=scale, window=window)
+            outs.append(o[s - ql:])
+        return torch.cat(outs)
+
+
+ATTENTION_CASES = [
+    # the reference's own cases (tests/test_triton.py:83-154): uniform, ragged around a page, one key
+    dict(seq_lens=[16] * 4, q_lens=[1] * 4, h=4, hk=4, d=64, page=8),
+    dict(seq_lens=[3, 8, 9, 17, 24], q_lens=[1] * 5, h=4, hk=4, d=64, page=8),
+    dict(seq_lens=[1, 1], q_lens=[1, 1], h=2, hk=2, d=64, page=8),
+    # other sizes: groups, head sizes in steps of 16, portions, pages of other sizes, long contexts
+    dict(seq_lens=[40, 7, 130], q_lens=[5, 7, 2], h=6, hk=2, d=48, page=4),
+    dict(seq_lens=[300, 65], q_lens=[1, 33], h=3, hk=1, d=16, page=16),
+    dict(seq_lens=[77, 200], q_lens=[77, 1], h=2, hk=2, d=128, page=32),
+    dict(seq_lens=[129], q_lens=[64], h=5, hk=5, d=80, page=16),
+]
+
+
+@pytest.mark.parametrize("window", [0, 5, 70])
+@pytest.mark.parametrize("case", range(len(ATTENTION_CASES)))
+@pytest.mark.parametrize("kernel", ["generic-float32", "generic-bfloat16", "split-bfloat16"])
+def test_paged_attention(kernel, case, window):
+    name, dtype = kernel.split("-")
+    c = PagedCase(**ATTENTION_CASES[case], dtype=dtype, seed=case)
+    scale = 0.37 if case % 2 else 1.0 / math.sqrt(c.d)
+    out = torch.full((c.n, c.h * c.d), float("nan"), dtype=TDT[dtype], device=DEV)
+    args = (c.q_flat, out, c.kp, c.vp, c.bt, c.cu, c.sl, c.q_req, c.n, len(c.seq_lens), c.h, scale, window)
+    if name == "generic":
+        kernels.paged_attention_generic(*args, fast_exp=dtype == "bfloat16")
+    else:
+        assert kernels.paged_attention_split_bf16(*args)
+    helpers.assert_close(out, c.want(scale, window), dtype, f"{kernel} case {case} window {window}")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_kv_write_and_padding(dtype):
+    g = torch.Generator().manual_seed(7)
+    n, hk, d, page, pages = 5, 3, 16, 4, 6
+    qkv = rnd(g, n, 7 + 2 * hk * d, dtype=dtype).to(DEV)
+    kp = torch.full((pages, hk, page, d), float("nan"), dtype=TDT[dtype], device=DEV)
+    vp = kp.clone()
+    slots = [9, 0, -1, 23, 10]
+    kernels.kv_write(qkv, 7, 7 + hk * d, kp, vp, i32(slots), n)
+    for t, s in enumerate(slots):
+        if s < 0:
+            continue
+        assert torch.equal(kp[s // page, :, s % page].reshape(-1), qkv[t, 7:7 + hk * d])
+        assert torch.equal(vp[s // page, :, s % page].reshape(-1), qkv[t, 7 + hk * d:])
+    assert torch.isnan(kp.float()).sum().item() == (pages * page - 4) * hk * d
+    # a padded token (q_req = -1) is skipped by attention: its output row is left alone
+    c = PagedCase(seq_lens=[9], q_lens=[2], h=3, hk=3, d=16, page=4, dtype=dtype)
+    out = torch.full((3, 48), 7.0, dtype=TDT[dtype], device=DEV)
+    q = torch.cat([c.q_flat, c.q_flat[:1]])
+    kernels.paged_attention_generic(q, out, c.kp, c.vp, c.bt, c.cu, c.sl, i32([0, 0, -1]), 3, 1, 3, 0.25, 0)
+    assert (out[2] == 7.0).all() and torch.isfinite(out[:2].float()).all()
+
+
+# ----------------------------------------------------------------------------- sampling
+def _sample(logits, temperature, top_k=None, top_p=None, seeds=None, idx=None, engine_seed=0, real_vocab=None):
+    m, v = logits.shape
+    out = torch.full((m,), -1, dtype=torch.int32, device=DEV)
+    kernels.sample(logits.to(DEV), m, real_vocab or v, torch.tensor(temperature, dtype=torch.float32, device=DEV),
+                   None if top_k is None else i32(top_k),
+                   None if top_p is None else torch.tensor(top_p, dtype=torch.float32, device=DEV),
+                   None if seeds is None else torch.tensor(seeds, dtype=torch.int64, device=DEV),
+                   None if idx is None else i32(idx), engine_seed, out)
+    return out.cpu().tolist()
+
+
+def test_greedy_is_argmax_with_the_lowest_index_on_ties_and_respects_the_vocabulary_mask():
+    g = torch.Generator().manual_seed(8)
+    logits = rnd(g, 6, 50304)
+    logits[1, 777] = logits[1, 40000] = 50.0
+    logits[2, 50300] = 99.0                       # beyond the real vocabulary
+    got = _sample(logits, [0.0] * 6, real_vocab=50257)
+    want = [P.plain_sample(row.numpy(), 0.0, None, None, 0.0, 50257)[0] for row in logits]
+    assert got == want and got[1] == 777 and got[2] < 50257
+
+
+@pytest.mark.parametrize("vocab", [257, 503, 5000])
+def test_seeded_sampling_matches_the_plain_sampler(vocab):
+    g = torch.Generator().manual_seed(9)
+    m = 24
+    logits = rnd(g, m, vocab, scale=2.0)
+    temps = [0.8, 1.0, 0.3, 1.7] * (m // 4)
+    top_k = [0, 5, 0, 40, 1, 0] * (m // 6)
+    top_p = [1.0, 1.0, 0.7, 0.9, 1.0, 0.2] * (m // 6)
+    seeds, idx = list(range(100, 100 + m)), [3 * i for i in range(m)]
+    got = _sample(logits, temps, top_k, top_p, seeds, idx, engine_seed=42)
+    assert got == _sample(logits, temps, top_k, top_p, seeds, idx, engine_seed=42)       # deterministic
+    for r in range(m):
+        u = P.plain_uniform(42, seeds[r], idx[r])
+        tok, lo, hi, total = P.plain_sample(logits[r].numpy(), temps[r], top_k[r] or None,
+                                            top_p[r] if top_p[r] < 1 else None, u)
+        if got[r] != tok:
+            # float32 prefix sums may move a boundary by rounding: then u must sit on that boundary
+            edge = min(abs(u * total - lo), abs(u * total - hi))
+            assert edge <= 1e-4 * total, f"row {r}: kernel {got[r]}, plain {tok}, u {u}"
+
+
+def test_reference_vectors_top_k_top_p():
+    # reference tests/test_sampling.py:25-38
+    logits = torch.tensor([[1.0, 5.0, 3.0, 2.0, 4.0]] * 64)
+    got = set(_sample(logits, [1.0] * 64, top_k=[2] * 64, seeds=list(range(64)), idx=[0] * 64))
+    assert got == {1, 4}
+    logits = torch.tensor([[10.0, 0.0, 0.0, 0.0]] * 64)
+    assert set(_sample(logits, [1.0] * 64, top_p=[1e-6] * 64, seeds=list(range(64)), idx=[0] * 64)) == {0}
+    # mixed rows: greedy beside stochastic (reference test_sampling.py:56-63)
+    g = torch.Generator().manual_seed(10)
+    logits = rnd(g, 2, 30)
+    assert _sample(logits, [0.0, 1.0], seeds=[1, 2], idx=[0, 0])[0] == int(torch.argmax(logits[0]))
+
+
+def test_sampling_follows_the_distribution():
+    probs = torch.tensor([0.5, 0.25, 0.125, 0.125])
+    m = 4096
+    logits = probs.log().repeat(m, 1)
+    got = np.bincount(_sample(logits, [1.0] * m, seeds=[7] * m, idx=list(range(m))), minlength=4) / m
+    assert np.abs(got - probs.numpy()).max() < 0.03
