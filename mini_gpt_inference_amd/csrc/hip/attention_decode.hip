@@ -148,3 +148,162 @@ extern "C" int mgpt_paged_attention_split_bf16(
                      page_size, scale, window);
   return mgpt_last_error();
 }
+
+// ---------------------------------------------------------------------------------------------
+// The same computation for head sizes 16, 32, 64 and 128 with every load 16 bytes wide and all
+// loads of a chunk in flight at once.  D/8 lanes share a key: lane L of instruction i holds
+// channels (L % (D/8))*8 .. +8 of key c0 + i*(512/D) + L/(D/8), for the key's score (a short
+// cross-lane sum) and, with the same mapping, for its value row, so a key's weight never leaves
+// the lanes that need it.  Partial sums over keys are combined across lanes once, at the end.
+template <int D>
+__global__ __launch_bounds__(256) void paged_attention_split_fast_kernel(
+    const bf16_t* __restrict__ q, long ldq, bf16_t* __restrict__ out, long ldo,
+    const bf16_t* __restrict__ kpool, const bf16_t* __restrict__ vpool,
+    const int* __restrict__ block_tables, int max_blocks, const int* __restrict__ cu_q,
+    const int* __restrict__ seq_lens, const int* __restrict__ q_req, int n_tokens, int n_head,
+    int n_kv_head, int page_size, float scale, int window) {
+  constexpr int LPK = D / 8;     // lanes per key
+  constexpr int KPI = 64 / LPK;  // keys per load instruction
+  __shared__ float m_s[AD_WAVES], l_s[AD_WAVES];
+  __shared__ float acc_s[AD_WAVES][D];
+
+  const int n = blockIdx.x, h = blockIdx.y;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  if (n >= n_tokens) return;
+  const int r = q_req[n];
+  if (r < 0) return;  // padded token
+  const int seq_len = seq_lens[r];
+  const int q_start = cu_q[r], q_len = cu_q[r + 1] - q_start;
+  const int qpos = seq_len - q_len + (n - q_start);
+  const int kv_end = qpos + 1;
+  const int kv_begin = (window > 0 && qpos - window + 1 > 0) ? qpos - window + 1 : 0;
+  const int hk = h / (n_head / n_kv_head);
+  const int* bt = block_tables + (long)r * max_blocks;
+  const int sub = lane / LPK, dg = lane % LPK;
+
+  float qv[8];
+  {
+    const uint4 raw = *reinterpret_cast<const uint4*>(q + (long)n * ldq + (long)h * D + dg * 8);
+    const unsigned int w[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      qv[2 * e] = __uint_as_float(w[e] << 16) * scale;
+      qv[2 * e + 1] = __uint_as_float(w[e] & 0xffff0000u) * scale;
+    }
+  }
+
+  float m = -INFINITY, l = 0.f;
+  float acc[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) acc[e] = 0.f;
+
+  const int first_chunk = kv_begin / 64;
+  for (int c0 = (first_chunk + wave) * 64; c0 < kv_end; c0 += 64 * AD_WAVES) {
+    long base[LPK];
+    bool valid[LPK];
+#pragma unroll
+    for (int i = 0; i < LPK; ++i) {
+      const int j = c0 + i * KPI + sub;
+      valid[i] = (j >= kv_begin) && (j < kv_end);
+      base[i] = 0;
+      if (valid[i]) {
+        const int page = bt[j / page_size];
+        base[i] = (((long)page * n_kv_head + hk) * page_size + (j % page_size)) * (long)D + dg * 8;
+      }
+    }
+    uint4 kraw[LPK], vraw[LPK];
+#pragma unroll
+    for (int i = 0; i < LPK; ++i) {
+      kraw[i] = valid[i] ? *reinterpret_cast<const uint4*>(kpool + base[i]) : make_uint4(0, 0, 0, 0);
+      vraw[i] = valid[i] ? *reinterpret_cast<const uint4*>(vpool + base[i]) : make_uint4(0, 0, 0, 0);
+    }
+    float s[LPK];
+    float cmax = -INFINITY;
+#pragma unroll
+    for (int i = 0; i < LPK; ++i) {
+      const unsigned int w[4] = {kraw[i].x, kraw[i].y, kraw[i].z, kraw[i].w};
+      float dot = 0.f;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        dot = fmaf(qv[2 * e], __uint_as_float(w[e] << 16), dot);
+        dot = fmaf(qv[2 * e + 1], __uint_as_float(w[e] & 0xffff0000u), dot);
+      }
+#pragma unroll
+      for (int off = 1; off < LPK; off <<= 1) dot += __shfl_xor(dot, off, 64);
+      s[i] = valid[i] ? dot : -INFINITY;
+      cmax = fmaxf(cmax, s[i]);
+    }
+    const float m_new = fmaxf(m, wave_max(cmax));
+    const float alpha = (m == -INFINITY) ? 0.f : __expf(m - m_new);
+    float psum = 0.f;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc[e] *= alpha;
+#pragma unroll
+    for (int i = 0; i < LPK; ++i) {
+      const float p = valid[i] ? __expf(s[i] - m_new) : 0.f;
+      psum += p;
+      const unsigned int w[4] = {vraw[i].x, vraw[i].y, vraw[i].z, vraw[i].w};
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        acc[2 * e] = fmaf(p, __uint_as_float(w[e] << 16), acc[2 * e]);
+        acc[2 * e + 1] = fmaf(p, __uint_as_float(w[e] & 0xffff0000u), acc[2 * e + 1]);
+      }
+    }
+    // every key's weight sits on LPK lanes
+    l = l * alpha + wave_sum(psum) * (1.0f / LPK);
+    m = m_new;
+  }
+
+  // add the partial sums of the 64/LPK key subgroups: lanes with equal dg
+#pragma unroll
+  for (int e = 0; e < 8; ++e)
+#pragma unroll
+    for (int off = LPK; off < 64; off <<= 1) acc[e] += __shfl_xor(acc[e], off, 64);
+  if (lane == 0) {
+    m_s[wave] = m;
+    l_s[wave] = l;
+  }
+  if (lane < LPK) {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc_s[wave][lane * 8 + e] = acc[e];
+  }
+  __syncthreads();
+  if (tid < D) {
+    float mx = m_s[0];
+    for (int w = 1; w < AD_WAVES; ++w) mx = fmaxf(mx, m_s[w]);
+    float lt = 0.f, a = 0.f;
+    for (int w = 0; w < AD_WAVES; ++w) {
+      const float f = (m_s[w] == -INFINITY) ? 0.f : __expf(m_s[w] - mx);
+      lt += l_s[w] * f;
+      a += acc_s[w][tid] * f;
+    }
+    out[(long)n * ldo + (long)h * D + tid] = float_to_bf16(a / lt);
+  }
+}
+
+extern "C" int mgpt_paged_attention_split_fast_bf16(
+    const void* q, long ldq, void* out, long ldo, const void* kpool, const void* vpool,
+    const int* block_tables, int max_blocks, const int* cu_q, const int* seq_lens, const int* q_req,
+    int n_tokens, int n_head, int n_kv_head, int head_dim, int page_size, float scale, int window,
+    hipStream_t stream) {
+  if (n_tokens == 0) return MGPT_OK;
+  if (!q || !out || !kpool || !vpool || !block_tables || !cu_q || !seq_lens || !q_req) return MGPT_ERR_NULL;
+  if (n_tokens < 0 || n_head <= 0 || n_kv_head <= 0 || (n_head % n_kv_head) != 0 || page_size <= 0 ||
+      max_blocks <= 0 || window < 0 || (ldq % 8) != 0)
+    return MGPT_ERR_BAD_SHAPE;
+  if (n_head > 65535) return MGPT_ERR_TOO_LARGE;
+  dim3 grid(n_tokens, n_head), block(256);
+#define AD_LAUNCH(DD)                                                                                   \
+  hipLaunchKernelGGL(paged_attention_split_fast_kernel<DD>, grid, block, 0, stream, (const bf16_t*)q, ldq, \
+                     (bf16_t*)out, ldo, (const bf16_t*)kpool, (const bf16_t*)vpool, block_tables,       \
+                     max_blocks, cu_q, seq_lens, q_req, n_tokens, n_head, n_kv_head, page_size, scale, window)
+  switch (head_dim) {
+    case 16: AD_LAUNCH(16); break;
+    case 32: AD_LAUNCH(32); break;
+    case 64: AD_LAUNCH(64); break;
+    case 128: AD_LAUNCH(128); break;
+    default: return MGPT_ERR_BAD_SHAPE;  // other head sizes: the kernel above
+  }
+#undef AD_LAUNCH
+  return mgpt_last_error();
+}

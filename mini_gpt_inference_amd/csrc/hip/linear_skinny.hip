@@ -26,7 +26,9 @@ typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4_t;
 #define SK_EPI_RESIDUAL 2
 #define SK_EPI_QKV 3
 
-#define SK_WAVES 4
+#define SK_WAVES 4        // waves of a workgroup without a prologue
+#define SK_LN_WAVES 16    // waves of a workgroup with the LayerNorm prologue: one row each
+#define SK_LN_MAX_PER_LANE 32  // a prologue row is held in registers: k_dim <= 64 * 32
 #define SK_PAD 8  // bfloat16 elements of padding per LDS row: keeps the 16 rows a MFMA reads on distinct banks
 
 struct SkinnyArgs {
@@ -55,10 +57,11 @@ __device__ __forceinline__ bf16x8_t load8(const bf16_t* p) {
 }
 
 template <int NT, bool LN, int EPI, typename OT>
-__global__ __launch_bounds__(256) void linear_skinny_kernel(SkinnyArgs a) {
+__global__ __launch_bounds__(LN ? SK_LN_WAVES * 64 : SK_WAVES * 64) void linear_skinny_kernel(SkinnyArgs a) {
   extern __shared__ __align__(16) unsigned char smem[];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int ks = a.ksplit, cw_per_wg = SK_WAVES / ks;
+  constexpr int WAVES = LN ? SK_LN_WAVES : SK_WAVES;
+  const int ks = a.ksplit, cw_per_wg = WAVES / ks;
   const int cw = wave / ks, kw = wave - cw * ks;
   const int o0 = (blockIdx.x * cw_per_wg + cw) * 16;
   const int K = a.k_dim;
@@ -67,31 +70,44 @@ __global__ __launch_bounds__(256) void linear_skinny_kernel(SkinnyArgs a) {
   float* red = reinterpret_cast<float*>(smem + (LN ? (size_t)NT * 16 * ldh * sizeof(bf16_t) : 0));
 
   if (LN) {
-    // LayerNorm of up to NT*16 rows: one wave per row, rows round-robin over the waves
-    for (int r = wave; r < NT * 16; r += SK_WAVES) {
-      bf16_t* hr = hs + (long)r * ldh;
-      if (r < a.n_rows) {
-        const float* xr = a.x + (long)(a.rows ? a.rows[r] : r) * K;
-        float s = 0.f;
-        for (int c = lane; c < K; c += 64) s += xr[c];
-        const float mean = wave_sum(s) / (float)K;
-        float e = 0.f;
-        for (int c = lane; c < K; c += 64) e += xr[c] - mean;
-        const float corr = wave_sum(e) / (float)K;  // what the first sum lost to rounding, kept apart
-        float v = 0.f;
-        for (int c = lane; c < K; c += 64) {
-          float d = (xr[c] - mean) - corr;
-          v += d * d;
-        }
-        const float rstd = 1.0f / sqrtf(wave_sum(v) / (float)K + a.eps);
-        for (int c = lane; c < K; c += 64) {
-          float y = ((xr[c] - mean) - corr) * rstd * a.ln_w[c];
+    // LayerNorm of up to 16 rows, one wave per row; the row is read once and kept in registers
+    // (the launcher sends more than 16 rows through a LayerNorm kernel of their own)
+    const int r = wave;
+    bf16_t* hr = hs + (long)r * ldh;
+    if (r < a.n_rows) {
+      const float* xr = a.x + (long)(a.rows ? a.rows[r] : r) * K;
+      float xv[SK_LN_MAX_PER_LANE];
+      float s = 0.f;
+#pragma unroll
+      for (int i = 0; i < SK_LN_MAX_PER_LANE; ++i) {
+        const int c = lane + i * 64;
+        xv[i] = c < K ? xr[c] : 0.f;
+        s += xv[i];
+      }
+      const float mean = wave_sum(s) / (float)K;
+      float e = 0.f;
+#pragma unroll
+      for (int i = 0; i < SK_LN_MAX_PER_LANE; ++i) e += (lane + i * 64 < K) ? xv[i] - mean : 0.f;
+      const float corr = wave_sum(e) / (float)K;  // what the first sum lost to rounding, kept apart
+      float v = 0.f;
+#pragma unroll
+      for (int i = 0; i < SK_LN_MAX_PER_LANE; ++i) {
+        const float d = (lane + i * 64 < K) ? (xv[i] - mean) - corr : 0.f;
+        xv[i] = d;
+        v += d * d;
+      }
+      const float rstd = 1.0f / sqrtf(wave_sum(v) / (float)K + a.eps);
+#pragma unroll
+      for (int i = 0; i < SK_LN_MAX_PER_LANE; ++i) {
+        const int c = lane + i * 64;
+        if (c < K) {
+          float y = xv[i] * rstd * a.ln_w[c];
           if (a.ln_b) y += a.ln_b[c];
           hr[c] = float_to_bf16(y);
         }
-      } else {
-        for (int c = lane; c < K; c += 64) hr[c] = 0;
       }
+    } else {
+      for (int c = lane; c < K; c += 64) hr[c] = 0;
     }
     __syncthreads();
   }
@@ -195,7 +211,7 @@ __global__ __launch_bounds__(256) void linear_skinny_kernel(SkinnyArgs a) {
 template <int NT, bool LN>
 static int launch_nt(const SkinnyArgs& a, int epi, int out_dtype, dim3 grid, size_t smem, hipStream_t s) {
 #define SK_LAUNCH(E, OT) \
-  hipLaunchKernelGGL((linear_skinny_kernel<NT, LN, E, OT>), grid, dim3(256), smem, s, a)
+  hipLaunchKernelGGL((linear_skinny_kernel<NT, LN, E, OT>), grid, dim3((LN ? SK_LN_WAVES : SK_WAVES) * 64), smem, s, a)
   if (epi == SK_EPI_NONE && out_dtype == MGPT_BF16) SK_LAUNCH(SK_EPI_NONE, bf16_t);
   else if (epi == SK_EPI_NONE && out_dtype == MGPT_F32) SK_LAUNCH(SK_EPI_NONE, float);
   else if (epi == SK_EPI_GELU && out_dtype == MGPT_BF16) SK_LAUNCH(SK_EPI_GELU, bf16_t);
@@ -208,7 +224,8 @@ static int launch_nt(const SkinnyArgs& a, int epi, int out_dtype, dim3 grid, siz
 
 // LayerNorm prologue when x is given (then act is ignored), plain bfloat16 activations otherwise.
 // Refuses (MGPT_ERR_BAD_SHAPE) more than 64 rows, k_dim that is no multiple of 16, and a LayerNorm
-// prologue whose rows do not fit 64 KB of LDS; the caller then takes the general kernels.
+// prologue for more than 16 rows or rows that do not fit 64 KB of LDS; the caller then runs the
+// LayerNorm by itself, or takes the general kernels.
 extern "C" int mgpt_linear_skinny(const void* act, long lda, const float* x, const int* rows,
                                   const float* ln_w, const float* ln_b, float eps, const void* w,
                                   const float* bias, void* out, int out_dtype, long ldo, int n_rows,
@@ -221,6 +238,8 @@ extern "C" int mgpt_linear_skinny(const void* act, long lda, const float* x, con
     return MGPT_ERR_BAD_SHAPE;
   const bool ln = x != nullptr;
   if (ln && !ln_w) return MGPT_ERR_NULL;
+  // the prologue normalises at most 16 rows (one per wave), each held in registers
+  if (ln && (n_rows > 16 || k_dim > 64 * SK_LN_MAX_PER_LANE)) return MGPT_ERR_BAD_SHAPE;
   if (!ln && (lda < k_dim || (lda % 8) != 0)) return MGPT_ERR_BAD_SHAPE;
   if (epilogue == SK_EPI_QKV) {
     if (!kpool || !vpool || !slot_mapping) return MGPT_ERR_NULL;
@@ -229,12 +248,13 @@ extern "C" int mgpt_linear_skinny(const void* act, long lda, const float* x, con
       return MGPT_ERR_BAD_SHAPE;
   }
   const int nt = (n_rows + 15) / 16;
+  const int waves = ln ? SK_LN_WAVES : SK_WAVES;
   // waves sharing a column tile: as many as keep every wave at least 64 k wide and the grid large
   int ks = 1;
   const int tiles = (n_out + 15) / 16;
-  while (ks < 4 && (k_dim % (64 * ks)) == 0 && k_dim / (ks * 2) >= 64 && tiles / (SK_WAVES / ks) < 1024) ks *= 2;
-  const size_t hs_bytes = ln ? (size_t)nt * 16 * (k_dim + SK_PAD) * sizeof(bf16_t) : 0;
-  size_t red_bytes = ks > 1 ? (size_t)SK_WAVES * nt * 4 * 64 * sizeof(float) : 0;
+  while (ks < 4 && (k_dim % (64 * ks)) == 0 && k_dim / (ks * 2) >= 64 && tiles / (waves / ks) < 1024) ks *= 2;
+  const size_t hs_bytes = ln ? (size_t)16 * (k_dim + SK_PAD) * sizeof(bf16_t) : 0;
+  size_t red_bytes = ks > 1 ? (size_t)waves * nt * 4 * 64 * sizeof(float) : 0;
   if (hs_bytes + red_bytes > 64 * 1024) {  // give up the k split before giving up the kernel
     ks = 1;
     red_bytes = 0;
@@ -246,7 +266,7 @@ extern "C" int mgpt_linear_skinny(const void* act, long lda, const float* x, con
   a.k_dim = k_dim; a.ksplit = ks; a.kpool = (bf16_t*)kpool; a.vpool = (bf16_t*)vpool;
   a.slot_mapping = slot_mapping; a.q_width = q_width; a.kv_width = kv_width; a.head_dim = head_dim;
   a.n_kv_head = n_kv_head; a.page_size = page_size;
-  const int cw_per_wg = SK_WAVES / ks;
+  const int cw_per_wg = waves / ks;
   dim3 grid((tiles + cw_per_wg - 1) / cw_per_wg);
   const size_t smem = hs_bytes + red_bytes;
 #define SK_NT(N)                                                                         \

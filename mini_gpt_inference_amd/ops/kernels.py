@@ -273,15 +273,19 @@ def linear_skinny(a: Optional[torch.Tensor], w: torch.Tensor, bias: Optional[tor
 def paged_attention_split_bf16(q: torch.Tensor, out: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor,
                                block_tables: torch.Tensor, cu_q: torch.Tensor, seq_lens: torch.Tensor,
                                q_req: torch.Tensor, n_tokens: int, n_req: int, n_head: int, scale: float,
-                               window: int = 0) -> bool:
-    """bfloat16 attention with each (token, head)'s keys split over four waves.  False if refused."""
+                               window: int = 0, fast: bool = True) -> bool:
+    """bfloat16 attention with each (token, head)'s keys split over four waves.  False if refused.
+    fast=False keeps to the variant that takes every head size."""
     if q.dtype != torch.bfloat16:
         return False
     n_kv_head, page_size, head_dim = _check_attention_args(
         q, out, k_pool, v_pool, block_tables, cu_q, seq_lens, q_req, n_tokens, n_req, n_head)
     if head_dim % 8 != 0 or head_dim > 256 or k_pool.data_ptr() % 16 != 0:
         return False
-    rc = library.kernels().mgpt_paged_attention_split_bf16(
+    fn = library.kernels().mgpt_paged_attention_split_bf16
+    if fast and head_dim in (16, 32, 64, 128) and q.stride(0) % 8 == 0 and q.data_ptr() % 16 == 0:
+        fn = library.kernels().mgpt_paged_attention_split_fast_bf16   # all loads 16 bytes wide
+    rc = fn(
         _ptr(q), q.stride(0), _ptr(out), out.stride(0), _ptr(k_pool), _ptr(v_pool), _ptr(block_tables),
         block_tables.shape[1], _ptr(cu_q), _ptr(seq_lens), _ptr(q_req), n_tokens, n_head, n_kv_head, head_dim,
         page_size, float(scale), int(window), _stream())
@@ -294,7 +298,27 @@ def paged_attention_split_bf16(q: torch.Tensor, out: torch.Tensor, k_pool: torch
 def linear_mfma(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor,
                 n_rows: int, epilogue: int) -> bool:
     """Tiled bfloat16 MFMA product for many rows.  False when it does not take the shape."""
-    return False
+    if a.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
+        return False
+    n_out, k_dim = w.shape
+    if k_dim % 16 != 0 or a.stride(0) % 8 != 0 or a.data_ptr() % 16 != 0 or w.data_ptr() % 16 != 0:
+        return False
+    if (epilogue, out.dtype) not in ((EPI_NONE, torch.bfloat16), (EPI_NONE, torch.float32),
+                                     (EPI_GELU, torch.bfloat16), (EPI_RESIDUAL, torch.float32)):
+        return False
+    _need_cuda(a, w, bias, out)
+    _need(w.is_contiguous(), "weight must be dense [out, in]")
+    _need(a.dim() == 2 and a.stride(1) == 1 and a.shape[1] == k_dim and a.shape[0] >= n_rows,
+          "activation must be [>=n_rows, inner] with unit inner stride")
+    _need(out.dim() == 2 and out.stride(1) == 1 and out.shape[1] >= n_out and out.shape[0] >= n_rows,
+          "output must be [>=n_rows, >=out] with unit inner stride")
+    _need(bias is None or (bias.dtype == torch.float32 and bias.numel() == n_out), "bias must be float32 [out]")
+    rc = library.kernels().mgpt_linear_mfma(_ptr(a), a.stride(0), _ptr(w), _ptr(bias), _ptr(out), _dtype_code(out),
+                                            out.stride(0), n_rows, n_out, k_dim, epilogue, _stream())
+    if rc == -2:
+        return False
+    _check(rc, "linear_mfma")
+    return True
 
 
 def prefill_attention_bf16(ctx, q, out, k_pool, v_pool, group, n_head: int, scale: float, window: int) -> bool:

@@ -54,6 +54,7 @@ def _declare_optional(lib: ctypes.CDLL) -> None:
     table = {
         "mgpt_linear_skinny": [P, L, P, P, P, P, F, P, P, P, I, L, I, I, I, I, P, P, P, I, I, I, I, I, P],
         "mgpt_paged_attention_split_bf16": [P, L, P, L, P, P, P, I, P, P, P, I, I, I, I, I, F, I, P],
+        "mgpt_paged_attention_split_fast_bf16": [P, L, P, L, P, P, P, I, P, P, P, I, I, I, I, I, F, I, P],
         "mgpt_linear_mfma": [P, L, P, P, P, I, L, I, I, I, I, P],
         "mgpt_prefill_attention_bf16": [P, L, P, L, P, P, P, I, P, P, P, I, I, I, I, I, I, F, I, P],
     }

@@ -105,8 +105,26 @@ def test_linear_skinny(n, k, o, epi, o_dt):
     helpers.assert_close(out2, _linear_want(a, w, None, epi, prev), "bfloat16", "skinny without bias")
 
 
+@pytest.mark.parametrize("n,k,o", [(65, 64, 257), (300, 512, 1536), (129, 96, 503), (2048, 80, 48), (128, 2048, 128),
+                                   (1000, 48, 130)])
+@pytest.mark.parametrize("epi,o_dt", [(kernels.EPI_NONE, "bfloat16"), (kernels.EPI_NONE, "float32"),
+                                      (kernels.EPI_GELU, "bfloat16"), (kernels.EPI_RESIDUAL, "float32")])
+def test_linear_mfma(n, k, o, epi, o_dt):
+    g = torch.Generator().manual_seed(6)
+    a, w, bias = rnd(g, n, k, dtype="bfloat16"), rnd(g, o, k, dtype="bfloat16", scale=k ** -0.5), rnd(g, o)
+    prev = rnd(g, n, o, dtype=o_dt)
+    out = prev.clone().to(DEV)
+    assert kernels.linear_mfma(a.to(DEV), w.to(DEV), bias.to(DEV), out, n, epi)
+    helpers.assert_close(out, _linear_want(a, w, bias, epi, prev), "bfloat16", f"mfma {n}x{k}x{o}")
+    # rows beyond n_rows are left alone
+    out2 = prev.clone().to(DEV)
+    assert kernels.linear_mfma(a.to(DEV), w.to(DEV), None, out2, n - 3, epi)
+    assert torch.equal(out2[n - 3:], prev[n - 3:].to(DEV))
+    helpers.assert_close(out2[:n - 3], _linear_want(a, w, None, epi, prev)[:n - 3], "bfloat16", "mfma partial rows")
+
+
 @pytest.mark.parametrize("n,k,o,ln_bias,gather", [(8, 512, 1536, True, False), (3, 96, 503, False, True),
-                                                  (40, 80, 257, True, True), (64, 448, 64, False, False)])
+                                                  (16, 80, 257, True, True), (12, 1600, 64, False, False)])
 def test_linear_skinny_with_layer_norm_prologue(n, k, o, ln_bias, gather):
     g = torch.Generator().manual_seed(4)
     x = rnd(g, 70, k, scale=2.0) + 0.5
@@ -153,10 +171,14 @@ def test_linear_skinny_refuses_what_it_cannot_do():
     a = torch.zeros(65, 64, dtype=torch.bfloat16, device=DEV)
     assert not kernels.linear_skinny(a, w, None, torch.zeros(65, 32, dtype=torch.bfloat16, device=DEV), 65)
     assert not kernels.linear_skinny(a.float(), w, None, torch.zeros(65, 32, dtype=torch.bfloat16, device=DEV), 4)
-    big = torch.zeros(64, 2048, device=DEV)      # 64 normed rows of 2048 do not fit the prologue's LDS
+    big = torch.zeros(17, 2048, device=DEV)      # the prologue normalises at most 16 rows
     wbig = torch.zeros(32, 2048, dtype=torch.bfloat16, device=DEV)
-    assert not kernels.linear_skinny(None, wbig, None, torch.zeros(64, 32, dtype=torch.bfloat16, device=DEV), 64,
+    assert not kernels.linear_skinny(None, wbig, None, torch.zeros(17, 32, dtype=torch.bfloat16, device=DEV), 17,
                                      ln_x=big, ln_weight=torch.ones(2048, device=DEV), ln_eps=1e-5)
+    huge = torch.zeros(4, 4096, device=DEV)      # and rows that fit its registers and 64 KB of LDS
+    whuge = torch.zeros(32, 4096, dtype=torch.bfloat16, device=DEV)
+    assert not kernels.linear_skinny(None, whuge, None, torch.zeros(4, 32, dtype=torch.bfloat16, device=DEV), 4,
+                                     ln_x=huge, ln_weight=torch.ones(4096, device=DEV), ln_eps=1e-5)
 
 
 # ----------------------------------------------------------------------------- cache write and attention
@@ -220,7 +242,7 @@ ATTENTION_CASES = [
 
 @pytest.mark.parametrize("window", [0, 5, 70])
 @pytest.mark.parametrize("case", range(len(ATTENTION_CASES)))
-@pytest.mark.parametrize("kernel", ["generic-float32", "generic-bfloat16", "split-bfloat16"])
+@pytest.mark.parametrize("kernel", ["generic-float32", "generic-bfloat16", "split-bfloat16", "splitfast-bfloat16"])
 def test_paged_attention(kernel, case, window):
     name, dtype = kernel.split("-")
     c = PagedCase(**ATTENTION_CASES[case], dtype=dtype, seed=case)
@@ -230,7 +252,9 @@ def test_paged_attention(kernel, case, window):
     if name == "generic":
         kernels.paged_attention_generic(*args, fast_exp=dtype == "bfloat16")
     else:
-        assert kernels.paged_attention_split_bf16(*args)
+        if name == "splitfast" and c.d not in (16, 32, 64, 128):
+            pytest.skip("the wide-load variant takes head sizes 16, 32, 64, 128")
+        assert kernels.paged_attention_split_bf16(*args, fast=name == "splitfast")
     helpers.assert_close(out, c.want(scale, window), dtype, f"{kernel} case {case} window {window}")
 
 
