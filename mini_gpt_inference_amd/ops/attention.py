@@ -16,8 +16,9 @@ def paged_attention(ctx, q: torch.Tensor, out: torch.Tensor, k_pool: torch.Tenso
     refuse use the general kernel, whose order of sums depends only on a query's position."""
     n, r = ctx.n_rows, ctx.cu_q.numel() - 1
     if q.dtype == torch.bfloat16 and not ctx.exact:
-        if not ctx.decode_only and kernels.prefill_attention_bf16(ctx, q, out, k_pool, v_pool, group, n_head,
-                                                                  scale, window):
+        if not ctx.decode_only and ctx.n_rows == ctx.n_tokens and kernels.prefill_attention_bf16(
+                q, out, k_pool, v_pool, group.block_tables, ctx.cu_q, ctx.seq_lens, ctx.n_req, ctx.max_q_len,
+                n_head, scale, window):
             return
         if kernels.paged_attention_split_bf16(q, out, k_pool, v_pool, group.block_tables, ctx.cu_q, ctx.seq_lens,
                                               ctx.q_req, n, r, n_head, scale, window):

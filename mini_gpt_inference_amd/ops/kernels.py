@@ -321,6 +321,34 @@ def linear_mfma(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], 
     return True
 
 
-def prefill_attention_bf16(ctx, q, out, k_pool, v_pool, group, n_head: int, scale: float, window: int) -> bool:
-    """MFMA tile attention for steps with prompt portions.  False when it does not take the case."""
-    return False
+def prefill_attention_bf16(q: torch.Tensor, out: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor,
+                           block_tables: torch.Tensor, cu_q: torch.Tensor, seq_lens: torch.Tensor, n_req: int,
+                           max_q_len: int, n_head: int, scale: float, window: int = 0) -> bool:
+    """MFMA tile attention for steps with prompt portions (every request's tokens are consecutive
+    rows of q from cu_q).  False when it does not take the case."""
+    if q.dtype != torch.bfloat16:
+        return False
+    _need_cuda(q, out, k_pool, v_pool, block_tables, cu_q, seq_lens)
+    _need(k_pool.shape == v_pool.shape and k_pool.dim() == 4 and k_pool.is_contiguous() and v_pool.is_contiguous(),
+          "key and value pools must be dense [pages, kv_heads, page_size, head_dim]")
+    _, n_kv_head, page_size, head_dim = k_pool.shape
+    if head_dim not in (32, 64, 96, 128) or q.stride(0) % 8 != 0 or q.data_ptr() % 16 != 0 \
+            or k_pool.data_ptr() % 16 != 0 or v_pool.data_ptr() % 16 != 0:
+        return False
+    _need(q.dtype == out.dtype == k_pool.dtype == v_pool.dtype, "queries, output and pools must share a dtype")
+    _need(q.stride(1) == 1 and out.stride(1) == 1, "query and output rows must have unit inner stride")
+    _need(q.shape[1] >= n_head * head_dim and out.shape[1] >= n_head * head_dim,
+          "query/output rows are narrower than n_head * head_dim")
+    _need(n_head % n_kv_head == 0, "n_head must be a multiple of the number of key/value heads")
+    _need(block_tables.dim() == 2 and block_tables.dtype == torch.int32 and block_tables.is_contiguous()
+          and block_tables.shape[0] >= n_req, "block_tables must be dense int32 [>=requests, max_blocks]")
+    _need_i32("cu_q", cu_q, n_req + 1)
+    _need_i32("seq_lens", seq_lens, n_req)
+    rc = library.kernels().mgpt_prefill_attention_bf16(
+        _ptr(q), q.stride(0), _ptr(out), out.stride(0), _ptr(k_pool), _ptr(v_pool), _ptr(block_tables),
+        block_tables.shape[1], _ptr(cu_q), _ptr(seq_lens), n_req, max_q_len, n_head, n_kv_head, head_dim,
+        page_size, float(scale), int(window), _stream())
+    if rc == -2:
+        return False
+    _check(rc, "prefill_attention_bf16")
+    return True

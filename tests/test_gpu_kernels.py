@@ -237,12 +237,15 @@ ATTENTION_CASES = [
     dict(seq_lens=[300, 65], q_lens=[1, 33], h=3, hk=1, d=16, page=16),
     dict(seq_lens=[77, 200], q_lens=[77, 1], h=2, hk=2, d=128, page=32),
     dict(seq_lens=[129], q_lens=[64], h=5, hk=5, d=80, page=16),
+    dict(seq_lens=[333, 70, 200], q_lens=[333, 3, 130], h=4, hk=2, d=32, page=16),
+    dict(seq_lens=[500], q_lens=[190], h=2, hk=1, d=96, page=8),
 ]
 
 
 @pytest.mark.parametrize("window", [0, 5, 70])
 @pytest.mark.parametrize("case", range(len(ATTENTION_CASES)))
-@pytest.mark.parametrize("kernel", ["generic-float32", "generic-bfloat16", "split-bfloat16", "splitfast-bfloat16"])
+@pytest.mark.parametrize("kernel", ["generic-float32", "generic-bfloat16", "split-bfloat16", "splitfast-bfloat16",
+                                    "prefill-bfloat16"])
 def test_paged_attention(kernel, case, window):
     name, dtype = kernel.split("-")
     c = PagedCase(**ATTENTION_CASES[case], dtype=dtype, seed=case)
@@ -251,6 +254,11 @@ def test_paged_attention(kernel, case, window):
     args = (c.q_flat, out, c.kp, c.vp, c.bt, c.cu, c.sl, c.q_req, c.n, len(c.seq_lens), c.h, scale, window)
     if name == "generic":
         kernels.paged_attention_generic(*args, fast_exp=dtype == "bfloat16")
+    elif name == "prefill":
+        if c.d not in (32, 64, 96, 128):
+            pytest.skip("the MFMA tile kernel takes head sizes 32, 64, 96, 128")
+        assert kernels.prefill_attention_bf16(c.q_flat, out, c.kp, c.vp, c.bt, c.cu, c.sl, len(c.seq_lens),
+                                              max(c.q_lens), c.h, scale, window)
     else:
         if name == "splitfast" and c.d not in (16, 32, 64, 128):
             pytest.skip("the wide-load variant takes head sizes 16, 32, 64, 128")
