@@ -1,0 +1,190 @@
+"""Generation through the entry points: greedy tokens against the plain implementation, seeded
+sampling, what happens when pages run out, graph replay against eager steps, the command line."""
+
+import os
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+import helpers
+import plain_gpt as P
+from mini_gpt_inference_amd import EngineConfig, Request, SamplingParams
+from mini_gpt_inference_amd.engine.llm_engine import LLMEngine
+from mini_gpt_inference_amd.engine.scheduler import SchedulerError
+
+pytestmark = pytest.mark.gpu
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _prompts(name, lengths, seed=0):
+    rng = np.random.default_rng(seed)
+    return [helpers.random_ids(rng, helpers.CONFIGS[name].vocab_size, n) for n in lengths]
+
+
+def _plain_greedy(folder, prompts, n_new):
+    cfg, w = P.read_model_folder(folder)
+    return [P.plain_greedy_generate(w, cfg, p, n_new) for p in prompts]
+
+
+def _assert_greedy_within_tolerance(folder, prompt, tokens, dtype):
+    """Every token the engine chose is, for the plain implementation's logits on the engine's own
+    prefix, the best one or within twice the logit tolerance of the best: what a greedy choice can
+    be when each logit is only known to that tolerance."""
+    cfg, w = P.read_model_folder(folder)
+    ids = list(prompt)
+    exact = 0
+    for tok in tokens:
+        logits = P.plain_forward(w, cfg, ids)[-1].numpy()
+        margin = 2 * helpers.TOL[dtype] * max(1.0, np.abs(logits).max())
+        assert logits[tok] >= logits.max() - margin, (len(ids), tok, int(np.argmax(logits)))
+        exact += tok == int(np.argmax(logits))
+        ids.append(tok)
+    return exact
+
+
+@pytest.mark.parametrize("use_graph", [True, False])
+def test_greedy_generation_32bit_equals_plain_tokens(model_folders, use_graph):
+    # BASELINE configuration 1: three requests of 5/17/30 tokens, 12 greedy tokens, pages of 4
+    prompts = _prompts("A", [5, 17, 30])
+    want = _plain_greedy(model_folders["A"], prompts, 12)
+    engine = LLMEngine.from_folder(model_folders["A"], EngineConfig(block_size=4, num_blocks=64, max_batch_size=4,
+                                                                    dtype="float32", use_graph=use_graph))
+    assert engine.generate(prompts, SamplingParams(max_tokens=12, temperature=0.0)) == want
+    assert engine.cache.num_free_pages() == 64 and engine.cache.check() == 0      # nothing leaked
+    assert (engine.stats()["graph_steps"] > 0) == use_graph
+
+
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_greedy_generation_bfloat16_chooses_the_plain_argmax_up_to_rounding(model_folders, name):
+    lengths = {"A": [5, 17, 30, 2], "B": [1, 9, 33, 64, 100]}[name]
+    prompts = _prompts(name, lengths, seed=4)
+    n_new = 16
+    engine = LLMEngine.from_folder(model_folders[name], EngineConfig(block_size=8, num_blocks=128, max_batch_size=8,
+                                                                     prefill_chunk=16, dtype="bfloat16"))
+    got = engine.generate(prompts, SamplingParams(max_tokens=n_new, temperature=0.0))
+    exact = 0
+    for prompt, tokens in zip(prompts, got):
+        assert len(tokens) == n_new
+        exact += _assert_greedy_within_tolerance(model_folders[name], prompt, tokens, "bfloat16")
+    assert exact >= 0.9 * n_new * len(prompts)      # and nearly always it is the argmax itself
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_chunked_mixed_and_whole_prompt_policies_give_the_same_tokens(model_folders, dtype):
+    prompts = _prompts("B", [1, 9, 33, 64, 100], seed=2)
+    sp = SamplingParams(max_tokens=16, temperature=0.0)
+    outs = []
+    for kw in (dict(prefill_chunk=0, mixed_batches=False), dict(prefill_chunk=16, mixed_batches=True),
+               dict(prefill_chunk=7, max_num_batched_tokens=24, mixed_batches=True, use_graph=False)):
+        engine = LLMEngine.from_folder(model_folders["B"], EngineConfig(block_size=8, num_blocks=96, max_batch_size=4,
+                                                                        dtype=dtype, **kw))
+        outs.append(engine.generate(prompts, sp))
+    if dtype == "float32":
+        assert outs[0] == outs[1] == outs[2]
+    else:   # bfloat16 kernels differ between few and many rows; the first tokens still agree
+        assert [o[:4] for o in outs[0]] == [o[:4] for o in outs[1]] == [o[:4] for o in outs[2]]
+
+
+def test_seeded_temperature_sampling_is_reproducible_and_independent_of_batching(model_folders):
+    # BASELINE configuration 2: five requests of 1/9/33/64/100 tokens, 16 tokens at temperature 0.8 from a
+    # fixed sampler seed, prompt portions of 16, pages of 8
+    prompts = _prompts("B", [1, 9, 33, 64, 100], seed=3)
+    params = [SamplingParams(max_tokens=16, temperature=0.8, seed=100 + i) for i in range(5)]
+
+    def run(**kw):
+        cfg = EngineConfig(block_size=8, num_blocks=128, dtype="float32", seed=7, **kw)
+        return LLMEngine.from_folder(model_folders["B"], cfg).generate(prompts, params)
+
+    together = run(max_batch_size=8, prefill_chunk=16)
+    assert together == run(max_batch_size=8, prefill_chunk=16)
+    assert together == run(max_batch_size=2, prefill_chunk=0, mixed_batches=False)    # other batches, same tokens
+    assert together != LLMEngine.from_folder(model_folders["B"], EngineConfig(
+        block_size=8, num_blocks=128, dtype="float32", seed=8)).generate(prompts, params)
+    # each token is the plain sampler's choice for the plain logits and the same uniform number
+    cfg, w = P.read_model_folder(model_folders["B"])
+    for i in (0, 2):
+        ids = list(prompts[i])
+        for k, tok in enumerate(together[i][:6]):
+            logits = P.plain_forward(w, cfg, ids)[-1].numpy()
+            u = P.plain_uniform(7, 100 + i, k)
+            want, lo, hi, total = P.plain_sample(logits, 0.8, None, None, u)
+            assert tok == want or min(abs(u * total - lo), abs(u * total - hi)) < 1e-3 * total
+            ids.append(tok)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_pages_run_out_preempted_request_is_recomputed_and_ends_with_the_same_tokens(model_folders, dtype):
+    # reference tests/test_paged.py:107-143: pages of 2, four pages, two prompts of 2, 4 new tokens each
+    prompts = [[1, 2], [4, 5]]
+    sp = SamplingParams(max_tokens=4, temperature=0.0)
+    roomy = LLMEngine.from_folder(model_folders["A"], EngineConfig(block_size=2, num_blocks=64, max_batch_size=2,
+                                                                   dtype=dtype)).generate(prompts, sp)
+    engine = LLMEngine.from_folder(model_folders["A"], EngineConfig(block_size=2, num_blocks=4, max_batch_size=2,
+                                                                    dtype=dtype))
+    tight = engine.generate(prompts, sp)
+    assert engine.stats()["num_preemptions"] > 0
+    assert engine.cache.num_free_pages() == 4 and engine.cache.check() == 0
+    if dtype == "float32":
+        assert tight == roomy == _plain_greedy(model_folders["A"], prompts, 4)
+    else:
+        assert [t[:2] for t in tight] == [r[:2] for r in roomy]
+
+
+def test_step_outputs_finish_reasons_eot_and_cancel(model_folders):
+    engine = LLMEngine.from_folder(model_folders["A"], EngineConfig(block_size=4, num_blocks=32, max_batch_size=4,
+                                                                    dtype="float32"))
+    # a prompt whose greedy continuation changes token somewhere, so that an end token can be told apart
+    for seed in range(20):
+        prompt = _prompts("A", [7], seed=seed)[0]
+        first = _plain_greedy(model_folders["A"], [prompt], 8)[0]
+        k = next((i for i, t in enumerate(first) if t not in first[:i] and i > 0), None)
+        if k is not None:
+            break
+    assert k is not None
+    engine.add_request(Request("len", prompt, SamplingParams(max_tokens=2, temperature=0.0)))
+    engine.add_request(Request("eot", prompt, SamplingParams(max_tokens=20, temperature=0.0), eot_token_id=first[k]))
+    engine.add_request(Request("gone", prompt, SamplingParams(max_tokens=20, temperature=0.0)))
+    seen = {}
+    steps = 0
+    while engine.has_unfinished_requests():
+        for out in engine.step():
+            assert len(out.new_token_ids) == 1      # one token per request and step (reference engine.py:177-183)
+            seen.setdefault(out.request_id, []).append(out)
+        steps += 1
+        if steps == 1:
+            assert engine.cancel_request("gone") and not engine.cancel_request("nobody")
+    assert [o.new_token_ids[0] for o in seen["len"]] == first[:2] and seen["len"][-1].finish_reason == "length"
+    assert [o.new_token_ids[0] for o in seen["eot"]] == first[:k + 1] and seen["eot"][-1].finish_reason == "eot"
+    assert len(seen["gone"]) == 1 and not seen["gone"][0].finished
+    assert engine.cache.num_free_pages() == 32
+    with pytest.raises(SchedulerError, match="block_size"):          # reference engine.py:83-88
+        engine.add_request(Request("long", list(range(60)), SamplingParams(max_tokens=10)))
+    with pytest.raises(ValueError, match="token id"):
+        engine.add_request(Request("bad", [1, 999], SamplingParams(max_tokens=2)))
+
+
+def test_real_vocabulary_bound_is_never_crossed(model_folders):
+    engine = LLMEngine.from_folder(model_folders["A"], EngineConfig(block_size=4, num_blocks=32, max_batch_size=4,
+                                                                    dtype="float32", real_vocab_size=40))
+    outs = engine.generate(_prompts("A", [6, 9]), SamplingParams(max_tokens=10, temperature=1.5, seed=1))
+    assert all(t < 40 for o in outs for t in o)
+
+
+def test_from_random_and_the_command_line(tmp_path, model_folders):
+    cfg = helpers.CONFIGS["A"]
+    a = LLMEngine.from_random(cfg, 3, EngineConfig(dtype="float32", num_blocks=32, max_batch_size=2))
+    b = LLMEngine.from_random(cfg, 3, EngineConfig(dtype="float32", num_blocks=32, max_batch_size=2))
+    sp = SamplingParams(max_tokens=5, temperature=0.0)
+    assert a.generate([[1, 2, 3]], sp) == b.generate([[1, 2, 3]], sp)
+    want = _plain_greedy(model_folders["A"], [[5, 17, 3, 200]], 6)[0]
+    proc = subprocess.run([sys.executable, "-m", "mini_gpt_inference_amd.generate", "--model", model_folders["A"],
+                           "--prompt-ids", "5,17,3,200", "--max-new-tokens", "6", "--temperature", "0",
+                           "--dtype", "float32", "--kv-block-size", "4", "--num-kv-blocks", "32"],
+                          cwd=ROOT, capture_output=True, text=True, timeout=300)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    assert "config: GPTConfig(" in proc.stdout
+    line = next(l for l in proc.stdout.splitlines() if l.startswith("sample:"))
+    assert [int(t) for t in line.split()[1:]] == want

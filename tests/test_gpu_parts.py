@@ -1,0 +1,362 @@
+"""The parts of a model, each alone and put together in other ways than the one architecture
+does: other sizes and constants, key/value groups, a window, an untied head, no positions, a
+layer that runs twice, a layer that reads another layer's cache, and a toy mixer with state of
+its own that is defined here and registered without touching the framework."""
+
+import math
+
+import numpy as np
+import pytest
+import torch
+
+import helpers
+import plain_gpt as P
+from mini_gpt_inference_amd import EngineConfig, SamplingParams
+from mini_gpt_inference_amd.cache.kv_store import KVStore
+from mini_gpt_inference_amd.cache.manager import CacheManager, GroupGeometry
+from mini_gpt_inference_amd.engine.llm_engine import LLMEngine
+from mini_gpt_inference_amd.engine.step import ModelRunner
+from mini_gpt_inference_amd.ops.linear import LazyNorm, as_tensor
+from mini_gpt_inference_amd.parts.base import (CacheBinding, MATRIX, PartSpec, StateNeed, WeightRequest,
+                                               register_mixer)
+from mini_gpt_inference_amd.parts.mixers import Mixer
+from mini_gpt_inference_amd.parts.model import DecoderModel, LayerRun, LayerSpec, ModelSpec
+
+pytestmark = pytest.mark.gpu
+DEV = torch.device("cuda")
+TDT = {"float32": torch.float32, "bfloat16": torch.bfloat16}
+
+
+# ----------------------------------------------------------------------------- a toy mixer with state
+@register_mixer("toy_decay")
+class ToyDecayMixer(Mixer):
+    """s_t = decay * s_{t-1} + h_t (s starts at zero with a request's first token); out_t = s_t W^T.
+    One float32 vector of state per request, kept in the engine's state slots.  Written with
+    library calls: it is a test's part, not the product's."""
+
+    def __init__(self, width: int, decay: float) -> None:
+        self.width, self.decay = int(width), float(decay)
+        self.mix_weight = None
+
+    def weight_requests(self):
+        return {"mix_weight": WeightRequest((self.width, self.width), MATRIX)}
+
+    def cache_need(self):
+        return StateNeed(self.width)
+
+    def forward_add(self, ctx, h, x, binding, position):
+        assert binding.kind == "state"
+        pool = ctx.state_pools[binding.index]
+        hn = as_tensor(ctx, h)[:ctx.n_tokens].float()
+        w = self.mix_weight.float()
+        t = 0
+        for slot, ctx_len, q_len in zip(ctx.host_state_slots, ctx.host_ctx_lens, ctx.host_q_lens):
+            s = torch.zeros(self.width, device=x.device) if ctx_len == 0 else pool[slot].clone()
+            for j in range(q_len):
+                s = self.decay * s + hn[t]
+                x[t] += s @ w.t()
+                t += 1
+            pool[slot] = s
+
+
+def plain_toy(h, w, decay):
+    s = torch.zeros(h.shape[1], dtype=P.DT)
+    out = []
+    for t in range(h.shape[0]):
+        s = decay * s + h[t]
+        out.append(s @ w.t())
+    return torch.stack(out)
+
+
+# ----------------------------------------------------------------------------- building small models
+def _norm(prefix, c, eps, bias=True):
+    w = {"weight": prefix + "weight"}
+    if bias:
+        w["bias"] = prefix + "bias"
+    return PartSpec("layer_norm", {"width": c, "eps": eps, "bias": bias}, w)
+
+
+def _attn_layer(i, c, h, hk, d, window, scale, hidden, eps):
+    p = f"L{i}."
+    return LayerSpec(
+        arrangement=PartSpec("pre_norm", {"width": c}),
+        norm1=_norm(p + "n1.", c, eps),
+        mixer=PartSpec("paged_causal_attention",
+                       {"width": c, "n_head": h, "head_dim": d, "bias": True, "n_kv_head": hk, "scale": scale,
+                        "window": window},
+                       {"qkv_weight": p + "qkv.w", "qkv_bias": p + "qkv.b", "proj_weight": p + "o.w",
+                        "proj_bias": p + "o.b"}),
+        norm2=_norm(p + "n2.", c, eps),
+        feed_forward=PartSpec("dense_mlp", {"width": c, "hidden": hidden, "bias": True, "activation": "gelu_tanh"},
+                              {"fc_weight": p + "fc.w", "fc_bias": p + "fc.b", "proj_weight": p + "pr.w",
+                               "proj_bias": p + "pr.b"}))
+
+
+def _toy_layer(i, c, decay, hidden, eps):
+    p = f"L{i}."
+    base = _attn_layer(i, c, 1, 1, 16, 0, 1.0, hidden, eps)
+    return LayerSpec(base.arrangement, base.norm1,
+                     PartSpec("toy_decay", {"width": c, "decay": decay}, {"mix_weight": p + "mix.w"}),
+                     base.norm2, base.feed_forward)
+
+
+def _random_weights(model, seed, scale=0.12):
+    """Matrices of standard deviation about 1/sqrt(width): every linear map keeps magnitudes, so
+    that five runs deep a bfloat16 rounding is not amplified from layer to layer."""
+    g = torch.Generator().manual_seed(seed)
+    out = {}
+    for name, req in model.weight_requests().items():
+        t = torch.randn(req.shape, generator=g) * (scale if len(req.shape) == 2 else 0.1)
+        if name.endswith("n1.weight") or name.endswith("n2.weight") or name.endswith("nf.weight"):
+            t = 1 + t
+        out[name] = t.to(torch.bfloat16)      # values that both dtypes hold exactly
+    return out
+
+
+def _bind(model, weights, dtype):
+    tensors = {}
+    for name, req in model.weight_requests().items():
+        t = weights[name]
+        tensors[name] = t.to(torch.float32 if (req.role == "vector" or dtype == "float32") else torch.bfloat16).to(DEV)
+    model.bind(tensors)
+
+
+def _runner(model, dtype, page_size=4, num_pages=64, max_requests=4, poison=True):
+    geo = [GroupGeometry(page_size, num_pages, g.window) for g in model.cache_layout.groups]
+    cache = CacheManager(geo, max_requests)
+    store = KVStore(model.cache_layout, geo, max_requests, TDT[dtype], DEV, poison=poison)
+    return ModelRunner(model, cache, store, TDT[dtype], DEV, model.spec.max_positions), cache
+
+
+# the plain counterparts of the parts, from the functions of plain_gpt
+def _pl_norm(x, w, prefix, eps):
+    return P.plain_layer_norm(x, w[prefix + "weight"].double(), w[prefix + "bias"].double(), eps)
+
+
+def _pl_attn(h, w, p, n_head, hk, scale, window, kv_from=None):
+    qkv = P.plain_linear(h, w[p + "qkv.w"].double(), w[p + "qkv.b"].double())
+    q, k, v = P.plain_split_heads(qkv, n_head, hk)
+    if kv_from is not None:
+        k, v = kv_from
+    y = P.plain_causal_attention(q, k, v, scale=scale, window=window)
+    return P.plain_linear(y, w[p + "o.w"].double(), w[p + "o.b"].double()), (k, v)
+
+
+def _pl_mlp(h, w, p):
+    u = P.plain_gelu_tanh(P.plain_linear(h, w[p + "fc.w"].double(), w[p + "fc.b"].double()))
+    return P.plain_linear(u, w[p + "pr.w"].double(), w[p + "pr.b"].double())
+
+
+# ----------------------------------------------------------------------------- the model under test
+C, H, HK, D, HID, EPS, V, WINDOW, SCALE = 96, 6, 2, 16, 80, 3e-4, 91, 7, 0.31
+
+
+def _spec(order, positions="learned_absolute", tied=False):
+    layers = (_attn_layer(0, C, H, HK, D, WINDOW, SCALE, HID, EPS),      # grouped heads, a window, its own scale
+              _toy_layer(1, C, 0.5, HID, EPS),                            # state instead of keys and values
+              _attn_layer(2, C, H, H, D, 0, 1 / math.sqrt(D), HID, EPS))  # all keys: another cache group
+    pos = (PartSpec("learned_absolute", {"max_positions": 50, "width": C}, {"weight": "pos.w"})
+           if positions == "learned_absolute" else PartSpec("none"))
+    return ModelSpec(width=C, vocab_size=V,
+                     embedding=PartSpec("token_embedding", {"vocab_size": V, "width": C}, {"weight": "emb.w"}),
+                     position=pos, layers=layers, order=tuple(order), final_norm=_norm("nf.", C, EPS),
+                     head=PartSpec("linear_head", {"vocab_size": V, "width": C, "tied": tied},
+                                   {"weight": "emb.w" if tied else "head.w"}),
+                     max_positions=50 if positions == "learned_absolute" else None)
+
+
+ORDER = (LayerRun(0), LayerRun(1), LayerRun(2), LayerRun(0), LayerRun(2, reads_cache_of=2))
+
+
+def _plain_model(w, ids, order=ORDER, positions=True, tied=False):
+    x = P.plain_embed(torch.tensor(ids), w["emb.w"].double(), w["pos.w"].double() if positions else None)
+    caches = {}
+    for i, run in enumerate(order):
+        p = f"L{run.layer}."
+        h = _pl_norm(x, w, p + "n1.", EPS)
+        if run.layer == 1:
+            x = x + plain_toy(h, w[p + "mix.w"].double(), 0.5)
+        else:
+            hk, window, scale = (HK, WINDOW, SCALE) if run.layer == 0 else (H, 0, 1 / math.sqrt(D))
+            kv = caches[run.reads_cache_of] if run.reads_cache_of is not None else None
+            a, caches[i] = _pl_attn(h, w, p, H, hk, scale, window, kv_from=kv)
+            x = x + a
+        x = x + _pl_mlp(_pl_norm(x, w, p + "n2.", EPS), w, p)
+    return _pl_norm(x, w, "nf.", EPS) @ w["emb.w" if tied else "head.w"].double().t()
+
+
+def test_cache_layout_groups_runs_by_what_their_mixers_keep():
+    layout = DecoderModel(_spec(ORDER)).cache_layout
+    assert [(g.n_kv_head, g.window, g.n_pools) for g in layout.groups] == [(HK, WINDOW, 2), (H, 0, 1)]
+    assert layout.state_numels == [C]
+    kinds = [(b.kind, b.group, b.index, b.writes) for b in layout.bindings]
+    assert kinds == [("kv", 0, 0, True), ("state", -1, 0, True), ("kv", 1, 0, True), ("kv", 0, 1, True),
+                     ("kv", 1, 0, False)]
+    with pytest.raises(ValueError, match="earlier run"):
+        DecoderModel(_spec((LayerRun(0, reads_cache_of=0),)))
+    with pytest.raises(ValueError, match="different needs"):
+        DecoderModel(_spec((LayerRun(0), LayerRun(2, reads_cache_of=0))))
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("variant", ["full", "no-positions-tied-head"])
+def test_mixed_layers_repeated_layer_shared_cache_and_toy_state(dtype, variant):
+    positions, tied = variant == "full", variant != "full"
+    model = DecoderModel(_spec(ORDER, "learned_absolute" if positions else "none", tied))
+    weights = _random_weights(model, 5)
+    _bind(model, weights, dtype)
+    rng = np.random.default_rng(1)
+    reqs = [rng.integers(0, V, n).tolist() for n in (23, 9, 40)]
+    want = [_plain_model(weights, ids, positions=positions, tied=tied).numpy() for ids in reqs]
+
+    # whole, then in portions beside single tokens of the others, with pages of the window group returning
+    runner, cache = _runner(model, dtype)
+    slots = [cache.acquire_slot() for _ in reqs]
+    for s, ids in zip(slots, reqs):
+        assert cache.reserve(s, len(ids))
+    whole = runner.step(slots, [0] * 3, [len(r) for r in reqs], sum(reqs, []), list(range(sum(map(len, reqs)))))
+    off = 0
+    for ids, w_ in zip(reqs, want):
+        helpers.assert_close(whole[off:off + len(ids)], w_, dtype, f"whole {variant}")
+        off += len(ids)
+    for s in slots:
+        cache.free_slot(s)
+
+    slots = [cache.acquire_slot() for _ in reqs]
+    done = [0, 0, 0]
+    got = [[] for _ in reqs]
+    sizes = [[5, 1, 1, 7, 2, 1, 6], [2, 3, 1, 1, 2], [16, 1, 9, 1, 1, 12]]
+    step = 0
+    while any(d < len(r) for d, r in zip(done, reqs)):
+        batch = []
+        for i, ids in enumerate(reqs):
+            if done[i] < len(ids) and (step + i) % 4 != 3:        # now and then a request sits a step out
+                q = min(sizes[i][step % len(sizes[i])], len(ids) - done[i])
+                batch.append((i, q))
+        step += 1
+        if not batch:
+            continue
+        for i, q in batch:
+            assert cache.reserve(slots[i], done[i] + q)
+        toks = sum((reqs[i][done[i]:done[i] + q] for i, q in batch), [])
+        out = runner.step([slots[i] for i, _ in batch], [done[i] for i, _ in batch], [q for _, q in batch], toks,
+                          list(range(len(toks))))
+        o = 0
+        for i, q in batch:
+            got[i].append(out[o:o + q].cpu())
+            o += q
+            done[i] += q
+            cache.release_passed(slots[i], done[i])
+    for i in range(3):
+        helpers.assert_close(torch.cat(got[i]), want[i], dtype, f"cut {variant} request {i}")
+    # the window group gave pages back while the request was still running
+    assert cache.held_pages(slots[2], 0) < cache.pages_needed(40, 0) == cache.held_pages(slots[2], 1)
+    assert cache.check() == 0
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_each_part_alone(dtype):
+    """Norm, feed-forward, mixer, embedding with and without positions, head: called directly."""
+    model = DecoderModel(_spec((LayerRun(0),)))
+    weights = _random_weights(model, 9)
+    _bind(model, weights, dtype)
+    runner, cache = _runner(model, dtype)
+    tdt = TDT[dtype]
+    ids = np.random.default_rng(2).integers(0, V, 20).tolist()
+    slot = cache.acquire_slot()
+    cache.reserve(slot, 20)
+    w64 = {k: v.double() for k, v in weights.items()}
+
+    def ctx_for(start, q):
+        arena = runner.arena(q, 1, q)
+        shape = runner.describe(arena, [slot], [start], [q], ids[start:start + q], list(range(q)))
+        arena.upload()
+        return runner.context(arena, shape, padded=False)
+
+    ctx = ctx_for(0, 13)
+    layer = model.layers[0]
+    g = torch.Generator().manual_seed(0)
+    x0 = torch.randn(13, C, generator=g)
+
+    # embedding, with the learned positions and with none
+    x = torch.empty(13, C, device=DEV)
+    model.embedding.forward(ctx, model.position, x)
+    helpers.assert_close(x, P.plain_embed(torch.tensor(ids[:13]), w64["emb.w"], w64["pos.w"]), "float32", "embed+pos")
+    from mini_gpt_inference_amd.parts.positions import NoPositions
+    model.embedding.forward(ctx, NoPositions(), x)
+    helpers.assert_close(x, P.plain_embed(torch.tensor(ids[:13]), w64["emb.w"], None), "float32", "embed")
+
+    # norm
+    out = torch.empty(13, C, dtype=tdt, device=DEV)
+    layer.norm1.forward(ctx, x0.to(DEV), out, 13)
+    helpers.assert_close(out, _pl_norm(x0.double(), w64, "L0.n1.", EPS), dtype, "norm")
+
+    # feed-forward: adds into the residual stream, from an uncomputed norm and from a tensor
+    for lazy in (True, False):
+        xr = x0.clone().to(DEV)
+        h = LazyNorm(layer.norm2, xr, 13) if lazy else out
+        layer.feed_forward.forward_add(ctx, h, xr)
+        hn = _pl_norm(x0.double(), w64, "L0.n2." if lazy else "L0.n1.", EPS)
+        helpers.assert_close(xr, x0.double() + _pl_mlp(hn, w64, "L0."), dtype, f"feed-forward lazy={lazy}")
+
+    # mixer: a portion of 13, then 7 more one by one, against the whole sequence at once
+    x_all = torch.randn(20, C, generator=g)
+    h_all = _pl_norm(x_all.double(), w64, "L0.n1.", EPS)
+    want = x_all.double() + _pl_attn(h_all, w64, "L0.", H, HK, SCALE, WINDOW)[0]
+    binding = model.cache_layout.bindings[0]
+    xr = x_all[:13].clone().to(DEV)
+    layer.mixer.forward_add(ctx, LazyNorm(layer.norm1, xr, 13), xr, binding, model.position)
+    helpers.assert_close(xr, want[:13], dtype, "mixer portion")
+    for t in range(13, 20):
+        c1 = ctx_for(t, 1)
+        xr = x_all[t:t + 1].clone().to(DEV)
+        layer.mixer.forward_add(c1, LazyNorm(layer.norm1, xr, 1), xr, binding, model.position)
+        helpers.assert_close(xr, want[t:t + 1], dtype, f"mixer decode {t}")
+
+    # head (untied here), float32 logits
+    logits = torch.empty(13, V, device=DEV)
+    model.head.forward(ctx, out, logits, 13)
+    helpers.assert_close(logits, _pl_norm(x0.double(), w64, "L0.n1.", EPS) @ w64["head.w"].t(), dtype, "head")
+    assert model.head.weight.data_ptr() != model.embedding.weight.data_ptr()
+
+
+def test_part_constructors_refuse_what_the_kernels_cannot_do():
+    from mini_gpt_inference_amd.parts.base import FEED_FORWARDS, MIXERS
+    with pytest.raises(ValueError, match="multiples of 16"):
+        MIXERS.build(PartSpec("paged_causal_attention", {"width": 40, "n_head": 2, "head_dim": 20, "bias": False}))
+    with pytest.raises(ValueError, match="multiple of n_kv_head"):
+        MIXERS.build(PartSpec("paged_causal_attention", {"width": 96, "n_head": 6, "head_dim": 16, "bias": False,
+                                                         "n_kv_head": 4}))
+    with pytest.raises(ValueError, match="no kernel epilogue"):
+        FEED_FORWARDS.build(PartSpec("dense_mlp", {"width": 32, "hidden": 64, "bias": False, "activation": "relu"}))
+    with pytest.raises(KeyError, match="no mixer of kind"):
+        MIXERS.build(PartSpec("nonexistent"))
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_toy_model_generates_through_the_engine(dtype):
+    """The engine, scheduler, state slots and (for decode steps) graph capture work for a model that
+    no registered architecture describes; eviction resets the toy's state because it starts over."""
+    model = DecoderModel(_spec(ORDER))
+    weights = _random_weights(model, 12, scale=0.2)
+    _bind(model, weights, dtype)
+    prompts = [np.random.default_rng(3).integers(0, V, n).tolist() for n in (6, 11, 3)]
+    sp = SamplingParams(max_tokens=8, temperature=0.0)
+    # the toy mixer reads host-side lists, so its steps cannot be replayed from a graph
+    engine = LLMEngine(model, None, EngineConfig(block_size=4, num_blocks=40, max_batch_size=3, dtype=dtype,
+                                                 prefill_chunk=4, use_graph=False))
+    got = engine.generate(prompts, sp)
+    tight = LLMEngine(model, None, EngineConfig(block_size=4, num_blocks=9, max_batch_size=3, dtype=dtype,
+                                                use_graph=False))
+    got_tight = tight.generate(prompts, sp)
+    assert tight.stats()["num_preemptions"] > 0
+    for prompt, tokens, tokens_tight in zip(prompts, got, got_tight):
+        ids = list(prompt)
+        for k, tok in enumerate(tokens):
+            logits = _plain_model(weights, ids)[-1].numpy()
+            margin = 2 * helpers.TOL[dtype] * max(1.0, np.abs(logits).max())
+            assert logits[tok] >= logits.max() - margin
+            ids.append(tok)
+        if dtype == "float32":
+            assert tokens_tight == tokens
+    assert engine.cache.check() == 0 and engine.cache.num_free_pages(0) == 40 and engine.cache.num_free_pages(1) == 40
