@@ -41,10 +41,13 @@ extern "C" int mgpt_embed(const int* ids, const int* pos, const void* tok, const
   return mgpt_last_error();
 }
 
-// One wave per row; four rows per workgroup.  Mean (with one correction pass),
-// then centred variance, then the normalised row: passes over a row that stays
-// in cache, so any width works and the variance is never a difference of large
-// numbers.
+// One wave per row; four rows per workgroup.  A row of up to 64 * LN_CACHE values is read once
+// and kept in registers.  First the mean; then, together, the centred sum of squares and what
+// the mean lost to rounding (kept apart: the mean is a sum of two floats), so the variance is
+// never a difference of large numbers and a row of nearly equal values far from zero stays exact.
+// Wider rows take the same steps with the row re-read from cache.
+#define LN_CACHE 16
+
 template <typename OT>
 __global__ void layernorm_kernel(const float* __restrict__ x, const float* __restrict__ w,
                                  const float* __restrict__ b, OT* __restrict__ out,
@@ -54,22 +57,57 @@ __global__ void layernorm_kernel(const float* __restrict__ x, const float* __res
   if (row >= n_rows) return;
   long src = rows ? rows[row] : row;
   const float* xr = x + src * (long)width;
+  OT* orow = out + (long)row * width;
+  if (width <= MGPT_WAVE * LN_CACHE) {
+    float xv[LN_CACHE];
+    float s = 0.f;
+#pragma unroll
+    for (int i = 0; i < LN_CACHE; ++i) {
+      const int c = lane + i * MGPT_WAVE;
+      const float v = xr[c < width ? c : 0];
+      xv[i] = c < width ? v : 0.f;
+      s += xv[i];
+    }
+    const float mean = wave_sum(s) / (float)width;
+    float e = 0.f, v2 = 0.f;
+#pragma unroll
+    for (int i = 0; i < LN_CACHE; ++i) {
+      const float d = (lane + i * MGPT_WAVE < width) ? xv[i] - mean : 0.f;
+      xv[i] = d;
+      e += d;
+      v2 = fmaf(d, d, v2);
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+      e += __shfl_xor(e, off, MGPT_WAVE);
+      v2 += __shfl_xor(v2, off, MGPT_WAVE);
+    }
+    const float corr = e / (float)width;
+    const float var = fmaxf(v2 / (float)width - corr * corr, 0.f);
+    const float rstd = 1.0f / sqrtf(var + eps);
+#pragma unroll
+    for (int i = 0; i < LN_CACHE; ++i) {
+      const int c = lane + i * MGPT_WAVE;
+      if (c < width) {
+        float y = (xv[i] - corr) * rstd * w[c];
+        if (b) y += b[c];
+        orow[c] = from_float<OT>(y);
+      }
+    }
+    return;
+  }
   float s = 0.f;
   for (int c = lane; c < width; c += MGPT_WAVE) s += xr[c];
   const float mean = wave_sum(s) / (float)width;
-  // The mean as a sum of two floats: what the first pass lost to rounding is kept apart, so that
-  // x - mean stays exact for a row whose values are close together and far from zero.
-  float e = 0.f;
-  for (int c = lane; c < width; c += MGPT_WAVE) e += xr[c] - mean;
-  const float corr = wave_sum(e) / (float)width;
-  float v = 0.f;
+  float e = 0.f, v2 = 0.f;
   for (int c = lane; c < width; c += MGPT_WAVE) {
-    float d = (xr[c] - mean) - corr;
-    v += d * d;
+    const float d = xr[c] - mean;
+    e += d;
+    v2 = fmaf(d, d, v2);
   }
-  float var = wave_sum(v) / (float)width;
-  float rstd = 1.0f / sqrtf(var + eps);
-  OT* orow = out + (long)row * width;
+  const float corr = wave_sum(e) / (float)width;
+  const float var = fmaxf(wave_sum(v2) / (float)width - corr * corr, 0.f);
+  const float rstd = 1.0f / sqrtf(var + eps);
   for (int c = lane; c < width; c += MGPT_WAVE) {
     float y = ((xr[c] - mean) - corr) * rstd * w[c];
     if (b) y += b[c];

@@ -28,7 +28,7 @@ typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4_t;
 
 #define SK_WAVES 4        // waves of a workgroup without a prologue
 #define SK_LN_WAVES 16    // waves of a workgroup with the LayerNorm prologue: one row each
-#define SK_LN_MAX_PER_LANE 32  // a prologue row is held in registers: k_dim <= 64 * 32
+#define SK_LN_MAX_PER_LANE 16  // a prologue row is held in registers: k_dim <= 64 * 32
 #define SK_PAD 8  // bfloat16 elements of padding per LDS row: keeps the 16 rows a MFMA reads on distinct banks
 
 struct SkinnyArgs {
@@ -56,55 +56,111 @@ __device__ __forceinline__ bf16x8_t load8(const bf16_t* p) {
   return *reinterpret_cast<const bf16x8_t*>(p);
 }
 
+
 template <int NT, bool LN, int EPI, typename OT>
 __global__ __launch_bounds__(LN ? SK_LN_WAVES * 64 : SK_WAVES * 64) void linear_skinny_kernel(SkinnyArgs a) {
   extern __shared__ __align__(16) unsigned char smem[];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   constexpr int WAVES = LN ? SK_LN_WAVES : SK_WAVES;
+  constexpr int SK_BATCH = 4;  // k steps whose loads are issued together; the next batch is in flight meanwhile
   const int ks = a.ksplit, cw_per_wg = WAVES / ks;
   const int cw = wave / ks, kw = wave - cw * ks;
-  const int o0 = (blockIdx.x * cw_per_wg + cw) * 16;
   const int K = a.k_dim;
   const int ldh = K + SK_PAD;
-  bf16_t* hs = reinterpret_cast<bf16_t*>(smem);                       // [NT*16][ldh] when LN
-  float* red = reinterpret_cast<float*>(smem + (LN ? (size_t)NT * 16 * ldh * sizeof(bf16_t) : 0));
+  bf16_t* hs = reinterpret_cast<bf16_t*>(smem);                       // [16][ldh] when LN
+  float* red = reinterpret_cast<float*>(smem + (LN ? (size_t)16 * ldh * sizeof(bf16_t) : 0));
+
+  // this wave's k range, in steps of 32
+  const int k_per = ((K / ks + 31) / 32) * 32;
+  const int k_begin = kw * k_per;
+  const int k_end = (k_begin + k_per < K) ? k_begin + k_per : K;
+  const int steps = (k_end - k_begin + 31) / 32;
+  const int lrow = lane & 15, lk = (lane >> 4) * 8;
+  const int tiles = (a.n_out + 15) / 16;
+  const int n_groups = (tiles + cw_per_wg - 1) / cw_per_wg;
+  const bf16x8_t zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+
+  // Loads are unconditional (a lane that has nothing to load reads the start of its row and
+  // discards it), so that a whole batch of them is in flight before the first is waited for.
+  bf16x8_t wv[SK_BATCH], wn[SK_BATCH];
+  bf16x8_t av[NT][SK_BATCH], an[NT][SK_BATCH];
+  auto load_w = [&](bf16x8_t (&dst)[SK_BATCH], int o0, int sb) {
+    const int wo = o0 + lrow;
+    const bool w_ok = wo < a.n_out;
+    const bf16_t* wp = a.w + (long)(w_ok ? wo : 0) * K;
+#pragma unroll
+    for (int i = 0; i < SK_BATCH; ++i) {
+      const int k0 = k_begin + (sb + i) * 32 + lk;
+      const bool ok = w_ok && (sb + i) < steps && k0 + 8 <= k_end;
+      const bf16x8_t v = load8(wp + (ok ? k0 : 0));
+      dst[i] = ok ? v : zero8;
+    }
+  };
+  auto load_a = [&](bf16x8_t (&dst)[NT][SK_BATCH], int sb) {
+    if (LN) return;
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+      const int n = t * 16 + lrow;
+      const bool n_ok = n < a.n_rows;
+      const bf16_t* ap = a.act + (long)(n_ok ? n : 0) * a.lda;
+#pragma unroll
+      for (int i = 0; i < SK_BATCH; ++i) {
+        const int k0 = k_begin + (sb + i) * 32 + lk;
+        const bool ok = n_ok && (sb + i) < steps && k0 + 8 <= k_end;
+        const bf16x8_t v = load8(ap + (ok ? k0 : 0));
+        dst[t][i] = ok ? v : zero8;
+      }
+    }
+  };
+
+  int group = blockIdx.x;
+  // the first batch does not depend on the prologue: start it now
+  load_w(wv, (group * cw_per_wg + cw) * 16, 0);
+  load_a(av, 0);
 
   if (LN) {
-    // LayerNorm of up to 16 rows, one wave per row; the row is read once and kept in registers
-    // (the launcher sends more than 16 rows through a LayerNorm kernel of their own)
+    // LayerNorm of up to 16 rows, one wave per row, the row read once and kept in registers:
+    // the mean, then together the centred sum of squares and what the mean lost to rounding.
     const int r = wave;
     bf16_t* hr = hs + (long)r * ldh;
     if (r < a.n_rows) {
       const float* xr = a.x + (long)(a.rows ? a.rows[r] : r) * K;
-      float xv[SK_LN_MAX_PER_LANE];
-      float s = 0.f;
+      float xv[SK_LN_MAX_PER_LANE], gw[SK_LN_MAX_PER_LANE], gb[SK_LN_MAX_PER_LANE];
 #pragma unroll
       for (int i = 0; i < SK_LN_MAX_PER_LANE; ++i) {
         const int c = lane + i * 64;
-        xv[i] = c < K ? xr[c] : 0.f;
-        s += xv[i];
+        const bool ok = c < K;
+        xv[i] = xr[ok ? c : 0];
+        gw[i] = a.ln_w[ok ? c : 0];
+        gb[i] = a.ln_b ? a.ln_b[ok ? c : 0] : 0.f;
       }
-      const float mean = wave_sum(s) / (float)K;
-      float e = 0.f;
-#pragma unroll
-      for (int i = 0; i < SK_LN_MAX_PER_LANE; ++i) e += (lane + i * 64 < K) ? xv[i] - mean : 0.f;
-      const float corr = wave_sum(e) / (float)K;  // what the first sum lost to rounding, kept apart
-      float v = 0.f;
+      float s0 = 0.f;
 #pragma unroll
       for (int i = 0; i < SK_LN_MAX_PER_LANE; ++i) {
-        const float d = (lane + i * 64 < K) ? (xv[i] - mean) - corr : 0.f;
+        if (lane + i * 64 >= K) xv[i] = 0.f;
+        s0 += xv[i];
+      }
+      const float mean = wave_sum(s0) / (float)K;
+      float e = 0.f, v2 = 0.f;
+#pragma unroll
+      for (int i = 0; i < SK_LN_MAX_PER_LANE; ++i) {
+        const float d = (lane + i * 64 < K) ? xv[i] - mean : 0.f;
         xv[i] = d;
-        v += d * d;
+        e += d;
+        v2 = fmaf(d, d, v2);
       }
-      const float rstd = 1.0f / sqrtf(wave_sum(v) / (float)K + a.eps);
+#pragma unroll
+      for (int off = 32; off > 0; off >>= 1) {
+        e += __shfl_xor(e, off, 64);
+        v2 += __shfl_xor(v2, off, 64);
+      }
+      const float corr = e / (float)K;  // what the mean lost to rounding, kept apart
+      const float var = fmaxf(v2 / (float)K - corr * corr, 0.f);
+      const float rstd = 1.0f / sqrtf(var + a.eps);
 #pragma unroll
       for (int i = 0; i < SK_LN_MAX_PER_LANE; ++i) {
         const int c = lane + i * 64;
-        if (c < K) {
-          float y = xv[i] * rstd * a.ln_w[c];
-          if (a.ln_b) y += a.ln_b[c];
-          hr[c] = float_to_bf16(y);
-        }
+        if (c < K) hr[c] = float_to_bf16((xv[i] - corr) * rstd * gw[i] + gb[i]);
       }
     } else {
       for (int c = lane; c < K; c += 64) hr[c] = 0;
@@ -112,96 +168,104 @@ __global__ __launch_bounds__(LN ? SK_LN_WAVES * 64 : SK_WAVES * 64) void linear_
     __syncthreads();
   }
 
-  // this wave's k range, in steps of 32
-  const int k_per = ((K / ks + 31) / 32) * 32;
-  const int k_begin = kw * k_per;
-  const int k_end = (k_begin + k_per < K) ? k_begin + k_per : K;
-  const int lrow = lane & 15, lk = (lane >> 4) * 8;
-
-  f32x4_t acc[NT];
+  for (bool first = true; group < n_groups; group += gridDim.x, first = false) {
+    const int o0 = (group * cw_per_wg + cw) * 16;
+    f32x4_t acc[NT];
 #pragma unroll
-  for (int t = 0; t < NT; ++t) acc[t] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
-
-  const int wo = o0 + lrow;
-  const bool w_ok = wo < a.n_out;
-  const bf16_t* wp = a.w + (long)(w_ok ? wo : 0) * K + lk;
-  const bf16x8_t zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
-
-  if (o0 < a.n_out) {
-#pragma unroll 4
-    for (int k0 = k_begin; k0 < k_end; k0 += 32) {
-      const bool k_ok = k0 + lk + 8 <= k_end;
-      bf16x8_t wv = (w_ok && k_ok) ? load8(wp + k0) : zero8;
+    for (int t = 0; t < NT; ++t) acc[t] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+    if (!first) {
+      load_w(wv, o0, 0);
+      load_a(av, 0);
+    }
+    for (int sb = 0; sb < steps; sb += SK_BATCH) {
+      const bool more = sb + SK_BATCH < steps;
+      if (more) {
+        load_w(wn, o0, sb + SK_BATCH);
+        load_a(an, sb + SK_BATCH);
+      }
 #pragma unroll
-      for (int t = 0; t < NT; ++t) {
-        bf16x8_t av;
-        const int n = t * 16 + lrow;
-        if (LN) {
-          av = k_ok ? load8(hs + (long)n * ldh + k0 + lk) : zero8;
-        } else {
-          av = (k_ok && n < a.n_rows) ? load8(a.act + (long)n * a.lda + k0 + lk) : zero8;
+      for (int i = 0; i < SK_BATCH; ++i) {
+        const int k0 = k_begin + (sb + i) * 32 + lk;
+#pragma unroll
+        for (int t = 0; t < NT; ++t) {
+          bf16x8_t b;
+          if (LN) {
+            // rows of hs are readable up to K + SK_PAD; what lies past k_end meets zeros of W
+            b = load8(hs + (long)(t * 16 + lrow) * ldh + ((sb + i) < steps && k0 + 8 <= k_end ? k0 : 0));
+          } else {
+            b = av[t][i];
+          }
+          acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wv[i], b, acc[t], 0, 0, 0);
         }
-        acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wv, av, acc[t], 0, 0, 0);
+      }
+      if (more) {
+#pragma unroll
+        for (int i = 0; i < SK_BATCH; ++i) {
+          wv[i] = wn[i];
+#pragma unroll
+          for (int t = 0; t < NT; ++t) av[t][i] = an[t][i];
+        }
       }
     }
-  }
 
-  // waves that split k hand their sums to the first of them, which adds in wave order
-  if (ks > 1) {
-    if (kw > 0) {
-#pragma unroll
-      for (int t = 0; t < NT; ++t)
-#pragma unroll
-        for (int i = 0; i < 4; ++i) red[((wave * NT + t) * 4 + i) * 64 + lane] = acc[t][i];
-    }
-    __syncthreads();
-    if (kw == 0) {
-      for (int s = 1; s < ks; ++s)
+    // waves that split k hand their sums to the first of them, which adds in wave order
+    if (ks > 1) {
+      if (!first) __syncthreads();  // the previous group's sums have been read
+      if (kw > 0) {
 #pragma unroll
         for (int t = 0; t < NT; ++t)
 #pragma unroll
-          for (int i = 0; i < 4; ++i) acc[t][i] += red[(((wave + s) * NT + t) * 4 + i) * 64 + lane];
-    }
-  }
-  if (kw != 0 || o0 >= a.n_out) return;
-
-  // lane holds out[n = t*16 + (lane & 15)][o0 + (lane >> 4) * 4 + i], i = 0..3
-  const int oc = o0 + (lane >> 4) * 4;
+          for (int i = 0; i < 4; ++i) red[((wave * NT + t) * 4 + i) * 64 + lane] = acc[t][i];
+      }
+      __syncthreads();
+      if (kw == 0) {
+        for (int s = 1; s < ks; ++s)
 #pragma unroll
-  for (int t = 0; t < NT; ++t) {
-    const int n = t * 16 + lrow;
-    if (n >= a.n_rows) continue;
-    float v[4];
+          for (int t = 0; t < NT; ++t)
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      v[i] = acc[t][i];
-      if (a.bias && oc + i < a.n_out) v[i] += a.bias[oc + i];
-      if (EPI == SK_EPI_GELU) v[i] = gelu_tanh(v[i]);
-    }
-    OT* orow = reinterpret_cast<OT*>(a.out) + (long)n * a.ldo;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      if (oc + i >= a.n_out) continue;
-      if (EPI == SK_EPI_RESIDUAL) {
-        orow[oc + i] = from_float<OT>(to_float<OT>(orow[oc + i]) + v[i]);
-      } else {
-        orow[oc + i] = from_float<OT>(v[i]);
+            for (int i = 0; i < 4; ++i) acc[t][i] += red[(((wave + s) * NT + t) * 4 + i) * 64 + lane];
       }
     }
-    if (EPI == SK_EPI_QKV) {
-      const int slot = a.slot_mapping[n];
-      if (slot >= 0 && oc >= a.q_width) {
-        const long page = slot / a.page_size;
-        const int off = slot - (int)page * a.page_size;
+    if (kw != 0 || o0 >= a.n_out) continue;
+
+    // lane holds out[n = t*16 + (lane & 15)][o0 + (lane >> 4) * 4 + i], i = 0..3
+    const int oc = o0 + (lane >> 4) * 4;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const int c = oc + i - a.q_width;  // column among keys then values
-          if (oc + i >= a.n_out) continue;
-          const bool is_v = c >= a.kv_width;
-          const int cc = is_v ? c - a.kv_width : c;
-          const int h = cc / a.head_dim, d = cc - h * a.head_dim;
-          const long dst = ((page * a.n_kv_head + h) * a.page_size + off) * (long)a.head_dim + d;
-          (is_v ? a.vpool : a.kpool)[dst] = float_to_bf16(v[i]);
+    for (int t = 0; t < NT; ++t) {
+      const int n = t * 16 + lrow;
+      if (n >= a.n_rows) continue;
+      float v[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        v[i] = acc[t][i];
+        if (a.bias && oc + i < a.n_out) v[i] += a.bias[oc + i];
+        if (EPI == SK_EPI_GELU) v[i] = gelu_tanh(v[i]);
+      }
+      OT* orow = reinterpret_cast<OT*>(a.out) + (long)n * a.ldo;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        if (oc + i >= a.n_out) continue;
+        if (EPI == SK_EPI_RESIDUAL) {
+          orow[oc + i] = from_float<OT>(to_float<OT>(orow[oc + i]) + v[i]);
+        } else {
+          orow[oc + i] = from_float<OT>(v[i]);
+        }
+      }
+      if (EPI == SK_EPI_QKV) {
+        const int slot = a.slot_mapping[n];
+        if (slot >= 0 && oc >= a.q_width) {
+          const long page = slot / a.page_size;
+          const int off = slot - (int)page * a.page_size;
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const int c = oc + i - a.q_width;  // column among keys then values
+            if (oc + i >= a.n_out) continue;
+            const bool is_v = c >= a.kv_width;
+            const int cc = is_v ? c - a.kv_width : c;
+            const int h = cc / a.head_dim, d = cc - h * a.head_dim;
+            const long dst = ((page * a.n_kv_head + h) * a.page_size + off) * (long)a.head_dim + d;
+            (is_v ? a.vpool : a.kpool)[dst] = float_to_bf16(v[i]);
+          }
         }
       }
     }
@@ -267,7 +331,10 @@ extern "C" int mgpt_linear_skinny(const void* act, long lda, const float* x, con
   a.slot_mapping = slot_mapping; a.q_width = q_width; a.kv_width = kv_width; a.head_dim = head_dim;
   a.n_kv_head = n_kv_head; a.page_size = page_size;
   const int cw_per_wg = waves / ks;
-  dim3 grid((tiles + cw_per_wg - 1) / cw_per_wg);
+  const int n_groups = (tiles + cw_per_wg - 1) / cw_per_wg;
+  // with a prologue every workgroup repeats the LayerNorm, so few workgroups walk many column groups
+  const int max_wg = ln ? 256 : 2048;
+  dim3 grid(n_groups < max_wg ? n_groups : max_wg);
   const size_t smem = hs_bytes + red_bytes;
 #define SK_NT(N)                                                                         \
   (ln ? launch_nt<N, true>(a, epilogue, out_dtype, grid, smem, stream)                   \

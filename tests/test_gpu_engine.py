@@ -84,8 +84,10 @@ def test_chunked_mixed_and_whole_prompt_policies_give_the_same_tokens(model_fold
         outs.append(engine.generate(prompts, sp))
     if dtype == "float32":
         assert outs[0] == outs[1] == outs[2]
-    else:   # bfloat16 kernels differ between few and many rows; the first tokens still agree
-        assert [o[:4] for o in outs[0]] == [o[:4] for o in outs[1]] == [o[:4] for o in outs[2]]
+    else:   # bfloat16 kernels differ between few and many rows: each choice is the argmax up to rounding
+        for out in outs:
+            for prompt, tokens in zip(prompts, out):
+                _assert_greedy_within_tolerance(model_folders["B"], prompt, tokens, dtype)
 
 
 def test_seeded_temperature_sampling_is_reproducible_and_independent_of_batching(model_folders):
@@ -130,7 +132,8 @@ def test_pages_run_out_preempted_request_is_recomputed_and_ends_with_the_same_to
     if dtype == "float32":
         assert tight == roomy == _plain_greedy(model_folders["A"], prompts, 4)
     else:
-        assert [t[:2] for t in tight] == [r[:2] for r in roomy]
+        for prompt, tokens in zip(prompts, tight):
+            _assert_greedy_within_tolerance(model_folders["A"], prompt, tokens, dtype)
 
 
 def test_step_outputs_finish_reasons_eot_and_cancel(model_folders):
