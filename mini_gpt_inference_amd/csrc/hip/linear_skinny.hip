@@ -57,11 +57,10 @@ __device__ __forceinline__ bf16x8_t load8(const bf16_t* p) {
 }
 
 
-template <int NT, bool LN, int EPI, typename OT>
-__global__ __launch_bounds__(LN ? SK_LN_WAVES * 64 : SK_WAVES * 64) void linear_skinny_kernel(SkinnyArgs a) {
+template <int NT, bool LN, int WAVES, int EPI, typename OT>
+__global__ __launch_bounds__(WAVES * 64) void linear_skinny_kernel(SkinnyArgs a) {
   extern __shared__ __align__(16) unsigned char smem[];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  constexpr int WAVES = LN ? SK_LN_WAVES : SK_WAVES;
   constexpr int SK_BATCH = 4;  // k steps whose loads are issued together; the next batch is in flight meanwhile
   const int ks = a.ksplit, cw_per_wg = WAVES / ks;
   const int cw = wave / ks, kw = wave - cw * ks;
@@ -242,40 +241,56 @@ __global__ __launch_bounds__(LN ? SK_LN_WAVES * 64 : SK_WAVES * 64) void linear_
         if (EPI == SK_EPI_GELU) v[i] = gelu_tanh(v[i]);
       }
       OT* orow = reinterpret_cast<OT*>(a.out) + (long)n * a.ldo;
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        if (oc + i >= a.n_out) continue;
+      const bool whole = oc + 4 <= a.n_out && (a.ldo & 3) == 0;  // four columns, one aligned vector
+      if (whole && sizeof(OT) == 4) {
+        float4* dst = reinterpret_cast<float4*>(orow + oc);
+        float4 r = make_float4(v[0], v[1], v[2], v[3]);
         if (EPI == SK_EPI_RESIDUAL) {
-          orow[oc + i] = from_float<OT>(to_float<OT>(orow[oc + i]) + v[i]);
-        } else {
-          orow[oc + i] = from_float<OT>(v[i]);
+          const float4 old = *dst;
+          r = make_float4(old.x + v[0], old.y + v[1], old.z + v[2], old.w + v[3]);
+        }
+        *dst = r;
+      } else if (whole && EPI != SK_EPI_RESIDUAL) {
+        uint2 pk;
+        pk.x = (unsigned int)float_to_bf16(v[0]) | ((unsigned int)float_to_bf16(v[1]) << 16);
+        pk.y = (unsigned int)float_to_bf16(v[2]) | ((unsigned int)float_to_bf16(v[3]) << 16);
+        *reinterpret_cast<uint2*>(orow + oc) = pk;
+      } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          if (oc + i >= a.n_out) continue;
+          if (EPI == SK_EPI_RESIDUAL) {
+            orow[oc + i] = from_float<OT>(to_float<OT>(orow[oc + i]) + v[i]);
+          } else {
+            orow[oc + i] = from_float<OT>(v[i]);
+          }
         }
       }
       if (EPI == SK_EPI_QKV) {
         const int slot = a.slot_mapping[n];
-        if (slot >= 0 && oc >= a.q_width) {
+        if (slot >= 0 && oc >= a.q_width && oc < a.n_out) {
+          // the four columns lie in one head (head sizes are multiples of 4): one 8-byte store
           const long page = slot / a.page_size;
           const int off = slot - (int)page * a.page_size;
-#pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            const int c = oc + i - a.q_width;  // column among keys then values
-            if (oc + i >= a.n_out) continue;
-            const bool is_v = c >= a.kv_width;
-            const int cc = is_v ? c - a.kv_width : c;
-            const int h = cc / a.head_dim, d = cc - h * a.head_dim;
-            const long dst = ((page * a.n_kv_head + h) * a.page_size + off) * (long)a.head_dim + d;
-            (is_v ? a.vpool : a.kpool)[dst] = float_to_bf16(v[i]);
-          }
+          const int c = oc - a.q_width;  // column among keys then values
+          const bool is_v = c >= a.kv_width;
+          const int cc = is_v ? c - a.kv_width : c;
+          const int h = cc / a.head_dim, d = cc - h * a.head_dim;
+          const long dst = ((page * a.n_kv_head + h) * a.page_size + off) * (long)a.head_dim + d;
+          uint2 pk;
+          pk.x = (unsigned int)float_to_bf16(v[0]) | ((unsigned int)float_to_bf16(v[1]) << 16);
+          pk.y = (unsigned int)float_to_bf16(v[2]) | ((unsigned int)float_to_bf16(v[3]) << 16);
+          *reinterpret_cast<uint2*>((is_v ? a.vpool : a.kpool) + dst) = pk;
         }
       }
     }
   }
 }
 
-template <int NT, bool LN>
+template <int NT, bool LN, int WAVES>
 static int launch_nt(const SkinnyArgs& a, int epi, int out_dtype, dim3 grid, size_t smem, hipStream_t s) {
 #define SK_LAUNCH(E, OT) \
-  hipLaunchKernelGGL((linear_skinny_kernel<NT, LN, E, OT>), grid, dim3((LN ? SK_LN_WAVES : SK_WAVES) * 64), smem, s, a)
+  hipLaunchKernelGGL((linear_skinny_kernel<NT, LN, WAVES, E, OT>), grid, dim3(WAVES * 64), smem, s, a)
   if (epi == SK_EPI_NONE && out_dtype == MGPT_BF16) SK_LAUNCH(SK_EPI_NONE, bf16_t);
   else if (epi == SK_EPI_NONE && out_dtype == MGPT_F32) SK_LAUNCH(SK_EPI_NONE, float);
   else if (epi == SK_EPI_GELU && out_dtype == MGPT_BF16) SK_LAUNCH(SK_EPI_GELU, bf16_t);
@@ -312,17 +327,17 @@ extern "C" int mgpt_linear_skinny(const void* act, long lda, const float* x, con
       return MGPT_ERR_BAD_SHAPE;
   }
   const int nt = (n_rows + 15) / 16;
-  const int waves = ln ? SK_LN_WAVES : SK_WAVES;
-  // waves sharing a column tile: as many as keep every wave at least 64 k wide and the grid large
+  // Sixteen waves with the prologue (one per row) and for long inner sizes, where splitting k
+  // sixteen ways keeps every wave's loads to one batch; four otherwise.
+  const int waves = (ln || (k_dim >= 1024 && nt <= 2)) ? SK_LN_WAVES : SK_WAVES;  // more row tiles need the registers
+  // waves sharing a column tile: as many as keep every wave at least 128 k wide and the grid large
   int ks = 1;
   const int tiles = (n_out + 15) / 16;
-  while (ks < 4 && (k_dim % (64 * ks)) == 0 && k_dim / (ks * 2) >= 64 && tiles / (waves / ks) < 1024) ks *= 2;
+  while (ks < waves && (k_dim % (64 * ks)) == 0 && k_dim / (ks * 2) >= 128 && tiles / (waves / ks) < 1024) ks *= 2;
   const size_t hs_bytes = ln ? (size_t)16 * (k_dim + SK_PAD) * sizeof(bf16_t) : 0;
-  size_t red_bytes = ks > 1 ? (size_t)waves * nt * 4 * 64 * sizeof(float) : 0;
-  if (hs_bytes + red_bytes > 64 * 1024) {  // give up the k split before giving up the kernel
-    ks = 1;
-    red_bytes = 0;
-  }
+  auto red_of = [&](int k) { return k > 1 ? (size_t)waves * nt * 4 * 64 * sizeof(float) : (size_t)0; };
+  while (ks > 1 && hs_bytes + red_of(ks) > 64 * 1024) ks = 1;  // give up the k split before the kernel
+  const size_t red_bytes = red_of(ks);
   if (hs_bytes + red_bytes > 64 * 1024) return MGPT_ERR_BAD_SHAPE;
   SkinnyArgs a;
   a.act = (const bf16_t*)act; a.lda = lda; a.x = x; a.rows = rows; a.ln_w = ln_w; a.ln_b = ln_b; a.eps = eps;
@@ -336,9 +351,10 @@ extern "C" int mgpt_linear_skinny(const void* act, long lda, const float* x, con
   const int max_wg = ln ? 256 : 2048;
   dim3 grid(n_groups < max_wg ? n_groups : max_wg);
   const size_t smem = hs_bytes + red_bytes;
-#define SK_NT(N)                                                                         \
-  (ln ? launch_nt<N, true>(a, epilogue, out_dtype, grid, smem, stream)                   \
-      : launch_nt<N, false>(a, epilogue, out_dtype, grid, smem, stream))
+#define SK_NT(N)                                                                                   \
+  (ln ? launch_nt<N, true, SK_LN_WAVES>(a, epilogue, out_dtype, grid, smem, stream)                \
+      : (waves == SK_LN_WAVES ? launch_nt<N, false, SK_LN_WAVES>(a, epilogue, out_dtype, grid, smem, stream) \
+                              : launch_nt<N, false, SK_WAVES>(a, epilogue, out_dtype, grid, smem, stream)))
   switch (nt) {
     case 1: return SK_NT(1);
     case 2: return SK_NT(2);
