@@ -9,10 +9,12 @@
 // and 16 rows of activations into float32 sums.  Waves that split k add their
 // sums through LDS in a fixed order, so results do not depend on timing.
 //
-// Prologue (optional): LayerNorm of the float32 residual rows, statistics in
-// float32, result in bfloat16 in LDS (src/minigpt_infer/model.py:113-114: every
-// linear that reads the residual stream reads it through a LayerNorm), with an
-// optional gather of rows (the logit rows of the output head).
+// Reading the residual stream through a LayerNorm (src/minigpt_infer/model.py:113-114,186-187:
+// every linear that reads the residual stream does): the LayerNorm's gain and bias are folded
+// into W beforehand (fold_norm.hip), the kernel multiplies the raw float32 rows (rounded to
+// bfloat16 on the way into the MFMA, with an optional gather of rows for the output head),
+// gathers each row's sum and sum of squares from the very values it loads, and applies
+// rstd * (acc - mean * S[o]) + b'[o] in the epilogue.  Nothing waits for the statistics.
 // Epilogues: plain store (bfloat16 or float32), GELU-tanh, add into the float32
 // residual stream, or store plus scatter of the key and value columns into
 // their cache pages by slot_mapping (src/minigpt_infer/cache/paged.py:125-137).
@@ -28,19 +30,16 @@ typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4_t;
 
 #define SK_WAVES 4        // waves of a workgroup without a prologue
 #define SK_LN_WAVES 16    // waves of a workgroup with the LayerNorm prologue: one row each
-#define SK_LN_MAX_PER_LANE 16  // a prologue row is held in registers: k_dim <= 64 * 32
-#define SK_PAD 8  // bfloat16 elements of padding per LDS row: keeps the 16 rows a MFMA reads on distinct banks
 
 struct SkinnyArgs {
   const bf16_t* act;  // [n_rows, k_dim] bfloat16, row stride lda (no prologue)
   long lda;
-  const float* x;     // residual stream, float32, row stride k_dim (LayerNorm prologue)
+  const float* x;     // residual stream, float32, row stride k_dim (folded LayerNorm)
   const int* rows;    // optional gather of residual rows
-  const float* ln_w;
-  const float* ln_b;
+  const float* colsum;  // S[o] of the folded matrix
   float eps;
-  const bf16_t* w;    // [n_out, k_dim]
-  const float* bias;  // [n_out] or null
+  const bf16_t* w;    // [n_out, k_dim] (the folded matrix when x is given)
+  const float* bias;  // [n_out] or null (the folded bias when x is given)
   void* out;          // [n_rows, n_out], row stride ldo
   long ldo;
   int n_rows, n_out, k_dim;
@@ -65,9 +64,8 @@ __global__ __launch_bounds__(WAVES * 64) void linear_skinny_kernel(SkinnyArgs a)
   const int ks = a.ksplit, cw_per_wg = WAVES / ks;
   const int cw = wave / ks, kw = wave - cw * ks;
   const int K = a.k_dim;
-  const int ldh = K + SK_PAD;
-  bf16_t* hs = reinterpret_cast<bf16_t*>(smem);                       // [16][ldh] when LN
-  float* red = reinterpret_cast<float*>(smem + (LN ? (size_t)16 * ldh * sizeof(bf16_t) : 0));
+  float* red = reinterpret_cast<float*>(smem);   // [wave][NT][4 sums (+ 2 statistics)][64 lanes]
+  constexpr int RED_PER = LN ? 6 : 4;
 
   // this wave's k range, in steps of 32
   const int k_per = ((K / ks + 31) / 32) * 32;
@@ -83,6 +81,20 @@ __global__ __launch_bounds__(WAVES * 64) void linear_skinny_kernel(SkinnyArgs a)
   // discards it), so that a whole batch of them is in flight before the first is waited for.
   bf16x8_t wv[SK_BATCH], wn[SK_BATCH];
   bf16x8_t av[NT][SK_BATCH], an[NT][SK_BATCH];
+  // folded LayerNorm: sums of (x - x0) and (x - x0)^2 over what this lane loads of its rows
+  float x0[NT], sd[NT], sq[NT];
+  const float* xrow[NT];
+#pragma unroll
+  for (int t = 0; t < NT; ++t) {
+    sd[t] = sq[t] = x0[t] = 0.f;
+    xrow[t] = nullptr;
+    if (LN) {
+      const int n = t * 16 + lrow;
+      const int src = n < a.n_rows ? (a.rows ? a.rows[n] : n) : 0;
+      xrow[t] = a.x + (long)src * K;
+      x0[t] = xrow[t][0];
+    }
+  }
   auto load_w = [&](bf16x8_t (&dst)[SK_BATCH], int o0, int sb) {
     const int wo = o0 + lrow;
     const bool w_ok = wo < a.n_out;
@@ -95,115 +107,110 @@ __global__ __launch_bounds__(WAVES * 64) void linear_skinny_kernel(SkinnyArgs a)
       dst[i] = ok ? v : zero8;
     }
   };
-  auto load_a = [&](bf16x8_t (&dst)[NT][SK_BATCH], int sb) {
-    if (LN) return;
+  auto load_a = [&](bf16x8_t (&dst)[NT][SK_BATCH], int sb, bool stats) {
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
       const int n = t * 16 + lrow;
       const bool n_ok = n < a.n_rows;
-      const bf16_t* ap = a.act + (long)(n_ok ? n : 0) * a.lda;
+      if (LN) {
+        float4 lo[SK_BATCH], hi[SK_BATCH];
 #pragma unroll
-      for (int i = 0; i < SK_BATCH; ++i) {
-        const int k0 = k_begin + (sb + i) * 32 + lk;
-        const bool ok = n_ok && (sb + i) < steps && k0 + 8 <= k_end;
-        const bf16x8_t v = load8(ap + (ok ? k0 : 0));
-        dst[t][i] = ok ? v : zero8;
+        for (int i = 0; i < SK_BATCH; ++i) {
+          const int k0 = k_begin + (sb + i) * 32 + lk;
+          const bool ok = (sb + i) < steps && k0 + 8 <= k_end;
+          const float4* p = reinterpret_cast<const float4*>(xrow[t] + (ok ? k0 : 0));
+          lo[i] = p[0];
+          hi[i] = p[1];
+        }
+#pragma unroll
+        for (int i = 0; i < SK_BATCH; ++i) {
+          const int k0 = k_begin + (sb + i) * 32 + lk;
+          const bool ok = n_ok && (sb + i) < steps && k0 + 8 <= k_end;
+          const float f[8] = {lo[i].x, lo[i].y, lo[i].z, lo[i].w, hi[i].x, hi[i].y, hi[i].z, hi[i].w};
+          bf16x8_t v;
+#pragma unroll
+          for (int e = 0; e < 8; ++e) {
+            v[e] = (short)float_to_bf16(f[e]);
+            if (ok && stats) {
+              const float d = f[e] - x0[t];
+              sd[t] += d;
+              sq[t] = fmaf(d, d, sq[t]);
+            }
+          }
+          dst[t][i] = ok ? v : zero8;
+        }
+      } else {
+        const bf16_t* ap = a.act + (long)(n_ok ? n : 0) * a.lda;
+#pragma unroll
+        for (int i = 0; i < SK_BATCH; ++i) {
+          const int k0 = k_begin + (sb + i) * 32 + lk;
+          const bool ok = n_ok && (sb + i) < steps && k0 + 8 <= k_end;
+          const bf16x8_t v = load8(ap + (ok ? k0 : 0));
+          dst[t][i] = ok ? v : zero8;
+        }
       }
     }
   };
 
   int group = blockIdx.x;
-  // the first batch does not depend on the prologue: start it now
-  load_w(wv, (group * cw_per_wg + cw) * 16, 0);
-  load_a(av, 0);
-
-  if (LN) {
-    // LayerNorm of up to 16 rows, one wave per row, the row read once and kept in registers:
-    // the mean, then together the centred sum of squares and what the mean lost to rounding.
-    const int r = wave;
-    bf16_t* hr = hs + (long)r * ldh;
-    if (r < a.n_rows) {
-      const float* xr = a.x + (long)(a.rows ? a.rows[r] : r) * K;
-      float xv[SK_LN_MAX_PER_LANE], gw[SK_LN_MAX_PER_LANE], gb[SK_LN_MAX_PER_LANE];
-#pragma unroll
-      for (int i = 0; i < SK_LN_MAX_PER_LANE; ++i) {
-        const int c = lane + i * 64;
-        const bool ok = c < K;
-        xv[i] = xr[ok ? c : 0];
-        gw[i] = a.ln_w[ok ? c : 0];
-        gb[i] = a.ln_b ? a.ln_b[ok ? c : 0] : 0.f;
-      }
-      float s0 = 0.f;
-#pragma unroll
-      for (int i = 0; i < SK_LN_MAX_PER_LANE; ++i) {
-        if (lane + i * 64 >= K) xv[i] = 0.f;
-        s0 += xv[i];
-      }
-      const float mean = wave_sum(s0) / (float)K;
-      float e = 0.f, v2 = 0.f;
-#pragma unroll
-      for (int i = 0; i < SK_LN_MAX_PER_LANE; ++i) {
-        const float d = (lane + i * 64 < K) ? xv[i] - mean : 0.f;
-        xv[i] = d;
-        e += d;
-        v2 = fmaf(d, d, v2);
-      }
-#pragma unroll
-      for (int off = 32; off > 0; off >>= 1) {
-        e += __shfl_xor(e, off, 64);
-        v2 += __shfl_xor(v2, off, 64);
-      }
-      const float corr = e / (float)K;  // what the mean lost to rounding, kept apart
-      const float var = fmaxf(v2 / (float)K - corr * corr, 0.f);
-      const float rstd = 1.0f / sqrtf(var + a.eps);
-#pragma unroll
-      for (int i = 0; i < SK_LN_MAX_PER_LANE; ++i) {
-        const int c = lane + i * 64;
-        if (c < K) hr[c] = float_to_bf16((xv[i] - corr) * rstd * gw[i] + gb[i]);
-      }
-    } else {
-      for (int c = lane; c < K; c += 64) hr[c] = 0;
-    }
-    __syncthreads();
+  // When a wave's k range fits one batch its activations are loaded once and serve every column
+  // group the workgroup walks; the next group's W is then in flight while this one is multiplied.
+  const bool one_batch = steps <= SK_BATCH;
+  if (group < n_groups) {
+    load_w(wv, (group * cw_per_wg + cw) * 16, 0);
+    load_a(av, 0, true);
   }
-
   for (bool first = true; group < n_groups; group += gridDim.x, first = false) {
     const int o0 = (group * cw_per_wg + cw) * 16;
     f32x4_t acc[NT];
 #pragma unroll
     for (int t = 0; t < NT; ++t) acc[t] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
-    if (!first) {
-      load_w(wv, o0, 0);
-      load_a(av, 0);
-    }
-    for (int sb = 0; sb < steps; sb += SK_BATCH) {
-      const bool more = sb + SK_BATCH < steps;
-      if (more) {
-        load_w(wn, o0, sb + SK_BATCH);
-        load_a(an, sb + SK_BATCH);
+    if (one_batch) {
+      const int next = group + gridDim.x;
+      if (next < n_groups) load_w(wn, (next * cw_per_wg + cw) * 16, 0);
+#pragma unroll
+      for (int i = 0; i < SK_BATCH; ++i)
+#pragma unroll
+        for (int t = 0; t < NT; ++t)
+          acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wv[i], av[t][i], acc[t], 0, 0, 0);
+      if (next < n_groups) {
+#pragma unroll
+        for (int i = 0; i < SK_BATCH; ++i) wv[i] = wn[i];
       }
+    } else {
+      if (!first) {
+        load_w(wv, o0, 0);
+        load_a(av, 0, false);
+      }
+      for (int sb = 0; sb < steps; sb += SK_BATCH) {
+        const bool more = sb + SK_BATCH < steps;
+        if (more) {
+          load_w(wn, o0, sb + SK_BATCH);
+          load_a(an, sb + SK_BATCH, first);
+        }
 #pragma unroll
-      for (int i = 0; i < SK_BATCH; ++i) {
-        const int k0 = k_begin + (sb + i) * 32 + lk;
+        for (int i = 0; i < SK_BATCH; ++i)
 #pragma unroll
-        for (int t = 0; t < NT; ++t) {
-          bf16x8_t b;
-          if (LN) {
-            // rows of hs are readable up to K + SK_PAD; what lies past k_end meets zeros of W
-            b = load8(hs + (long)(t * 16 + lrow) * ldh + ((sb + i) < steps && k0 + 8 <= k_end ? k0 : 0));
-          } else {
-            b = av[t][i];
+          for (int t = 0; t < NT; ++t)
+            acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wv[i], av[t][i], acc[t], 0, 0, 0);
+        if (more) {
+#pragma unroll
+          for (int i = 0; i < SK_BATCH; ++i) {
+            wv[i] = wn[i];
+#pragma unroll
+            for (int t = 0; t < NT; ++t) av[t][i] = an[t][i];
           }
-          acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wv[i], b, acc[t], 0, 0, 0);
         }
       }
-      if (more) {
+    }
+    if (LN && first) {
+      // the four lanes that share a row hold parts of its sums: add them
 #pragma unroll
-        for (int i = 0; i < SK_BATCH; ++i) {
-          wv[i] = wn[i];
-#pragma unroll
-          for (int t = 0; t < NT; ++t) av[t][i] = an[t][i];
-        }
+      for (int t = 0; t < NT; ++t) {
+        sd[t] += __shfl_xor(sd[t], 16, 64);
+        sd[t] += __shfl_xor(sd[t], 32, 64);
+        sq[t] += __shfl_xor(sq[t], 16, 64);
+        sq[t] += __shfl_xor(sq[t], 32, 64);
       }
     }
 
@@ -212,17 +219,27 @@ __global__ __launch_bounds__(WAVES * 64) void linear_skinny_kernel(SkinnyArgs a)
       if (!first) __syncthreads();  // the previous group's sums have been read
       if (kw > 0) {
 #pragma unroll
-        for (int t = 0; t < NT; ++t)
+        for (int t = 0; t < NT; ++t) {
 #pragma unroll
-          for (int i = 0; i < 4; ++i) red[((wave * NT + t) * 4 + i) * 64 + lane] = acc[t][i];
+          for (int i = 0; i < 4; ++i) red[((wave * NT + t) * RED_PER + i) * 64 + lane] = acc[t][i];
+          if (LN && first) {
+            red[((wave * NT + t) * RED_PER + 4) * 64 + lane] = sd[t];
+            red[((wave * NT + t) * RED_PER + 5) * 64 + lane] = sq[t];
+          }
+        }
       }
       __syncthreads();
       if (kw == 0) {
         for (int s = 1; s < ks; ++s)
 #pragma unroll
-          for (int t = 0; t < NT; ++t)
+          for (int t = 0; t < NT; ++t) {
 #pragma unroll
-            for (int i = 0; i < 4; ++i) acc[t][i] += red[(((wave + s) * NT + t) * 4 + i) * 64 + lane];
+            for (int i = 0; i < 4; ++i) acc[t][i] += red[(((wave + s) * NT + t) * RED_PER + i) * 64 + lane];
+            if (LN && first) {
+              sd[t] += red[(((wave + s) * NT + t) * RED_PER + 4) * 64 + lane];
+              sq[t] += red[(((wave + s) * NT + t) * RED_PER + 5) * 64 + lane];
+            }
+          }
       }
     }
     if (kw != 0 || o0 >= a.n_out) continue;
@@ -234,9 +251,16 @@ __global__ __launch_bounds__(WAVES * 64) void linear_skinny_kernel(SkinnyArgs a)
       const int n = t * 16 + lrow;
       if (n >= a.n_rows) continue;
       float v[4];
+      float mean = 0.f, rstd = 1.f;
+      if (LN) {
+        const float md = sd[t] / (float)K;   // mean of x - x0
+        mean = x0[t] + md;
+        rstd = 1.0f / sqrtf(fmaxf(sq[t] / (float)K - md * md, 0.f) + a.eps);
+      }
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         v[i] = acc[t][i];
+        if (LN && oc + i < a.n_out) v[i] = rstd * (v[i] - mean * a.colsum[oc + i]);
         if (a.bias && oc + i < a.n_out) v[i] += a.bias[oc + i];
         if (EPI == SK_EPI_GELU) v[i] = gelu_tanh(v[i]);
       }
@@ -301,12 +325,12 @@ static int launch_nt(const SkinnyArgs& a, int epi, int out_dtype, dim3 grid, siz
   return mgpt_last_error();
 }
 
-// LayerNorm prologue when x is given (then act is ignored), plain bfloat16 activations otherwise.
-// Refuses (MGPT_ERR_BAD_SHAPE) more than 64 rows, k_dim that is no multiple of 16, and a LayerNorm
-// prologue for more than 16 rows or rows that do not fit 64 KB of LDS; the caller then runs the
-// LayerNorm by itself, or takes the general kernels.
+// With x given (then act is ignored) the rows are read from the float32 residual stream through
+// a LayerNorm whose gain and bias were folded into w, bias and colsum (fold_norm.hip); otherwise
+// act holds bfloat16 activations.  Refuses (MGPT_ERR_BAD_SHAPE) more than 64 rows and k_dim that
+// is no multiple of 16; the caller then takes the general kernels.
 extern "C" int mgpt_linear_skinny(const void* act, long lda, const float* x, const int* rows,
-                                  const float* ln_w, const float* ln_b, float eps, const void* w,
+                                  const float* colsum, float eps, const void* w,
                                   const float* bias, void* out, int out_dtype, long ldo, int n_rows,
                                   int n_out, int k_dim, int epilogue, void* kpool, void* vpool,
                                   const int* slot_mapping, int q_width, int kv_width, int head_dim,
@@ -316,9 +340,7 @@ extern "C" int mgpt_linear_skinny(const void* act, long lda, const float* x, con
   if (n_rows < 0 || n_rows > 64 || n_out < 0 || k_dim <= 0 || (k_dim % 16) != 0 || ldo < n_out)
     return MGPT_ERR_BAD_SHAPE;
   const bool ln = x != nullptr;
-  if (ln && !ln_w) return MGPT_ERR_NULL;
-  // the prologue normalises at most 16 rows (one per wave), each held in registers
-  if (ln && (n_rows > 16 || k_dim > 64 * SK_LN_MAX_PER_LANE)) return MGPT_ERR_BAD_SHAPE;
+  if (ln && !colsum) return MGPT_ERR_NULL;
   if (!ln && (lda < k_dim || (lda % 8) != 0)) return MGPT_ERR_BAD_SHAPE;
   if (epilogue == SK_EPI_QKV) {
     if (!kpool || !vpool || !slot_mapping) return MGPT_ERR_NULL;
@@ -327,36 +349,39 @@ extern "C" int mgpt_linear_skinny(const void* act, long lda, const float* x, con
       return MGPT_ERR_BAD_SHAPE;
   }
   const int nt = (n_rows + 15) / 16;
-  // Sixteen waves with the prologue (one per row) and for long inner sizes, where splitting k
-  // sixteen ways keeps every wave's loads to one batch; four otherwise.
-  const int waves = (ln || (k_dim >= 1024 && nt <= 2)) ? SK_LN_WAVES : SK_WAVES;  // more row tiles need the registers
-  // waves sharing a column tile: as many as keep every wave at least 128 k wide and the grid large
+  // Sixteen waves for long inner sizes, where splitting k sixteen ways keeps every wave's loads
+  // to one batch (only with one row tile of bfloat16 activations: more need the registers).
+  const int waves = (k_dim >= 1024 && nt == 1 && !ln) ? SK_LN_WAVES : SK_WAVES;
+  // waves sharing a column tile: as many as keep every wave at least 128 k wide
   int ks = 1;
   const int tiles = (n_out + 15) / 16;
-  while (ks < waves && (k_dim % (64 * ks)) == 0 && k_dim / (ks * 2) >= 128 && tiles / (waves / ks) < 1024) ks *= 2;
-  const size_t hs_bytes = ln ? (size_t)16 * (k_dim + SK_PAD) * sizeof(bf16_t) : 0;
-  auto red_of = [&](int k) { return k > 1 ? (size_t)waves * nt * 4 * 64 * sizeof(float) : (size_t)0; };
-  while (ks > 1 && hs_bytes + red_of(ks) > 64 * 1024) ks = 1;  // give up the k split before the kernel
-  const size_t red_bytes = red_of(ks);
-  if (hs_bytes + red_bytes > 64 * 1024) return MGPT_ERR_BAD_SHAPE;
+  // (a very wide output has waves enough without a split, and then needs no reduction through LDS)
+  while (tiles < 1024 && ks < waves && (k_dim % (64 * ks)) == 0 && k_dim / (ks * 2) >= 128) ks *= 2;
+  const int red_per = ln ? 6 : 4;
+  size_t red_bytes = ks > 1 ? (size_t)waves * nt * red_per * 64 * sizeof(float) : 0;
+  if (red_bytes > 64 * 1024) {  // give up the k split before giving up the kernel
+    ks = 1;
+    red_bytes = 0;
+  }
   SkinnyArgs a;
-  a.act = (const bf16_t*)act; a.lda = lda; a.x = x; a.rows = rows; a.ln_w = ln_w; a.ln_b = ln_b; a.eps = eps;
+  a.act = (const bf16_t*)act; a.lda = lda; a.x = x; a.rows = rows; a.colsum = colsum; a.eps = eps;
   a.w = (const bf16_t*)w; a.bias = bias; a.out = out; a.ldo = ldo; a.n_rows = n_rows; a.n_out = n_out;
   a.k_dim = k_dim; a.ksplit = ks; a.kpool = (bf16_t*)kpool; a.vpool = (bf16_t*)vpool;
   a.slot_mapping = slot_mapping; a.q_width = q_width; a.kv_width = kv_width; a.head_dim = head_dim;
   a.n_kv_head = n_kv_head; a.page_size = page_size;
   const int cw_per_wg = waves / ks;
   const int n_groups = (tiles + cw_per_wg - 1) / cw_per_wg;
-  // with a prologue every workgroup repeats the LayerNorm, so few workgroups walk many column groups
-  const int max_wg = ln ? 256 : 2048;
-  dim3 grid(n_groups < max_wg ? n_groups : max_wg);
-  const size_t smem = hs_bytes + red_bytes;
-#define SK_NT(N)                                                                                   \
-  (ln ? launch_nt<N, true, SK_LN_WAVES>(a, epilogue, out_dtype, grid, smem, stream)                \
-      : (waves == SK_LN_WAVES ? launch_nt<N, false, SK_LN_WAVES>(a, epilogue, out_dtype, grid, smem, stream) \
-                              : launch_nt<N, false, SK_WAVES>(a, epilogue, out_dtype, grid, smem, stream)))
+  // few enough workgroups that each walks several column groups and reuses its activations
+  dim3 grid(n_groups < 1024 ? n_groups : 1024);
+  const size_t smem = red_bytes;
+#define SK_NT(N)                                                                       \
+  (ln ? launch_nt<N, true, SK_WAVES>(a, epilogue, out_dtype, grid, smem, stream)       \
+      : launch_nt<N, false, SK_WAVES>(a, epilogue, out_dtype, grid, smem, stream))
   switch (nt) {
-    case 1: return SK_NT(1);
+    case 1:
+      if (waves == SK_LN_WAVES)
+        return launch_nt<1, false, SK_LN_WAVES>(a, epilogue, out_dtype, grid, smem, stream);
+      return SK_NT(1);
     case 2: return SK_NT(2);
     case 3: return SK_NT(3);
     default: return SK_NT(4);

@@ -62,6 +62,9 @@ class Scheduler:
         cap = max(max_batch_size, 1)
         self._e = [np.zeros(cap, dtype=np.int32) for _ in range(4)]
         self._o = [np.zeros(cap, dtype=np.int32) for _ in range(4)]
+        self._ep = [_p(a) for a in self._e]
+        self._op = [_p(a) for a in self._o]
+        self._cp = _p(self._counts)
 
     def __del__(self) -> None:
         h, self._h = getattr(self, "_h", None), None
@@ -88,28 +91,31 @@ class Scheduler:
 
     def schedule(self) -> Tuple[int, int, int]:
         """Plans the next step.  Returns (tokens, entries, entries that sample)."""
-        r = self._lib.mgpt_sched_schedule(self._h, _p(self._counts))
+        r = self._lib.mgpt_sched_schedule(self._h, self._cp)
         if r < 0:
             raise SchedulerError(library.host_error())
         return int(self._counts[0]), int(self._counts[1]), int(self._counts[2])
 
     def entries(self) -> List[StepEntry]:
-        n = self._lib.mgpt_sched_entries(self._h, *[_p(a) for a in self._e], self._e[0].size)
+        n = self._lib.mgpt_sched_entries(self._h, *self._ep, self._e[0].size)
         return [StepEntry(int(self._e[0][i]), int(self._e[1][i]), int(self._e[2][i]), bool(self._e[3][i]))
                 for i in range(n)]
 
     def entry_arrays(self) -> Tuple[np.ndarray, np.ndarray, np.ndarray, np.ndarray]:
-        n = self._lib.mgpt_sched_entries(self._h, *[_p(a) for a in self._e], self._e[0].size)
+        n = self._lib.mgpt_sched_entries(self._h, *self._ep, self._e[0].size)
         return tuple(a[:n] for a in self._e)
 
     def fill(self, arena) -> None:
         """Writes the planned step into a StepArena's host arrays."""
-        h = arena.h
-        rc = self._lib.mgpt_sched_fill(
-            self._h, self.cache.handle, arena.n_cap, arena.r_cap, arena.m_cap, arena.max_blocks,
-            _p(h["token_ids"]), _p(h["positions"]), _p(h["q_req"]), _p(h["cu_q"]), _p(h["seq_lens"]),
-            _p(h["slot_mapping"]), _p(h["block_tables"]), _p(h["state_slots"]), _p(h["logit_rows"]),
-            _p(h["temperature"]), _p(h["top_k"]), _p(h["top_p"]), _p(h["seeds"]), _p(h["out_index"]))
+        args = getattr(arena, "_fill_args", None)
+        if args is None:      # the arena's addresses never change: make the argument list once
+            h = arena.h
+            args = arena._fill_args = (
+                self._h, self.cache.handle, arena.n_cap, arena.r_cap, arena.m_cap, arena.max_blocks,
+                _p(h["token_ids"]), _p(h["positions"]), _p(h["q_req"]), _p(h["cu_q"]), _p(h["seq_lens"]),
+                _p(h["slot_mapping"]), _p(h["block_tables"]), _p(h["state_slots"]), _p(h["logit_rows"]),
+                _p(h["temperature"]), _p(h["top_k"]), _p(h["top_p"]), _p(h["seeds"]), _p(h["out_index"]))
+        rc = self._lib.mgpt_sched_fill(*args)
         if rc != 0:
             raise SchedulerError(f"filling the step failed ({rc}) {library.host_error()}")
 
@@ -117,7 +123,7 @@ class Scheduler:
         """Hands in the sampled tokens (entry order).  Returns (request, token, finished, reason)."""
         tokens = np.ascontiguousarray(tokens, dtype=np.int32)
         n = self._lib.mgpt_sched_commit(self._h, _p(tokens) if tokens.size else None, int(tokens.size),
-                                        *[_p(a) for a in self._o], self._o[0].size)
+                                        *self._op, self._o[0].size)
         if n < 0:
             raise SchedulerError(f"commit failed ({n}) {library.host_error()}")
         ids, toks, fin, why = self._o

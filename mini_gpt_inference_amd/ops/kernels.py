@@ -209,20 +209,40 @@ SK_EPI_QKV = 3
 _SKINNY_MAX_ROWS = 64
 
 
+def fold_layer_norm(w: torch.Tensor, gain: torch.Tensor, beta: Optional[torch.Tensor],
+                    bias: Optional[torch.Tensor]):
+    """Folds a LayerNorm's gain and bias into the bfloat16 matrix that reads it.  Returns
+    (w', colsum, bias'): LN(x) w^T + bias = rstd * (x w'^T - mean * colsum) + bias'."""
+    _need_cuda(w, gain, beta, bias)
+    n_out, k_dim = w.shape
+    _need(w.dtype == torch.bfloat16 and w.is_contiguous(), "the matrix must be dense bfloat16")
+    _need(gain.dtype == torch.float32 and gain.numel() == k_dim, "gain must be float32 [inner]")
+    _need(beta is None or (beta.dtype == torch.float32 and beta.numel() == k_dim), "beta must be float32 [inner]")
+    _need(bias is None or (bias.dtype == torch.float32 and bias.numel() == n_out), "bias must be float32 [out]")
+    w_out = torch.empty_like(w)
+    colsum = torch.empty(n_out, dtype=torch.float32, device=w.device)
+    bias_out = torch.empty(n_out, dtype=torch.float32, device=w.device)
+    rc = library.kernels().mgpt_fold_layernorm(_ptr(w), _ptr(gain), _ptr(beta), _ptr(bias), _ptr(w_out),
+                                               _ptr(colsum), _ptr(bias_out), n_out, k_dim, _stream())
+    _check(rc, "fold_layer_norm")
+    return w_out, colsum, bias_out
+
+
 def linear_skinny(a: Optional[torch.Tensor], w: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor,
                   n_rows: int, epilogue: int = EPI_NONE, *, ln_x: Optional[torch.Tensor] = None,
-                  ln_weight: Optional[torch.Tensor] = None, ln_bias: Optional[torch.Tensor] = None,
-                  ln_eps: float = 0.0, ln_rows: Optional[torch.Tensor] = None, scatter=None) -> bool:
-    """bfloat16 MFMA product for at most 64 rows, with an optional LayerNorm prologue (ln_x is the
-    float32 residual stream, ln_rows an optional gather) and an optional key/value scatter
-    (scatter = (k_pool, v_pool, slot_mapping, q_width, kv_width)).  Returns False, having launched
-    nothing, when the kernel does not take the shape."""
+                  ln_colsum: Optional[torch.Tensor] = None, ln_eps: float = 0.0,
+                  ln_rows: Optional[torch.Tensor] = None, scatter=None) -> bool:
+    """bfloat16 MFMA product for at most 64 rows.  With ln_x (the float32 residual stream; ln_rows an
+    optional gather) the rows are read through a LayerNorm that fold_layer_norm folded into w, bias
+    and ln_colsum.  scatter = (k_pool, v_pool, slot_mapping, q_width, kv_width) also stores the new
+    keys and values into their pages.  Returns False, having launched nothing, when the kernel does
+    not take the shape."""
     if n_rows > _SKINNY_MAX_ROWS or w.dtype != torch.bfloat16:
         return False
     n_out, k_dim = w.shape
     if k_dim % 16 != 0:
         return False
-    _need_cuda(a, w, bias, out, ln_x, ln_weight, ln_bias, ln_rows)
+    _need_cuda(a, w, bias, out, ln_x, ln_colsum, ln_rows)
     _need(w.is_contiguous(), "weight must be dense [out, in]")
     _need(out.dim() == 2 and out.stride(1) == 1 and out.shape[1] >= n_out and out.shape[0] >= n_rows,
           "output must be [>=n_rows, >=out] with unit inner stride")
@@ -234,11 +254,9 @@ def linear_skinny(a: Optional[torch.Tensor], w: torch.Tensor, bias: Optional[tor
     lda = 0
     if ln_x is not None:
         _need(ln_x.dtype == torch.float32 and ln_x.is_contiguous() and ln_x.shape[1] == k_dim,
-              "LayerNorm prologue reads dense float32 rows of the inner size")
-        _need(ln_weight is not None and ln_weight.dtype == torch.float32 and ln_weight.numel() == k_dim,
-              "LayerNorm weight must be float32 [inner]")
-        _need(ln_bias is None or (ln_bias.dtype == torch.float32 and ln_bias.numel() == k_dim),
-              "LayerNorm bias must be float32 [inner]")
+              "the residual stream must be dense float32 rows of the inner size")
+        _need(ln_colsum is not None and ln_colsum.dtype == torch.float32 and ln_colsum.numel() == n_out,
+              "the folded column sums must be float32 [out]")
         if ln_rows is None:
             _need(ln_x.shape[0] >= n_rows, "too few residual rows")
         else:
@@ -261,7 +279,7 @@ def linear_skinny(a: Optional[torch.Tensor], w: torch.Tensor, bias: Optional[tor
         _, n_kv_head, page_size, head_dim = kp.shape
         _need_i32("slot_mapping", sm, n_rows)
     rc = library.kernels().mgpt_linear_skinny(
-        _ptr(a if ln_x is None else None), lda, _ptr(ln_x), _ptr(ln_rows), _ptr(ln_weight), _ptr(ln_bias),
+        _ptr(a if ln_x is None else None), lda, _ptr(ln_x), _ptr(ln_rows), _ptr(ln_colsum),
         float(ln_eps), _ptr(w), _ptr(bias), _ptr(out), _dtype_code(out), out.stride(0), n_rows, n_out, k_dim,
         epilogue, _ptr(kp), _ptr(vp), _ptr(sm), q_width, kv_width, head_dim, n_kv_head, page_size, _stream())
     if rc == -2:

@@ -27,6 +27,20 @@ class LazyNorm:
         return self._tensor
 
 
+_folded = {}   # (matrix, gain, beta, bias) buffers -> (folded matrix, column sums, folded bias)
+
+
+def folded_layer_norm(norm, w: torch.Tensor, bias: Optional[torch.Tensor]):
+    """The matrix with the LayerNorm's gain and bias folded in, made once per (norm, matrix) pair."""
+    key = (w.data_ptr(), norm.weight.data_ptr(), 0 if norm.bias is None else norm.bias.data_ptr(),
+           0 if bias is None else bias.data_ptr())
+    hit = _folded.get(key)
+    if hit is None or hit[0] is not w:
+        hit = (w,) + kernels.fold_layer_norm(w, norm.weight, norm.bias, bias)
+        _folded[key] = hit
+    return hit[1:]
+
+
 def as_tensor(ctx, a: Union[torch.Tensor, LazyNorm]) -> torch.Tensor:
     return a.tensor(ctx) if isinstance(a, LazyNorm) else a
 
@@ -35,8 +49,8 @@ def linear(ctx, a: Union[torch.Tensor, LazyNorm], w: torch.Tensor, bias: Optiona
            out: torch.Tensor, n_rows: int, epilogue: int = kernels.EPI_NONE, scatter=None) -> bool:
     """out[:n_rows] = a[:n_rows] @ w.T (+ bias) with the epilogue.
 
-    On the bfloat16 path few rows go to the skinny MFMA kernel (with the LayerNorm in its prologue
-    when `a` is a LazyNorm of a fusable norm) and many rows to the tiled MFMA kernel; the 32-bit
+    On the bfloat16 path few rows go to the skinny MFMA kernel (reading the residual stream through
+    the folded LayerNorm when `a` is a LazyNorm of a fusable norm) and many rows to the tiled MFMA kernel; the 32-bit
     path, and every shape those refuse, go to the 32-bit FMA kernel.  `scatter` = (k_pool, v_pool,
     slot_mapping, q_width, kv_width) asks for the new keys and values to be stored into their
     pages by the same kernel; the return value says whether that was done."""
@@ -45,9 +59,13 @@ def linear(ctx, a: Union[torch.Tensor, LazyNorm], w: torch.Tensor, bias: Optiona
     fast = w.dtype == torch.bfloat16 and not ctx.exact and ctx.dtype == torch.bfloat16
     if fast and n_rows <= 64:
         epi = kernels.SK_EPI_QKV if scatter is not None else epilogue
-        if isinstance(a, LazyNorm) and getattr(a.norm, "fusable_layer_norm", False) and a._tensor is None:
-            if kernels.linear_skinny(None, w, bias, out, n_rows, epi, ln_x=a.x, ln_weight=a.norm.weight,
-                                     ln_bias=a.norm.bias, ln_eps=a.norm.eps, ln_rows=a.rows, scatter=scatter):
+        # every column tile converts the residual rows it multiplies: beyond 32 rows, or for a very
+        # wide output (the head), that costs more than a LayerNorm kernel of its own
+        if (isinstance(a, LazyNorm) and getattr(a.norm, "fusable_layer_norm", False) and a._tensor is None
+                and n_rows <= 32 and w.shape[0] <= 4096):
+            wf, colsum, bias_f = folded_layer_norm(a.norm, w, bias)
+            if kernels.linear_skinny(None, wf, bias_f, out, n_rows, epi, ln_x=a.x, ln_colsum=colsum,
+                                     ln_eps=a.norm.eps, ln_rows=a.rows, scatter=scatter):
                 return scatter is not None
         if kernels.linear_skinny(as_tensor(ctx, a), w, bias, out, n_rows, epi, scatter=scatter):
             return scatter is not None

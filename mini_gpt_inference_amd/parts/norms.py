@@ -17,7 +17,7 @@ class LayerNorm(Part):
     library default, here it is a parameter)."""
 
     category = "norm"
-    fusable_layer_norm = True   # a linear kernel may compute it in its prologue from weight, bias, eps
+    fusable_layer_norm = True   # a linear kernel may fold weight and bias into its matrix and apply mean, rstd itself
 
     def __init__(self, width: int, eps: float, bias: bool) -> None:
         self.width, self.eps, self.has_bias = int(width), float(eps), bool(bias)

@@ -124,17 +124,23 @@ def test_linear_mfma(n, k, o, epi, o_dt):
 
 
 @pytest.mark.parametrize("n,k,o,ln_bias,gather", [(8, 512, 1536, True, False), (3, 96, 503, False, True),
-                                                  (16, 80, 257, True, True), (12, 1024, 64, False, False)])
-def test_linear_skinny_with_layer_norm_prologue(n, k, o, ln_bias, gather):
+                                                  (40, 80, 257, True, True), (64, 2048, 64, False, False),
+                                                  (17, 1600, 48, True, False)])
+def test_linear_skinny_through_a_folded_layer_norm(n, k, o, ln_bias, gather):
     g = torch.Generator().manual_seed(4)
     x = rnd(g, 70, k, scale=2.0) + 0.5
+    x[:, 3] += 40.0                      # an outlier channel, as residual streams have
     lw, lb = 1 + 0.1 * rnd(g, k), rnd(g, k) if ln_bias else None
     w, bias = rnd(g, o, k, dtype="bfloat16", scale=k ** -0.5), rnd(g, o)
     rows = torch.randperm(70, generator=g)[:n].tolist() if gather else list(range(n))
+    wf, colsum, bias_f = kernels.fold_layer_norm(w.to(DEV), lw.to(DEV), lb.to(DEV) if ln_bias else None, bias.to(DEV))
+    # the fold itself: W' = W * gain, S = row sums of W', b' = b + W beta
+    helpers.assert_close(wf, w.double() * lw.double(), "bfloat16", "folded matrix")
+    helpers.assert_close(colsum, wf.double().sum(1), "float32", "column sums")
+    helpers.assert_close(bias_f, bias.double() + (w.double() @ lb.double() if ln_bias else 0), "float32", "folded bias")
     out = torch.empty(n, o, dtype=torch.float32, device=DEV)
-    assert kernels.linear_skinny(None, w.to(DEV), bias.to(DEV), out, n, kernels.EPI_NONE, ln_x=x.to(DEV),
-                                 ln_weight=lw.to(DEV), ln_bias=lb.to(DEV) if ln_bias else None, ln_eps=1e-5,
-                                 ln_rows=i32(rows) if gather else None)
+    assert kernels.linear_skinny(None, wf, bias_f, out, n, kernels.EPI_NONE, ln_x=x.to(DEV), ln_colsum=colsum,
+                                 ln_eps=1e-5, ln_rows=i32(rows) if gather else None)
     h = P.plain_layer_norm(x.double()[rows], lw.double(), lb.double() if ln_bias else None, 1e-5)
     helpers.assert_close(out, P.plain_linear(h, w.double(), bias.double()), "bfloat16", "LN + skinny")
 
@@ -171,14 +177,6 @@ def test_linear_skinny_refuses_what_it_cannot_do():
     a = torch.zeros(65, 64, dtype=torch.bfloat16, device=DEV)
     assert not kernels.linear_skinny(a, w, None, torch.zeros(65, 32, dtype=torch.bfloat16, device=DEV), 65)
     assert not kernels.linear_skinny(a.float(), w, None, torch.zeros(65, 32, dtype=torch.bfloat16, device=DEV), 4)
-    big = torch.zeros(17, 2048, device=DEV)      # the prologue normalises at most 16 rows
-    wbig = torch.zeros(32, 2048, dtype=torch.bfloat16, device=DEV)
-    assert not kernels.linear_skinny(None, wbig, None, torch.zeros(17, 32, dtype=torch.bfloat16, device=DEV), 17,
-                                     ln_x=big, ln_weight=torch.ones(2048, device=DEV), ln_eps=1e-5)
-    huge = torch.zeros(4, 1040, device=DEV)      # and rows of at most 1024 values (held in registers)
-    whuge = torch.zeros(32, 1040, dtype=torch.bfloat16, device=DEV)
-    assert not kernels.linear_skinny(None, whuge, None, torch.zeros(4, 32, dtype=torch.bfloat16, device=DEV), 4,
-                                     ln_x=huge, ln_weight=torch.ones(1040, device=DEV), ln_eps=1e-5)
 
 
 # ----------------------------------------------------------------------------- cache write and attention
