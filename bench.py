@@ -32,7 +32,7 @@ def build_engine(args, batch, dtype):
     pages = batch * (-(-args.positions // args.kv_block)) + 8
     ecfg = EngineConfig(block_size=args.kv_block, num_blocks=pages, max_batch_size=max(batch, 2),
                         max_num_batched_tokens=max(4096, batch * args.prompt), dtype=dtype,
-                        use_graph=not args.no_graph)
+                        use_graph=not args.no_graph, decode_burst=args.burst)
     return LLMEngine.from_random(cfg, seed=0, engine_config=ecfg), cfg
 
 
@@ -45,23 +45,31 @@ def decode_run(args, batch, steps, warmup, dtype):
 
     engine, cfg = build_engine(args, batch, dtype)
     rng = np.random.default_rng(0)
-    budget = steps + warmup + 2
+    budget = steps + warmup + 2 * args.burst + 2
     assert args.prompt + budget <= cfg.block_size, "prompt + decode steps exceed the model's positions"
     for i in range(batch):
         engine.add_request(Request(f"b{i}", rng.integers(0, cfg.vocab_size, args.prompt).tolist(),
                                    SamplingParams(max_tokens=budget, temperature=0.0)))
-    while engine.scheduler.num_decode_tokens == 0:      # prompts, untimed
+    sched = engine.scheduler
+    while sched.num_decode_tokens == 0:      # prompts, untimed
         engine.step()
-    for _ in range(warmup):
-        engine.step()
+
+    def run_decode_steps(n):
+        """engine.step() until exactly n more decode steps have run (a call may run a burst of them)."""
+        first, tokens = sched.num_steps, sched.num_decode_tokens
+        while sched.num_steps - first < n:
+            engine.step()
+        assert sched.num_steps - first == n, "the decode bursts do not divide the number of steps"
+        assert sched.num_decode_tokens - tokens == n * batch, "a request dropped out of the decode steps"
+
+    done = sched.num_steps
+    run_decode_steps(warmup)
     torch.cuda.synchronize()
-    start_ctx = args.prompt + 1 + warmup
+    start_ctx = args.prompt + 1 + (sched.num_steps - done)
     t0 = time.perf_counter()
-    for _ in range(steps):
-        outs = engine.step()
+    run_decode_steps(steps)
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
-    assert len(outs) == batch, "a request dropped out of the timed decode steps"
     mean_ctx = start_ctx + (steps - 1) / 2.0 + 1     # keys read per request and step, own token included
     return elapsed, mean_ctx, engine, cfg
 
@@ -120,6 +128,7 @@ def main() -> int:
     ap.add_argument("--prompt", type=int, default=128)
     ap.add_argument("--kv-block", type=int, default=16)
     ap.add_argument("--no-graph", action="store_true")
+    ap.add_argument("--burst", type=int, default=8, help="decode steps enqueued back to back (1 = off)")
     ap.add_argument("--no-extras", action="store_true", help="skip prefill and the batch 1 / 64 points")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -144,7 +153,7 @@ def main() -> int:
             "vocab_size": cfg.vocab_size, "block_size": cfg.block_size, "bias": True,
             "global_batch": args.batch, "seq_len": cfg.block_size, "prompt_len": args.prompt,
             "mean_context": round(mean_ctx, 1), "kv_block": args.kv_block, "weights": "random",
-            "hip_graph": bool(stats["graph_steps"]), "parallelism": "single-gpu",
+            "hip_graph": bool(stats["graph_steps"]), "decode_burst": args.burst, "parallelism": "single-gpu",
         },
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 5)},

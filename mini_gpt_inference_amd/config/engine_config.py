@@ -25,6 +25,8 @@ class EngineConfig:
                                      # as the reference does (scheduler.py:52-56)
     dtype: str = "bfloat16"          # "bfloat16" (serving) or "float32" (true 32-bit path)
     use_graph: bool = True           # replay decode-only steps from a captured HIP graph
+    decode_burst: int = 8            # decode steps enqueued back to back when nothing else is pending,
+                                     # tokens fed on the device from one to the next; 1 = off
     seed: int = 0                    # engine-wide sampler seed
     real_vocab_size: Optional[int] = None  # ids at or above it are never sampled
                                            # (src/minigpt_infer/tokenizer.py:37-46)

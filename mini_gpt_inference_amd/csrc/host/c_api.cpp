@@ -132,11 +132,13 @@ int mgpt_sched_entries(void* s, int* ids, int* ctx, int* q_len, int* sample, int
   return (int)e.size();
 }
 
-// Fills the arrays of the planned step.  Per-token arrays have n_stride entries, per-request
+// Fills the arrays of the planned step (step_offset = 0), or of step `step_offset` of a planned
+// burst: every entry then feeds position ctx + step_offset, and its token, which only the device
+// knows, is left 0 for the device to fill in.  Per-token arrays have n_stride entries, per-request
 // arrays r_stride (cu_q one more), per-logit-row arrays m_stride; what lies beyond the real
 // counts is padding that the kernels skip.  Returns 0, or a negative code.
-int mgpt_sched_fill(void* sv, void* cm, int n_stride, int r_stride, int m_stride, int max_blocks,
-                    int* token_ids, int* positions, int* q_req, int* cu_q, int* seq_lens,
+int mgpt_sched_fill(void* sv, void* cm, int step_offset, int n_stride, int r_stride, int m_stride,
+                    int max_blocks, int* token_ids, int* positions, int* q_req, int* cu_q, int* seq_lens,
                     int* slot_mapping, int* block_tables, int* state_slots, int* logit_rows,
                     float* temperature, int* top_k, float* top_p, unsigned long long* seeds,
                     int* out_index) {
@@ -150,7 +152,7 @@ int mgpt_sched_fill(void* sv, void* cm, int n_stride, int r_stride, int m_stride
   for (int i = 0; i < R; ++i) {
     const mgpt::Request* r = s->request(e[i].id);
     slots[i] = r->slot;
-    ctx[i] = e[i].ctx;
+    ctx[i] = e[i].ctx + step_offset;
     ql[i] = e[i].q_len;
   }
   int n = c->build_step(R, slots.data(), ctx.data(), ql.data(), n_stride, r_stride, max_blocks, positions,
@@ -160,7 +162,7 @@ int mgpt_sched_fill(void* sv, void* cm, int n_stride, int r_stride, int m_stride
   for (int i = 0; i < R; ++i) {
     const mgpt::Request* r = s->request(e[i].id);
     state_slots[i] = r->slot;
-    for (int j = 0; j < e[i].q_len; ++j) token_ids[t++] = r->token_at(e[i].ctx + j);
+    for (int j = 0; j < e[i].q_len; ++j) token_ids[t++] = step_offset ? 0 : r->token_at(e[i].ctx + j);
     if (e[i].sample) {
       if (m >= m_stride) return -4;
       logit_rows[m] = t - 1;
@@ -168,7 +170,7 @@ int mgpt_sched_fill(void* sv, void* cm, int n_stride, int r_stride, int m_stride
       top_k[m] = r->top_k;
       top_p[m] = r->top_p;
       seeds[m] = r->seed;
-      out_index[m] = (int)r->output.size();
+      out_index[m] = (int)r->output.size() + step_offset;
       ++m;
     }
   }
@@ -190,6 +192,27 @@ int mgpt_sched_commit(void* s, const int* tokens, int n_tokens, int* out_ids, in
                       int* out_finished, int* out_reason, int cap) {
   GUARD_BEGIN
   const auto& o = static_cast<Scheduler*>(s)->commit(tokens, n_tokens);
+  if ((int)o.size() > cap) return -1;
+  for (size_t i = 0; i < o.size(); ++i) {
+    out_ids[i] = o[i].id;
+    out_tokens[i] = o[i].token;
+    out_finished[i] = o[i].finished;
+    out_reason[i] = o[i].reason;
+  }
+  return (int)o.size();
+  GUARD_END(-100)
+}
+
+int mgpt_sched_plan_burst(void* s, int max_k) {
+  GUARD_BEGIN
+  return static_cast<Scheduler*>(s)->plan_burst(max_k);
+  GUARD_END(-100)
+}
+
+int mgpt_sched_commit_burst(void* s, const int* tokens, int k, int* out_ids, int* out_tokens, int* out_finished,
+                            int* out_reason, int cap) {
+  GUARD_BEGIN
+  const auto& o = static_cast<Scheduler*>(s)->commit_burst(tokens, k);
   if ((int)o.size() > cap) return -1;
   for (size_t i = 0; i < o.size(); ++i) {
     out_ids[i] = o[i].id;

@@ -202,6 +202,58 @@ const std::vector<StepOutput>& Scheduler::commit(const int* tokens, int n_tokens
   return outputs_;
 }
 
+int Scheduler::plan_burst(int max_k) {
+  if (max_k < 2 || running_.empty() || !waiting_.empty()) return 0;
+  int k = max_k;
+  for (int id : running_) {
+    const Request& r = *get(id);
+    if (r.num_tokens() - r.num_computed != 1) return 0;  // still in its prompt
+    k = std::min(k, r.max_tokens - (int)r.output.size());
+  }
+  if (k < 2) return 0;
+  // pages for k more tokens each, or no burst at all
+  for (int g = 0; g < cache_->num_groups(); ++g) {
+    long need = 0;
+    for (int id : running_) {
+      const Request& r = *get(id);
+      need += std::max(0, cache_->pages_needed(g, r.num_computed + k) - cache_->table_len(r.slot, g));
+    }
+    if (need > cache_->num_free_pages(g)) return 0;
+  }
+  entries_.clear();
+  for (int id : running_) {
+    Request& r = *get(id);
+    cache_->reserve(r.slot, r.num_computed + k);
+    entries_.push_back({id, r.num_computed, 1, true});
+  }
+  num_decode_tokens += (long)k * (long)entries_.size();
+  num_steps += k;
+  return k;
+}
+
+const std::vector<StepOutput>& Scheduler::commit_burst(const int* tokens, int k) {
+  outputs_.clear();
+  const std::vector<StepEntry> entries = entries_;
+  const int n = (int)entries.size();
+  for (int j = 0; j < k; ++j) {
+    for (int i = 0; i < n; ++i) {
+      Request& r = *get(entries[i].id);
+      if (r.status != RUNNING) continue;  // ended earlier in this burst
+      r.num_computed += 1;
+      cache_->release_passed(r.slot, r.num_computed);
+      const int token = tokens[(long)j * n + i];
+      r.output.push_back(token);
+      FinishReason why = NOT_FINISHED;
+      if (r.eot >= 0 && token == r.eot) why = FINISH_EOT;
+      else if ((int)r.output.size() >= r.max_tokens) why = FINISH_LENGTH;
+      if (why != NOT_FINISHED) finish(r, why);
+      outputs_.push_back({r.id, token, why != NOT_FINISHED, (int)why});
+    }
+  }
+  entries_.clear();
+  return outputs_;
+}
+
 void Scheduler::forget_finished() {
   for (auto& r : requests_)
     if (r && r->status == FINISHED) {

@@ -87,6 +87,17 @@ class Scheduler {
   // Takes the tokens sampled for the entries with sample = true, in entry order.
   const std::vector<StepOutput>& commit(const int* tokens, int n_tokens);
 
+  // A burst: up to max_k decode steps of the running requests planned at once, so that the device
+  // can run them back to back while it feeds each step's tokens to the next by itself.  Only when
+  // every running request is decoding, nobody waits, and pages for all k tokens are free; k stops
+  // one short of the first request's length limit, so nobody can end inside a burst except by its
+  // end token.  Returns k >= 2 with entries() set to step 0, or 0 when a burst is not possible
+  // (then nothing has changed).  Step j of a burst feeds position ctx + j.
+  int plan_burst(int max_k);
+  // tokens[j * n_entries + i]: what entry i sampled in step j.  A request that meets its end token
+  // in step j ends there; what the device computed for it afterwards is dropped.
+  const std::vector<StepOutput>& commit_burst(const int* tokens, int k);
+
   const Request* request(int id) const;
   const std::deque<int>& waiting() const { return waiting_; }
   const std::vector<int>& running() const { return running_; }

@@ -36,6 +36,7 @@ class _GraphedDecode:
         self.arena = StepArena(cap, cap, cap, runner.n_groups, runner.max_blocks, runner.device)
         self.workspace = Workspace(runner.device)
         self.graph: Optional[torch.cuda.CUDAGraph] = None
+        self.staging: List[StepArena] = []   # host sides of the steps of a burst
 
     def _launch(self, shape: StepShape) -> None:
         ctx = self.runner.context(self.arena, shape, padded=True, workspace=self.workspace)
@@ -130,7 +131,43 @@ class LLMEngine:
         return False if sid is None else self.scheduler.cancel(sid)
 
     # ------------------------------------------------------------------ stepping
+    def _try_burst(self) -> Optional[List[RequestOutput]]:
+        """Several decode steps enqueued at once: each is one upload, one on-device copy of the last
+        step's tokens into this step's inputs, one graph replay and one download, with no wait in
+        between; the host looks at the tokens only when all are done."""
+        ecfg = self.engine_config
+        if ecfg.decode_burst < 2 or not ecfg.use_graph or not self._graphs:
+            return None
+        running = len(self.scheduler.running)
+        graphed = self._graphs.get(_bucket(max(running, 1)))
+        if graphed is None or graphed.graph is None:
+            return None
+        k = self.scheduler.plan_burst(ecfg.decode_burst)
+        if k < 2:
+            return None
+        r = running
+        arena = graphed.arena
+        while len(graphed.staging) < k:
+            graphed.staging.append(StepArena(arena.n_cap, arena.r_cap, arena.m_cap, arena.n_groups,
+                                             arena.max_blocks, self.device))
+        for j in range(k):
+            stage = graphed.staging[j]
+            self.scheduler.fill(stage, j)
+            arena.dev_t.copy_(stage.host_t, non_blocking=True)
+            if j:
+                arena.d["token_ids"][:r].copy_(arena.tokens_out[:r], non_blocking=True)
+            graphed.graph.replay()
+            stage.tokens_host.copy_(arena.tokens_out, non_blocking=True)
+        torch.cuda.current_stream().synchronize()
+        tokens = np.stack([graphed.staging[j].tokens_host.numpy()[:r] for j in range(k)])
+        self.num_graph_steps += k
+        return [RequestOutput(self._ids[sid], [token], finished, reason)
+                for sid, token, finished, reason in self.scheduler.commit_burst(tokens, k)]
+
     def step(self) -> List[RequestOutput]:
+        burst = self._try_burst()
+        if burst is not None:
+            return burst
         n, r, m = self.scheduler.schedule()
         if r == 0:
             return []

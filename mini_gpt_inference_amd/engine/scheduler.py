@@ -105,17 +105,18 @@ class Scheduler:
         n = self._lib.mgpt_sched_entries(self._h, *self._ep, self._e[0].size)
         return tuple(a[:n] for a in self._e)
 
-    def fill(self, arena) -> None:
-        """Writes the planned step into a StepArena's host arrays."""
+    def fill(self, arena, step_offset: int = 0) -> None:
+        """Writes the planned step (or step `step_offset` of a planned burst) into a StepArena's
+        host arrays."""
         args = getattr(arena, "_fill_args", None)
         if args is None:      # the arena's addresses never change: make the argument list once
             h = arena.h
             args = arena._fill_args = (
-                self._h, self.cache.handle, arena.n_cap, arena.r_cap, arena.m_cap, arena.max_blocks,
+                arena.n_cap, arena.r_cap, arena.m_cap, arena.max_blocks,
                 _p(h["token_ids"]), _p(h["positions"]), _p(h["q_req"]), _p(h["cu_q"]), _p(h["seq_lens"]),
                 _p(h["slot_mapping"]), _p(h["block_tables"]), _p(h["state_slots"]), _p(h["logit_rows"]),
                 _p(h["temperature"]), _p(h["top_k"]), _p(h["top_p"]), _p(h["seeds"]), _p(h["out_index"]))
-        rc = self._lib.mgpt_sched_fill(*args)
+        rc = self._lib.mgpt_sched_fill(self._h, self.cache.handle, step_offset, *args)
         if rc != 0:
             raise SchedulerError(f"filling the step failed ({rc}) {library.host_error()}")
 
@@ -127,6 +128,24 @@ class Scheduler:
         if n < 0:
             raise SchedulerError(f"commit failed ({n}) {library.host_error()}")
         ids, toks, fin, why = self._o
+        return [(int(ids[i]), int(toks[i]), bool(fin[i]), FINISH_REASONS[int(why[i])]) for i in range(n)]
+
+    def plan_burst(self, max_k: int) -> int:
+        """Plans up to max_k decode steps at once (see csrc/host/scheduler.h).  Returns k >= 2, or 0."""
+        k = self._lib.mgpt_sched_plan_burst(self._h, int(max_k))
+        if k < 0:
+            raise SchedulerError(library.host_error())
+        return k
+
+    def commit_burst(self, tokens: np.ndarray, k: int) -> List[Tuple[int, int, bool, Optional[str]]]:
+        """tokens[j, i]: what entry i sampled in step j of the burst."""
+        tokens = np.ascontiguousarray(tokens, dtype=np.int32)
+        cap = tokens.size
+        out = [np.zeros(max(cap, 1), dtype=np.int32) for _ in range(4)]
+        n = self._lib.mgpt_sched_commit_burst(self._h, _p(tokens), int(k), *[_p(a) for a in out], cap)
+        if n < 0:
+            raise SchedulerError(f"commit_burst failed ({n}) {library.host_error()}")
+        ids, toks, fin, why = out
         return [(int(ids[i]), int(toks[i]), bool(fin[i]), FINISH_REASONS[int(why[i])]) for i in range(n)]
 
     # -------------------------------------------------------------- inspection

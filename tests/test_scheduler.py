@@ -223,3 +223,40 @@ def test_random_load_keeps_every_invariant(mixed, chunk):
     assert not s.has_work() and arrivals == 40
     assert all(s.info(rid).status == FINISHED and s.info(rid).finish_reason == "length" for rid in want)
     assert cm.num_free_pages() == 24 and cm.num_free_slots == 5
+
+
+def test_burst_is_planned_only_when_nothing_else_is_pending_and_ends_on_the_end_token():
+    cm, s = make(20, 4, max_batch=4, max_positions=64)
+    a = s.add_request([1, 2, 3], 10, eot=7)
+    b = s.add_request([1, 2, 3, 4, 5], 6)
+    assert s.plan_burst(8) == 0                  # nobody is running yet
+    step(s)                                      # both prompts, one token each
+    c = s.add_request([9], 5)
+    assert s.plan_burst(8) == 0                  # somebody waits
+    step(s)                                      # c's prompt beside the decode tokens of a and b
+    free_before = cm.num_free_pages()
+    k = s.plan_burst(8)
+    # a has 8 tokens left, b 4, c 4: the burst stops at the first length limit
+    assert k == 4
+    ents = s.entries()
+    assert [(e.request, e.ctx, e.q_len, e.sample) for e in ents] == [(a, 4, 1, True), (b, 6, 1, True), (c, 1, 1, True)]
+    for e in ents:       # pages for all four tokens are held before the burst starts
+        assert len(cm.table(s.info(e.request).slot)) * 4 >= e.ctx + k
+    assert cm.num_free_pages() <= free_before
+    # a meets its end token in the burst's second step: what came after is dropped
+    tokens = np.array([[5, 5, 5], [7, 5, 5], [6, 5, 5], [6, 5, 5]], dtype=np.int32)
+    outs = s.commit_burst(tokens, k)
+    assert [o for o in outs if o[0] == a] == [(a, 5, False, None), (a, 7, True, "eot")]
+    assert [o[1:] for o in outs if o[0] == b] == [(5, False, None)] * 3 + [(5, True, "length")]
+    assert s.output(a) == [100, 101, 5, 7] and s.info(b).status == FINISHED and s.info(c).status == FINISHED
+    assert not s.has_work() and cm.num_free_pages() == 20 and cm.check() == 0
+
+
+def test_burst_needs_pages_for_every_step_or_does_not_start():
+    cm, s = make(4, 4, max_batch=2, max_positions=64)
+    a = s.add_request([1, 2, 3], 12)
+    b = s.add_request([1, 2, 3], 12)
+    step(s)
+    free = cm.num_free_pages()
+    assert s.plan_burst(8) == 0 and cm.num_free_pages() == free     # 2 free pages, 4 would be needed
+    assert s.plan_burst(2) == 2                                      # two more tokens each fit
