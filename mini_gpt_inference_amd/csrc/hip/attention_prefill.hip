@@ -6,9 +6,10 @@
 // softmax and all sums in float32 (src/minigpt_infer/model.py:61-87).
 //
 // A workgroup of four waves takes 64 consecutive queries of one request and one head, 16 per
-// wave.  It walks the keys in blocks of 64 (aligned to multiples of 64 of the key position):
+// wave.  It walks the keys in blocks of 128 (aligned to multiples of 128 of the key position):
 // the block's key rows go to LDS as they are, its value rows transposed, gathered row by row
-// through the block table, so any page size works and nothing outside [begin, end) is loaded.
+// through the block table, so any page size works and nothing outside [begin, end) is loaded;
+// the next block is on its way from memory while the current one is multiplied.
 // S = K Q^T uses the keys as the first MFMA operand, so a lane holds, for one query, four
 // neighbouring keys of each 16-key tile; those are exactly the k-slots of the second MFMA
 // (values^T times P) if the transposed values are read with the same interleaving, so the
@@ -21,7 +22,7 @@ typedef __attribute__((__vector_size__(4 * sizeof(short)))) short bf16x4_t;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4_t;
 
 #define PF_QT 64   // queries per workgroup
-#define PF_KT 64   // keys per block
+#define PF_KT 128  // keys per block
 
 template <int D>
 __global__ __launch_bounds__(256) void prefill_attention_kernel(
@@ -38,7 +39,8 @@ __global__ __launch_bounds__(256) void prefill_attention_kernel(
 
   const int r = blockIdx.y, h = blockIdx.z;
   const int q_start = cu_q[r], q_len = cu_q[r + 1] - q_start;
-  const int q0 = blockIdx.x * PF_QT;
+  // later tiles see more keys: start them first
+  const int q0 = (int)blockIdx.x * PF_QT;
   if (q0 >= q_len) return;
   const int seq_len = seq_lens[r];
   const int ctx = seq_len - q_len;
@@ -68,35 +70,56 @@ __global__ __launch_bounds__(256) void prefill_attention_kernel(
 #pragma unroll
   for (int dt = 0; dt < DT; ++dt) o[dt] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
 
-  const int srow = tid >> 2, sc = tid & 3;  // staging: 4 threads per key row
-  for (int c0 = (kv_begin / PF_KT) * PF_KT; c0 < kv_end; c0 += PF_KT) {
-    __syncthreads();  // the previous block's readers are done
-    {
-      const int j = c0 + srow;
-      const bool valid = (j >= kv_begin) && (j < kv_end);
-      long base = 0;
-      if (valid) {
-        const int page = bt[j / page_size];
-        base = (((long)page * n_kv_head + hk) * page_size + (j % page_size)) * (long)D;
-      }
-#pragma unroll
-      for (int c = sc; c < D / 8; c += 4) {
-        bf16x8_t kv8 = zero8, vv8 = zero8;
-        if (valid) {
-          kv8 = *reinterpret_cast<const bf16x8_t*>(kpool + base + c * 8);
-          vv8 = *reinterpret_cast<const bf16x8_t*>(vpool + base + c * 8);
-        }
-        *reinterpret_cast<bf16x8_t*>(&ks[srow * KLD + c * 8]) = kv8;
-#pragma unroll
-        for (int e = 0; e < 8; ++e) vt[(c * 8 + e) * VLD + srow] = (bf16_t)vv8[e];
-      }
+  // Staging: 256 / PF_KT threads per key row, each 16 bytes (8 channels) of the key row and of the
+  // value row at a time; keys go to LDS as they are, values transposed.  The next block's rows
+  // are fetched into registers while the current block is multiplied.
+  constexpr int TPR = 256 / PF_KT;                 // threads per row
+  constexpr int NC = (D / 8 + TPR - 1) / TPR;      // chunks per thread
+  const int srow = tid / TPR, sc = tid % TPR;
+  bf16x8_t kst[NC], vst[NC];
+
+  auto fetch = [&](int c0) {
+    const int j = c0 + srow;
+    const bool valid = (j >= kv_begin) && (j < kv_end);
+    long base = 0;
+    if (valid) {
+      const int page = bt[j / page_size];
+      base = (((long)page * n_kv_head + hk) * page_size + (j % page_size)) * (long)D;
     }
+#pragma unroll
+    for (int u = 0; u < NC; ++u) {
+      const int c = sc + u * TPR;
+      const bool ok = valid && c < D / 8;
+      const bf16x8_t kv8 = *reinterpret_cast<const bf16x8_t*>(kpool + base + (ok ? c * 8 : 0));
+      const bf16x8_t vv8 = *reinterpret_cast<const bf16x8_t*>(vpool + base + (ok ? c * 8 : 0));
+      kst[u] = ok ? kv8 : zero8;
+      vst[u] = ok ? vv8 : zero8;
+    }
+  };
+  auto deposit = [&]() {
+#pragma unroll
+    for (int u = 0; u < NC; ++u) {
+      const int c = sc + u * TPR;
+      if (c >= D / 8) continue;
+      *reinterpret_cast<bf16x8_t*>(&ks[srow * KLD + c * 8]) = kst[u];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) vt[(c * 8 + e) * VLD + srow] = (bf16_t)vst[u][e];
+    }
+  };
+
+  const int c_first = (kv_begin / PF_KT) * PF_KT;
+  fetch(c_first);
+  for (int c0 = c_first; c0 < kv_end; c0 += PF_KT) {
+    __syncthreads();  // the previous block's readers are done
+    deposit();
     __syncthreads();
+    if (c0 + PF_KT < kv_end) fetch(c0 + PF_KT);
 
     // scores of this wave's 16 queries against the block's 64 keys
-    f32x4_t s[4];
+    constexpr int NKT = PF_KT / 16;   // 16-key tiles per block
+    f32x4_t s[NKT];
 #pragma unroll
-    for (int kt = 0; kt < 4; ++kt) {
+    for (int kt = 0; kt < NKT; ++kt) {
       s[kt] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int kk = 0; kk < KK; ++kk) {
@@ -104,31 +127,49 @@ __global__ __launch_bounds__(256) void prefill_attention_kernel(
         s[kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[kk], s[kt], 0, 0, 0);
       }
     }
-    // lane: query qi, keys c0 + kt*16 + g*4 + i
+    // lane: query qi, keys c0 + kt*16 + g*4 + i.  Scores are kept in units of log2(e), so that
+    // the exponential is one v_exp_f32.  A block that every query of this wave sees whole (the
+    // common case away from the diagonal) needs no mask.
+    const float sc2 = scale * 1.4426950408889634f;
+    const int wave_pos_lo = ctx + q0 + wave * 16;   // first query position of this wave
+    const bool whole = c0 + PF_KT - 1 <= wave_pos_lo && c0 >= kv_begin && wave_pos_lo + 15 < ctx + q_len &&
+                       (window <= 0 || c0 > wave_pos_lo + 15 - window);
     float mx = -INFINITY;
+    if (whole) {
 #pragma unroll
-    for (int kt = 0; kt < 4; ++kt)
+      for (int kt = 0; kt < NKT; ++kt)
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int key = c0 + kt * 16 + g * 4 + i;
-        const bool see = q_ok && key <= my_pos && key >= kv_begin && (window <= 0 || key > my_pos - window);
-        const float v = see ? s[kt][i] * scale : -INFINITY;
-        s[kt][i] = v;
-        mx = fmaxf(mx, v);
-      }
+        for (int i = 0; i < 4; ++i) {
+          s[kt][i] *= sc2;
+          mx = fmaxf(mx, s[kt][i]);
+        }
+    } else {
+#pragma unroll
+      for (int kt = 0; kt < NKT; ++kt)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int key = c0 + kt * 16 + g * 4 + i;
+          const bool see = q_ok && key <= my_pos && key >= kv_begin && (window <= 0 || key > my_pos - window);
+          const float v = see ? s[kt][i] * sc2 : -INFINITY;
+          s[kt][i] = v;
+          mx = fmaxf(mx, v);
+        }
+    }
     mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
     mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
     const float m_new = fmaxf(m, mx);
-    const float alpha = (m == -INFINITY) ? ((m_new == -INFINITY) ? 1.f : 0.f) : __expf(m - m_new);
+    const float alpha = (m == -INFINITY) ? ((m_new == -INFINITY) ? 1.f : 0.f) : __builtin_amdgcn_exp2f(m - m_new);
+    const float m_sub = (m_new == -INFINITY) ? 0.f : m_new;   // exp2(-inf - 0) = 0 for masked scores
     float rs = 0.f;
-    bf16x8_t pf[2];
+    bf16x8_t pf[NKT / 2];
 #pragma unroll
-    for (int kt = 0; kt < 4; ++kt)
+    for (int kt = 0; kt < NKT; ++kt)
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        const float p = (s[kt][i] == -INFINITY) ? 0.f : __expf(s[kt][i] - m_new);
+        const float p = __builtin_amdgcn_exp2f(s[kt][i] - m_sub);
         rs += p;
-        pf[kt >> 1][(kt & 1) * 4 + i] = (short)float_to_bf16(p);
+        // p lies in [0, 1]: rounding to bfloat16 by adding half an ulp and truncating
+        pf[kt >> 1][(kt & 1) * 4 + i] = (short)((__float_as_uint(p) + 0x8000u) >> 16);
       }
     rs += __shfl_xor(rs, 16, 64);
     rs += __shfl_xor(rs, 32, 64);
@@ -139,7 +180,7 @@ __global__ __launch_bounds__(256) void prefill_attention_kernel(
 #pragma unroll
       for (int i = 0; i < 4; ++i) o[dt][i] *= alpha;
 #pragma unroll
-      for (int b = 0; b < 2; ++b) {
+      for (int b = 0; b < NKT / 2; ++b) {
         // k-slot (g, e): key b*32 + g*4 + e for e < 4, key b*32 + 16 + g*4 + (e - 4) otherwise
         const bf16_t* vrow = &vt[(dt * 16 + qi) * VLD + b * 32 + g * 4];
         const bf16x4_t lo = *reinterpret_cast<const bf16x4_t*>(vrow);

@@ -6,7 +6,7 @@
 // A workgroup of four waves owns a 128 x 128 (or, for small problems, 64 x 64)
 // tile of the output; each wave a quarter of it, as 4 x 4 (2 x 2)
 // v_mfma_f32_16x16x32_bf16 accumulators.  Per step of 32 along k the workgroup
-// stages a slice of the activations and of W
+// stages a slice (32 or 64 along k) of the activations and of W
 // in LDS (rows padded by 16 bytes so the 16 rows a MFMA operand reads fall on
 // distinct banks), with the next slice's global loads in flight while the
 // current one is multiplied.  W is the first MFMA operand, so a lane ends up
@@ -21,16 +21,17 @@ typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4_t;
 #define MM_EPI_GELU 1
 #define MM_EPI_RESIDUAL 2
 
-#define MM_BK 32
-#define MM_LD (MM_BK + 8)  // LDS row stride in elements
-
 // WT: 16-wide tiles per wave in each direction.  4 -> 128 x 128 per workgroup, 2 -> 64 x 64.
 template <int WT, int EPI, typename OT>
 __global__ __launch_bounds__(256) void linear_mfma_kernel(
     const bf16_t* __restrict__ act, long lda, const bf16_t* __restrict__ w,
     const float* __restrict__ bias, OT* __restrict__ out, long ldo, int n_rows, int n_out, int k_dim) {
   constexpr int TILE = 2 * WT * 16;   // rows and columns of the workgroup's tile
-  constexpr int PASSES = TILE / 64;   // staging passes of 64 rows
+  constexpr int MM_BK = WT == 2 ? 64 : 32;   // k per step: what fits LDS twice over
+  constexpr int MM_LD = MM_BK + 8;           // LDS row stride in elements (16 bytes of padding)
+  constexpr int TPR = MM_BK / 8;             // threads per staged row (16 bytes each)
+  constexpr int RPP = 256 / TPR;             // rows per staging pass
+  constexpr int PASSES = TILE / RPP;
   __shared__ __align__(16) bf16_t as[2][TILE * MM_LD];
   __shared__ __align__(16) bf16_t ws[2][TILE * MM_LD];
 
@@ -39,15 +40,15 @@ __global__ __launch_bounds__(256) void linear_mfma_kernel(
   const int wr = (wave >> 1) * (WT * 16), wc = (wave & 1) * (WT * 16);  // this wave's quarter
   const int lrow = lane & 15, lk = (lane >> 4) * 8;
 
-  // staging: thread t copies 16 bytes of rows (t >> 2) + 64 * pass, k offset (t & 3) * 8
-  const int srow = tid >> 2, sk = (tid & 3) * 8;
+  // staging: thread t copies 16 bytes of rows (t / TPR) + RPP * pass, k offset (t % TPR) * 8
+  const int srow = tid / TPR, sk = (tid % TPR) * 8;
   const bf16x8_t zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
   bf16x8_t ga[PASSES], gw[PASSES];
 
   auto load_global = [&](int k0) {
 #pragma unroll
     for (int p = 0; p < PASSES; ++p) {
-      const int r = srow + p * 64;
+      const int r = srow + p * RPP;
       const bool k_ok = k0 + sk + 8 <= k_dim;
       const int an = row0 + r, wo = col0 + r;
       const bool a_ok = k_ok && an < n_rows, w_ok = k_ok && wo < n_out;
@@ -60,7 +61,7 @@ __global__ __launch_bounds__(256) void linear_mfma_kernel(
   auto store_lds = [&](int buf) {
 #pragma unroll
     for (int p = 0; p < PASSES; ++p) {
-      const int r = srow + p * 64;
+      const int r = srow + p * RPP;
       *reinterpret_cast<bf16x8_t*>(&as[buf][r * MM_LD + sk]) = ga[p];
       *reinterpret_cast<bf16x8_t*>(&ws[buf][r * MM_LD + sk]) = gw[p];
     }
@@ -79,17 +80,20 @@ __global__ __launch_bounds__(256) void linear_mfma_kernel(
   for (int s = 0; s < k_steps; ++s) {
     const int buf = s & 1;
     if (s + 1 < k_steps) load_global((s + 1) * MM_BK);
-    bf16x8_t wf[WT], af[WT];
 #pragma unroll
-    for (int i = 0; i < WT; ++i) {
-      wf[i] = *reinterpret_cast<const bf16x8_t*>(&ws[buf][(wc + i * 16 + lrow) * MM_LD + lk]);
-      af[i] = *reinterpret_cast<const bf16x8_t*>(&as[buf][(wr + i * 16 + lrow) * MM_LD + lk]);
+    for (int kk = 0; kk < MM_BK; kk += 32) {
+      bf16x8_t wf[WT], af[WT];
+#pragma unroll
+      for (int i = 0; i < WT; ++i) {
+        wf[i] = *reinterpret_cast<const bf16x8_t*>(&ws[buf][(wc + i * 16 + lrow) * MM_LD + kk + lk]);
+        af[i] = *reinterpret_cast<const bf16x8_t*>(&as[buf][(wr + i * 16 + lrow) * MM_LD + kk + lk]);
+      }
+#pragma unroll
+      for (int i = 0; i < WT; ++i)
+#pragma unroll
+        for (int j = 0; j < WT; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[i], af[j], acc[i][j], 0, 0, 0);
     }
-#pragma unroll
-    for (int i = 0; i < WT; ++i)
-#pragma unroll
-      for (int j = 0; j < WT; ++j)
-        acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[i], af[j], acc[i][j], 0, 0, 0);
     if (s + 1 < k_steps) {
       store_lds(buf ^ 1);  // the other buffer: its readers finished before the last barrier
       __syncthreads();
