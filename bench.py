@@ -130,10 +130,16 @@ def main() -> int:
     ap.add_argument("--no-graph", action="store_true")
     ap.add_argument("--burst", type=int, default=8, help="decode steps enqueued back to back (1 = off)")
     ap.add_argument("--no-extras", action="store_true", help="skip prefill and the batch 1 / 64 points")
+    ap.add_argument("--prefill-only", action="store_true",
+                    help="run only the 2,048-token prefill and print its record (for profiling)")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
         return 2
+
+    if args.prefill_only:
+        print(json.dumps({"prefill": prefill_run(args, args.dtype, reps=10)}))
+        return 0
 
     elapsed, mean_ctx, engine, cfg = decode_run(args, args.batch, args.steps, args.warmup, args.dtype)
     itemsize = 2 if args.dtype == "bfloat16" else 4
