@@ -20,13 +20,18 @@ CONFIGS: Dict[str, GPTConfig] = {
                    layer_norm_eps=1e-5),
     "B": GPTConfig("gpt2-mini", n_layer=3, n_embd=96, n_head=3, vocab_size=503, block_size=128, bias=False,
                    layer_norm_eps=1e-6),
+    # head sizes that are no power of two (48, 80) and a width that is no multiple of 64
+    "C": GPTConfig("gpt2-mini", n_layer=2, n_embd=144, n_head=3, vocab_size=131, block_size=96, bias=True,
+                   layer_norm_eps=1e-4),
+    "D": GPTConfig("gpt2-mini", n_layer=1, n_embd=80, n_head=1, vocab_size=77, block_size=200, bias=False,
+                   layer_norm_eps=1e-5),
     "LONG": GPTConfig("gpt2-mini", n_layer=1, n_embd=48, n_head=1, vocab_size=61, block_size=640, bias=True,
                       layer_norm_eps=1e-3),
 }
-SEEDS = {"A": 0, "B": 1, "LONG": 2}
+SEEDS = {"A": 0, "B": 1, "C": 3, "D": 4, "LONG": 2}
 # The init rule's standard deviations give nearly uniform attention and tiny logits, which hides
 # faults; the tests scale them up so that softmax is peaked and every path carries signal.
-STD_SCALE = {"A": 5.0, "B": 5.0, "LONG": 6.0}
+STD_SCALE = {"A": 5.0, "B": 5.0, "C": 4.0, "D": 5.0, "LONG": 6.0}
 
 # Tolerances, fixed before any kernel was measured.  float32: summation order only.  bfloat16:
 # activations and weights carry 8 bits of mantissa (relative 2^-9 per rounding, a handful of

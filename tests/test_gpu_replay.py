@@ -17,7 +17,8 @@ from mini_gpt_inference_amd.engine.replay import TraceError, TraceReplayer
 
 pytestmark = pytest.mark.gpu
 
-LENGTHS = {"A": [5, 17, 30, 64, 41, 23], "B": [1, 9, 33, 64, 100, 128]}
+LENGTHS = {"A": [5, 17, 30, 64, 41, 23], "B": [1, 9, 33, 64, 100, 128], "C": [2, 96, 40, 71, 18],
+           "D": [200, 3, 130, 77, 150]}
 
 
 def _requests(name, rng):
@@ -58,6 +59,23 @@ def test_every_way_of_cutting_matches_the_plain_implementation(model_folders, na
     if way == "mixed":
         total = sum(-(-len(t) // page_size) for t in reqs.values())
         assert total > replayer.num_pages, "the pool is so large that no page was used twice"
+
+
+@pytest.mark.parametrize("way", ["whole", "tail", "portions", "mixed"])
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["C", "D"])
+def test_head_sizes_that_are_no_power_of_two(model_folders, name, dtype, way):
+    """Head sizes 48 and 80 and widths 144 and 80: the kernels that only take some head sizes must
+    hand over to the general ones, never compute something else."""
+    reqs = _requests(name, np.random.default_rng(17))
+    want = _plain_logits(model_folders[name], name, reqs)
+    plan = helpers.PLANS[way](reqs, np.random.default_rng(6))
+    replayer = TraceReplayer(model_folders[name], dtype, plan.tight_tokens(16), poison=True)
+    got = plan.assemble(helpers.run_plan_in_process(replayer, plan), {r: len(t) for r, t in reqs.items()},
+                        helpers.CONFIGS[name].vocab_size)
+    for rid in reqs:
+        helpers.assert_close(got[rid], want[rid], dtype, f"{name} {dtype} {way} {rid}")
+    assert replayer.cache.check() == 0 and replayer.cache.num_free_pages() == replayer.num_pages
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
