@@ -42,7 +42,8 @@ class TraceReplayer:
 
     def run_step(self, record: dict) -> Optional[torch.Tensor]:
         """One line of a trace.  Returns float32 logits [wanted, vocab] on the device, or None when
-        the step wants none."""
+        the step wants none.  The result lives in the step function's workspace: the next step
+        overwrites it, so copy what is to be kept."""
         step = record.get("step")
         slots, ctx_lens, q_lens, tokens, rows, ids = [], [], [], [], [], []
         for entry in record.get("entries", []):

@@ -116,6 +116,7 @@ class Scheduler:
                 _p(h["token_ids"]), _p(h["positions"]), _p(h["q_req"]), _p(h["cu_q"]), _p(h["seq_lens"]),
                 _p(h["slot_mapping"]), _p(h["block_tables"]), _p(h["state_slots"]), _p(h["logit_rows"]),
                 _p(h["temperature"]), _p(h["top_k"]), _p(h["top_p"]), _p(h["seeds"]), _p(h["out_index"]))
+        arena.host_ready()
         rc = self._lib.mgpt_sched_fill(self._h, self.cache.handle, step_offset, *args)
         if rc != 0:
             raise SchedulerError(f"filling the step failed ({rc}) {library.host_error()}")

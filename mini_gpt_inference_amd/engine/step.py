@@ -66,9 +66,20 @@ class StepArena:
         self.d["seeds"] = self.d["seeds"].view(torch.int64)
         self.tokens_out = torch.zeros(m_cap, dtype=torch.int32, device=device)
         self.tokens_host = torch.zeros(m_cap, dtype=torch.int32, pin_memory=device.type == "cuda")
+        self._uploaded: Optional[torch.cuda.Event] = None
 
     def upload(self) -> None:
         self.dev_t.copy_(self.host_t, non_blocking=True)
+        if self.dev_t.is_cuda:
+            if self._uploaded is None:
+                self._uploaded = torch.cuda.Event()
+            self._uploaded.record()
+
+    def host_ready(self) -> None:
+        """Call before writing the host arrays: the copy of the last upload reads them when the
+        device gets there, which may be later than the host's next step."""
+        if self._uploaded is not None:
+            self._uploaded.synchronize()
 
 
 @dataclass
@@ -116,6 +127,7 @@ class ModelRunner:
                  tokens: Sequence[int], logit_rows: Sequence[int]) -> StepShape:
         """Fills the arena for requests given by their cache slots: request i brings q_lens[i] tokens
         (its part of the flat `tokens`) on top of ctx_lens[i] cached ones.  logit_rows index `tokens`."""
+        arena.host_ready()
         h = arena.h
         self.check_positions(ctx_lens, q_lens)
         n = self.cache.build_step(slots, ctx_lens, q_lens, arena.n_cap, arena.r_cap, arena.max_blocks,

@@ -226,3 +226,34 @@ def test_a_far_key_among_hundreds_decides_the_result(tmp_path, dtype, far):
     other[far] = 7
     moved = np.abs(P.plain_forward(w, pcfg, other).numpy()[-1] - want[-1]).max()
     assert moved > 10 * helpers.TOL[dtype] * max(1.0, np.abs(want[-1]).max())
+
+
+FAMILY = {
+    # the reference family's real widths, head counts and odd vocabulary, with few layers to keep it quick
+    "small": dict(n_layer=2, n_embd=768, n_head=12, vocab_size=50257, block_size=1024, bias=True),
+    "xl": dict(n_layer=1, n_embd=1600, n_head=25, vocab_size=50257, block_size=1024, bias=True),
+    "50M": dict(n_layer=2, n_embd=512, n_head=8, vocab_size=50304, block_size=1024, bias=True),
+}
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("shape", ["small", "xl", "50M"])
+def test_real_family_sizes(tmp_path, shape, dtype):
+    """Widths 512/768/1600, 25 heads, vocabularies 50257 and 50304: a prompt portion, a second
+    portion over the cache, and single tokens, against the plain implementation."""
+    from mini_gpt_inference_amd import GPTConfig
+    from mini_gpt_inference_amd.weights.random_init import write_random_model
+    cfg = GPTConfig("gpt2-mini", layer_norm_eps=1e-5, **FAMILY[shape])
+    folder = write_random_model(str(tmp_path / shape), cfg, 7, std_scale=2.0)
+    rng = np.random.default_rng(1)
+    ids = helpers.random_ids(rng, cfg.vocab_size, 90)
+    pcfg, w = P.read_model_folder(folder)
+    want = P.plain_forward(w, pcfg, ids).numpy()
+    rep = TraceReplayer(folder, dtype, 128, poison=True)
+    # no wait between the steps, and each result copied on the device: a step must not disturb the
+    # inputs of the one before it while the device is still behind
+    got = [rep.run_step({"step": 0, "entries": [{"id": "x", "tokens": ids[:70], "want": [0, 33, 69]}], "end": []}).clone(),
+           rep.run_step({"step": 1, "entries": [{"id": "x", "tokens": ids[70:87], "want": [0, 16]}], "end": []}).clone()]
+    for i in range(87, 90):
+        got.append(rep.run_step({"step": i, "entries": [{"id": "x", "tokens": ids[i:i + 1], "want": [0]}], "end": []}).clone())
+    helpers.assert_close(torch.cat(got), want[[0, 33, 69, 70, 86, 87, 88, 89]], dtype, f"{shape} {dtype}")
