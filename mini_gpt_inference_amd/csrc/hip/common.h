@@ -25,12 +25,19 @@ __device__ __forceinline__ float bf16_to_float(bf16_t v) {
   return __uint_as_float(((unsigned int)v) << 16);
 }
 
-// round-to-nearest-even, NaN kept quiet
+// round-to-nearest-even, NaN kept quiet: gfx950 converts in hardware (v_cvt_pk_bf16_f32)
 __device__ __forceinline__ bf16_t float_to_bf16(float f) {
-  unsigned int u = __float_as_uint(f);
-  if ((u & 0x7fffffffu) > 0x7f800000u) return (bf16_t)0x7fc0;
-  u += 0x7fffu + ((u >> 16) & 1u);
-  return (bf16_t)(u >> 16);
+  const __bf16 b = (__bf16)f;
+  return __builtin_bit_cast(bf16_t, b);
+}
+
+// two floats to two bfloat16 in one register, `lo` in the low half
+__device__ __forceinline__ unsigned int pack_bf16x2(float lo, float hi) {
+  typedef __attribute__((__vector_size__(2 * sizeof(float)))) float f32x2_t;
+  typedef __attribute__((__vector_size__(2 * sizeof(__bf16)))) __bf16 bf16x2_t;
+  const f32x2_t f = {lo, hi};
+  const bf16x2_t b = __builtin_convertvector(f, bf16x2_t);
+  return __builtin_bit_cast(unsigned int, b);
 }
 
 template <typename T> __device__ __forceinline__ float to_float(T v);

@@ -18,38 +18,7 @@
 // Epilogues: plain store (bfloat16 or float32), GELU-tanh, add into the float32
 // residual stream, or store plus scatter of the key and value columns into
 // their cache pages by slot_mapping (src/minigpt_infer/cache/paged.py:125-137).
-#include "common.h"
-
-typedef __attribute__((__vector_size__(8 * sizeof(short)))) short bf16x8_t;
-typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4_t;
-
-#define SK_EPI_NONE 0
-#define SK_EPI_GELU 1
-#define SK_EPI_RESIDUAL 2
-#define SK_EPI_QKV 3
-
-#define SK_WAVES 4        // waves of a workgroup without a prologue
-#define SK_LN_WAVES 16    // waves of a workgroup with the LayerNorm prologue: one row each
-
-struct SkinnyArgs {
-  const bf16_t* act;  // [n_rows, k_dim] bfloat16, row stride lda (no prologue)
-  long lda;
-  const float* x;     // residual stream, float32, row stride k_dim (folded LayerNorm)
-  const int* rows;    // optional gather of residual rows
-  const float* colsum;  // S[o] of the folded matrix
-  float eps;
-  const bf16_t* w;    // [n_out, k_dim] (the folded matrix when x is given)
-  const float* bias;  // [n_out] or null (the folded bias when x is given)
-  void* out;          // [n_rows, n_out], row stride ldo
-  long ldo;
-  int n_rows, n_out, k_dim;
-  int ksplit;         // waves of a workgroup that share a column tile: 1, 2 or 4
-  // key/value scatter (SK_EPI_QKV)
-  bf16_t* kpool;
-  bf16_t* vpool;
-  const int* slot_mapping;
-  int q_width, kv_width, head_dim, n_kv_head, page_size;
-};
+#include "linear_skinny.h"
 
 __device__ __forceinline__ bf16x8_t load8(const bf16_t* p) {
   return *reinterpret_cast<const bf16x8_t*>(p);
@@ -276,8 +245,8 @@ __global__ __launch_bounds__(WAVES * 64) void linear_skinny_kernel(SkinnyArgs a)
         *dst = r;
       } else if (whole && EPI != SK_EPI_RESIDUAL) {
         uint2 pk;
-        pk.x = (unsigned int)float_to_bf16(v[0]) | ((unsigned int)float_to_bf16(v[1]) << 16);
-        pk.y = (unsigned int)float_to_bf16(v[2]) | ((unsigned int)float_to_bf16(v[3]) << 16);
+        pk.x = pack_bf16x2(v[0], v[1]);
+        pk.y = pack_bf16x2(v[2], v[3]);
         *reinterpret_cast<uint2*>(orow + oc) = pk;
       } else {
 #pragma unroll
@@ -302,8 +271,8 @@ __global__ __launch_bounds__(WAVES * 64) void linear_skinny_kernel(SkinnyArgs a)
           const int h = cc / a.head_dim, d = cc - h * a.head_dim;
           const long dst = ((page * a.n_kv_head + h) * a.page_size + off) * (long)a.head_dim + d;
           uint2 pk;
-          pk.x = (unsigned int)float_to_bf16(v[0]) | ((unsigned int)float_to_bf16(v[1]) << 16);
-          pk.y = (unsigned int)float_to_bf16(v[2]) | ((unsigned int)float_to_bf16(v[3]) << 16);
+          pk.x = pack_bf16x2(v[0], v[1]);
+          pk.y = pack_bf16x2(v[2], v[3]);
           *reinterpret_cast<uint2*>((is_v ? a.vpool : a.kpool) + dst) = pk;
         }
       }
@@ -328,13 +297,14 @@ static int launch_nt(const SkinnyArgs& a, int epi, int out_dtype, dim3 grid, siz
 // With x given (then act is ignored) the rows are read from the float32 residual stream through
 // a LayerNorm whose gain and bias were folded into w, bias and colsum (fold_norm.hip); otherwise
 // act holds bfloat16 activations.  Refuses (MGPT_ERR_BAD_SHAPE) more than 64 rows and k_dim that
-// is no multiple of 16; the caller then takes the general kernels.
+// is no multiple of 16; the caller then takes the general kernels.  general_only != 0 keeps to this
+// file's kernel also where linear_decode.hip would take the shape.
 extern "C" int mgpt_linear_skinny(const void* act, long lda, const float* x, const int* rows,
                                   const float* colsum, float eps, const void* w,
                                   const float* bias, void* out, int out_dtype, long ldo, int n_rows,
                                   int n_out, int k_dim, int epilogue, void* kpool, void* vpool,
                                   const int* slot_mapping, int q_width, int kv_width, int head_dim,
-                                  int n_kv_head, int page_size, hipStream_t stream) {
+                                  int n_kv_head, int page_size, int general_only, hipStream_t stream) {
   if (n_rows == 0 || n_out == 0) return MGPT_OK;
   if (!w || !out || (!act && !x)) return MGPT_ERR_NULL;
   if (n_rows < 0 || n_rows > 64 || n_out < 0 || k_dim <= 0 || (k_dim % 16) != 0 || ldo < n_out)
@@ -369,6 +339,11 @@ extern "C" int mgpt_linear_skinny(const void* act, long lda, const float* x, con
   a.k_dim = k_dim; a.ksplit = ks; a.kpool = (bf16_t*)kpool; a.vpool = (bf16_t*)vpool;
   a.slot_mapping = slot_mapping; a.q_width = q_width; a.kv_width = kv_width; a.head_dim = head_dim;
   a.n_kv_head = n_kv_head; a.page_size = page_size;
+  if (!general_only) {
+    // the rows of a decode step: the kernel laid out for latency, where it takes the shape
+    const int rc = mgpt_launch_linear_decode(a, epilogue, out_dtype, stream);
+    if (rc != MGPT_ERR_BAD_SHAPE) return rc;
+  }
   const int cw_per_wg = waves / ks;
   const int n_groups = (tiles + cw_per_wg - 1) / cw_per_wg;
   // few enough workgroups that each walks several column groups and reuses its activations

@@ -231,12 +231,13 @@ def fold_layer_norm(w: torch.Tensor, gain: torch.Tensor, beta: Optional[torch.Te
 def linear_skinny(a: Optional[torch.Tensor], w: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor,
                   n_rows: int, epilogue: int = EPI_NONE, *, ln_x: Optional[torch.Tensor] = None,
                   ln_colsum: Optional[torch.Tensor] = None, ln_eps: float = 0.0,
-                  ln_rows: Optional[torch.Tensor] = None, scatter=None) -> bool:
+                  ln_rows: Optional[torch.Tensor] = None, scatter=None, general_only: bool = False) -> bool:
     """bfloat16 MFMA product for at most 64 rows.  With ln_x (the float32 residual stream; ln_rows an
     optional gather) the rows are read through a LayerNorm that fold_layer_norm folded into w, bias
     and ln_colsum.  scatter = (k_pool, v_pool, slot_mapping, q_width, kv_width) also stores the new
-    keys and values into their pages.  Returns False, having launched nothing, when the kernel does
-    not take the shape."""
+    keys and values into their pages.  Up to 16 rows with an inner size that is a multiple of 32 go
+    to the kernel laid out for a decode step's latency unless general_only is set.  Returns False,
+    having launched nothing, when the kernel does not take the shape."""
     if n_rows > _SKINNY_MAX_ROWS or w.dtype != torch.bfloat16:
         return False
     n_out, k_dim = w.shape
@@ -281,7 +282,8 @@ def linear_skinny(a: Optional[torch.Tensor], w: torch.Tensor, bias: Optional[tor
     rc = library.kernels().mgpt_linear_skinny(
         _ptr(a if ln_x is None else None), lda, _ptr(ln_x), _ptr(ln_rows), _ptr(ln_colsum),
         float(ln_eps), _ptr(w), _ptr(bias), _ptr(out), _dtype_code(out), out.stride(0), n_rows, n_out, k_dim,
-        epilogue, _ptr(kp), _ptr(vp), _ptr(sm), q_width, kv_width, head_dim, n_kv_head, page_size, _stream())
+        epilogue, _ptr(kp), _ptr(vp), _ptr(sm), q_width, kv_width, head_dim, n_kv_head, page_size,
+        1 if general_only else 0, _stream())
     if rc == -2:
         return False
     _check(rc, "linear_skinny")

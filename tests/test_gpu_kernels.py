@@ -89,20 +89,25 @@ def test_linear_generic_refuses_bad_inner_size():
         kernels.linear_generic(a.cpu(), w, None, torch.zeros(4, 8, device=DEV), 4)
 
 
+# general=False lets the kernel for a decode step's rows (at most 16, inner size a multiple of 32)
+# take what it can; general=True keeps every case on the kernel for up to 64 rows
+@pytest.mark.parametrize("general", [False, True])
 @pytest.mark.parametrize("n,k,o", [(1, 64, 257), (8, 512, 1536), (17, 96, 503), (33, 80, 48), (64, 2048, 512),
-                                   (5, 48, 16)])
+                                   (5, 48, 16), (16, 160, 503), (12, 1600, 48), (7, 2048, 512), (3, 32, 20),
+                                   (9, 768, 130)])
 @pytest.mark.parametrize("epi,o_dt", [(kernels.EPI_NONE, "bfloat16"), (kernels.EPI_NONE, "float32"),
                                       (kernels.EPI_GELU, "bfloat16"), (kernels.EPI_RESIDUAL, "float32")])
-def test_linear_skinny(n, k, o, epi, o_dt):
+def test_linear_skinny(n, k, o, epi, o_dt, general):
     g = torch.Generator().manual_seed(3)
-    a, w, bias = rnd(g, n, k, dtype="bfloat16"), rnd(g, o, k, dtype="bfloat16", scale=k ** -0.5), rnd(g, o)
-    prev = rnd(g, n, o, dtype=o_dt)
+    a, w, bias = rnd(g, n + 2, k, dtype="bfloat16"), rnd(g, o, k, dtype="bfloat16", scale=k ** -0.5), rnd(g, o)
+    prev = rnd(g, n + 2, o, dtype=o_dt)
     out = prev.clone().to(DEV)
-    assert kernels.linear_skinny(a.to(DEV), w.to(DEV), bias.to(DEV), out, n, epi)
-    helpers.assert_close(out, _linear_want(a, w, bias, epi, prev), "bfloat16", f"skinny {n}x{k}x{o}")
+    assert kernels.linear_skinny(a.to(DEV), w.to(DEV), bias.to(DEV), out, n, epi, general_only=general)
+    helpers.assert_close(out[:n], _linear_want(a, w, bias, epi, prev)[:n], "bfloat16", f"skinny {n}x{k}x{o}")
+    assert torch.equal(out[n:], prev[n:].to(DEV)), "rows beyond n_rows were written"
     out2 = prev.clone().to(DEV)
-    assert kernels.linear_skinny(a.to(DEV), w.to(DEV), None, out2, n, epi)
-    helpers.assert_close(out2, _linear_want(a, w, None, epi, prev), "bfloat16", "skinny without bias")
+    assert kernels.linear_skinny(a.to(DEV), w.to(DEV), None, out2, n, epi, general_only=general)
+    helpers.assert_close(out2[:n], _linear_want(a, w, None, epi, prev)[:n], "bfloat16", "skinny without bias")
 
 
 @pytest.mark.parametrize("n,k,o", [(65, 64, 257), (300, 512, 1536), (129, 96, 503), (2048, 80, 48), (128, 2048, 128),
@@ -123,10 +128,12 @@ def test_linear_mfma(n, k, o, epi, o_dt):
     helpers.assert_close(out2[:n - 3], _linear_want(a, w, None, epi, prev)[:n - 3], "bfloat16", "mfma partial rows")
 
 
+@pytest.mark.parametrize("general", [False, True])
 @pytest.mark.parametrize("n,k,o,ln_bias,gather", [(8, 512, 1536, True, False), (3, 96, 503, False, True),
                                                   (40, 80, 257, True, True), (64, 2048, 64, False, False),
-                                                  (17, 1600, 48, True, False)])
-def test_linear_skinny_through_a_folded_layer_norm(n, k, o, ln_bias, gather):
+                                                  (17, 1600, 48, True, False), (16, 1600, 130, True, True),
+                                                  (1, 160, 48, False, False), (5, 768, 2050, True, True)])
+def test_linear_skinny_through_a_folded_layer_norm(n, k, o, ln_bias, gather, general):
     g = torch.Generator().manual_seed(4)
     x = rnd(g, 70, k, scale=2.0) + 0.5
     x[:, 3] += 40.0                      # an outlier channel, as residual streams have
@@ -140,12 +147,13 @@ def test_linear_skinny_through_a_folded_layer_norm(n, k, o, ln_bias, gather):
     helpers.assert_close(bias_f, bias.double() + (w.double() @ lb.double() if ln_bias else 0), "float32", "folded bias")
     out = torch.empty(n, o, dtype=torch.float32, device=DEV)
     assert kernels.linear_skinny(None, wf, bias_f, out, n, kernels.EPI_NONE, ln_x=x.to(DEV), ln_colsum=colsum,
-                                 ln_eps=1e-5, ln_rows=i32(rows) if gather else None)
+                                 ln_eps=1e-5, ln_rows=i32(rows) if gather else None, general_only=general)
     h = P.plain_layer_norm(x.double()[rows], lw.double(), lb.double() if ln_bias else None, 1e-5)
     helpers.assert_close(out, P.plain_linear(h, w.double(), bias.double()), "bfloat16", "LN + skinny")
 
 
-def test_linear_skinny_stores_keys_and_values():
+@pytest.mark.parametrize("general", [False, True])
+def test_linear_skinny_stores_keys_and_values(general):
     g = torch.Generator().manual_seed(5)
     n, k, h, hk, d, page, pages = 6, 64, 4, 2, 16, 4, 9
     qw, kvw = h * d, hk * d
@@ -155,7 +163,7 @@ def test_linear_skinny_stores_keys_and_values():
     slots = [4 * 8 + 3, 0, 7, -1, 4 * 2 + 1, 4 * 8 + 0]
     out = torch.empty(n, qw + 2 * kvw, dtype=torch.bfloat16, device=DEV)
     assert kernels.linear_skinny(a.to(DEV), w.to(DEV), bias.to(DEV), out, n, kernels.SK_EPI_QKV,
-                                 scatter=(kp, vp, i32(slots), qw, kvw))
+                                 scatter=(kp, vp, i32(slots), qw, kvw), general_only=general)
     want = P.plain_linear(a.double(), w.double(), bias.double())
     helpers.assert_close(out, want, "bfloat16", "qkv")
     written = torch.zeros(pages * page, dtype=torch.bool)
