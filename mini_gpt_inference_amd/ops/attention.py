@@ -11,11 +11,16 @@ def paged_attention(ctx, q: torch.Tensor, out: torch.Tensor, k_pool: torch.Tenso
                     group, n_head: int, scale: float, window: int) -> None:
     """Attention of the step's tokens (rows of q) over their requests' pages.
 
-    On the bfloat16 path steps with prompt portions use the MFMA tile kernel and the rest the
-    kernel that splits a query's keys over four waves; the 32-bit path and every shape those
-    refuse use the general kernel, whose order of sums depends only on a query's position."""
+    On the bfloat16 path a decode-only step (token n is request n's one token) uses the kernel
+    laid out for a decode step's latency, steps with prompt portions the MFMA tile kernel and the
+    rest the kernel that splits a query's keys over four waves; the 32-bit path and every shape
+    those refuse use the general kernel, whose order of sums depends only on a query's position."""
     n, r = ctx.n_rows, ctx.cu_q.numel() - 1
     if q.dtype == torch.bfloat16 and not ctx.exact:
+        if ctx.decode_only and kernels.paged_attention_decode_bf16(
+                q, out, k_pool, v_pool, group.block_tables, ctx.positions, ctx.q_req, n, n_head, scale, window,
+                identity=True):
+            return
         if not ctx.decode_only and ctx.n_rows == ctx.n_tokens and kernels.prefill_attention_bf16(
                 q, out, k_pool, v_pool, group.block_tables, ctx.cu_q, ctx.seq_lens, ctx.n_req, ctx.max_q_len,
                 n_head, scale, window):

@@ -315,6 +315,45 @@ def paged_attention_split_bf16(q: torch.Tensor, out: torch.Tensor, k_pool: torch
     return True
 
 
+def paged_attention_decode_bf16(q: torch.Tensor, out: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor,
+                                block_tables: torch.Tensor, positions: torch.Tensor, q_req: torch.Tensor,
+                                n_tokens: int, n_head: int, scale: float, window: int = 0,
+                                identity: bool = False) -> bool:
+    """bfloat16 attention for single tokens (one query per request and step), keys split over eight
+    waves.  positions[n] is token n's absolute position, q_req[n] its block table row or -1 for a
+    padded token; identity=True promises q_req[n] in (n, -1).  False if refused (other head sizes
+    than 16, 32, 64, 128)."""
+    if q.dtype != torch.bfloat16:
+        return False
+    _need_cuda(q, out, k_pool, v_pool, block_tables, positions, q_req)
+    _need(k_pool.shape == v_pool.shape and k_pool.dim() == 4 and k_pool.is_contiguous() and v_pool.is_contiguous()
+          and k_pool.dtype == torch.bfloat16 and v_pool.dtype == torch.bfloat16,
+          "key and value pools must be dense bfloat16 [pages, kv_heads, page_size, head_dim]")
+    num_pages, n_kv_head, page_size, head_dim = k_pool.shape
+    if head_dim not in (16, 32, 64, 128) or q.stride(0) % 8 != 0 or q.data_ptr() % 16 != 0 \
+            or k_pool.data_ptr() % 16 != 0 or v_pool.data_ptr() % 16 != 0:
+        return False
+    _need(q.dim() == 2 and q.stride(1) == 1 and q.shape[0] >= n_tokens and q.shape[1] >= n_head * head_dim,
+          "q must be [>=n_tokens, >=heads*head_dim] with unit inner stride")
+    _need(out.dtype == torch.bfloat16 and out.dim() == 2 and out.stride(1) == 1 and out.shape[0] >= n_tokens
+          and out.shape[1] >= n_head * head_dim, "out must be bfloat16 [>=n_tokens, >=heads*head_dim]")
+    _need(n_head % n_kv_head == 0, "query heads must be a multiple of key/value heads")
+    _need(block_tables.dtype == torch.int32 and block_tables.dim() == 2 and block_tables.is_contiguous(),
+          "block_tables must be dense int32 [requests, blocks]")
+    _need_i32("positions", positions, n_tokens)
+    _need_i32("q_req", q_req, n_tokens)
+    if identity:
+        _need(block_tables.shape[0] >= n_tokens, "a decode-only step needs a block table row per token")
+    rc = library.kernels().mgpt_paged_attention_decode_bf16(
+        _ptr(q), q.stride(0), _ptr(out), out.stride(0), _ptr(k_pool), _ptr(v_pool), _ptr(block_tables),
+        block_tables.shape[1], _ptr(positions), _ptr(q_req), n_tokens, n_head, n_kv_head, head_dim, page_size,
+        num_pages, float(scale), int(window), 1 if identity else 0, _stream())
+    if rc == -2:
+        return False
+    _check(rc, "paged_attention_decode_bf16")
+    return True
+
+
 def linear_mfma(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor,
                 n_rows: int, epilogue: int) -> bool:
     """Tiled bfloat16 MFMA product for many rows.  False when it does not take the shape."""

@@ -272,6 +272,49 @@ def test_paged_attention(kernel, case, window):
     helpers.assert_close(out, c.want(scale, window), dtype, f"{kernel} case {case} window {window}")
 
 
+DECODE_CASES = [
+    dict(seq_lens=[600, 1, 64, 65, 513, 300], q_lens=[1] * 6, h=4, hk=2, d=64, page=16),
+    dict(seq_lens=[130, 1030, 7], q_lens=[1] * 3, h=3, hk=3, d=128, page=32),
+    dict(seq_lens=[257, 31, 512, 511], q_lens=[1] * 4, h=6, hk=2, d=32, page=8),
+    dict(seq_lens=[90, 700], q_lens=[1] * 2, h=2, hk=1, d=16, page=4),
+    dict(seq_lens=[100, 550, 13], q_lens=[1] * 3, h=2, hk=2, d=64, page=12),   # a page size that is no power of two
+]
+
+
+@pytest.mark.parametrize("window", [0, 5, 70])
+@pytest.mark.parametrize("case", range(len(ATTENTION_CASES) + len(DECODE_CASES)))
+def test_paged_attention_decode(case, window):
+    """The decode step's kernel: by position and block table row, for any token; with identity=True
+    where every request brings one token.  Unused block table entries hold numbers far outside the
+    pool, and a padded token leaves its output row alone."""
+    spec = (ATTENTION_CASES + DECODE_CASES)[case]
+    if spec["d"] not in (16, 32, 64, 128):
+        pytest.skip("head sizes 16, 32, 64, 128")
+    c = PagedCase(**spec, dtype="bfloat16", seed=case)
+    scale = 0.37 if case % 2 else 1.0 / math.sqrt(c.d)
+    bt = c.bt.clone()
+    bt[bt < 0] = 10 ** 6
+    positions = i32([p for s, ql in zip(c.seq_lens, c.q_lens) for p in range(s - ql, s)] + [0])
+    q_req = torch.cat([c.q_req, i32([-1])])
+    q = torch.cat([c.q_flat, c.q_flat[:1]])
+    want = c.want(scale, window)
+    modes = [False, True] if all(ql == 1 for ql in c.q_lens) else [False]
+    for identity in modes:
+        out = torch.full((c.n + 1, c.h * c.d), 7.0, dtype=torch.bfloat16, device=DEV)
+        if identity:   # the padded token's row of the block table exists, as in a padded step
+            bt_i = torch.cat([bt, torch.full_like(bt[:1], 10 ** 6)])
+        else:
+            bt_i = bt
+        took = kernels.paged_attention_decode_bf16(q, out, c.kp, c.vp, bt_i, positions, q_req, c.n + 1, c.h, scale,
+                                                   window, identity=identity)
+        if c.page & (c.page - 1):
+            assert not took, "page sizes that are no power of two go to the general kernels"
+            return
+        assert took
+        helpers.assert_close(out[:c.n], want, "bfloat16", f"decode case {case} window {window} identity {identity}")
+        assert (out[c.n] == 7.0).all(), "a padded token's row was written"
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_kv_write_and_padding(dtype):
     g = torch.Generator().manual_seed(7)
