@@ -1,0 +1,283 @@
+// The kernel of linear_decode.hip and linear_decode_rows.hip: a matrix product for the rows of a
+// decode step in bfloat16 on the MFMA units, laid out for latency.
+//
+// out[n, o] = sum_k act[n, k] * W[o, k] (+ bias[o]), nn.Linear as in
+// src/minigpt_infer/model.py:43-44,96-101.
+//
+// A decode step is a chain of some forty dependent kernels that each read a megabyte or two,
+// so what counts is how soon a kernel is over, and that is set by the bytes one compute unit
+// has to pull through its own cache.  Hence: one workgroup of four waves per 16 output
+// columns (as many workgroups, on as many compute units, as the matrix has column tiles), the
+// waves split k four ways, every lane issues all its loads (W, activations, and what the
+// epilogue will need: bias, column sums, the old residual values, the cache slot) before it
+// waits for any, rows beyond n_rows are not loaded at all, one v_mfma_f32_16x16x32_bf16 per 32
+// k and 16 rows, the four waves' sums are added through LDS in wave order, and the first wave
+// stores.  NT tiles of 16 rows share the W a lane has loaded.  A wave's k range longer than SMAX
+// steps of 32 takes several passes of loads.
+//
+// Folded LayerNorm, epilogues and the key/value scatter are those of linear_skinny.hip (the
+// LayerNorm of src/minigpt_infer/model.py:113-114,186-187 folded into W by fold_norm.hip;
+// scatter as src/minigpt_infer/cache/paged.py:125-137).
+#pragma once
+#include "linear_skinny.h"
+
+// VEC: n_out is a multiple of 16 and bias, column sums and output rows are aligned for vectors of
+// four; otherwise every access of the epilogue is a single element with its own bound check.
+template <int NT, int SMAX, bool LN, int EPI, typename OT, bool VEC>
+__global__ __launch_bounds__(256) void linear_decode_kernel(SkinnyArgs a) {
+  __shared__ float red[3 * NT * 6 * 64];  // waves 1..3: per row tile four sums and two statistics per lane
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // the same in all lanes: branches on it are scalar
+  const int lrow = lane & 15, g = lane >> 4;
+  const int K = a.k_dim;
+  const int steps_total = K >> 5;
+  const int per = (steps_total + 3) >> 2;
+  const int steps = max(0, min(per, steps_total - wave * per));  // the last waves of a short k may have none
+  const int kb = steps > 0 ? wave * per * 32 : 0;
+  const int o0 = blockIdx.x * 16;
+  const int wo = min(o0 + lrow, a.n_out - 1);  // a column past the end reads the last row; never stored
+  const int oc = o0 + g * 4;  // this lane's four output columns, of rows lrow + 16 t
+  bool row_ok[NT];
+#pragma unroll
+  for (int t = 0; t < NT; ++t) row_ok[t] = t * 16 + lrow < a.n_rows;
+
+  // ---- every load this lane will need, issued before anything waits.  Loads are unconditional
+  // within a row (a k step past this wave's range reads the range's first step again and is not
+  // multiplied), so that nothing but the data stands between one load and the next.
+  int src[NT];
+#pragma unroll
+  for (int t = 0; t < NT; ++t) {
+    src[t] = t * 16 + lrow;
+    if (LN && a.rows != nullptr && row_ok[t]) src[t] = a.rows[t * 16 + lrow];
+  }
+  // the epilogue's inputs (first wave only)
+  const bool col_writer = wave == 0 && oc < a.n_out;
+  float bias4[4] = {0.f, 0.f, 0.f, 0.f}, cs4[4] = {0.f, 0.f, 0.f, 0.f};
+  float old4[NT][4];
+  int slot[NT];
+#pragma unroll
+  for (int t = 0; t < NT; ++t) {
+    slot[t] = -1;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) old4[t][i] = 0.f;
+  }
+  OT* const out = reinterpret_cast<OT*>(a.out);
+  if (col_writer) {
+    if (VEC) {
+      if (a.bias != nullptr) {
+        const float4 b4 = *reinterpret_cast<const float4*>(a.bias + oc);
+        bias4[0] = b4.x; bias4[1] = b4.y; bias4[2] = b4.z; bias4[3] = b4.w;
+      }
+      if (LN) {
+        const float4 c4 = *reinterpret_cast<const float4*>(a.colsum + oc);
+        cs4[0] = c4.x; cs4[1] = c4.y; cs4[2] = c4.z; cs4[3] = c4.w;
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int o = min(oc + i, a.n_out - 1);
+        if (a.bias != nullptr) bias4[i] = a.bias[o];
+        if (LN) cs4[i] = a.colsum[o];
+      }
+    }
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+      if (!row_ok[t]) continue;
+      const OT* orow = out + (long)(t * 16 + lrow) * a.ldo;
+      if (EPI == SK_EPI_RESIDUAL) {
+        if (VEC) {
+          const float4 o4 = *reinterpret_cast<const float4*>(orow + oc);
+          old4[t][0] = o4.x; old4[t][1] = o4.y; old4[t][2] = o4.z; old4[t][3] = o4.w;
+        } else {
+#pragma unroll
+          for (int i = 0; i < 4; ++i) old4[t][i] = to_float<OT>(orow[min(oc + i, a.n_out - 1)]);
+        }
+      }
+      if (EPI == SK_EPI_QKV) slot[t] = a.slot_mapping[t * 16 + lrow];
+    }
+  }
+
+  const bf16x8_t zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+  f32x4_t acc[NT];
+  float x0[NT], sd[NT], sq[NT];  // sums of (x - x0) and (x - x0)^2 over what this lane loads of its rows
+#pragma unroll
+  for (int t = 0; t < NT; ++t) {
+    acc[t] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+    x0[t] = sd[t] = sq[t] = 0.f;
+    if (LN && row_ok[t]) x0[t] = a.x[(long)src[t] * K];
+  }
+  const bf16_t* wp = a.w + (long)wo * K + kb + g * 8;
+  for (int s0 = 0; s0 < steps; s0 += SMAX) {
+    bf16x8_t wv[SMAX], av[NT][SMAX];
+#pragma unroll
+    for (int i = 0; i < SMAX; ++i)
+      wv[i] = *reinterpret_cast<const bf16x8_t*>(wp + (s0 + i < steps ? s0 + i : 0) * 32);
+    if (LN) {
+      float4 lo[NT][SMAX], hi[NT][SMAX];
+#pragma unroll
+      for (int t = 0; t < NT; ++t) {
+#pragma unroll
+        for (int i = 0; i < SMAX; ++i) lo[t][i] = hi[t][i] = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (row_ok[t]) {
+          const float* xr = a.x + (long)src[t] * K + kb + g * 8;
+#pragma unroll
+          for (int i = 0; i < SMAX; ++i) {
+            const float4* p = reinterpret_cast<const float4*>(xr + (s0 + i < steps ? s0 + i : 0) * 32);
+            lo[t][i] = p[0];
+            hi[t][i] = p[1];
+          }
+        }
+      }
+#pragma unroll
+      for (int t = 0; t < NT; ++t) {
+#pragma unroll
+        for (int i = 0; i < SMAX; ++i) {
+          const float f[8] = {lo[t][i].x, lo[t][i].y, lo[t][i].z, lo[t][i].w,
+                              hi[t][i].x, hi[t][i].y, hi[t][i].z, hi[t][i].w};
+          typedef __attribute__((__vector_size__(4 * sizeof(unsigned int)))) unsigned int u32x4_t;
+          const u32x4_t pk = {pack_bf16x2(f[0], f[1]), pack_bf16x2(f[2], f[3]), pack_bf16x2(f[4], f[5]),
+                              pack_bf16x2(f[6], f[7])};
+          av[t][i] = __builtin_bit_cast(bf16x8_t, pk);
+          if (s0 + i < steps) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+              const float d = f[e] - x0[t];
+              sd[t] += d;
+              sq[t] = fmaf(d, d, sq[t]);
+            }
+          }
+        }
+      }
+    } else {
+#pragma unroll
+      for (int t = 0; t < NT; ++t) {
+#pragma unroll
+        for (int i = 0; i < SMAX; ++i) av[t][i] = zero8;
+        if (row_ok[t]) {
+          const bf16_t* ap = a.act + (long)(t * 16 + lrow) * a.lda + kb + g * 8;
+#pragma unroll
+          for (int i = 0; i < SMAX; ++i)
+            av[t][i] = *reinterpret_cast<const bf16x8_t*>(ap + (s0 + i < steps ? s0 + i : 0) * 32);
+        }
+      }
+    }
+    // ---- multiply
+#pragma unroll
+    for (int i = 0; i < SMAX; ++i)
+      if (s0 + i < steps) {
+#pragma unroll
+        for (int t = 0; t < NT; ++t) acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wv[i], av[t][i], acc[t], 0, 0, 0);
+      }
+  }
+  if (LN) {
+    // the four lanes that share a row hold parts of its sums
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+      sd[t] += __shfl_xor(sd[t], 16, 64);
+      sd[t] += __shfl_xor(sd[t], 32, 64);
+      sq[t] += __shfl_xor(sq[t], 16, 64);
+      sq[t] += __shfl_xor(sq[t], 32, 64);
+    }
+  }
+
+  // ---- the four waves' parts, added in wave order by the first
+  if (wave > 0) {
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+      float* r = red + ((wave - 1) * NT + t) * 6 * 64 + lane;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) r[i * 64] = acc[t][i];
+      if (LN) {
+        r[4 * 64] = sd[t];
+        r[5 * 64] = sq[t];
+      }
+    }
+  }
+  __syncthreads();
+  if (!col_writer) return;
+#pragma unroll
+  for (int s = 0; s < 3; ++s) {
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+      const float* r = red + (s * NT + t) * 6 * 64 + lane;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) acc[t][i] += r[i * 64];
+      if (LN) {
+        sd[t] += r[4 * 64];
+        sq[t] += r[5 * 64];
+      }
+    }
+  }
+
+  // ---- epilogue: lane holds out[t * 16 + lrow][oc + i], i = 0..3
+#pragma unroll
+  for (int t = 0; t < NT; ++t) {
+    if (!row_ok[t]) continue;
+    OT* orow = out + (long)(t * 16 + lrow) * a.ldo;
+    float v[4];
+    float mean = 0.f, rstd = 1.f;
+    if (LN) {
+      const float inv_k = 1.0f / (float)K;
+      const float md = sd[t] * inv_k;  // mean of x - x0
+      mean = x0[t] + md;
+      rstd = 1.0f / sqrtf(fmaxf(sq[t] * inv_k - md * md, 0.f) + a.eps);
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      v[i] = acc[t][i];
+      if (LN) v[i] = rstd * (v[i] - mean * cs4[i]);
+      v[i] += bias4[i];
+      if (EPI == SK_EPI_GELU) v[i] = gelu_tanh(v[i]);
+      if (EPI == SK_EPI_RESIDUAL) v[i] += old4[t][i];
+    }
+    if (VEC && sizeof(OT) == 4) {
+      *reinterpret_cast<float4*>(orow + oc) = make_float4(v[0], v[1], v[2], v[3]);
+    } else if (VEC) {
+      uint2 pk;
+      pk.x = pack_bf16x2(v[0], v[1]);
+      pk.y = pack_bf16x2(v[2], v[3]);
+      *reinterpret_cast<uint2*>(orow + oc) = pk;
+    } else {
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        if (oc + i < a.n_out) orow[oc + i] = from_float<OT>(v[i]);
+    }
+    if (EPI == SK_EPI_QKV) {
+      if (slot[t] >= 0 && oc >= a.q_width) {
+        // the four columns lie in one head (head sizes and widths are multiples of 4): one 8-byte store
+        const long page = slot[t] / a.page_size;
+        const int off = slot[t] - (int)page * a.page_size;
+        const int c = oc - a.q_width;  // column among keys then values
+        const bool is_v = c >= a.kv_width;
+        const int cc = is_v ? c - a.kv_width : c;
+        const int h = cc / a.head_dim, d = cc - h * a.head_dim;
+        const long dst = ((page * a.n_kv_head + h) * a.page_size + off) * (long)a.head_dim + d;
+        uint2 pk;
+        pk.x = pack_bf16x2(v[0], v[1]);
+        pk.y = pack_bf16x2(v[2], v[3]);
+        *reinterpret_cast<uint2*>((is_v ? a.vpool : a.kpool) + dst) = pk;
+      }
+    }
+  }
+}
+
+template <int NT, int SMAX, bool LN, bool VEC>
+static int launch_decode_epi(const SkinnyArgs& a, int epi, int out_dtype, dim3 grid, hipStream_t s) {
+#define LD_LAUNCH(E, OT) \
+  hipLaunchKernelGGL((linear_decode_kernel<NT, SMAX, LN, E, OT, VEC>), grid, dim3(256), 0, s, a)
+  if (epi == SK_EPI_NONE && out_dtype == MGPT_BF16) LD_LAUNCH(SK_EPI_NONE, bf16_t);
+  else if (epi == SK_EPI_NONE && out_dtype == MGPT_F32) LD_LAUNCH(SK_EPI_NONE, float);
+  else if (epi == SK_EPI_GELU && out_dtype == MGPT_BF16) LD_LAUNCH(SK_EPI_GELU, bf16_t);
+  else if (epi == SK_EPI_RESIDUAL && out_dtype == MGPT_F32) LD_LAUNCH(SK_EPI_RESIDUAL, float);
+  else if (epi == SK_EPI_QKV && out_dtype == MGPT_BF16) LD_LAUNCH(SK_EPI_QKV, bf16_t);
+  else return MGPT_ERR_BAD_DTYPE;
+#undef LD_LAUNCH
+  return mgpt_last_error();
+}
+
+// whether the epilogue may use vectors of four (see VEC above)
+static inline bool decode_vec_ok(const SkinnyArgs& a) {
+  const size_t align = sizeof(float) * 4 - 1;  // bfloat16 rows are stored 8 bytes at a time: covered as well
+  return (a.n_out % 16) == 0 && (a.ldo % 4) == 0 &&
+         ((((size_t)a.bias) | ((size_t)a.colsum) | ((size_t)a.out)) & align) == 0;
+}

@@ -33,6 +33,6 @@ struct SkinnyArgs {
   int q_width, kv_width, head_dim, n_kv_head, page_size;
 };
 
-// linear_decode.hip: at most 16 rows, k_dim a multiple of 32 and at most 2048.  Returns
+// linear_decode.hip: at most 64 rows, k_dim a multiple of 32.  Returns
 // MGPT_ERR_BAD_SHAPE for what it does not take (the general kernel then runs).
 int mgpt_launch_linear_decode(const SkinnyArgs& a, int epilogue, int out_dtype, hipStream_t stream);

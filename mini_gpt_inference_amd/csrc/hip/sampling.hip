@@ -103,11 +103,51 @@ __device__ __forceinline__ void scan_row(const float* __restrict__ lg, int nv, F
   }
 }
 
+// After a decode-only step (token n is request n's one token and every row is sampled) the row's
+// first thread can prepare the next step on the device: the sampled token becomes the next input,
+// position, length and output index go up by one, the cache slot of the new position is looked up
+// in the block tables (which already hold the pages of the steps planned ahead), and the token is
+// also appended to the row's column of a history that the host reads once at the end.  Then
+// several decode steps run back to back with no copy between them.  token_ids == nullptr: off.
+struct AdvanceArgs {
+  int* token_ids;
+  int* positions;
+  int* seq_lens;
+  int* out_index;
+  const int* q_req;         // -1: a padded row, left alone
+  int* slot_mapping;        // [n_groups][n_stride]
+  const int* block_tables;  // [n_groups][r_stride][max_blocks]
+  const int* page_sizes;    // [n_groups]
+  int n_groups, n_stride, r_stride, max_blocks;
+  int* history;             // [history_rows][history_stride]
+  int* history_pos;         // per row: how many tokens it has appended
+  int history_rows, history_stride;
+};
+
+__device__ __forceinline__ void finish_row(int row, int token, int* out_tokens, const AdvanceArgs& adv) {
+  out_tokens[row] = token;
+  if (adv.token_ids == nullptr || adv.q_req[row] < 0) return;
+  adv.token_ids[row] = token;
+  const int pos = adv.positions[row] + 1;
+  adv.positions[row] = pos;
+  adv.seq_lens[row] += 1;
+  adv.out_index[row] += 1;
+  for (int g = 0; g < adv.n_groups; ++g) {
+    const int ps = adv.page_sizes[g];
+    const int idx = pos / ps;
+    const int page = idx < adv.max_blocks ? adv.block_tables[((long)g * adv.r_stride + row) * adv.max_blocks + idx] : -1;
+    adv.slot_mapping[(long)g * adv.n_stride + row] = page >= 0 ? page * ps + pos % ps : -1;
+  }
+  const int j = adv.history_pos[row];
+  if (j < adv.history_rows) adv.history[(long)j * adv.history_stride + row] = token;
+  adv.history_pos[row] = j + 1;
+}
+
 __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
     const float* __restrict__ logits, long ld, int vocab, int real_vocab,
     const float* __restrict__ temperature, const int* __restrict__ top_k,
     const float* __restrict__ top_p, const uint64_t* __restrict__ request_seed,
-    const int* __restrict__ out_index, uint64_t engine_seed, int* __restrict__ out_tokens) {
+    const int* out_index, uint64_t engine_seed, int* out_tokens, AdvanceArgs adv) {
   __shared__ float red_f[SAMPLE_WAVES];
   __shared__ int red_i[SAMPLE_WAVES];
   __shared__ float part[SAMPLE_THREADS];
@@ -136,7 +176,7 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
     if (tid == 0) {
       for (int i = 1; i < SAMPLE_WAVES; ++i)
         if (red_f[i] > best || (red_f[i] == best && red_i[i] < best_i)) { best = red_f[i]; best_i = red_i[i]; }
-      out_tokens[row] = best_i == 0x7fffffff ? 0 : best_i;
+      finish_row(row, best_i == 0x7fffffff ? 0 : best_i, out_tokens, adv);
     }
     return;
   }
@@ -242,21 +282,52 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
       c = 0;
       for (int i = 0; i < SAMPLE_WAVES; ++i) c = max(c, red_i[i]);
     }
-    out_tokens[row] = c;
+    finish_row(row, c, out_tokens, adv);
   }
 }
 
 // logits: [n_rows, vocab] floats with row stride ld.  top_k (0 = off), top_p (1 = off),
 // request_seed and out_index may be null.
-extern "C" int mgpt_sample(const float* logits, long ld, int n_rows, int vocab, int real_vocab,
-                           const float* temperature, const int* top_k, const float* top_p,
-                           const uint64_t* request_seed, const int* out_index, uint64_t engine_seed,
-                           int* out_tokens, hipStream_t stream) {
+static int launch_sample(const float* logits, long ld, int n_rows, int vocab, int real_vocab,
+                         const float* temperature, const int* top_k, const float* top_p,
+                         const uint64_t* request_seed, const int* out_index, uint64_t engine_seed,
+                         int* out_tokens, const AdvanceArgs& adv, hipStream_t stream) {
   if (n_rows == 0) return MGPT_OK;
   if (!logits || !temperature || !out_tokens) return MGPT_ERR_NULL;
   if (n_rows < 0 || vocab <= 0 || real_vocab <= 0 || ld < vocab) return MGPT_ERR_BAD_SHAPE;
   hipLaunchKernelGGL(sample_kernel, dim3(n_rows), dim3(SAMPLE_THREADS), 0, stream, logits, ld, vocab,
                      real_vocab, temperature, top_k, top_p, request_seed, out_index, engine_seed,
-                     out_tokens);
+                     out_tokens, adv);
   return mgpt_last_error();
+}
+
+extern "C" int mgpt_sample(const float* logits, long ld, int n_rows, int vocab, int real_vocab,
+                           const float* temperature, const int* top_k, const float* top_p,
+                           const uint64_t* request_seed, const int* out_index, uint64_t engine_seed,
+                           int* out_tokens, hipStream_t stream) {
+  AdvanceArgs adv = {};
+  return launch_sample(logits, ld, n_rows, vocab, real_vocab, temperature, top_k, top_p, request_seed,
+                       out_index, engine_seed, out_tokens, adv, stream);
+}
+
+// mgpt_sample, then each row prepares the next decode step on the device (AdvanceArgs above).
+// Rows are requests: n_rows <= n_stride, r_stride.
+extern "C" int mgpt_sample_advance(const float* logits, long ld, int n_rows, int vocab, int real_vocab,
+                                   const float* temperature, const int* top_k, const float* top_p,
+                                   const uint64_t* request_seed, int* out_index, uint64_t engine_seed,
+                                   int* out_tokens, int* token_ids, int* positions, int* seq_lens,
+                                   const int* q_req, int* slot_mapping, const int* block_tables,
+                                   const int* page_sizes, int n_groups, int n_stride, int r_stride,
+                                   int max_blocks, int* history, int* history_pos, int history_rows,
+                                   int history_stride, hipStream_t stream) {
+  if (!token_ids || !positions || !seq_lens || !out_index || !q_req || !slot_mapping || !block_tables ||
+      !page_sizes || !history || !history_pos)
+    return MGPT_ERR_NULL;
+  if (n_groups <= 0 || n_rows > n_stride || n_rows > r_stride || max_blocks <= 0 || history_rows <= 0 ||
+      history_stride < n_rows)
+    return MGPT_ERR_BAD_SHAPE;
+  AdvanceArgs adv = {token_ids, positions, seq_lens, out_index, q_req, slot_mapping, block_tables, page_sizes,
+                     n_groups, n_stride, r_stride, max_blocks, history, history_pos, history_rows, history_stride};
+  return launch_sample(logits, ld, n_rows, vocab, real_vocab, temperature, top_k, top_p, request_seed,
+                       out_index, engine_seed, out_tokens, adv, stream);
 }

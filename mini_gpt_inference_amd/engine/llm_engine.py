@@ -28,42 +28,66 @@ _TORCH_DTYPES = {"bfloat16": torch.bfloat16, "float32": torch.float32}
 
 
 class _GraphedDecode:
-    """One captured HIP graph: a decode-only step (model + sampling) for up to `cap` requests.
-    The arena and the workspace are its own, so their addresses never change."""
+    """Captured HIP graphs of a decode-only step (model + sampling) for up to `cap` requests.  The
+    arena and the workspace are its own, so their addresses never change.  The sampling kernel also
+    turns the arena's device arrays into the next step's (its token, position, length, cache slot)
+    and appends the tokens to `history`, so that steps can follow each other with no copy between
+    them: `burst` of them are captured as one graph as well."""
 
-    def __init__(self, runner: ModelRunner, sampler: Sampler, cap: int) -> None:
-        self.runner, self.sampler, self.cap = runner, sampler, cap
+    def __init__(self, runner: ModelRunner, sampler: Sampler, cap: int, burst: int) -> None:
+        self.runner, self.sampler, self.cap, self.burst = runner, sampler, cap, max(burst, 1)
         self.arena = StepArena(cap, cap, cap, runner.n_groups, runner.max_blocks, runner.device)
         self.workspace = Workspace(runner.device)
+        self.history = torch.zeros(self.burst, cap, dtype=torch.int32, device=runner.device)
+        self.history_host = torch.zeros(self.burst, cap, dtype=torch.int32, pin_memory=runner.device.type == "cuda")
         self.graph: Optional[torch.cuda.CUDAGraph] = None
-        self.staging: List[StepArena] = []   # host sides of the steps of a burst
+        self.burst_graph: Optional[torch.cuda.CUDAGraph] = None
 
     def _launch(self, shape: StepShape) -> None:
         ctx = self.runner.context(self.arena, shape, padded=True, workspace=self.workspace)
         # launch geometry must not depend on this step's lengths: size it for the longest sequence
         ctx.max_seq_len = self.runner.max_positions or ctx.max_seq_len
         logits = self.runner.model.forward(ctx)
-        self.sampler.sample(logits, self.arena, self.cap)
+        self.sampler.sample(logits, self.arena, self.cap, advance=(self.runner.page_sizes, self.history))
+
+    def _capture(self, shape: StepShape, times: int) -> torch.cuda.CUDAGraph:
+        graph = torch.cuda.CUDAGraph()
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            graph.capture_begin()
+            for _ in range(times):
+                self._launch(shape)
+            graph.capture_end()
+        torch.cuda.current_stream().wait_stream(side)
+        return graph
 
     def run(self, shape: StepShape) -> None:
+        """One step from the uploaded arena."""
         self.arena.upload()
         if self.graph is None:
             # once eagerly, so that every workspace buffer exists before capture
             self._launch(shape)
             torch.cuda.synchronize()
             self.workspace.frozen = True
-            graph = torch.cuda.CUDAGraph()
-            side = torch.cuda.Stream()
-            side.wait_stream(torch.cuda.current_stream())
-            with torch.cuda.stream(side):
-                graph.capture_begin()
-                self._launch(shape)
-                graph.capture_end()
-            torch.cuda.current_stream().wait_stream(side)
-            self.graph = graph
-            # the eager launch above already did this step's work (and wrote its keys and values);
-            # replaying it writes the same values again
+            self.graph = self._capture(shape, 1)
+            # the eager launch above did this step's work and moved the device arrays on to the
+            # next step: upload this step's again
+            self.arena.upload()
+        self.shape = shape
         self.graph.replay()
+
+    def run_burst(self, k: int) -> None:
+        """k steps from the uploaded arena, each feeding the next on the device; their tokens are in
+        history[:k] afterwards."""
+        self.arena.upload()
+        if k == self.burst:
+            if self.burst_graph is None:
+                self.burst_graph = self._capture(self.shape, k)
+            self.burst_graph.replay()
+        else:
+            for _ in range(k):
+                self.graph.replay()
 
 
 class LLMEngine:
@@ -132,34 +156,23 @@ class LLMEngine:
 
     # ------------------------------------------------------------------ stepping
     def _try_burst(self) -> Optional[List[RequestOutput]]:
-        """Several decode steps enqueued at once: each is one upload, one on-device copy of the last
-        step's tokens into this step's inputs, one graph replay and one download, with no wait in
-        between; the host looks at the tokens only when all are done."""
+        """Several decode steps enqueued at once: one upload, the captured steps (each prepares the
+        next one's inputs on the device), one download of all their tokens."""
         ecfg = self.engine_config
         if ecfg.decode_burst < 2 or not ecfg.use_graph or not self._graphs:
             return None
-        running = len(self.scheduler.running)
-        graphed = self._graphs.get(_bucket(max(running, 1)))
+        r = len(self.scheduler.running)
+        graphed = self._graphs.get(_bucket(max(r, 1)))
         if graphed is None or graphed.graph is None:
             return None
         k = self.scheduler.plan_burst(ecfg.decode_burst)
         if k < 2:
             return None
-        r = running
-        arena = graphed.arena
-        while len(graphed.staging) < k:
-            graphed.staging.append(StepArena(arena.n_cap, arena.r_cap, arena.m_cap, arena.n_groups,
-                                             arena.max_blocks, self.device))
-        for j in range(k):
-            stage = graphed.staging[j]
-            self.scheduler.fill(stage, j)
-            arena.dev_t.copy_(stage.host_t, non_blocking=True)
-            if j:
-                arena.d["token_ids"][:r].copy_(arena.tokens_out[:r], non_blocking=True)
-            graphed.graph.replay()
-            stage.tokens_host.copy_(arena.tokens_out, non_blocking=True)
+        self.scheduler.fill(graphed.arena)
+        graphed.run_burst(k)
+        graphed.history_host[:k].copy_(graphed.history[:k], non_blocking=True)
         torch.cuda.current_stream().synchronize()
-        tokens = np.stack([graphed.staging[j].tokens_host.numpy()[:r] for j in range(k)])
+        tokens = np.ascontiguousarray(graphed.history_host.numpy()[:k, :r])
         self.num_graph_steps += k
         return [RequestOutput(self._ids[sid], [token], finished, reason)
                 for sid, token, finished, reason in self.scheduler.commit_burst(tokens, k)]
@@ -177,7 +190,8 @@ class LLMEngine:
             cap = _bucket(r)
             graphed = self._graphs.get(cap)
             if graphed is None:
-                graphed = self._graphs[cap] = _GraphedDecode(self.runner, self.sampler, cap)
+                graphed = self._graphs[cap] = _GraphedDecode(self.runner, self.sampler, cap,
+                                                             self.engine_config.decode_burst)
             arena = graphed.arena
         else:
             arena = self.runner.arena(n, r, m)

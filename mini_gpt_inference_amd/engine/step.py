@@ -49,6 +49,7 @@ class StepArena:
             ("block_tables", n_groups * r_cap * max_blocks, np.int32),
             ("temperature", m_cap, np.float32), ("top_k", m_cap, np.int32), ("top_p", m_cap, np.float32),
             ("out_index", m_cap, np.int32),
+            ("history_pos", m_cap, np.int32),   # stays zero on the host: every upload restarts the device's count
         ]
         total = sum(_round_up(n, 4) for _, n, _ in fields)
         self.host_t = torch.zeros(total, dtype=torch.int32, pin_memory=device.type == "cuda")
@@ -107,6 +108,7 @@ class ModelRunner:
         self.workspace = Workspace(device)
         self._arenas: Dict[Tuple[int, int, int], StepArena] = {}
         self.n_groups = len(cache.groups)
+        self.page_sizes = torch.tensor([g.page_size for g in cache.groups], dtype=torch.int32, device=device)
         # enough block-table columns for the longest sequence this model can hold
         if max_positions is not None:
             self.max_blocks = max(1, max(-(-max_positions // g.page_size) for g in cache.groups))

@@ -183,8 +183,13 @@ def paged_attention_generic(q: torch.Tensor, out: torch.Tensor, k_pool: torch.Te
 
 def sample(logits: torch.Tensor, n_rows: int, real_vocab: int, temperature: torch.Tensor,
            top_k: Optional[torch.Tensor], top_p: Optional[torch.Tensor], request_seed: Optional[torch.Tensor],
-           out_index: Optional[torch.Tensor], engine_seed: int, out_tokens: torch.Tensor) -> None:
-    """One token per row of float32 logits: argmax where temperature <= 0, else seeded sampling."""
+           out_index: Optional[torch.Tensor], engine_seed: int, out_tokens: torch.Tensor, advance=None) -> None:
+    """One token per row of float32 logits: argmax where temperature <= 0, else seeded sampling.
+
+    advance = (token_ids, positions, seq_lens, q_req, slot_mapping [groups, n_stride], block_tables
+    [groups, r_stride, max_blocks], page_sizes [groups], history [rows, stride], history_pos): after
+    a decode-only step each row also prepares the next step on the device (token, position, length,
+    output index, cache slot) and appends its token to the history."""
     _need_cuda(logits, temperature, top_k, top_p, request_seed, out_index, out_tokens)
     _need(logits.dtype == torch.float32 and logits.dim() == 2 and logits.stride(1) == 1 and logits.shape[0] >= n_rows,
           "logits must be float32 [>=n_rows, vocab] with unit inner stride")
@@ -198,6 +203,31 @@ def sample(logits: torch.Tensor, n_rows: int, real_vocab: int, temperature: torc
     _need(out_index is None or (out_index.dtype == torch.int32 and out_index.numel() >= n_rows),
           "out_index must be int32 [rows]")
     _need_i32("out_tokens", out_tokens, n_rows)
+    if advance is not None:
+        token_ids, positions, seq_lens, q_req, slot_mapping, block_tables, page_sizes, history, history_pos = advance
+        _need_cuda(*advance)
+        _need(out_index is not None, "advancing needs the output index array")
+        _need(slot_mapping.dtype == torch.int32 and slot_mapping.dim() == 2 and slot_mapping.is_contiguous(),
+              "slot_mapping must be dense int32 [groups, tokens]")
+        n_groups, n_stride = slot_mapping.shape
+        _need(block_tables.dtype == torch.int32 and block_tables.dim() == 3 and block_tables.is_contiguous()
+              and block_tables.shape[0] == n_groups, "block_tables must be dense int32 [groups, requests, blocks]")
+        _, r_stride, max_blocks = block_tables.shape
+        _need(n_rows <= n_stride and n_rows <= r_stride, "more rows than the step's arrays hold")
+        _need_i32("page_sizes", page_sizes, n_groups)
+        _need(history.dtype == torch.int32 and history.dim() == 2 and history.is_contiguous()
+              and history.shape[1] >= n_rows, "history must be dense int32 [steps, >=rows]")
+        for name, t in (("token_ids", token_ids), ("positions", positions), ("seq_lens", seq_lens),
+                        ("q_req", q_req), ("history_pos", history_pos)):
+            _need_i32(name, t, n_rows)
+        rc = library.kernels().mgpt_sample_advance(
+            _ptr(logits), logits.stride(0), n_rows, vocab, real_vocab, _ptr(temperature), _ptr(top_k), _ptr(top_p),
+            _ptr(request_seed), _ptr(out_index), ctypes.c_ulonglong(engine_seed & (2**64 - 1)), _ptr(out_tokens),
+            _ptr(token_ids), _ptr(positions), _ptr(seq_lens), _ptr(q_req), _ptr(slot_mapping), _ptr(block_tables),
+            _ptr(page_sizes), n_groups, n_stride, r_stride, max_blocks, _ptr(history), _ptr(history_pos),
+            history.shape[0], history.stride(0), _stream())
+        _check(rc, "sample_advance")
+        return
     rc = library.kernels().mgpt_sample(_ptr(logits), logits.stride(0), n_rows, vocab, real_vocab,
                                        _ptr(temperature), _ptr(top_k), _ptr(top_p), _ptr(request_seed),
                                        _ptr(out_index), ctypes.c_ulonglong(engine_seed & (2**64 - 1)),

@@ -16,10 +16,19 @@ class Sampler:
             raise ValueError("real_vocab_size must lie in 1..vocab_size")
         self.engine_seed = int(engine_seed)
 
-    def sample(self, logits: torch.Tensor, arena, n_rows: int) -> torch.Tensor:
+    def sample(self, logits: torch.Tensor, arena, n_rows: int, advance=None) -> torch.Tensor:
         """Writes one token per logits row into arena.tokens_out, using the arena's per-row sampling
-        arrays.  Returns arena.tokens_out."""
+        arrays.  Returns arena.tokens_out.  advance = (page_sizes, history): after a decode-only
+        step, also turn the arena's device arrays into those of the next step and append the
+        tokens to history [steps, rows] (see kernels.sample)."""
         d = arena.d
+        adv = None
+        if advance is not None:
+            page_sizes, history = advance
+            adv = (d["token_ids"], d["positions"], d["seq_lens"], d["q_req"],
+                   d["slot_mapping"].view(arena.n_groups, arena.n_cap),
+                   d["block_tables"].view(arena.n_groups, arena.r_cap, arena.max_blocks), page_sizes, history,
+                   d["history_pos"])
         kernels.sample(logits, n_rows, self.real_vocab, d["temperature"], d["top_k"], d["top_p"], d["seeds"],
-                       d["out_index"], self.engine_seed, arena.tokens_out)
+                       d["out_index"], self.engine_seed, arena.tokens_out, advance=adv)
         return arena.tokens_out

@@ -92,7 +92,7 @@ def test_linear_generic_refuses_bad_inner_size():
 # general=False lets the kernel for a decode step's rows (at most 16, inner size a multiple of 32)
 # take what it can; general=True keeps every case on the kernel for up to 64 rows
 @pytest.mark.parametrize("general", [False, True])
-@pytest.mark.parametrize("n,k,o", [(1, 64, 257), (8, 512, 1536), (17, 96, 503), (33, 80, 48), (64, 2048, 512),
+@pytest.mark.parametrize("n,k,o", [(1, 64, 257), (8, 512, 1536), (17, 96, 503), (33, 80, 48), (64, 2048, 512), (40, 512, 1536), (24, 768, 48), (60, 96, 64),
                                    (5, 48, 16), (16, 160, 503), (12, 1600, 48), (7, 2048, 512), (3, 32, 20),
                                    (9, 768, 130)])
 @pytest.mark.parametrize("epi,o_dt", [(kernels.EPI_NONE, "bfloat16"), (kernels.EPI_NONE, "float32"),
@@ -130,7 +130,7 @@ def test_linear_mfma(n, k, o, epi, o_dt):
 
 @pytest.mark.parametrize("general", [False, True])
 @pytest.mark.parametrize("n,k,o,ln_bias,gather", [(8, 512, 1536, True, False), (3, 96, 503, False, True),
-                                                  (40, 80, 257, True, True), (64, 2048, 64, False, False),
+                                                  (40, 80, 257, True, True), (64, 2048, 64, False, False), (64, 512, 2048, True, False), (33, 768, 96, True, True),
                                                   (17, 1600, 48, True, False), (16, 1600, 130, True, True),
                                                   (1, 160, 48, False, False), (5, 768, 2050, True, True)])
 def test_linear_skinny_through_a_folded_layer_norm(n, k, o, ln_bias, gather, general):
@@ -358,6 +358,54 @@ def test_greedy_is_argmax_with_the_lowest_index_on_ties_and_respects_the_vocabul
     got = _sample(logits, [0.0] * 6, real_vocab=50257)
     want = [P.plain_sample(row.numpy(), 0.0, None, None, 0.0, 50257)[0] for row in logits]
     assert got == want and got[1] == 777 and got[2] < 50257
+
+
+def test_sampling_prepares_the_next_decode_step_on_the_device():
+    """Greedy and seeded rows; two cache groups with pages of 4 and 8 slots; a padded row is left alone;
+    a position past the block table's end gets slot -1."""
+    g = torch.Generator().manual_seed(21)
+    rows, vocab, n_stride, r_stride, max_blocks = 5, 300, 8, 6, 4
+    page_sizes = [4, 8]
+    positions = [3, 7, 0, 15, 9]
+    q_req = [0, 1, -1, 3, 4]
+    bt = torch.randint(0, 50, (2, r_stride, max_blocks), generator=g, dtype=torch.int32)
+    bt[0, 1, 2] = -1                     # request 1 has no page yet for position 8 in group 0
+    tok0 = torch.randint(0, vocab, (n_stride,), generator=g, dtype=torch.int32)
+    d = dict(token_ids=tok0.clone().to(DEV), positions=i32(positions + [0] * 3),
+             seq_lens=i32([p + 1 for p in positions] + [0]), q_req=i32(q_req + [-1] * 3),
+             slot_mapping=torch.full((2, n_stride), -7, dtype=torch.int32, device=DEV), block_tables=bt.to(DEV),
+             page_sizes=i32(page_sizes), history=torch.full((3, 6), -5, dtype=torch.int32, device=DEV),
+             history_pos=torch.zeros(6, dtype=torch.int32, device=DEV))
+    out_index = i32([0, 4, 2, 9, 1])
+    temps = torch.tensor([0.0, 0.9, 0.0, 1.3, 0.0], device=DEV)
+    seeds = torch.tensor([5, 6, 7, 8, 9], dtype=torch.int64, device=DEV)
+    out = torch.full((rows,), -1, dtype=torch.int32, device=DEV)
+    advance = tuple(d[k] for k in ("token_ids", "positions", "seq_lens", "q_req", "slot_mapping", "block_tables",
+                                   "page_sizes", "history", "history_pos"))
+    want_tokens = []
+    for step in range(2):
+        logits = rnd(g, rows, vocab, scale=2.0)
+        idx_before = out_index.cpu().tolist()
+        kernels.sample(logits.to(DEV), rows, vocab, temps, None, None, seeds, out_index, 3, out, advance=advance)
+        plain = torch.full((rows,), -1, dtype=torch.int32, device=DEV)
+        kernels.sample(logits.to(DEV), rows, vocab, temps, None, None, seeds, i32(idx_before), 3, plain)
+        assert torch.equal(out, plain), "advancing must not change what is sampled"
+        want_tokens.append(plain.cpu().tolist())
+        for r in range(rows):
+            if q_req[r] < 0:
+                assert d["token_ids"][r].item() == tok0[r].item() and d["positions"][r].item() == positions[r]
+                assert d["history_pos"][r].item() == 0 and out_index[r].item() == 2
+                assert d["slot_mapping"][:, r].cpu().tolist() == [-7, -7]
+                continue
+            pos = positions[r] + step + 1
+            assert d["token_ids"][r].item() == want_tokens[step][r]
+            assert d["positions"][r].item() == pos and d["seq_lens"][r].item() == pos + 1
+            assert out_index[r].item() == idx_before[r] + 1
+            assert d["history_pos"][r].item() == step + 1 and d["history"][step, r].item() == want_tokens[step][r]
+            for grp, ps in enumerate(page_sizes):
+                page = bt[grp, r, pos // ps].item() if pos // ps < max_blocks else -1
+                assert d["slot_mapping"][grp, r].item() == (page * ps + pos % ps if page >= 0 else -1)
+    assert (d["history"][2] == -5).all() and (d["history"][:, 5] == -5).all()
 
 
 @pytest.mark.parametrize("vocab", [257, 503, 5000])
