@@ -242,6 +242,19 @@ class LLMEngine:
         return [got[name] for name in names]
 
     # ------------------------------------------------------------------ counters
+    def fragmentation_stats(self, group: int = 0) -> Dict[str, int]:
+        """Free and allocated pages of a cache group and the slots that allocated pages hold beyond the
+        tokens computed into them (src/minigpt_infer/cache/paged.py:83-94)."""
+        geometry = self.cache.groups[group]
+        free = self.cache.num_free_pages(group)
+        allocated = geometry.num_pages - free
+        computed = 0
+        for sid in self.scheduler.running:
+            n = self.scheduler.info(sid).num_computed
+            computed += min(n, geometry.window) if geometry.window else n
+        return {"free_blocks": free, "allocated_blocks": allocated,
+                "internal_fragmentation_slots": max(0, allocated * geometry.page_size - computed)}
+
     def stats(self) -> Dict[str, int]:
         s = self.scheduler
         return {

@@ -136,6 +136,25 @@ def test_pages_run_out_preempted_request_is_recomputed_and_ends_with_the_same_to
             _assert_greedy_within_tolerance(model_folders["A"], prompt, tokens, dtype)
 
 
+def test_fragmentation_stats_follow_the_requests(model_folders):
+    # src/minigpt_infer/cache/paged.py:83-94: free, allocated, and slots allocated beyond the computed tokens
+    engine = LLMEngine.from_folder(model_folders["A"], EngineConfig(block_size=4, num_blocks=32, max_batch_size=4,
+                                                                    decode_burst=1, dtype="float32"))
+    assert engine.fragmentation_stats() == {"free_blocks": 32, "allocated_blocks": 0,
+                                            "internal_fragmentation_slots": 0}
+    engine.add_request(Request("a", [1, 2, 3, 4, 5], SamplingParams(max_tokens=6, temperature=0.0)))
+    engine.add_request(Request("b", [7], SamplingParams(max_tokens=3, temperature=0.0)))
+    engine.step()      # both prompts: 5 and 1 tokens computed, pages for 5 and 1 tokens
+    assert engine.fragmentation_stats() == {"free_blocks": 29, "allocated_blocks": 3,
+                                            "internal_fragmentation_slots": 3 * 4 - 6}
+    engine.step()      # one decoded token each: 6 and 2 computed
+    assert engine.fragmentation_stats()["internal_fragmentation_slots"] == 3 * 4 - 8
+    while engine.has_unfinished_requests():
+        engine.step()
+    assert engine.fragmentation_stats() == {"free_blocks": 32, "allocated_blocks": 0,
+                                            "internal_fragmentation_slots": 0}
+
+
 def test_step_outputs_finish_reasons_eot_and_cancel(model_folders):
     engine = LLMEngine.from_folder(model_folders["A"], EngineConfig(block_size=4, num_blocks=32, max_batch_size=4,
                                                                     dtype="float32"))
