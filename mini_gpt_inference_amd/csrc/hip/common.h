@@ -48,22 +48,45 @@ template <typename T> __device__ __forceinline__ T from_float(float v);
 template <> __device__ __forceinline__ float from_float<float>(float v) { return v; }
 template <> __device__ __forceinline__ bf16_t from_float<bf16_t>(float v) { return float_to_bf16(v); }
 
+// Reductions over the 64 lanes of a wave, for waves whose lanes are all active.  Within each row
+// of 16 lanes by DPP moves (neighbours, pairs, halves of 8, halves of 16), then the four rows'
+// results through scalar registers: no trip through LDS, and the result is the same in all lanes.
+template <int CTRL>
+__device__ __forceinline__ int dpp_move(int v) {
+  return __builtin_amdgcn_update_dpp(0, v, CTRL, 0xf, 0xf, false);
+}
+#define MGPT_DPP_XOR1 0xB1          // quad_perm [1,0,3,2]
+#define MGPT_DPP_XOR2 0x4E          // quad_perm [2,3,0,1]
+#define MGPT_DPP_HALF_MIRROR 0x141  // lane i of each 8 reads lane 7 - i
+#define MGPT_DPP_MIRROR 0x140       // lane i of each 16 reads lane 15 - i
+
 __device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-  for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, MGPT_WAVE);
-  return v;
+  v += __int_as_float(dpp_move<MGPT_DPP_XOR1>(__float_as_int(v)));
+  v += __int_as_float(dpp_move<MGPT_DPP_XOR2>(__float_as_int(v)));
+  v += __int_as_float(dpp_move<MGPT_DPP_HALF_MIRROR>(__float_as_int(v)));
+  v += __int_as_float(dpp_move<MGPT_DPP_MIRROR>(__float_as_int(v)));
+  const int b = __float_as_int(v);
+  return (__int_as_float(__builtin_amdgcn_readlane(b, 0)) + __int_as_float(__builtin_amdgcn_readlane(b, 16))) +
+         (__int_as_float(__builtin_amdgcn_readlane(b, 32)) + __int_as_float(__builtin_amdgcn_readlane(b, 48)));
 }
 
 __device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-  for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, MGPT_WAVE));
-  return v;
+  v = fmaxf(v, __int_as_float(dpp_move<MGPT_DPP_XOR1>(__float_as_int(v))));
+  v = fmaxf(v, __int_as_float(dpp_move<MGPT_DPP_XOR2>(__float_as_int(v))));
+  v = fmaxf(v, __int_as_float(dpp_move<MGPT_DPP_HALF_MIRROR>(__float_as_int(v))));
+  v = fmaxf(v, __int_as_float(dpp_move<MGPT_DPP_MIRROR>(__float_as_int(v))));
+  const int b = __float_as_int(v);
+  return fmaxf(fmaxf(__int_as_float(__builtin_amdgcn_readlane(b, 0)), __int_as_float(__builtin_amdgcn_readlane(b, 16))),
+               fmaxf(__int_as_float(__builtin_amdgcn_readlane(b, 32)), __int_as_float(__builtin_amdgcn_readlane(b, 48))));
 }
 
 __device__ __forceinline__ int wave_sum_int(int v) {
-#pragma unroll
-  for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, MGPT_WAVE);
-  return v;
+  v += dpp_move<MGPT_DPP_XOR1>(v);
+  v += dpp_move<MGPT_DPP_XOR2>(v);
+  v += dpp_move<MGPT_DPP_HALF_MIRROR>(v);
+  v += dpp_move<MGPT_DPP_MIRROR>(v);
+  return (__builtin_amdgcn_readlane(v, 0) + __builtin_amdgcn_readlane(v, 16)) +
+         (__builtin_amdgcn_readlane(v, 32) + __builtin_amdgcn_readlane(v, 48));
 }
 
 // GELU with the tanh approximation, as F.gelu(approximate="tanh"):

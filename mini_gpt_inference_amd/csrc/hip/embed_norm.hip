@@ -59,13 +59,20 @@ __global__ void layernorm_kernel(const float* __restrict__ x, const float* __res
   const float* xr = x + src * (long)width;
   OT* orow = out + (long)row * width;
   if (width <= MGPT_WAVE * LN_CACHE) {
-    float xv[LN_CACHE];
+    // the row, the gain and the bias are all asked for before anything is waited for
+    float xv[LN_CACHE], gv[LN_CACHE], bv[LN_CACHE];
     float s = 0.f;
 #pragma unroll
     for (int i = 0; i < LN_CACHE; ++i) {
       const int c = lane + i * MGPT_WAVE;
-      const float v = xr[c < width ? c : 0];
-      xv[i] = c < width ? v : 0.f;
+      const int cc = c < width ? c : 0;
+      xv[i] = xr[cc];
+      gv[i] = w[cc];
+      bv[i] = b ? b[cc] : 0.f;
+    }
+#pragma unroll
+    for (int i = 0; i < LN_CACHE; ++i) {
+      if (lane + i * MGPT_WAVE >= width) xv[i] = 0.f;
       s += xv[i];
     }
     const float mean = wave_sum(s) / (float)width;
@@ -77,22 +84,13 @@ __global__ void layernorm_kernel(const float* __restrict__ x, const float* __res
       e += d;
       v2 = fmaf(d, d, v2);
     }
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) {
-      e += __shfl_xor(e, off, MGPT_WAVE);
-      v2 += __shfl_xor(v2, off, MGPT_WAVE);
-    }
-    const float corr = e / (float)width;
-    const float var = fmaxf(v2 / (float)width - corr * corr, 0.f);
+    const float corr = wave_sum(e) / (float)width;
+    const float var = fmaxf(wave_sum(v2) / (float)width - corr * corr, 0.f);
     const float rstd = 1.0f / sqrtf(var + eps);
 #pragma unroll
     for (int i = 0; i < LN_CACHE; ++i) {
       const int c = lane + i * MGPT_WAVE;
-      if (c < width) {
-        float y = (xv[i] - corr) * rstd * w[c];
-        if (b) y += b[c];
-        orow[c] = from_float<OT>(y);
-      }
+      if (c < width) orow[c] = from_float<OT>((xv[i] - corr) * rstd * gv[i] + bv[i]);
     }
     return;
   }

@@ -1,7 +1,4 @@
-// Next-token choice from 32-bit logits: one workgroup per row; a greedy row may be split over
-// several workgroups (its argmax is a pass over 200 KB, more than one compute unit reads fast):
-// each writes its part's best to a scratch array, and the one that arrives last, by a counter,
-// takes the best of the parts.
+// Next-token choice from 32-bit logits: one workgroup per row.
 //
 // Order of operations as the reference (src/minigpt_infer/sampling.py:97-137,
 // src/minigpt_infer/engine/engine.py:154-159): ids at or above real_vocab are
@@ -19,8 +16,7 @@
 
 #define SAMPLE_THREADS 1024
 #define SAMPLE_WAVES (SAMPLE_THREADS / MGPT_WAVE)
-#define SAMPLE_MAX_SPLIT 16                          // most workgroups that share a greedy row
-#define SAMPLE_SCRATCH_PER_ROW (1 + 2 * SAMPLE_MAX_SPLIT)  // ints of scratch per row: counter, values, indices
+static_assert(SAMPLE_WAVES <= 16, "the greedy path reduces the waves' results within one row of 16 lanes");
 
 __device__ __forceinline__ unsigned int float_key(float f) {
   unsigned int u = __float_as_uint(f);
@@ -73,6 +69,26 @@ __device__ float block_max(float v, float* red) {
   return t;
 }
 
+// DPP move within rows of 16 lanes
+template <int CTRL>
+__device__ __forceinline__ int dpp_i(int v) { return __builtin_amdgcn_update_dpp(0, v, CTRL, 0xf, 0xf, false); }
+
+// (value, index) of the largest value, the lowest index among equals, over each row of 16 lanes;
+// every lane of the row gets it.  Four DPP exchanges: neighbours, pairs, halves of 8, halves of 16.
+__device__ __forceinline__ void argmax_rows16(float& best, int& best_i) {
+#define ARGMAX_STEP(CTRL)                                                         \
+  {                                                                               \
+    const float ov = __int_as_float(dpp_i<CTRL>(__float_as_int(best)));           \
+    const int oi = dpp_i<CTRL>(best_i);                                           \
+    if (ov > best || (ov == best && oi < best_i)) { best = ov; best_i = oi; }     \
+  }
+  ARGMAX_STEP(0xB1)   // quad_perm [1,0,3,2]
+  ARGMAX_STEP(0x4E)   // quad_perm [2,3,0,1]
+  ARGMAX_STEP(0x141)  // row_half_mirror
+  ARGMAX_STEP(0x140)  // row_mirror
+#undef ARGMAX_STEP
+}
+
 // Calls f(index, value) for every logit below nv, each thread taking indices 1024 apart.  When the
 // row is 16-byte aligned the loads are four floats wide and eight of them are issued before any
 // is used, so one pass over the vocabulary costs a few memory latencies, not one per element.
@@ -82,7 +98,7 @@ __device__ __forceinline__ void scan_row(const float* __restrict__ lg, int nv, F
   if ((reinterpret_cast<uintptr_t>(lg) & 15) == 0) {
     const int n4 = nv >> 2;
     const float4* lg4 = reinterpret_cast<const float4*>(lg);
-    constexpr int U = 8;
+    constexpr int U = 16;
     for (int base = tid; base < n4; base += SAMPLE_THREADS * U) {
       float4 v[U];
 #pragma unroll
@@ -152,8 +168,7 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
     const float* __restrict__ logits, long ld, int vocab, int real_vocab,
     const float* __restrict__ temperature, const int* __restrict__ top_k,
     const float* __restrict__ top_p, const uint64_t* __restrict__ request_seed,
-    const int* out_index, uint64_t engine_seed, int* out_tokens, int* scratch, int scratch_rows,
-    AdvanceArgs adv) {
+    const int* out_index, uint64_t engine_seed, int* out_tokens, AdvanceArgs adv) {
   __shared__ float red_f[SAMPLE_WAVES];
   __shared__ int red_i[SAMPLE_WAVES];
   __shared__ float part[SAMPLE_THREADS];
@@ -165,57 +180,64 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
   const int nv = real_vocab < vocab ? real_vocab : vocab;
   const float temp = temperature[row];
 
-  const int split = blockIdx.y, n_split = gridDim.y;
   if (temp <= 0.f) {
-    // this workgroup's share of the row: a multiple of 4 logits, so that aligned rows stay aligned
-    const int share = (((nv + n_split - 1) / n_split) + 3) & ~3;
-    const int lo = split * share < nv ? split * share : nv;
-    const int len = lo + share < nv ? share : nv - lo;
+    // argmax, the lowest index among equals.  A thread meets its indices in rising order, so a
+    // strictly larger value is all it has to look for; four logits are compared as their maximum.
     float best = -INFINITY;
     int best_i = 0x7fffffff;
-    scan_row(lg + lo, len, [&](int i, float v) {
-      if (v > best || (v == best && lo + i < best_i)) { best = v; best_i = lo + i; }
-    });
+    if ((reinterpret_cast<uintptr_t>(lg) & 15) == 0) {
+      const int n4 = nv >> 2;
+      const float4* lg4 = reinterpret_cast<const float4*>(lg);
+      constexpr int U = 16;  // loads in flight per thread: one pass covers 64 Ki logits
+      for (int base = tid; base < n4; base += SAMPLE_THREADS * U) {
+        float4 v[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+          const int i4 = base + u * SAMPLE_THREADS;
+          v[u] = lg4[i4 < n4 ? i4 : base];
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+          const int i4 = base + u * SAMPLE_THREADS;
+          const float m = fmaxf(fmaxf(v[u].x, v[u].y), fmaxf(v[u].z, v[u].w));
+          if (i4 < n4 && m > best) {
+            best = m;
+            best_i = 4 * i4 + (v[u].x == m ? 0 : (v[u].y == m ? 1 : (v[u].z == m ? 2 : 3)));
+          }
+        }
+      }
+      const int i = 4 * n4 + tid;  // the row's last one to three logits
+      if (i < nv && lg[i] > best) { best = lg[i]; best_i = i; }
+    } else {
+      for (int i = tid; i < nv; i += SAMPLE_THREADS)
+        if (lg[i] > best) { best = lg[i]; best_i = i; }
+    }
     // NaN-free rows always have a candidate; a row of -inf falls back to index 0
-    for (int off = 32; off > 0; off >>= 1) {
-      float ov = __shfl_xor(best, off, MGPT_WAVE);
-      int oi = __shfl_xor(best_i, off, MGPT_WAVE);
-      if (ov > best || (ov == best && oi < best_i)) { best = ov; best_i = oi; }
+    argmax_rows16(best, best_i);
+    // lanes 0, 16, 32, 48 hold their rows' best: the wave's best through scalar registers
+    {
+      float wb = best;
+      int wi = best_i;
+#pragma unroll
+      for (int r = 1; r < 4; ++r) {
+        const float ov = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(best), 16 * r));
+        const int oi = __builtin_amdgcn_readlane(best_i, 16 * r);
+        if (ov > wb || (ov == wb && oi < wi)) { wb = ov; wi = oi; }
+      }
+      best = wb;  // right in lane 0 (and in every lane of the first row)
+      best_i = wi;
     }
     if ((tid & 63) == 0) { red_f[tid >> 6] = best; red_i[tid >> 6] = best_i; }
     __syncthreads();
-    if (tid == 0) {
-      for (int i = 1; i < SAMPLE_WAVES; ++i)
-        if (red_f[i] > best || (red_f[i] == best && red_i[i] < best_i)) { best = red_f[i]; best_i = red_i[i]; }
-      if (n_split == 1) {
-        finish_row(row, best_i == 0x7fffffff ? 0 : best_i, out_tokens, adv);
-      } else {
-        // scratch, for scratch_rows rows whatever this launch's number: [rows] counters (zero between
-        // launches), [rows][16] values, [rows][16] indices
-        int* counter = scratch + row;
-        float* part_v = reinterpret_cast<float*>(scratch) + scratch_rows + (long)row * SAMPLE_MAX_SPLIT;
-        int* part_i = scratch + scratch_rows * (1L + SAMPLE_MAX_SPLIT) + (long)row * SAMPLE_MAX_SPLIT;
-        __hip_atomic_store(part_v + split, best, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        __hip_atomic_store(part_i + split, best_i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        // release what was written, count this part in; whoever counts the last part has, after the
-        // acquire, every part's values before it
-        const int arrived = __hip_atomic_fetch_add(counter, 1, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
-        if (arrived == n_split - 1) {
-          best = -INFINITY;
-          best_i = 0x7fffffff;
-          for (int p = 0; p < n_split; ++p) {
-            const float pv = __hip_atomic_load(part_v + p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            const int pi = __hip_atomic_load(part_i + p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            if (pv > best || (pv == best && pi < best_i)) { best = pv; best_i = pi; }
-          }
-          __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // for the next launch
-          finish_row(row, best_i == 0x7fffffff ? 0 : best_i, out_tokens, adv);
-        }
-      }
+    if (tid < MGPT_WAVE) {
+      // the sixteen waves' results, one per lane of the first row, reduced the same way
+      best = tid < SAMPLE_WAVES ? red_f[tid] : -INFINITY;
+      best_i = tid < SAMPLE_WAVES ? red_i[tid] : 0x7fffffff;
+      argmax_rows16(best, best_i);
     }
+    if (tid == 0) finish_row(row, best_i == 0x7fffffff ? 0 : best_i, out_tokens, adv);
     return;
   }
-  if (split != 0) return;  // a sampled row is one workgroup's work
 
   const float t_safe = fmaxf(temp, 1e-6f);
   // largest scaled logit
@@ -323,37 +345,27 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
 }
 
 // logits: [n_rows, vocab] floats with row stride ld.  top_k (0 = off), top_p (1 = off),
-// request_seed and out_index may be null.  scratch: scratch_ints ints of device memory (33 a row
-// for as many rows as will ever be sampled at once), all zero before the first launch and used
-// by no other launch at the same time (the kernel leaves its counters zero again); null, or
-// fewer rows than n_rows: every row is one workgroup's work.
+// request_seed and out_index may be null.
 static int launch_sample(const float* logits, long ld, int n_rows, int vocab, int real_vocab,
                          const float* temperature, const int* top_k, const float* top_p,
                          const uint64_t* request_seed, const int* out_index, uint64_t engine_seed,
-                         int* out_tokens, int* scratch, int scratch_ints, const AdvanceArgs& adv,
-                         hipStream_t stream) {
+                         int* out_tokens, const AdvanceArgs& adv, hipStream_t stream) {
   if (n_rows == 0) return MGPT_OK;
   if (!logits || !temperature || !out_tokens) return MGPT_ERR_NULL;
   if (n_rows < 0 || vocab <= 0 || real_vocab <= 0 || ld < vocab) return MGPT_ERR_BAD_SHAPE;
-  // greedy rows over several workgroups: one per 4096 logits, at most 16, if the scratch array holds them
-  const int nv = real_vocab < vocab ? real_vocab : vocab;
-  int n_split = nv / 4096;
-  n_split = n_split < 1 ? 1 : (n_split > SAMPLE_MAX_SPLIT ? SAMPLE_MAX_SPLIT : n_split);
-  const int scratch_rows = scratch ? scratch_ints / SAMPLE_SCRATCH_PER_ROW : 0;
-  if (n_rows > scratch_rows) n_split = 1;
-  hipLaunchKernelGGL(sample_kernel, dim3(n_rows, n_split), dim3(SAMPLE_THREADS), 0, stream, logits, ld, vocab,
+  hipLaunchKernelGGL(sample_kernel, dim3(n_rows), dim3(SAMPLE_THREADS), 0, stream, logits, ld, vocab,
                      real_vocab, temperature, top_k, top_p, request_seed, out_index, engine_seed,
-                     out_tokens, scratch, scratch_rows, adv);
+                     out_tokens, adv);
   return mgpt_last_error();
 }
 
 extern "C" int mgpt_sample(const float* logits, long ld, int n_rows, int vocab, int real_vocab,
                            const float* temperature, const int* top_k, const float* top_p,
                            const uint64_t* request_seed, const int* out_index, uint64_t engine_seed,
-                           int* out_tokens, int* scratch, int scratch_ints, hipStream_t stream) {
+                           int* out_tokens, hipStream_t stream) {
   AdvanceArgs adv = {};
   return launch_sample(logits, ld, n_rows, vocab, real_vocab, temperature, top_k, top_p, request_seed,
-                       out_index, engine_seed, out_tokens, scratch, scratch_ints, adv, stream);
+                       out_index, engine_seed, out_tokens, adv, stream);
 }
 
 // mgpt_sample, then each row prepares the next decode step on the device (AdvanceArgs above).
@@ -365,7 +377,7 @@ extern "C" int mgpt_sample_advance(const float* logits, long ld, int n_rows, int
                                    const int* q_req, int* slot_mapping, const int* block_tables,
                                    const int* page_sizes, int n_groups, int n_stride, int r_stride,
                                    int max_blocks, int* history, int* history_pos, int history_rows,
-                                   int history_stride, int* scratch, int scratch_ints, hipStream_t stream) {
+                                   int history_stride, hipStream_t stream) {
   if (!token_ids || !positions || !seq_lens || !out_index || !q_req || !slot_mapping || !block_tables ||
       !page_sizes || !history || !history_pos)
     return MGPT_ERR_NULL;
@@ -375,5 +387,5 @@ extern "C" int mgpt_sample_advance(const float* logits, long ld, int n_rows, int
   AdvanceArgs adv = {token_ids, positions, seq_lens, out_index, q_req, slot_mapping, block_tables, page_sizes,
                      n_groups, n_stride, r_stride, max_blocks, history, history_pos, history_rows, history_stride};
   return launch_sample(logits, ld, n_rows, vocab, real_vocab, temperature, top_k, top_p, request_seed,
-                       out_index, engine_seed, out_tokens, scratch, scratch_ints, adv, stream);
+                       out_index, engine_seed, out_tokens, adv, stream);
 }

@@ -183,18 +183,13 @@ def paged_attention_generic(q: torch.Tensor, out: torch.Tensor, k_pool: torch.Te
 
 def sample(logits: torch.Tensor, n_rows: int, real_vocab: int, temperature: torch.Tensor,
            top_k: Optional[torch.Tensor], top_p: Optional[torch.Tensor], request_seed: Optional[torch.Tensor],
-           out_index: Optional[torch.Tensor], engine_seed: int, out_tokens: torch.Tensor, advance=None,
-           scratch: Optional[torch.Tensor] = None) -> None:
+           out_index: Optional[torch.Tensor], engine_seed: int, out_tokens: torch.Tensor, advance=None) -> None:
     """One token per row of float32 logits: argmax where temperature <= 0, else seeded sampling.
 
     advance = (token_ids, positions, seq_lens, q_req, slot_mapping [groups, n_stride], block_tables
     [groups, r_stride, max_blocks], page_sizes [groups], history [rows, stride], history_pos): after
     a decode-only step each row also prepares the next step on the device (token, position, length,
-    output index, cache slot) and appends its token to the history.
-
-    scratch: int32 device memory of SAMPLE_SCRATCH_PER_ROW ints for every row that may be sampled at
-    once, zero before its first use and shared with no launch that may run at the same time; with it
-    a greedy row over a large vocabulary is scanned by several workgroups."""
+    output index, cache slot) and appends its token to the history."""
     _need_cuda(logits, temperature, top_k, top_p, request_seed, out_index, out_tokens)
     _need(logits.dtype == torch.float32 and logits.dim() == 2 and logits.stride(1) == 1 and logits.shape[0] >= n_rows,
           "logits must be float32 [>=n_rows, vocab] with unit inner stride")
@@ -208,11 +203,6 @@ def sample(logits: torch.Tensor, n_rows: int, real_vocab: int, temperature: torc
     _need(out_index is None or (out_index.dtype == torch.int32 and out_index.numel() >= n_rows),
           "out_index must be int32 [rows]")
     _need_i32("out_tokens", out_tokens, n_rows)
-    scratch_ints = 0
-    if scratch is not None:
-        _need_cuda(scratch)
-        _need(scratch.dtype == torch.int32 and scratch.is_contiguous(), "scratch must be contiguous int32")
-        scratch_ints = scratch.numel()
     if advance is not None:
         token_ids, positions, seq_lens, q_req, slot_mapping, block_tables, page_sizes, history, history_pos = advance
         _need_cuda(*advance)
@@ -235,17 +225,16 @@ def sample(logits: torch.Tensor, n_rows: int, real_vocab: int, temperature: torc
             _ptr(request_seed), _ptr(out_index), ctypes.c_ulonglong(engine_seed & (2**64 - 1)), _ptr(out_tokens),
             _ptr(token_ids), _ptr(positions), _ptr(seq_lens), _ptr(q_req), _ptr(slot_mapping), _ptr(block_tables),
             _ptr(page_sizes), n_groups, n_stride, r_stride, max_blocks, _ptr(history), _ptr(history_pos),
-            history.shape[0], history.stride(0), _ptr(scratch), scratch_ints, _stream())
+            history.shape[0], history.stride(0), _stream())
         _check(rc, "sample_advance")
         return
     rc = library.kernels().mgpt_sample(_ptr(logits), logits.stride(0), n_rows, vocab, real_vocab,
                                        _ptr(temperature), _ptr(top_k), _ptr(top_p), _ptr(request_seed),
                                        _ptr(out_index), ctypes.c_ulonglong(engine_seed & (2**64 - 1)),
-                                       _ptr(out_tokens), _ptr(scratch), scratch_ints, _stream())
+                                       _ptr(out_tokens), _stream())
     _check(rc, "sample")
 
 
-SAMPLE_SCRATCH_PER_ROW = 33   # ints of scratch per row for the split argmax (counter, 16 values, 16 indices)
 SK_EPI_QKV = 3
 _SKINNY_MAX_ROWS = 64
 

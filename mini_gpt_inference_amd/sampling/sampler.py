@@ -15,8 +15,6 @@ class Sampler:
         if not (0 < self.real_vocab <= vocab_size):
             raise ValueError("real_vocab_size must lie in 1..vocab_size")
         self.engine_seed = int(engine_seed)
-        self._retired = []
-        self._scratch = None   # device memory for the greedy rows' split argmax; grows with the rows seen
 
     def sample(self, logits: torch.Tensor, arena, n_rows: int, advance=None) -> torch.Tensor:
         """Writes one token per logits row into arena.tokens_out, using the arena's per-row sampling
@@ -24,12 +22,6 @@ class Sampler:
         step, also turn the arena's device arrays into those of the next step and append the
         tokens to history [steps, rows] (see kernels.sample)."""
         d = arena.d
-        if self._scratch is None or self._scratch.numel() < n_rows * kernels.SAMPLE_SCRATCH_PER_ROW:
-            if torch.cuda.is_current_stream_capturing():
-                raise RuntimeError("the sampler's scratch memory must exist before a graph is captured")
-            rows = max(n_rows, 64)
-            self._retired.append(self._scratch)   # captured graphs may still point at it
-            self._scratch = torch.zeros(rows * kernels.SAMPLE_SCRATCH_PER_ROW, dtype=torch.int32, device=logits.device)
         adv = None
         if advance is not None:
             page_sizes, history = advance
@@ -38,5 +30,5 @@ class Sampler:
                    d["block_tables"].view(arena.n_groups, arena.r_cap, arena.max_blocks), page_sizes, history,
                    d["history_pos"])
         kernels.sample(logits, n_rows, self.real_vocab, d["temperature"], d["top_k"], d["top_p"], d["seeds"],
-                       d["out_index"], self.engine_seed, arena.tokens_out, advance=adv, scratch=self._scratch)
+                       d["out_index"], self.engine_seed, arena.tokens_out, advance=adv)
         return arena.tokens_out

@@ -339,15 +339,14 @@ def test_kv_write_and_padding(dtype):
 
 
 # ----------------------------------------------------------------------------- sampling
-def _sample(logits, temperature, top_k=None, top_p=None, seeds=None, idx=None, engine_seed=0, real_vocab=None,
-            scratch=None):
+def _sample(logits, temperature, top_k=None, top_p=None, seeds=None, idx=None, engine_seed=0, real_vocab=None):
     m, v = logits.shape
     out = torch.full((m,), -1, dtype=torch.int32, device=DEV)
     kernels.sample(logits.to(DEV), m, real_vocab or v, torch.tensor(temperature, dtype=torch.float32, device=DEV),
                    None if top_k is None else i32(top_k),
                    None if top_p is None else torch.tensor(top_p, dtype=torch.float32, device=DEV),
                    None if seeds is None else torch.tensor(seeds, dtype=torch.int64, device=DEV),
-                   None if idx is None else i32(idx), engine_seed, out, scratch=scratch)
+                   None if idx is None else i32(idx), engine_seed, out)
     return out.cpu().tolist()
 
 
@@ -361,26 +360,19 @@ def test_greedy_is_argmax_with_the_lowest_index_on_ties_and_respects_the_vocabul
     assert got == want and got[1] == 777 and got[2] < 50257
 
 
-def test_greedy_rows_split_over_workgroups_agree_with_one_workgroup():
-    """With scratch memory a greedy row over a large vocabulary is scanned in parts; ties between parts
-    go to the lowest index; the counters are left zero, so the next launch (other rows, other number
-    of rows) works too; sampled rows are untouched by the split."""
+def test_greedy_ties_at_every_distance_and_rows_that_are_not_aligned():
+    """Equal maxima in one vector of four, in one thread's vectors, in different waves; the last id that
+    may be chosen; a vocabulary that leaves rows unaligned and a tail of one to three logits."""
     g = torch.Generator().manual_seed(12)
-    scratch = torch.zeros(7 * kernels.SAMPLE_SCRATCH_PER_ROW, dtype=torch.int32, device=DEV)
-    for rows, vocab, real in ((6, 50304, 50257), (3, 50257, 50257), (7, 9000, 9000), (2, 300, 300)):
+    for rows, vocab, real in ((6, 50304, 50257), (3, 50257, 50257), (7, 9003, 9001), (3, 300, 300)):
         logits = rnd(g, rows, vocab)
-        logits[0, vocab - 5] = logits[0, 11] = 60.0             # equal maxima in the first and the last part
-        logits[1, real - 1] = 70.0                              # the last id that may be chosen
-        temps = [0.0] * rows
-        temps[-1] = 0.7
-        seeds, idx = list(range(rows)), [5] * rows
-        want = _sample(logits, temps, None, None, seeds, idx, 9, real)
-        assert _sample(logits, temps, None, None, seeds, idx, 9, real, scratch=scratch) == want
-        assert want[0] == 11 and want[1] == real - 1
-        assert (scratch[:7] == 0).all(), "a counter was left standing"
-    # more rows than the scratch memory was made for: every row by one workgroup, same result
-    logits = rnd(g, 9, 50304)
-    assert _sample(logits, [0.0] * 9, scratch=scratch) == _sample(logits, [0.0] * 9)
+        logits[0, real - 5] = logits[0, 11] = 60.0
+        logits[1, real - 1] = 70.0
+        far = 4096 + 5 if real > 4101 else 200
+        logits[-1, 5] = logits[-1, 6] = logits[-1, far] = 65.0
+        got = _sample(logits, [0.0] * rows, real_vocab=real)
+        want = [P.plain_sample(row.numpy(), 0.0, None, None, 0.0, real)[0] for row in logits]
+        assert got == want and got[0] == 11 and got[1] == real - 1 and got[-1] == 5
 
 
 def test_sampling_prepares_the_next_decode_step_on_the_device():
