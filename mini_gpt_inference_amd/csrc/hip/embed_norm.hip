@@ -113,6 +113,72 @@ __global__ void layernorm_kernel(const float* __restrict__ x, const float* __res
   }
 }
 
+// The same for widths that are multiples of 4 up to 64 * 4 * LN_VEC with 16-byte aligned rows: every
+// lane loads and stores vectors of four (a row of 512 is two loads per lane instead of eight).
+#define LN_VEC 4
+
+template <typename OT>
+__global__ void layernorm_vec_kernel(const float* __restrict__ x, const float* __restrict__ w,
+                                     const float* __restrict__ b, OT* __restrict__ out,
+                                     const int* __restrict__ rows, int n_rows, int width, float eps) {
+  const int lane = threadIdx.x & (MGPT_WAVE - 1);
+  const int row = blockIdx.x * (blockDim.x / MGPT_WAVE) + (threadIdx.x / MGPT_WAVE);
+  if (row >= n_rows) return;
+  const long src = rows ? rows[row] : row;
+  const float4* xr = reinterpret_cast<const float4*>(x + src * (long)width);
+  const float4* w4 = reinterpret_cast<const float4*>(w);
+  const float4* b4 = reinterpret_cast<const float4*>(b);
+  const int n4 = width >> 2;
+  float4 xv[LN_VEC], gv[LN_VEC], bv[LN_VEC];
+#pragma unroll
+  for (int i = 0; i < LN_VEC; ++i) {
+    const int c = lane + i * MGPT_WAVE;
+    const int cc = c < n4 ? c : 0;
+    xv[i] = xr[cc];
+    gv[i] = w4[cc];
+    bv[i] = b ? b4[cc] : make_float4(0.f, 0.f, 0.f, 0.f);
+  }
+  float s = 0.f;
+#pragma unroll
+  for (int i = 0; i < LN_VEC; ++i) {
+    if (lane + i * MGPT_WAVE >= n4) xv[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+    s += (xv[i].x + xv[i].y) + (xv[i].z + xv[i].w);
+  }
+  const float mean = wave_sum(s) / (float)width;
+  float e = 0.f, v2 = 0.f;
+#pragma unroll
+  for (int i = 0; i < LN_VEC; ++i) {
+    const bool in = lane + i * MGPT_WAVE < n4;
+    float* p = reinterpret_cast<float*>(&xv[i]);
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const float d = in ? p[k] - mean : 0.f;
+      p[k] = d;
+      e += d;
+      v2 = fmaf(d, d, v2);
+    }
+  }
+  const float corr = wave_sum(e) / (float)width;
+  const float var = fmaxf(wave_sum(v2) / (float)width - corr * corr, 0.f);
+  const float rstd = 1.0f / sqrtf(var + eps);
+  OT* orow = out + (long)row * width;
+#pragma unroll
+  for (int i = 0; i < LN_VEC; ++i) {
+    const int c = lane + i * MGPT_WAVE;
+    if (c >= n4) continue;
+    const float y0 = (xv[i].x - corr) * rstd * gv[i].x + bv[i].x, y1 = (xv[i].y - corr) * rstd * gv[i].y + bv[i].y;
+    const float y2 = (xv[i].z - corr) * rstd * gv[i].z + bv[i].z, y3 = (xv[i].w - corr) * rstd * gv[i].w + bv[i].w;
+    if (sizeof(OT) == 4) {
+      reinterpret_cast<float4*>(orow)[c] = make_float4(y0, y1, y2, y3);
+    } else {
+      uint2 pk;
+      pk.x = pack_bf16x2(y0, y1);
+      pk.y = pack_bf16x2(y2, y3);
+      reinterpret_cast<uint2*>(orow)[c] = pk;
+    }
+  }
+}
+
 // rows: optional gather list (n_rows entries) of source rows of x; out row i <- x row rows[i].
 extern "C" int mgpt_layernorm(const float* x, const float* w, const float* b, void* out,
                               const int* rows, int n_rows, int width, float eps, int out_dtype,
@@ -122,7 +188,15 @@ extern "C" int mgpt_layernorm(const float* x, const float* w, const float* b, vo
   if (n_rows < 0 || width <= 0) return MGPT_ERR_BAD_SHAPE;
   const int rows_per_block = 4;
   dim3 grid((n_rows + rows_per_block - 1) / rows_per_block), block(rows_per_block * MGPT_WAVE);
-  if (out_dtype == MGPT_F32) {
+  const bool vec = (width % 4) == 0 && width <= MGPT_WAVE * 4 * LN_VEC &&
+                   ((((size_t)x) | ((size_t)w) | ((size_t)b) | ((size_t)out)) & 15) == 0;
+  if (vec && out_dtype == MGPT_F32) {
+    hipLaunchKernelGGL(layernorm_vec_kernel<float>, grid, block, 0, stream, x, w, b, (float*)out, rows,
+                       n_rows, width, eps);
+  } else if (vec && out_dtype == MGPT_BF16) {
+    hipLaunchKernelGGL(layernorm_vec_kernel<bf16_t>, grid, block, 0, stream, x, w, b, (bf16_t*)out,
+                       rows, n_rows, width, eps);
+  } else if (out_dtype == MGPT_F32) {
     hipLaunchKernelGGL(layernorm_kernel<float>, grid, block, 0, stream, x, w, b, (float*)out, rows,
                        n_rows, width, eps);
   } else if (out_dtype == MGPT_BF16) {

@@ -8,8 +8,8 @@
 // v_mfma_f32_16x16x32_bf16 accumulators.  Per step of 32 along k the workgroup
 // stages a slice (32 or 64 along k) of the activations and of W
 // in LDS (rows padded by 16 bytes so the 16 rows a MFMA operand reads fall on
-// distinct banks), with the next slice's global loads in flight while the
-// current one is multiplied.  W is the first MFMA operand, so a lane ends up
+// distinct banks), with the global loads of the next two to four slices in
+// flight while the current one is multiplied.  W is the first MFMA operand, so a lane ends up
 // with four neighbouring output columns of one row and stores them as one
 // vector.
 #include "common.h"
@@ -36,16 +36,32 @@ __global__ __launch_bounds__(256) void linear_mfma_kernel(
   __shared__ __align__(16) bf16_t ws[2][TILE * MM_LD];
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int row0 = blockIdx.y * TILE, col0 = blockIdx.x * TILE;
+  // Workgroups go to the eight XCDs in turn by their id, and each XCD has an L2 of its own.  The ids
+  // are therefore dealt out so that an XCD's workgroups are neighbours in tile order: they walk the
+  // column tiles of the same few row tiles, whose activations then come from memory once instead
+  // of once per XCD.
+  int tile_id;
+  {
+    const int total = gridDim.x, pid = blockIdx.x;
+    const int per_xcd = (total + 7) >> 3, tall = (total & 7) ? (total & 7) : 8;
+    const int xcd = pid & 7, local = pid >> 3;
+    tile_id = xcd < tall ? xcd * per_xcd + local : tall * per_xcd + (xcd - tall) * (per_xcd - 1) + local;
+  }
+  const int col_tiles = (n_out + TILE - 1) / TILE;
+  const int row0 = (tile_id / col_tiles) * TILE, col0 = (tile_id % col_tiles) * TILE;
   const int wr = (wave >> 1) * (WT * 16), wc = (wave & 1) * (WT * 16);  // this wave's quarter
   const int lrow = lane & 15, lk = (lane >> 4) * 8;
 
   // staging: thread t copies 16 bytes of rows (t / TPR) + RPP * pass, k offset (t % TPR) * 8
   const int srow = tid / TPR, sk = (tid % TPR) * 8;
   const bf16x8_t zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
-  bf16x8_t ga[PASSES], gw[PASSES];
+  // PD slices along k are on their way from memory at any time, each in registers of its own: with
+  // few workgroups on a compute unit the latency of a load is what a step costs, and it is paid
+  // once per PD - 1 steps
+  constexpr int PD = WT == 2 ? 4 : 2;
+  bf16x8_t ga[PD][PASSES], gw[PD][PASSES];
 
-  auto load_global = [&](int k0) {
+  auto load_global = [&](int set, int k0) {
 #pragma unroll
     for (int p = 0; p < PASSES; ++p) {
       const int r = srow + p * RPP;
@@ -54,16 +70,16 @@ __global__ __launch_bounds__(256) void linear_mfma_kernel(
       const bool a_ok = k_ok && an < n_rows, w_ok = k_ok && wo < n_out;
       const bf16x8_t av = *reinterpret_cast<const bf16x8_t*>(act + (a_ok ? (long)an * lda + k0 + sk : 0));
       const bf16x8_t wv = *reinterpret_cast<const bf16x8_t*>(w + (w_ok ? (long)wo * k_dim + k0 + sk : 0));
-      ga[p] = a_ok ? av : zero8;
-      gw[p] = w_ok ? wv : zero8;
+      ga[set][p] = a_ok ? av : zero8;
+      gw[set][p] = w_ok ? wv : zero8;
     }
   };
-  auto store_lds = [&](int buf) {
+  auto store_lds = [&](int set, int buf) {
 #pragma unroll
     for (int p = 0; p < PASSES; ++p) {
       const int r = srow + p * RPP;
-      *reinterpret_cast<bf16x8_t*>(&as[buf][r * MM_LD + sk]) = ga[p];
-      *reinterpret_cast<bf16x8_t*>(&ws[buf][r * MM_LD + sk]) = gw[p];
+      *reinterpret_cast<bf16x8_t*>(&as[buf][r * MM_LD + sk]) = ga[set][p];
+      *reinterpret_cast<bf16x8_t*>(&ws[buf][r * MM_LD + sk]) = gw[set][p];
     }
   };
 
@@ -74,52 +90,91 @@ __global__ __launch_bounds__(256) void linear_mfma_kernel(
     for (int j = 0; j < WT; ++j) acc[i][j] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
 
   const int k_steps = (k_dim + MM_BK - 1) / MM_BK;
-  load_global(0);
-  store_lds(0);
+#pragma unroll
+  for (int d = 0; d < PD; ++d)
+    if (d < k_steps) load_global(d, d * MM_BK);
+  store_lds(0, 0);
   __syncthreads();
-  for (int s = 0; s < k_steps; ++s) {
-    const int buf = s & 1;
-    if (s + 1 < k_steps) load_global((s + 1) * MM_BK);
+  for (int s0 = 0; s0 < k_steps; s0 += PD) {
 #pragma unroll
-    for (int kk = 0; kk < MM_BK; kk += 32) {
-      bf16x8_t wf[WT], af[WT];
+    for (int d = 0; d < PD; ++d) {
+      const int s = s0 + d;  // this step's slice sat in register set d and is in LDS buffer s & 1 now
+      if (s < k_steps) {
+        const int buf = s & 1;
+        if (s + PD < k_steps) load_global(d, (s + PD) * MM_BK);
 #pragma unroll
-      for (int i = 0; i < WT; ++i) {
-        wf[i] = *reinterpret_cast<const bf16x8_t*>(&ws[buf][(wc + i * 16 + lrow) * MM_LD + kk + lk]);
-        af[i] = *reinterpret_cast<const bf16x8_t*>(&as[buf][(wr + i * 16 + lrow) * MM_LD + kk + lk]);
+        for (int kk = 0; kk < MM_BK; kk += 32) {
+          bf16x8_t wf[WT], af[WT];
+#pragma unroll
+          for (int i = 0; i < WT; ++i) {
+            wf[i] = *reinterpret_cast<const bf16x8_t*>(&ws[buf][(wc + i * 16 + lrow) * MM_LD + kk + lk]);
+            af[i] = *reinterpret_cast<const bf16x8_t*>(&as[buf][(wr + i * 16 + lrow) * MM_LD + kk + lk]);
+          }
+#pragma unroll
+          for (int i = 0; i < WT; ++i)
+#pragma unroll
+            for (int j = 0; j < WT; ++j)
+              acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[i], af[j], acc[i][j], 0, 0, 0);
+        }
+        if (s + 1 < k_steps) {
+          store_lds((d + 1) % PD, buf ^ 1);  // the other buffer: its readers finished before the last barrier
+          __syncthreads();
+        }
       }
-#pragma unroll
-      for (int i = 0; i < WT; ++i)
-#pragma unroll
-        for (int j = 0; j < WT; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[i], af[j], acc[i][j], 0, 0, 0);
-    }
-    if (s + 1 < k_steps) {
-      store_lds(buf ^ 1);  // the other buffer: its readers finished before the last barrier
-      __syncthreads();
     }
   }
 
   // lane holds out[row0 + wr + j*16 + (lane & 15)][col0 + wc + i*16 + (lane >> 4)*4 + e], e = 0..3
+  const bool vec = (n_out & 3) == 0 && (ldo & 3) == 0 &&
+                   (((size_t)out | (size_t)bias) & 15) == 0;  // the four columns as one aligned vector
 #pragma unroll
-  for (int j = 0; j < WT; ++j) {
-    const int n = row0 + wr + j * 16 + lrow;
-    if (n >= n_rows) continue;
-    OT* orow = out + (long)n * ldo;
+  for (int i = 0; i < WT; ++i) {
+    const int oc = col0 + wc + i * 16 + (lane >> 4) * 4;
+    if (oc >= n_out) continue;
+    float b4[4] = {0.f, 0.f, 0.f, 0.f};
+    if (bias) {
+      if (vec) {
+        const float4 t = *reinterpret_cast<const float4*>(bias + oc);
+        b4[0] = t.x; b4[1] = t.y; b4[2] = t.z; b4[3] = t.w;
+      } else {
 #pragma unroll
-    for (int i = 0; i < WT; ++i) {
-      const int oc = col0 + wc + i * 16 + (lane >> 4) * 4;
+        for (int e = 0; e < 4; ++e) b4[e] = oc + e < n_out ? bias[oc + e] : 0.f;
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < WT; ++j) {
+      const int n = row0 + wr + j * 16 + lrow;
+      if (n >= n_rows) continue;
+      OT* orow = out + (long)n * ldo;
+      float v[4];
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
-        const int o = oc + e;
-        if (o >= n_out) continue;
-        float v = acc[i][j][e];
-        if (bias) v += bias[o];
-        if (EPI == MM_EPI_GELU) v = gelu_tanh(v);
+        v[e] = acc[i][j][e] + b4[e];
+        if (EPI == MM_EPI_GELU) v[e] = gelu_tanh(v[e]);
+      }
+      if (vec && sizeof(OT) == 4) {
+        float4* dst = reinterpret_cast<float4*>(orow + oc);
         if (EPI == MM_EPI_RESIDUAL) {
-          orow[o] = from_float<OT>(to_float<OT>(orow[o]) + v);
+          const float4 old = *dst;
+          *dst = make_float4(old.x + v[0], old.y + v[1], old.z + v[2], old.w + v[3]);
         } else {
-          orow[o] = from_float<OT>(v);
+          *dst = make_float4(v[0], v[1], v[2], v[3]);
+        }
+      } else if (vec && EPI != MM_EPI_RESIDUAL) {
+        uint2 pk;
+        pk.x = pack_bf16x2(v[0], v[1]);
+        pk.y = pack_bf16x2(v[2], v[3]);
+        *reinterpret_cast<uint2*>(orow + oc) = pk;
+      } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const int o = oc + e;
+          if (o >= n_out) continue;
+          if (EPI == MM_EPI_RESIDUAL) {
+            orow[o] = from_float<OT>(to_float<OT>(orow[o]) + v[e]);
+          } else {
+            orow[o] = from_float<OT>(v[e]);
+          }
         }
       }
     }
@@ -130,8 +185,9 @@ template <int WT>
 static int launch_tile(const void* act, long lda, const void* w, const float* bias, void* out, int out_dtype,
                        long ldo, int n_rows, int n_out, int k_dim, int epilogue, hipStream_t stream) {
   constexpr int TILE = 2 * WT * 16;
-  dim3 grid((n_out + TILE - 1) / TILE, (n_rows + TILE - 1) / TILE), block(256);
-  if (grid.y > 65535) return MGPT_ERR_TOO_LARGE;
+  const long tiles = (long)((n_out + TILE - 1) / TILE) * ((n_rows + TILE - 1) / TILE);
+  if (tiles > 0x7fffffffL) return MGPT_ERR_TOO_LARGE;
+  dim3 grid((unsigned int)tiles), block(256);
 #define MM_LAUNCH(E, OT)                                                                               \
   hipLaunchKernelGGL((linear_mfma_kernel<WT, E, OT>), grid, block, 0, stream, (const bf16_t*)act, lda, \
                      (const bf16_t*)w, bias, (OT*)out, ldo, n_rows, n_out, k_dim)
