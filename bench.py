@@ -9,6 +9,10 @@ random weights in bfloat16, a batch of 8 requests with 128-token random prompts,
 tokens.  It prints one JSON line; `value` is decoded tokens per second.  Beside it: the
 prefill of 2,048 tokens (2 prompts of 1,024) as one step, the decode step's bytes against the
 HBM peak, and decode throughput at batch 1 and 64.
+
+    python bench.py --workload small-mixed | xl-preempt
+
+runs one of the family's other two named workloads end to end (see WORKLOADS) and prints its own line.
 """
 
 from __future__ import annotations
@@ -113,6 +117,65 @@ def prefill_run(args, dtype, reps=5):
             "frac": round(flops / best / MFMA_PEAK[dtype], 5)}
 
 
+WORKLOADS = {
+    # the reference family's other two named workloads (shapes of GPT-2 small and GPT-2 XL, random weights)
+    "small-mixed": dict(layers=12, width=768, heads=12, vocab=50257, positions=1024, requests=64,
+                        prompt=(16, 1024), output=(16, 256), prefill_chunk=512, pool_frac=1.0),
+    "xl-preempt": dict(layers=48, width=1600, heads=25, vocab=50257, positions=1024, requests=256,
+                       prompt=(512, 512), output=(512, 512), prefill_chunk=0, pool_frac=0.55),
+}
+
+
+def serve_run(args, name):
+    """A whole continuous-batching run: all requests arrive at once, prompts are cut into portions
+    beside the decoding of others, requests end at their own lengths; with pool_frac < 1 the page
+    pool is smaller than the requests' full demand, so the newest are evicted and recomputed."""
+    import numpy as np
+    import torch
+
+    from mini_gpt_inference_amd import EngineConfig, GPTConfig, Request, SamplingParams
+    from mini_gpt_inference_amd.engine.llm_engine import LLMEngine
+
+    w = dict(WORKLOADS[name])
+    if args.workload_layers:
+        w["layers"] = args.workload_layers
+    if args.workload_requests:
+        w["requests"] = args.workload_requests
+    cfg = GPTConfig("gpt2-mini", n_layer=w["layers"], n_embd=w["width"], n_head=w["heads"], vocab_size=w["vocab"],
+                    block_size=w["positions"], bias=True, layer_norm_eps=1e-5)
+    rng = np.random.default_rng(2)
+    requests = []
+    for i in range(w["requests"]):
+        p = int(rng.integers(w["prompt"][0], w["prompt"][1] + 1))
+        o = int(rng.integers(w["output"][0], w["output"][1] + 1))
+        p = min(p, cfg.block_size - o)          # prompt + output within the model's positions
+        requests.append((rng.integers(0, cfg.vocab_size, p).tolist(), o))
+    demand = sum(-(-(len(p) + o) // args.kv_block) for p, o in requests)
+    pages = max(int(demand * w["pool_frac"]), -(-cfg.block_size // args.kv_block) + 1)
+    ecfg = EngineConfig(block_size=args.kv_block, num_blocks=pages, max_batch_size=w["requests"],
+                        max_num_batched_tokens=4096, prefill_chunk=w["prefill_chunk"], dtype=args.dtype,
+                        use_graph=not args.no_graph, decode_burst=args.burst)
+    engine = LLMEngine.from_random(cfg, seed=0, engine_config=ecfg)
+    for i, (p, o) in enumerate(requests):
+        engine.add_request(Request(f"r{i}", p, SamplingParams(max_tokens=o, temperature=0.0)))
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    produced = 0
+    while engine.has_unfinished_requests():
+        produced += len(engine.step())
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    stats = engine.stats()
+    assert produced == sum(o for _, o in requests), "a request ended early or late"
+    assert stats["free_blocks"] == pages, "pages were lost"
+    return {"workload": name, "value": round(produced / elapsed, 1), "unit": "generated tokens/s",
+            "seconds": round(elapsed, 3), "requests": len(requests), "generated_tokens": produced,
+            "prompt_tokens": sum(len(p) for p, _ in requests), "n_layer": cfg.n_layer, "n_embd": cfg.n_embd,
+            "n_head": cfg.n_head, "vocab_size": cfg.vocab_size, "pages": pages, "page_demand": demand,
+            "steps": stats["num_steps"], "preemptions": stats["num_preemptions"],
+            "prompt_tokens_computed": stats["num_prompt_tokens"], "dtype": args.dtype, "weights": "random"}
+
+
 def main() -> int:
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
     ap.add_argument("--gpus", type=int, default=1)
@@ -130,6 +193,12 @@ def main() -> int:
     ap.add_argument("--no-graph", action="store_true")
     ap.add_argument("--burst", type=int, default=8, help="decode steps enqueued back to back (1 = off)")
     ap.add_argument("--no-extras", action="store_true", help="skip prefill and the batch 1 / 64 points")
+    ap.add_argument("--workload", choices=sorted(WORKLOADS), default=None,
+                    help="instead of the decode measurement: a whole continuous-batching run with the shape "
+                         "of GPT-2 small (64 mixed requests, prompt portions of 512) or of GPT-2 XL (256 "
+                         "requests, a page pool too small for them: evictions)")
+    ap.add_argument("--workload-layers", type=int, default=0, help="fewer layers for --workload (0 = the shape's)")
+    ap.add_argument("--workload-requests", type=int, default=0, help="fewer requests for --workload")
     ap.add_argument("--prefill-only", action="store_true",
                     help="run only the 2,048-token prefill and print its record (for profiling)")
     args = ap.parse_args()
@@ -139,6 +208,9 @@ def main() -> int:
 
     if args.prefill_only:
         print(json.dumps({"prefill": prefill_run(args, args.dtype, reps=10)}))
+        return 0
+    if args.workload:
+        print(json.dumps(serve_run(args, args.workload)))
         return 0
 
     elapsed, mean_ctx, engine, cfg = decode_run(args, args.batch, args.steps, args.warmup, args.dtype)
