@@ -115,9 +115,8 @@ __global__ void layernorm_kernel(const float* __restrict__ x, const float* __res
 
 // The same for widths that are multiples of 4 up to 64 * 4 * LN_VEC with 16-byte aligned rows: every
 // lane loads and stores vectors of four (a row of 512 is two loads per lane instead of eight).
-#define LN_VEC 4
-
-template <typename OT>
+// LN_VEC is 4 for rows up to 1024 wide and 8 for rows up to 2048.
+template <typename OT, int LN_VEC>
 __global__ void layernorm_vec_kernel(const float* __restrict__ x, const float* __restrict__ w,
                                      const float* __restrict__ b, OT* __restrict__ out,
                                      const int* __restrict__ rows, int n_rows, int width, float eps) {
@@ -188,14 +187,16 @@ extern "C" int mgpt_layernorm(const float* x, const float* w, const float* b, vo
   if (n_rows < 0 || width <= 0) return MGPT_ERR_BAD_SHAPE;
   const int rows_per_block = 4;
   dim3 grid((n_rows + rows_per_block - 1) / rows_per_block), block(rows_per_block * MGPT_WAVE);
-  const bool vec = (width % 4) == 0 && width <= MGPT_WAVE * 4 * LN_VEC &&
+  const bool vec = (width % 4) == 0 && width <= MGPT_WAVE * 4 * 8 &&
                    ((((size_t)x) | ((size_t)w) | ((size_t)b) | ((size_t)out)) & 15) == 0;
+  const bool narrow = width <= MGPT_WAVE * 4 * 4;
+#define LN_LAUNCH(OT, V) \
+  hipLaunchKernelGGL((layernorm_vec_kernel<OT, V>), grid, block, 0, stream, x, w, b, (OT*)out, rows, n_rows, width, eps)
   if (vec && out_dtype == MGPT_F32) {
-    hipLaunchKernelGGL(layernorm_vec_kernel<float>, grid, block, 0, stream, x, w, b, (float*)out, rows,
-                       n_rows, width, eps);
+    if (narrow) LN_LAUNCH(float, 4); else LN_LAUNCH(float, 8);
   } else if (vec && out_dtype == MGPT_BF16) {
-    hipLaunchKernelGGL(layernorm_vec_kernel<bf16_t>, grid, block, 0, stream, x, w, b, (bf16_t*)out,
-                       rows, n_rows, width, eps);
+    if (narrow) LN_LAUNCH(bf16_t, 4); else LN_LAUNCH(bf16_t, 8);
+#undef LN_LAUNCH
   } else if (out_dtype == MGPT_F32) {
     hipLaunchKernelGGL(layernorm_kernel<float>, grid, block, 0, stream, x, w, b, (float*)out, rows,
                        n_rows, width, eps);
