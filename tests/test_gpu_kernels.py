@@ -93,7 +93,7 @@ def test_linear_generic_refuses_bad_inner_size():
 # general=False lets the kernel for a decode step's rows (at most 16, inner size a multiple of 32)
 # take what it can; general=True keeps every case on the kernel for up to 64 rows
 @pytest.mark.parametrize("general", [False, True])
-@pytest.mark.parametrize("n,k,o", [(1, 64, 257), (8, 512, 1536), (17, 96, 503), (33, 80, 48), (64, 2048, 512), (40, 512, 1536), (24, 768, 48), (60, 96, 64),
+@pytest.mark.parametrize("n,k,o", [(1, 64, 257), (8, 512, 1536), (17, 96, 503), (33, 80, 48), (64, 2048, 512), (40, 512, 1536), (24, 768, 48), (60, 96, 64), (50, 768, 1003),
                                    (5, 48, 16), (16, 160, 503), (12, 1600, 48), (7, 2048, 512), (3, 32, 20),
                                    (9, 768, 130)])
 @pytest.mark.parametrize("epi,o_dt", [(kernels.EPI_NONE, "bfloat16"), (kernels.EPI_NONE, "float32"),
