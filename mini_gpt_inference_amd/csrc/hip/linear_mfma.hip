@@ -61,17 +61,35 @@ __global__ __launch_bounds__(256) void linear_mfma_kernel(
   constexpr int PD = WT == 2 ? 4 : 2;
   bf16x8_t ga[PD][PASSES], gw[PD][PASSES];
 
-  auto load_global = [&](int set, int k0) {
+  // Rows past the end are read from the last row (their results are never stored), so that a
+  // load's value is used only when the slice is multiplied: a select on it right after the load
+  // would wait for it and leave nothing in flight.  Only a last, partial slice along k needs zeros.
+  const bf16_t* ap[PASSES];
+  const bf16_t* wp[PASSES];
 #pragma unroll
-    for (int p = 0; p < PASSES; ++p) {
-      const int r = srow + p * RPP;
+  for (int p = 0; p < PASSES; ++p) {
+    const int r = srow + p * RPP;
+    const int an = row0 + r < n_rows ? row0 + r : n_rows - 1;
+    const int wo = col0 + r < n_out ? col0 + r : n_out - 1;
+    ap[p] = act + (long)an * lda + sk;
+    wp[p] = w + (long)wo * k_dim + sk;
+  }
+  auto load_global = [&](int set, int k0) {
+    if (k0 + MM_BK <= k_dim) {
+#pragma unroll
+      for (int p = 0; p < PASSES; ++p) {
+        ga[set][p] = *reinterpret_cast<const bf16x8_t*>(ap[p] + k0);
+        gw[set][p] = *reinterpret_cast<const bf16x8_t*>(wp[p] + k0);
+      }
+    } else {
       const bool k_ok = k0 + sk + 8 <= k_dim;
-      const int an = row0 + r, wo = col0 + r;
-      const bool a_ok = k_ok && an < n_rows, w_ok = k_ok && wo < n_out;
-      const bf16x8_t av = *reinterpret_cast<const bf16x8_t*>(act + (a_ok ? (long)an * lda + k0 + sk : 0));
-      const bf16x8_t wv = *reinterpret_cast<const bf16x8_t*>(w + (w_ok ? (long)wo * k_dim + k0 + sk : 0));
-      ga[set][p] = a_ok ? av : zero8;
-      gw[set][p] = w_ok ? wv : zero8;
+#pragma unroll
+      for (int p = 0; p < PASSES; ++p) {
+        const bf16x8_t av = *reinterpret_cast<const bf16x8_t*>(ap[p] + (k_ok ? k0 : 0));
+        const bf16x8_t wv = *reinterpret_cast<const bf16x8_t*>(wp[p] + (k_ok ? k0 : 0));
+        ga[set][p] = k_ok ? av : zero8;
+        gw[set][p] = k_ok ? wv : zero8;
+      }
     }
   };
   auto store_lds = [&](int set, int buf) {
