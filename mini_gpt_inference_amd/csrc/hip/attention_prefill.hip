@@ -77,6 +77,8 @@ __global__ __launch_bounds__(256) void prefill_attention_kernel(
   constexpr int NC = (D / 8 + TPR - 1) / TPR;      // chunks per thread
   const int srow = tid / TPR, sc = tid % TPR;
   bf16x8_t kst[NC], vst[NC];
+  bool st_ok[NC];  // whether the fetched chunk is a visible key's; decided at fetch, applied at deposit,
+                   // so that nothing touches a loaded value while the current block is multiplied
 
   auto fetch = [&](int c0) {
     const int j = c0 + srow;
@@ -92,8 +94,9 @@ __global__ __launch_bounds__(256) void prefill_attention_kernel(
       const bool ok = valid && c < D / 8;
       const bf16x8_t kv8 = *reinterpret_cast<const bf16x8_t*>(kpool + base + (ok ? c * 8 : 0));
       const bf16x8_t vv8 = *reinterpret_cast<const bf16x8_t*>(vpool + base + (ok ? c * 8 : 0));
-      kst[u] = ok ? kv8 : zero8;
-      vst[u] = ok ? vv8 : zero8;
+      kst[u] = kv8;
+      vst[u] = vv8;
+      st_ok[u] = ok;
     }
   };
   auto deposit = [&]() {
@@ -101,9 +104,10 @@ __global__ __launch_bounds__(256) void prefill_attention_kernel(
     for (int u = 0; u < NC; ++u) {
       const int c = sc + u * TPR;
       if (c >= D / 8) continue;
-      *reinterpret_cast<bf16x8_t*>(&ks[srow * KLD + c * 8]) = kst[u];
+      const bf16x8_t k8 = st_ok[u] ? kst[u] : zero8, v8 = st_ok[u] ? vst[u] : zero8;
+      *reinterpret_cast<bf16x8_t*>(&ks[srow * KLD + c * 8]) = k8;
 #pragma unroll
-      for (int e = 0; e < 8; ++e) vt[(c * 8 + e) * VLD + srow] = (bf16_t)vst[u][e];
+      for (int e = 0; e < 8; ++e) vt[(c * 8 + e) * VLD + srow] = (bf16_t)v8[e];
     }
   };
 

@@ -97,4 +97,14 @@ __device__ __forceinline__ float gelu_tanh(float u) {
   return 0.5f * u * (1.0f + tanhf(inner));
 }
 
+// The same with tanh(z) = 1 - 2 / (exp(2z) + 1) on the hardware's exp2 and reciprocal (a few ulp
+// of float32): for the kernels whose results are rounded to bfloat16 anyway.
+__device__ __forceinline__ float gelu_tanh_fast(float u) {
+  const float k = 0.7978845608028654f;  // sqrt(2/pi)
+  const float inner = k * (u + 0.044715f * u * u * u);
+  const float e = __builtin_amdgcn_exp2f(inner * 2.8853900817779268f);  // exp(2 inner); inf and 0 at the ends are right
+  const float t = 1.0f - 2.0f * __builtin_amdgcn_rcpf(e + 1.0f);
+  return 0.5f * u * (1.0f + t);
+}
+
 static inline int mgpt_last_error() { return (int)hipGetLastError(); }

@@ -227,7 +227,7 @@ __global__ __launch_bounds__(256) void linear_decode_kernel(SkinnyArgs a) {
       v[i] = acc[t][i];
       if (LN) v[i] = rstd * (v[i] - mean * cs4[i]);
       v[i] += bias4[i];
-      if (EPI == SK_EPI_GELU) v[i] = gelu_tanh(v[i]);
+      if (EPI == SK_EPI_GELU) v[i] = gelu_tanh_fast(v[i]);
       if (EPI == SK_EPI_RESIDUAL) v[i] += old4[t][i];
     }
     if (VEC && sizeof(OT) == 4) {

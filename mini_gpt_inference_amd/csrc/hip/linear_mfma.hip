@@ -168,7 +168,7 @@ __global__ __launch_bounds__(256) void linear_mfma_kernel(
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
         v[e] = acc[i][j][e] + b4[e];
-        if (EPI == MM_EPI_GELU) v[e] = gelu_tanh(v[e]);
+        if (EPI == MM_EPI_GELU) v[e] = gelu_tanh_fast(v[e]);
       }
       if (vec && sizeof(OT) == 4) {
         float4* dst = reinterpret_cast<float4*>(orow + oc);
@@ -232,7 +232,7 @@ extern "C" int mgpt_linear_mfma(const void* act, long lda, const void* w, const 
   // large tiles reuse operands better, small tiles fill the 256 compute units: take the large
   // ones only when they alone give every unit several workgroups
   const long big = (long)((n_out + 127) / 128) * ((n_rows + 127) / 128);
-  if (big >= 1024)
+  if (big >= 384)
     return launch_tile<4>(act, lda, w, bias, out, out_dtype, ldo, n_rows, n_out, k_dim, epilogue, stream);
   return launch_tile<2>(act, lda, w, bias, out, out_dtype, ldo, n_rows, n_out, k_dim, epilogue, stream);
 }

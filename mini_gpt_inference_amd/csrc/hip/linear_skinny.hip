@@ -231,7 +231,7 @@ __global__ __launch_bounds__(WAVES * 64) void linear_skinny_kernel(SkinnyArgs a)
         v[i] = acc[t][i];
         if (LN && oc + i < a.n_out) v[i] = rstd * (v[i] - mean * a.colsum[oc + i]);
         if (a.bias && oc + i < a.n_out) v[i] += a.bias[oc + i];
-        if (EPI == SK_EPI_GELU) v[i] = gelu_tanh(v[i]);
+        if (EPI == SK_EPI_GELU) v[i] = gelu_tanh_fast(v[i]);
       }
       OT* orow = reinterpret_cast<OT*>(a.out) + (long)n * a.ldo;
       const bool whole = oc + 4 <= a.n_out && (a.ldo & 3) == 0;  // four columns, one aligned vector
