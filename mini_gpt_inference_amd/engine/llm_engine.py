@@ -42,6 +42,7 @@ class _GraphedDecode:
         self.history_host = torch.zeros(self.burst, cap, dtype=torch.int32, pin_memory=runner.device.type == "cuda")
         self.graph: Optional[torch.cuda.CUDAGraph] = None
         self.burst_graph: Optional[torch.cuda.CUDAGraph] = None
+        self.shape: Optional[StepShape] = None   # of the last single step; launch geometry for captures
 
     def _launch(self, shape: StepShape) -> None:
         ctx = self.runner.context(self.arena, shape, padded=True, workspace=self.workspace)
@@ -80,6 +81,8 @@ class _GraphedDecode:
     def run_burst(self, k: int) -> None:
         """k steps from the uploaded arena, each feeding the next on the device; their tokens are in
         history[:k] afterwards."""
+        if self.graph is None:
+            raise RuntimeError("a burst needs the single step's graph, which the first decode step captures")
         self.arena.upload()
         if k == self.burst:
             if self.burst_graph is None:
