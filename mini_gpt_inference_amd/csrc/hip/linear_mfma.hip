@@ -21,13 +21,13 @@ typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4_t;
 #define MM_EPI_GELU 1
 #define MM_EPI_RESIDUAL 2
 
-// WT: 16-wide tiles per wave in each direction.  4 -> 128 x 128 per workgroup, 2 -> 64 x 64.
+// WT: 16-wide tiles per wave in each direction.  4 -> 128 x 128 per workgroup, 2 -> 64 x 64, 1 -> 32 x 32.
 template <int WT, int EPI, typename OT>
 __global__ __launch_bounds__(256) void linear_mfma_kernel(
     const bf16_t* __restrict__ act, long lda, const bf16_t* __restrict__ w,
     const float* __restrict__ bias, OT* __restrict__ out, long ldo, int n_rows, int n_out, int k_dim) {
   constexpr int TILE = 2 * WT * 16;   // rows and columns of the workgroup's tile
-  constexpr int MM_BK = WT == 2 ? 64 : 32;   // k per step: what fits LDS twice over
+  constexpr int MM_BK = WT == 4 ? 32 : 64;   // k per step: what fits LDS twice over
   constexpr int MM_LD = MM_BK + 8;           // LDS row stride in elements (16 bytes of padding)
   constexpr int TPR = MM_BK / 8;             // threads per staged row (16 bytes each)
   constexpr int RPP = 256 / TPR;             // rows per staging pass
@@ -58,7 +58,7 @@ __global__ __launch_bounds__(256) void linear_mfma_kernel(
   // PD slices along k are on their way from memory at any time, each in registers of its own: with
   // few workgroups on a compute unit the latency of a load is what a step costs, and it is paid
   // once per PD - 1 steps
-  constexpr int PD = WT == 2 ? 4 : 2;
+  constexpr int PD = WT == 4 ? 2 : 4;
   bf16x8_t ga[PD][PASSES], gw[PD][PASSES];
 
   // Rows past the end are read from the last row (their results are never stored), so that a
@@ -234,5 +234,10 @@ extern "C" int mgpt_linear_mfma(const void* act, long lda, const void* w, const 
   const long big = (long)((n_out + 127) / 128) * ((n_rows + 127) / 128);
   if (big >= 384)
     return launch_tile<4>(act, lda, w, bias, out, out_dtype, ldo, n_rows, n_out, k_dim, epilogue, stream);
+  // and tiles of 32 x 32 where the 64 x 64 ones would leave most of the units idle (a prompt
+  // portion of a few hundred tokens)
+  const long mid = (long)((n_out + 63) / 64) * ((n_rows + 63) / 64);
+  if (mid < 192)
+    return launch_tile<1>(act, lda, w, bias, out, out_dtype, ldo, n_rows, n_out, k_dim, epilogue, stream);
   return launch_tile<2>(act, lda, w, bias, out, out_dtype, ldo, n_rows, n_out, k_dim, epilogue, stream);
 }
