@@ -20,12 +20,22 @@ typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4_t;
 #define MM_EPI_NONE 0
 #define MM_EPI_GELU 1
 #define MM_EPI_RESIDUAL 2
+#define MM_EPI_QKV 3   // store, and scatter the key and value columns into their cache pages
+
+// where the key and value columns of a fused QKV product go (src/minigpt_infer/cache/paged.py:125-137)
+struct MfmaScatter {
+  bf16_t* kpool;
+  bf16_t* vpool;
+  const int* slot_mapping;  // per row: page * page_size + offset, or -1 for a padded row
+  int q_width, kv_width, head_dim, n_kv_head, page_size;
+};
 
 // WT: 16-wide tiles per wave in each direction.  4 -> 128 x 128 per workgroup, 2 -> 64 x 64, 1 -> 32 x 32.
 template <int WT, int EPI, typename OT>
 __global__ __launch_bounds__(256) void linear_mfma_kernel(
     const bf16_t* __restrict__ act, long lda, const bf16_t* __restrict__ w,
-    const float* __restrict__ bias, OT* __restrict__ out, long ldo, int n_rows, int n_out, int k_dim) {
+    const float* __restrict__ bias, OT* __restrict__ out, long ldo, int n_rows, int n_out, int k_dim,
+    MfmaScatter sc) {
   constexpr int TILE = 2 * WT * 16;   // rows and columns of the workgroup's tile
   constexpr int MM_BK = WT == 4 ? 32 : 64;   // k per step: what fits LDS twice over
   constexpr int MM_LD = MM_BK + 8;           // LDS row stride in elements (16 bytes of padding)
@@ -183,6 +193,20 @@ __global__ __launch_bounds__(256) void linear_mfma_kernel(
         pk.x = pack_bf16x2(v[0], v[1]);
         pk.y = pack_bf16x2(v[2], v[3]);
         *reinterpret_cast<uint2*>(orow + oc) = pk;
+        if (EPI == MM_EPI_QKV && oc >= sc.q_width) {
+          // the four columns lie in one head (the launcher checks that sizes are multiples of 4)
+          const int slot = sc.slot_mapping[n];
+          if (slot >= 0) {
+            const long page = slot / sc.page_size;
+            const int off = slot - (int)page * sc.page_size;
+            const int c = oc - sc.q_width;  // column among keys then values
+            const bool is_v = c >= sc.kv_width;
+            const int cc = is_v ? c - sc.kv_width : c;
+            const int h = cc / sc.head_dim, d = cc - h * sc.head_dim;
+            const long dst = ((page * sc.n_kv_head + h) * sc.page_size + off) * (long)sc.head_dim + d;
+            *reinterpret_cast<uint2*>((is_v ? sc.vpool : sc.kpool) + dst) = pk;
+          }
+        }
       } else {
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
@@ -201,18 +225,20 @@ __global__ __launch_bounds__(256) void linear_mfma_kernel(
 
 template <int WT>
 static int launch_tile(const void* act, long lda, const void* w, const float* bias, void* out, int out_dtype,
-                       long ldo, int n_rows, int n_out, int k_dim, int epilogue, hipStream_t stream) {
+                       long ldo, int n_rows, int n_out, int k_dim, int epilogue, const MfmaScatter& sc,
+                       hipStream_t stream) {
   constexpr int TILE = 2 * WT * 16;
   const long tiles = (long)((n_out + TILE - 1) / TILE) * ((n_rows + TILE - 1) / TILE);
   if (tiles > 0x7fffffffL) return MGPT_ERR_TOO_LARGE;
   dim3 grid((unsigned int)tiles), block(256);
 #define MM_LAUNCH(E, OT)                                                                               \
   hipLaunchKernelGGL((linear_mfma_kernel<WT, E, OT>), grid, block, 0, stream, (const bf16_t*)act, lda, \
-                     (const bf16_t*)w, bias, (OT*)out, ldo, n_rows, n_out, k_dim)
+                     (const bf16_t*)w, bias, (OT*)out, ldo, n_rows, n_out, k_dim, sc)
   if (epilogue == MM_EPI_NONE && out_dtype == MGPT_BF16) MM_LAUNCH(MM_EPI_NONE, bf16_t);
   else if (epilogue == MM_EPI_NONE && out_dtype == MGPT_F32) MM_LAUNCH(MM_EPI_NONE, float);
   else if (epilogue == MM_EPI_GELU && out_dtype == MGPT_BF16) MM_LAUNCH(MM_EPI_GELU, bf16_t);
   else if (epilogue == MM_EPI_RESIDUAL && out_dtype == MGPT_F32) MM_LAUNCH(MM_EPI_RESIDUAL, float);
+  else if (epilogue == MM_EPI_QKV && out_dtype == MGPT_BF16) MM_LAUNCH(MM_EPI_QKV, bf16_t);
   else return MGPT_ERR_BAD_DTYPE;
 #undef MM_LAUNCH
   return mgpt_last_error();
@@ -221,9 +247,9 @@ static int launch_tile(const void* act, long lda, const void* w, const float* bi
 // act: [n_rows, k_dim] bfloat16 with row stride lda (a multiple of 8, 16-byte aligned base);
 // w: [n_out, k_dim] dense bfloat16; out: [n_rows, n_out] with row stride ldo.  k_dim must be a
 // multiple of 16.  Refuses other layouts with MGPT_ERR_BAD_SHAPE.
-extern "C" int mgpt_linear_mfma(const void* act, long lda, const void* w, const float* bias, void* out,
-                                int out_dtype, long ldo, int n_rows, int n_out, int k_dim, int epilogue,
-                                hipStream_t stream) {
+static int linear_mfma_any(const void* act, long lda, const void* w, const float* bias, void* out,
+                           int out_dtype, long ldo, int n_rows, int n_out, int k_dim, int epilogue,
+                           const MfmaScatter& sc, hipStream_t stream) {
   if (n_rows == 0 || n_out == 0) return MGPT_OK;
   if (!act || !w || !out) return MGPT_ERR_NULL;
   if (n_rows < 0 || n_out < 0 || k_dim <= 0 || (k_dim % 16) != 0 || lda < k_dim || (lda % 8) != 0 ||
@@ -233,11 +259,36 @@ extern "C" int mgpt_linear_mfma(const void* act, long lda, const void* w, const 
   // ones only when they alone give every unit several workgroups
   const long big = (long)((n_out + 127) / 128) * ((n_rows + 127) / 128);
   if (big >= 384)
-    return launch_tile<4>(act, lda, w, bias, out, out_dtype, ldo, n_rows, n_out, k_dim, epilogue, stream);
+    return launch_tile<4>(act, lda, w, bias, out, out_dtype, ldo, n_rows, n_out, k_dim, epilogue, sc, stream);
   // and tiles of 32 x 32 where the 64 x 64 ones would leave most of the units idle (a prompt
   // portion of a few hundred tokens)
   const long mid = (long)((n_out + 63) / 64) * ((n_rows + 63) / 64);
   if (mid < 192)
-    return launch_tile<1>(act, lda, w, bias, out, out_dtype, ldo, n_rows, n_out, k_dim, epilogue, stream);
-  return launch_tile<2>(act, lda, w, bias, out, out_dtype, ldo, n_rows, n_out, k_dim, epilogue, stream);
+    return launch_tile<1>(act, lda, w, bias, out, out_dtype, ldo, n_rows, n_out, k_dim, epilogue, sc, stream);
+  return launch_tile<2>(act, lda, w, bias, out, out_dtype, ldo, n_rows, n_out, k_dim, epilogue, sc, stream);
+}
+
+extern "C" int mgpt_linear_mfma(const void* act, long lda, const void* w, const float* bias, void* out,
+                                int out_dtype, long ldo, int n_rows, int n_out, int k_dim, int epilogue,
+                                hipStream_t stream) {
+  if (epilogue == MM_EPI_QKV) return MGPT_ERR_BAD_SHAPE;  // mgpt_linear_mfma_qkv brings the pools
+  MfmaScatter sc = {};
+  return linear_mfma_any(act, lda, w, bias, out, out_dtype, ldo, n_rows, n_out, k_dim, epilogue, sc, stream);
+}
+
+// The fused QKV product of a step with prompt portions: out[n] = act[n] W^T + bias in bfloat16, and
+// the key and value columns (after the first q_width) of every row with a slot also go into the
+// cache pools [pages, n_kv_head, page_size, head_dim].  Refuses (MGPT_ERR_BAD_SHAPE) sizes that
+// are no multiples of 4 and outputs that are not aligned for 8-byte stores.
+extern "C" int mgpt_linear_mfma_qkv(const void* act, long lda, const void* w, const float* bias, void* out,
+                                    long ldo, int n_rows, int n_out, int k_dim, void* kpool, void* vpool,
+                                    const int* slot_mapping, int q_width, int kv_width, int head_dim,
+                                    int n_kv_head, int page_size, hipStream_t stream) {
+  if (!kpool || !vpool || !slot_mapping) return MGPT_ERR_NULL;
+  if (head_dim <= 0 || (head_dim % 4) != 0 || (q_width % 4) != 0 || q_width + 2 * kv_width != n_out ||
+      kv_width != n_kv_head * head_dim || page_size <= 0 || (n_out % 4) != 0 || (ldo % 4) != 0 ||
+      (((size_t)out | (size_t)bias) & 15) != 0)
+    return MGPT_ERR_BAD_SHAPE;
+  MfmaScatter sc = {(bf16_t*)kpool, (bf16_t*)vpool, slot_mapping, q_width, kv_width, head_dim, n_kv_head, page_size};
+  return linear_mfma_any(act, lda, w, bias, out, MGPT_BF16, ldo, n_rows, n_out, k_dim, MM_EPI_QKV, sc, stream);
 }

@@ -385,12 +385,16 @@ def paged_attention_decode_bf16(q: torch.Tensor, out: torch.Tensor, k_pool: torc
 
 
 def linear_mfma(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor,
-                n_rows: int, epilogue: int) -> bool:
-    """Tiled bfloat16 MFMA product for many rows.  False when it does not take the shape."""
+                n_rows: int, epilogue: int, scatter=None) -> bool:
+    """Tiled bfloat16 MFMA product for many rows.  scatter = (k_pool, v_pool, slot_mapping, q_width,
+    kv_width) also stores the new keys and values into their pages (bfloat16 output, no other
+    epilogue).  False when it does not take the shape."""
     if a.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
         return False
     n_out, k_dim = w.shape
     if k_dim % 16 != 0 or a.stride(0) % 8 != 0 or a.data_ptr() % 16 != 0 or w.data_ptr() % 16 != 0:
+        return False
+    if scatter is not None and (epilogue != EPI_NONE or out.dtype != torch.bfloat16):
         return False
     if (epilogue, out.dtype) not in ((EPI_NONE, torch.bfloat16), (EPI_NONE, torch.float32),
                                      (EPI_GELU, torch.bfloat16), (EPI_RESIDUAL, torch.float32)):
@@ -402,8 +406,21 @@ def linear_mfma(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], 
     _need(out.dim() == 2 and out.stride(1) == 1 and out.shape[1] >= n_out and out.shape[0] >= n_rows,
           "output must be [>=n_rows, >=out] with unit inner stride")
     _need(bias is None or (bias.dtype == torch.float32 and bias.numel() == n_out), "bias must be float32 [out]")
-    rc = library.kernels().mgpt_linear_mfma(_ptr(a), a.stride(0), _ptr(w), _ptr(bias), _ptr(out), _dtype_code(out),
-                                            out.stride(0), n_rows, n_out, k_dim, epilogue, _stream())
+    if scatter is not None:
+        kp, vp, sm, q_width, kv_width = scatter
+        _need_cuda(kp, vp, sm)
+        _need(kp.shape == vp.shape and kp.dim() == 4 and kp.is_contiguous() and vp.is_contiguous()
+              and kp.dtype == torch.bfloat16 and vp.dtype == torch.bfloat16,
+              "key and value pools must be dense bfloat16 [pages, kv_heads, page_size, head_dim]")
+        _, n_kv_head, page_size, head_dim = kp.shape
+        _need_i32("slot_mapping", sm, n_rows)
+        rc = library.kernels().mgpt_linear_mfma_qkv(
+            _ptr(a), a.stride(0), _ptr(w), _ptr(bias), _ptr(out), out.stride(0), n_rows, n_out, k_dim, _ptr(kp),
+            _ptr(vp), _ptr(sm), q_width, kv_width, head_dim, n_kv_head, page_size, _stream())
+    else:
+        rc = library.kernels().mgpt_linear_mfma(_ptr(a), a.stride(0), _ptr(w), _ptr(bias), _ptr(out),
+                                                _dtype_code(out), out.stride(0), n_rows, n_out, k_dim, epilogue,
+                                                _stream())
     if rc == -2:
         return False
     _check(rc, "linear_mfma")

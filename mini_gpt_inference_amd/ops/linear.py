@@ -70,6 +70,8 @@ def linear(ctx, a: Union[torch.Tensor, LazyNorm], w: torch.Tensor, bias: Optiona
         if kernels.linear_skinny(as_tensor(ctx, a), w, bias, out, n_rows, epi, scatter=scatter):
             return scatter is not None
     a = as_tensor(ctx, a)
+    if fast and scatter is not None and kernels.linear_mfma(a, w, bias, out, n_rows, epilogue, scatter=scatter):
+        return True
     if fast and kernels.linear_mfma(a, w, bias, out, n_rows, epilogue):
         return False
     kernels.linear_generic(a, w, bias, out, n_rows, epilogue)

@@ -181,6 +181,36 @@ def test_linear_skinny_stores_keys_and_values(general):
     assert torch.isnan(untouched).all(), "a slot that no token owns was written"
 
 
+@pytest.mark.parametrize("n", [70, 300, 1100])
+def test_linear_mfma_stores_keys_and_values(n):
+    """The tiled kernel's fused QKV product: all three tile sizes; groups of heads; padded rows (slot -1)
+    leave the pools alone."""
+    g = torch.Generator().manual_seed(15)
+    k, h, hk, d, page = 96, 6, 2, 16, 8
+    pages = n // page + 3
+    qw, kvw = h * d, hk * d
+    a, w, bias = rnd(g, n, k, dtype="bfloat16"), rnd(g, qw + 2 * kvw, k, dtype="bfloat16", scale=0.2), rnd(g, qw + 2 * kvw)
+    kp = torch.full((pages, hk, page, d), float("nan"), dtype=torch.bfloat16, device=DEV)
+    vp = kp.clone()
+    slots = torch.randperm(pages * page, generator=g)[:n].tolist()
+    for t in range(0, n, 7):
+        slots[t] = -1
+    out = torch.empty(n, qw + 2 * kvw, dtype=torch.bfloat16, device=DEV)
+    assert kernels.linear_mfma(a.to(DEV), w.to(DEV), bias.to(DEV), out, n, kernels.EPI_NONE,
+                               scatter=(kp, vp, i32(slots), qw, kvw))
+    want = P.plain_linear(a.double(), w.double(), bias.double())
+    helpers.assert_close(out, want, "bfloat16", "qkv")
+    kflat = kp.float().cpu().permute(0, 2, 1, 3).reshape(pages * page, kvw)
+    vflat = vp.float().cpu().permute(0, 2, 1, 3).reshape(pages * page, kvw)
+    live = torch.tensor([s for s in slots if s >= 0])
+    rows = torch.tensor([t for t, s in enumerate(slots) if s >= 0])
+    helpers.assert_close(kflat[live], want[rows, qw:qw + kvw], "bfloat16", "stored keys")
+    helpers.assert_close(vflat[live], want[rows, qw + kvw:], "bfloat16", "stored values")
+    untouched = torch.ones(pages * page, dtype=torch.bool)
+    untouched[live] = False
+    assert torch.isnan(kflat[untouched]).all() and torch.isnan(vflat[untouched]).all()
+
+
 def test_linear_skinny_refuses_what_it_cannot_do():
     w = torch.zeros(32, 64, dtype=torch.bfloat16, device=DEV)
     a = torch.zeros(65, 64, dtype=torch.bfloat16, device=DEV)
