@@ -240,3 +240,48 @@ def test_decode_bursts_change_nothing_but_the_pace(model_folders, dtype):
     assert steps[1] < steps[0]                      # the bursts were taken
     if dtype == "float32":
         assert outs[0]["r0"] == plain_first[:plain_first.index(eot) + 1]
+
+
+@pytest.mark.parametrize("name,seed", [("A", 0), ("B", 1), ("C", 2)])
+def test_arrivals_evictions_bursts_and_cancels_together_32bit(model_folders, name, seed):
+    """Requests arrive while others decode, the page pool is too small for all of them, prompts are
+    cut into portions, decode steps run in bursts, one request is cancelled on the way: every
+    request that ends has exactly the plain implementation's greedy tokens, and nothing is left
+    allocated."""
+    cfg = helpers.CONFIGS[name]
+    rng = np.random.default_rng(100 + seed)
+    n_req = 9
+    lens = [int(rng.integers(1, cfg.block_size // 2)) for _ in range(n_req)]
+    news = [int(rng.integers(3, min(24, cfg.block_size - n))) for n in lens]
+    prompts = [helpers.random_ids(rng, cfg.vocab_size, n) for n in lens]
+    page = 4
+    worst = max(-(-(n + m) // page) for n, m in zip(lens, news))
+    engine = LLMEngine.from_folder(model_folders[name], EngineConfig(
+        block_size=page, num_blocks=worst + 6, max_batch_size=4, max_num_batched_tokens=24, prefill_chunk=7,
+        dtype="float32", decode_burst=4))
+    got = {i: [] for i in range(n_req)}
+    arrivals = sorted((int(rng.integers(0, 25)), i) for i in range(n_req))
+    cancelled, step = None, 0
+    while arrivals or engine.has_unfinished_requests():
+        while arrivals and arrivals[0][0] <= step:
+            _, i = arrivals.pop(0)
+            engine.add_request(Request(f"r{i}", prompts[i], SamplingParams(max_tokens=news[i], temperature=0.0)))
+        if step == 12 and cancelled is None:
+            live = [i for i in range(n_req) if f"r{i}" in engine._rids and len(got[i]) < news[i]]
+            if live:
+                cancelled = live[-1]
+                engine.cancel_request(f"r{cancelled}")
+        for out in engine.step():
+            got[int(out.request_id[1:])].extend(out.new_token_ids)
+        step += 1
+        assert step < 2000, "the engine makes no progress"
+    want = _plain_greedy(model_folders[name], prompts, max(news))
+    for i in range(n_req):
+        if i == cancelled:
+            assert got[i] == want[i][:len(got[i])]
+        else:
+            assert got[i] == want[i][:news[i]], f"request {i}"
+    stats = engine.stats()
+    assert stats["free_blocks"] == worst + 6 and engine.cache.check() == 0
+    # with these draws every configuration evicts, replays graphs and runs eager (prompt) steps
+    assert stats["num_preemptions"] > 0 and stats["graph_steps"] > 0 and stats["eager_steps"] > 0
