@@ -220,7 +220,7 @@ def main() -> int:
     achieved = decode_bytes(cfg, args.batch, mean_ctx, itemsize) / step_s / 1e9
     stats = engine.stats()
     record = {
-        "metric": "decode tokens/s (50.9M GPT-2-style, batch 8, 128-token prompts)",
+        "metric": f"decode tokens/s (50.9M GPT-2-style, batch {args.batch}, {args.prompt}-token prompts)",
         "value": round(value, 1), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(step_s * 1e3, 4), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": round(value / REFERENCE_DECODE_B8, 2) if args.batch == 8 else None,

@@ -23,18 +23,21 @@
 
 // VEC: n_out is a multiple of 16 and bias, column sums and output rows are aligned for vectors of
 // four; otherwise every access of the epilogue is a single element with its own bound check.
-template <int NT, int SMAX, bool LN, int EPI, typename OT, bool VEC>
+// SPLIT: k is also split over a.k_parts workgroups per column tile; each stores its raw sums to
+// a.partials (no LayerNorm, no epilogue: linear_partials_epilogue_kernel finishes the job).
+template <int NT, int SMAX, bool LN, int EPI, typename OT, bool VEC, bool SPLIT = false>
 __global__ __launch_bounds__(256) void linear_decode_kernel(SkinnyArgs a) {
   __shared__ float red[3 * NT * 6 * 64];  // waves 1..3: per row tile four sums and two statistics per lane
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // the same in all lanes: branches on it are scalar
   const int lrow = lane & 15, g = lane >> 4;
   const int K = a.k_dim;
-  const int steps_total = K >> 5;
+  const int part = SPLIT ? (int)(blockIdx.x % a.k_parts) : 0;
+  const int steps_total = SPLIT ? (K >> 5) / a.k_parts : K >> 5;   // of this workgroup
   const int per = (steps_total + 3) >> 2;
   const int steps = max(0, min(per, steps_total - wave * per));  // the last waves of a short k may have none
-  const int kb = steps > 0 ? wave * per * 32 : 0;
-  const int o0 = blockIdx.x * 16;
+  const int kb = (steps > 0 ? wave * per * 32 : 0) + part * steps_total * 32;
+  const int o0 = (SPLIT ? (int)(blockIdx.x / a.k_parts) : (int)blockIdx.x) * 16;
   const int wo = min(o0 + lrow, a.n_out - 1);  // a column past the end reads the last row; never stored
   const int oc = o0 + g * 4;  // this lane's four output columns, of rows lrow + 16 t
   bool row_ok[NT];
@@ -62,7 +65,7 @@ __global__ __launch_bounds__(256) void linear_decode_kernel(SkinnyArgs a) {
     for (int i = 0; i < 4; ++i) old4[t][i] = 0.f;
   }
   OT* const out = reinterpret_cast<OT*>(a.out);
-  if (col_writer) {
+  if (col_writer && !SPLIT) {
     if (VEC) {
       if (a.bias != nullptr) {
         const float4 b4 = *reinterpret_cast<const float4*>(a.bias + oc);
@@ -210,6 +213,15 @@ __global__ __launch_bounds__(256) void linear_decode_kernel(SkinnyArgs a) {
   }
 
   // ---- epilogue: lane holds out[t * 16 + lrow][oc + i], i = 0..3
+  if (SPLIT) {
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+      if (!row_ok[t]) continue;
+      float* prow = a.partials + ((long)part * a.n_rows + t * 16 + lrow) * a.n_out + oc;
+      *reinterpret_cast<float4*>(prow) = make_float4(acc[t][0], acc[t][1], acc[t][2], acc[t][3]);
+    }
+    return;
+  }
 #pragma unroll
   for (int t = 0; t < NT; ++t) {
     if (!row_ok[t]) continue;

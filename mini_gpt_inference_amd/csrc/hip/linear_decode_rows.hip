@@ -31,8 +31,89 @@ static int launch_tiles_unaligned_head(const SkinnyArgs& a, hipStream_t s) {
   return mgpt_last_error();
 }
 
+// ---- k split over workgroups, for a long k and few column tiles: with 64 rows a workgroup that owns
+// 16 columns pulls all the activations (256 KB for k = 2048) through one compute unit; four
+// workgroups per tile pull a quarter each, write their sums, and a second kernel adds the parts in
+// order and applies bias, GELU or the residual add.
+#define LDR_PARTS 4
+
+long mgpt_linear_decode_partials(int n_rows, int n_out, int k_dim, bool ln, int epilogue) {
+  if (ln || epilogue == SK_EPI_QKV || n_rows <= 16 || n_rows > 64) return 0;
+  if (k_dim < 1024 || (k_dim % (32 * LDR_PARTS)) != 0 || (n_out % 16) != 0 || n_out / 16 >= 128) return 0;
+  return (long)LDR_PARTS * n_rows * n_out;
+}
+
+template <int EPI, typename OT>
+__global__ __launch_bounds__(256) void linear_partials_epilogue_kernel(
+    const float* __restrict__ partials, const float* __restrict__ bias, OT* __restrict__ out, long ldo,
+    int n_rows, int n_out) {
+  const int quads = n_out >> 2;
+  const int idx = blockIdx.x * 256 + threadIdx.x;
+  if (idx >= n_rows * quads) return;
+  const int row = idx / quads, oc = (idx - row * quads) * 4;
+  float4 p[LDR_PARTS];
+#pragma unroll
+  for (int s = 0; s < LDR_PARTS; ++s)
+    p[s] = *reinterpret_cast<const float4*>(partials + ((long)s * n_rows + row) * n_out + oc);
+  float4 b4 = make_float4(0.f, 0.f, 0.f, 0.f);
+  if (bias) b4 = *reinterpret_cast<const float4*>(bias + oc);
+  OT* orow = out + (long)row * ldo + oc;
+  float4 old = make_float4(0.f, 0.f, 0.f, 0.f);
+  if (EPI == SK_EPI_RESIDUAL) old = *reinterpret_cast<const float4*>(orow);
+  float v[4] = {p[0].x, p[0].y, p[0].z, p[0].w};
+#pragma unroll
+  for (int s = 1; s < LDR_PARTS; ++s) {  // in the order of k, whatever order the parts were written in
+    v[0] += p[s].x; v[1] += p[s].y; v[2] += p[s].z; v[3] += p[s].w;
+  }
+  const float b[4] = {b4.x, b4.y, b4.z, b4.w};
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    v[i] += b[i];
+    if (EPI == SK_EPI_GELU) v[i] = gelu_tanh_fast(v[i]);
+  }
+  if (sizeof(OT) == 4) {
+    *reinterpret_cast<float4*>(orow) = make_float4(v[0] + old.x, v[1] + old.y, v[2] + old.z, v[3] + old.w);
+  } else {
+    uint2 pk;
+    pk.x = pack_bf16x2(v[0], v[1]);
+    pk.y = pack_bf16x2(v[2], v[3]);
+    *reinterpret_cast<uint2*>(orow) = pk;
+  }
+}
+
+template <int NT>
+static int launch_split(const SkinnyArgs& a0, int epilogue, int out_dtype, hipStream_t s) {
+  SkinnyArgs a = a0;
+  a.k_parts = LDR_PARTS;
+  const int per = (a.k_dim / 32 / LDR_PARTS + 3) / 4;
+  dim3 grid((a.n_out / 16) * LDR_PARTS);
+  if (per <= 4) hipLaunchKernelGGL((linear_decode_kernel<NT, 4, false, SK_EPI_NONE, float, true, true>), grid, dim3(256), 0, s, a);
+  else hipLaunchKernelGGL((linear_decode_kernel<NT, 8, false, SK_EPI_NONE, float, true, true>), grid, dim3(256), 0, s, a);
+  int rc = mgpt_last_error();
+  if (rc != MGPT_OK) return rc;
+  dim3 egrid((a.n_rows * (a.n_out / 4) + 255) / 256);
+#define LDR_EPI(E, OT) \
+  hipLaunchKernelGGL((linear_partials_epilogue_kernel<E, OT>), egrid, dim3(256), 0, s, a.partials, a.bias, (OT*)a.out, a.ldo, a.n_rows, a.n_out)
+  if (epilogue == SK_EPI_NONE && out_dtype == MGPT_BF16) LDR_EPI(SK_EPI_NONE, bf16_t);
+  else if (epilogue == SK_EPI_NONE && out_dtype == MGPT_F32) LDR_EPI(SK_EPI_NONE, float);
+  else if (epilogue == SK_EPI_GELU && out_dtype == MGPT_BF16) LDR_EPI(SK_EPI_GELU, bf16_t);
+  else if (epilogue == SK_EPI_RESIDUAL && out_dtype == MGPT_F32) LDR_EPI(SK_EPI_RESIDUAL, float);
+  else return MGPT_ERR_BAD_DTYPE;
+#undef LDR_EPI
+  return mgpt_last_error();
+}
+
 int mgpt_launch_linear_decode_rows(const SkinnyArgs& a, int epilogue, int out_dtype, hipStream_t stream) {
   const int nt = (a.n_rows + 15) / 16;
+  if (a.partials != nullptr && decode_vec_ok(a) &&
+      mgpt_linear_decode_partials(a.n_rows, a.n_out, a.k_dim, a.x != nullptr, epilogue) > 0) {
+    switch (nt) {
+      case 2: return launch_split<2>(a, epilogue, out_dtype, stream);
+      case 3: return launch_split<3>(a, epilogue, out_dtype, stream);
+      case 4: return launch_split<4>(a, epilogue, out_dtype, stream);
+      default: return MGPT_ERR_BAD_SHAPE;
+    }
+  }
   if (!decode_vec_ok(a)) {
     // odd widths with many rows: only the head's case here, the general kernel for the rest
     if (epilogue != SK_EPI_NONE || out_dtype != MGPT_F32) return MGPT_ERR_BAD_SHAPE;

@@ -26,6 +26,10 @@ struct SkinnyArgs {
   long ldo;
   int n_rows, n_out, k_dim;
   int ksplit;         // waves of a workgroup that share a column tile: 1, 2 or 4
+  // k split over workgroups (linear_decode_rows.hip): each writes its raw sums to
+  // partials[part][row][column] and a second kernel adds them and applies the epilogue
+  float* partials;
+  int k_parts;
   // key/value scatter (SK_EPI_QKV)
   bf16_t* kpool;
   bf16_t* vpool;
@@ -36,3 +40,5 @@ struct SkinnyArgs {
 // linear_decode.hip: at most 64 rows, k_dim a multiple of 32.  Returns
 // MGPT_ERR_BAD_SHAPE for what it does not take (the general kernel then runs).
 int mgpt_launch_linear_decode(const SkinnyArgs& a, int epilogue, int out_dtype, hipStream_t stream);
+// floats of partial sums the split over workgroups needs for this shape; 0: no split
+long mgpt_linear_decode_partials(int n_rows, int n_out, int k_dim, bool ln, int epilogue);

@@ -298,13 +298,16 @@ static int launch_nt(const SkinnyArgs& a, int epi, int out_dtype, dim3 grid, siz
 // a LayerNorm whose gain and bias were folded into w, bias and colsum (fold_norm.hip); otherwise
 // act holds bfloat16 activations.  Refuses (MGPT_ERR_BAD_SHAPE) more than 64 rows and k_dim that
 // is no multiple of 16; the caller then takes the general kernels.  general_only != 0 keeps to this
-// file's kernel also where linear_decode.hip would take the shape.
+// file's kernel also where linear_decode.hip would take the shape.  partials: optional scratch of
+// mgpt_linear_skinny_partials(...) floats; with it a long inner size with many rows is split over
+// workgroups (two launches).
 extern "C" int mgpt_linear_skinny(const void* act, long lda, const float* x, const int* rows,
                                   const float* colsum, float eps, const void* w,
                                   const float* bias, void* out, int out_dtype, long ldo, int n_rows,
                                   int n_out, int k_dim, int epilogue, void* kpool, void* vpool,
                                   const int* slot_mapping, int q_width, int kv_width, int head_dim,
-                                  int n_kv_head, int page_size, int general_only, hipStream_t stream) {
+                                  int n_kv_head, int page_size, int general_only, float* partials,
+                                  long partials_floats, hipStream_t stream) {
   if (n_rows == 0 || n_out == 0) return MGPT_OK;
   if (!w || !out || (!act && !x)) return MGPT_ERR_NULL;
   if (n_rows < 0 || n_rows > 64 || n_out < 0 || k_dim <= 0 || (k_dim % 16) != 0 || ldo < n_out)
@@ -339,6 +342,10 @@ extern "C" int mgpt_linear_skinny(const void* act, long lda, const float* x, con
   a.k_dim = k_dim; a.ksplit = ks; a.kpool = (bf16_t*)kpool; a.vpool = (bf16_t*)vpool;
   a.slot_mapping = slot_mapping; a.q_width = q_width; a.kv_width = kv_width; a.head_dim = head_dim;
   a.n_kv_head = n_kv_head; a.page_size = page_size;
+  // room for the parts of a split over workgroups, if the caller brought enough of it
+  a.k_parts = 1;
+  a.partials = (partials && partials_floats >= mgpt_linear_decode_partials(n_rows, n_out, k_dim, ln, epilogue))
+                   ? partials : nullptr;
   if (!general_only) {
     // the rows of a decode step: the kernel laid out for latency, where it takes the shape
     const int rc = mgpt_launch_linear_decode(a, epilogue, out_dtype, stream);
@@ -362,4 +369,9 @@ extern "C" int mgpt_linear_skinny(const void* act, long lda, const float* x, con
     default: return SK_NT(4);
   }
 #undef SK_NT
+}
+
+// floats of scratch with which mgpt_linear_skinny splits this shape's inner size over workgroups; 0: it would not
+extern "C" long mgpt_linear_skinny_partials(int n_rows, int n_out, int k_dim, int has_ln, int epilogue) {
+  return mgpt_linear_decode_partials(n_rows, n_out, k_dim, has_ln != 0, epilogue);
 }

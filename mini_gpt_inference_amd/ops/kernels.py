@@ -261,13 +261,16 @@ def fold_layer_norm(w: torch.Tensor, gain: torch.Tensor, beta: Optional[torch.Te
 def linear_skinny(a: Optional[torch.Tensor], w: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor,
                   n_rows: int, epilogue: int = EPI_NONE, *, ln_x: Optional[torch.Tensor] = None,
                   ln_colsum: Optional[torch.Tensor] = None, ln_eps: float = 0.0,
-                  ln_rows: Optional[torch.Tensor] = None, scatter=None, general_only: bool = False) -> bool:
+                  ln_rows: Optional[torch.Tensor] = None, scatter=None, general_only: bool = False,
+                  partials: Optional[torch.Tensor] = None) -> bool:
     """bfloat16 MFMA product for at most 64 rows.  With ln_x (the float32 residual stream; ln_rows an
     optional gather) the rows are read through a LayerNorm that fold_layer_norm folded into w, bias
     and ln_colsum.  scatter = (k_pool, v_pool, slot_mapping, q_width, kv_width) also stores the new
     keys and values into their pages.  Up to 16 rows with an inner size that is a multiple of 32 go
-    to the kernel laid out for a decode step's latency unless general_only is set.  Returns False,
-    having launched nothing, when the kernel does not take the shape."""
+    to the kernel laid out for a decode step's latency unless general_only is set.  partials:
+    float32 scratch of linear_skinny_partials(...) elements, with which a long inner size under many
+    rows is split over workgroups.  Returns False, having launched nothing, when the kernel does not
+    take the shape."""
     if n_rows > _SKINNY_MAX_ROWS or w.dtype != torch.bfloat16:
         return False
     n_out, k_dim = w.shape
@@ -300,6 +303,10 @@ def linear_skinny(a: Optional[torch.Tensor], w: torch.Tensor, bias: Optional[tor
         if a.stride(0) % 8 != 0 or a.data_ptr() % 16 != 0:
             return False
         lda = a.stride(0)
+    if partials is not None:
+        _need_cuda(partials)
+        _need(partials.dtype == torch.float32 and partials.is_contiguous() and partials.data_ptr() % 16 == 0,
+              "partials must be contiguous, 16-byte aligned float32")
     kp = vp = sm = None
     q_width = kv_width = head_dim = n_kv_head = page_size = 0
     if epilogue == SK_EPI_QKV:
@@ -313,11 +320,17 @@ def linear_skinny(a: Optional[torch.Tensor], w: torch.Tensor, bias: Optional[tor
         _ptr(a if ln_x is None else None), lda, _ptr(ln_x), _ptr(ln_rows), _ptr(ln_colsum),
         float(ln_eps), _ptr(w), _ptr(bias), _ptr(out), _dtype_code(out), out.stride(0), n_rows, n_out, k_dim,
         epilogue, _ptr(kp), _ptr(vp), _ptr(sm), q_width, kv_width, head_dim, n_kv_head, page_size,
-        1 if general_only else 0, _stream())
+        1 if general_only else 0, _ptr(partials), 0 if partials is None else partials.numel(), _stream())
     if rc == -2:
         return False
     _check(rc, "linear_skinny")
     return True
+
+
+def linear_skinny_partials(n_rows: int, n_out: int, k_dim: int, has_ln: bool, epilogue: int) -> int:
+    """float32 elements of scratch with which linear_skinny would split this shape's inner size over
+    workgroups; 0 if it would not."""
+    return int(library.kernels().mgpt_linear_skinny_partials(n_rows, n_out, k_dim, 1 if has_ln else 0, epilogue))
 
 
 def paged_attention_split_bf16(q: torch.Tensor, out: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor,

@@ -67,7 +67,11 @@ def linear(ctx, a: Union[torch.Tensor, LazyNorm], w: torch.Tensor, bias: Optiona
             if kernels.linear_skinny(None, wf, bias_f, out, n_rows, epi, ln_x=a.x, ln_colsum=colsum,
                                      ln_eps=a.norm.eps, ln_rows=a.rows, scatter=scatter):
                 return scatter is not None
-        if kernels.linear_skinny(as_tensor(ctx, a), w, bias, out, n_rows, epi, scatter=scatter):
+        partials = None
+        need = kernels.linear_skinny_partials(n_rows, w.shape[0], w.shape[1], False, epi) if n_rows > 16 else 0
+        if need:
+            partials = ctx.workspace.get("linear_partials", need, 1, torch.float32)
+        if kernels.linear_skinny(as_tensor(ctx, a), w, bias, out, n_rows, epi, scatter=scatter, partials=partials):
             return scatter is not None
     a = as_tensor(ctx, a)
     if fast and scatter is not None and kernels.linear_mfma(a, w, bias, out, n_rows, epilogue, scatter=scatter):

@@ -181,6 +181,33 @@ def test_linear_skinny_stores_keys_and_values(general):
     assert torch.isnan(untouched).all(), "a slot that no token owns was written"
 
 
+@pytest.mark.parametrize("n,k,o", [(64, 2048, 512), (40, 1024, 256), (17, 2048, 48), (33, 3072, 768)])
+@pytest.mark.parametrize("epi,o_dt", [(kernels.EPI_NONE, "bfloat16"), (kernels.EPI_NONE, "float32"),
+                                      (kernels.EPI_GELU, "bfloat16"), (kernels.EPI_RESIDUAL, "float32")])
+def test_linear_skinny_with_the_inner_size_split_over_workgroups(n, k, o, epi, o_dt):
+    """With scratch for the parts, a long inner size under more than 16 rows runs as two launches; the
+    result is the unsplit kernel's up to the order of four sums."""
+    g = torch.Generator().manual_seed(16)
+    need = kernels.linear_skinny_partials(n, o, k, False, epi)
+    assert need == 4 * n * o
+    assert kernels.linear_skinny_partials(16, o, k, False, epi) == 0          # few rows: one launch is as fast
+    assert kernels.linear_skinny_partials(n, o, 512, False, epi) == 0         # a short inner size
+    assert kernels.linear_skinny_partials(n, o, k, True, epi) == 0            # not through a folded LayerNorm
+    a, w, bias = rnd(g, n + 2, k, dtype="bfloat16"), rnd(g, o, k, dtype="bfloat16", scale=k ** -0.5), rnd(g, o)
+    prev = rnd(g, n + 2, o, dtype=o_dt)
+    partials = torch.full((need,), float("nan"), device=DEV)
+    for b in (bias, None):
+        out = prev.clone().to(DEV)
+        assert kernels.linear_skinny(a.to(DEV), w.to(DEV), None if b is None else b.to(DEV), out, n, epi,
+                                     partials=partials)
+        helpers.assert_close(out[:n], _linear_want(a, w, b, epi, prev)[:n], "bfloat16", f"split {n}x{k}x{o}")
+        assert torch.equal(out[n:], prev[n:].to(DEV)), "rows beyond n_rows were written"
+    # too little scratch: the unsplit kernel, same result
+    out2 = prev.clone().to(DEV)
+    assert kernels.linear_skinny(a.to(DEV), w.to(DEV), bias.to(DEV), out2, n, epi, partials=partials[:need // 2])
+    helpers.assert_close(out2[:n], _linear_want(a, w, bias, epi, prev)[:n], "bfloat16", "unsplit")
+
+
 @pytest.mark.parametrize("n", [70, 300, 1100])
 def test_linear_mfma_stores_keys_and_values(n):
     """The tiled kernel's fused QKV product: all three tile sizes; groups of heads; padded rows (slot -1)
