@@ -7,6 +7,30 @@ import torch
 from . import kernels
 
 
+def _mixed_step(ctx, q, out, k_pool, v_pool, group, n_head: int, scale: float, window: int) -> bool:
+    """A step with prompt portions.  The requests that lead the step with one token each (a scheduler
+    puts the decoding requests first) go to the decode kernel, token n being request n; the rest,
+    prompt portions mostly, to the MFMA tile kernel, which would spend a 64-query tile on a single
+    token.  False, having launched nothing, if the tile kernel does not take the case."""
+    q_lens = ctx.host_q_lens
+    lead = 0
+    if q_lens is not None:
+        while lead < len(q_lens) and q_lens[lead] == 1:
+            lead += 1
+    rest = ctx.n_req - lead
+    if lead and rest and kernels.prefill_attention_bf16(
+            q, out, k_pool, v_pool, group.block_tables[lead:], ctx.cu_q[lead:], ctx.seq_lens[lead:], rest,
+            ctx.max_q_len, n_head, scale, window):
+        if kernels.paged_attention_decode_bf16(q, out, k_pool, v_pool, group.block_tables, ctx.positions, ctx.q_req,
+                                               lead, n_head, scale, window, identity=True):
+            return True
+        # the decode kernel refuses this head or page size: the tile kernel for the leading requests too
+        return kernels.prefill_attention_bf16(q, out, k_pool, v_pool, group.block_tables, ctx.cu_q, ctx.seq_lens,
+                                              lead, 1, n_head, scale, window)
+    return kernels.prefill_attention_bf16(q, out, k_pool, v_pool, group.block_tables, ctx.cu_q, ctx.seq_lens,
+                                          ctx.n_req, ctx.max_q_len, n_head, scale, window)
+
+
 def paged_attention(ctx, q: torch.Tensor, out: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor,
                     group, n_head: int, scale: float, window: int) -> None:
     """Attention of the step's tokens (rows of q) over their requests' pages.
@@ -21,9 +45,8 @@ def paged_attention(ctx, q: torch.Tensor, out: torch.Tensor, k_pool: torch.Tenso
                 q, out, k_pool, v_pool, group.block_tables, ctx.positions, ctx.q_req, n, n_head, scale, window,
                 identity=True):
             return
-        if not ctx.decode_only and ctx.n_rows == ctx.n_tokens and kernels.prefill_attention_bf16(
-                q, out, k_pool, v_pool, group.block_tables, ctx.cu_q, ctx.seq_lens, ctx.n_req, ctx.max_q_len,
-                n_head, scale, window):
+        if not ctx.decode_only and ctx.n_rows == ctx.n_tokens and _mixed_step(ctx, q, out, k_pool, v_pool, group,
+                                                                               n_head, scale, window):
             return
         if kernels.paged_attention_split_bf16(q, out, k_pool, v_pool, group.block_tables, ctx.cu_q, ctx.seq_lens,
                                               ctx.q_req, n, r, n_head, scale, window):
