@@ -16,6 +16,7 @@ import torch
 from ..cache.kv_store import KVStore
 from ..cache.manager import CacheManager, GroupGeometry
 from ..config.engine_config import EngineConfig, SamplingParams
+from ..ops import kernels
 from ..parts.base import Workspace
 from ..sampling.sampler import Sampler
 from ..weights.loader import load_model
@@ -48,8 +49,9 @@ class _GraphedDecode:
         ctx = self.runner.context(self.arena, shape, padded=True, workspace=self.workspace)
         # launch geometry must not depend on this step's lengths: size it for the longest sequence
         ctx.max_seq_len = self.runner.max_positions or ctx.max_seq_len
-        logits = self.runner.model.forward(ctx)
-        self.sampler.sample(logits, self.arena, self.cap, advance=(self.runner.page_sizes, self.history))
+        with kernels.pinned_stream():
+            logits = self.runner.model.forward(ctx)
+            self.sampler.sample(logits, self.arena, self.cap, advance=(self.runner.page_sizes, self.history))
 
     def _capture(self, shape: StepShape, times: int) -> torch.cuda.CUDAGraph:
         graph = torch.cuda.CUDAGraph()

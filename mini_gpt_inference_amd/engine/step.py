@@ -18,6 +18,7 @@ import torch
 
 from ..cache.kv_store import KVStore
 from ..cache.manager import CacheManager
+from ..ops import kernels
 from ..parts.base import GroupView, StepContext, Workspace
 from ..parts.model import DecoderModel
 
@@ -194,7 +195,8 @@ class ModelRunner:
         """Uploads the arena and runs the model eagerly.  Returns float32 logits [n_logits, vocab]."""
         arena.upload()
         ctx = self.context(arena, shape, padded=False)
-        return self.model.forward(ctx)
+        with kernels.pinned_stream():
+            return self.model.forward(ctx)
 
     def step(self, slots: Sequence[int], ctx_lens: Sequence[int], q_lens: Sequence[int], tokens: Sequence[int],
              logit_rows: Sequence[int]) -> torch.Tensor:

@@ -8,6 +8,7 @@ operator computes anything here.
 
 from __future__ import annotations
 
+import contextlib
 import ctypes
 from typing import Optional
 
@@ -42,8 +43,27 @@ def _ptr(t: Optional[torch.Tensor]) -> ctypes.c_void_p:
     return ctypes.c_void_p(0 if t is None else t.data_ptr())
 
 
+_pinned_stream: Optional[ctypes.c_void_p] = None
+
+
 def _stream() -> ctypes.c_void_p:
+    if _pinned_stream is not None:
+        return _pinned_stream
     return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+@contextlib.contextmanager
+def pinned_stream():
+    """Inside the block every launch goes to the stream that is current on entry.  Asking torch for
+    the current stream costs about as much as a launch does, and a step is some hundred launches;
+    the block must not switch streams."""
+    global _pinned_stream
+    previous = _pinned_stream
+    _pinned_stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    try:
+        yield
+    finally:
+        _pinned_stream = previous
 
 
 def _check(rc: int, what: str) -> None:
