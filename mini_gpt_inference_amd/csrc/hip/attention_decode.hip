@@ -1,5 +1,8 @@
 // Paged attention for bfloat16 caches with the keys of one (token, head) split over the four
-// waves of a workgroup: the decode kernel.  Same rule as the general kernel (a query at
+// waves of a workgroup, for any number of tokens per request: what steps use that neither
+// attention_decode_wide.hip (one token per request) nor attention_prefill.hip (prompt portions)
+// takes, such as padded steps with several tokens per request or other head sizes.  Same rule as
+// the general kernel (a query at
 // position p sees the keys max(0, p-window+1)..p of its own request; scores, softmax and the
 // weighted sum in float32; reference: src/minigpt_infer/model.py:61-87 and the Triton decode
 // kernel src/minigpt_infer/attention/triton_paged.py:44-123, which walks the whole context in

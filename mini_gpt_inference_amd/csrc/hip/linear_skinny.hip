@@ -1,4 +1,7 @@
-// Matrix product for few rows (a decode step: 1..64 tokens) in bfloat16 on the MFMA units.
+// Matrix product for few rows (a decode step: 1..64 tokens) in bfloat16 on the MFMA units: the
+// general kernel, for every inner size that is a multiple of 16 and any alignment.  Shapes that
+// linear_decode.hip takes (inner sizes that are multiples of 32) go there from this file's
+// launcher.
 //
 // out[n, o] = sum_k act[n, k] * W[o, k] (+ bias[o]), nn.Linear as in
 // src/minigpt_infer/model.py:43-44,96-101 of the reference.  With so few rows the

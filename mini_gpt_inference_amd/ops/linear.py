@@ -49,9 +49,10 @@ def linear(ctx, a: Union[torch.Tensor, LazyNorm], w: torch.Tensor, bias: Optiona
            out: torch.Tensor, n_rows: int, epilogue: int = kernels.EPI_NONE, scatter=None) -> bool:
     """out[:n_rows] = a[:n_rows] @ w.T (+ bias) with the epilogue.
 
-    On the bfloat16 path few rows go to the skinny MFMA kernel (reading the residual stream through
-    the folded LayerNorm when `a` is a LazyNorm of a fusable norm) and many rows to the tiled MFMA kernel; the 32-bit
-    path, and every shape those refuse, go to the 32-bit FMA kernel.  `scatter` = (k_pool, v_pool,
+    On the bfloat16 path up to 64 rows go to the decode step's MFMA kernels (reading the residual
+    stream through the folded LayerNorm when `a` is a LazyNorm of a fusable norm and the rows are
+    few; splitting a long inner size over workgroups when the rows are many) and more rows to the
+    tiled MFMA kernel; the 32-bit path, and every shape those refuse, go to the 32-bit FMA kernel.  `scatter` = (k_pool, v_pool,
     slot_mapping, q_width, kv_width) asks for the new keys and values to be stored into their
     pages by the same kernel; the return value says whether that was done."""
     if n_rows == 0:
