@@ -44,3 +44,33 @@ extern "C" int mgpt_fold_layernorm(const void* w, const float* gain, const float
                      gain, beta, bias, (bf16_t*)w_out, colsum, bias_out, n_out, k_dim);
   return mgpt_last_error();
 }
+
+// The layout the decode step's product reads fastest: for every 16 rows of W and every 32 along k
+// one block of 1 KB, in which lane l of a wave finds its MFMA operand, the 8 values
+// W[16 t + (l & 15)][32 s + (l >> 4) * 8 ..], at offset 16 l.  A wave's load is then 1 KB in one piece
+// instead of sixteen pieces of 64 bytes.  Rows past n_out are zeros.  Made once per matrix.
+__global__ void pack_weight_kernel(const bf16_t* __restrict__ w, bf16_t* __restrict__ packed, int n_out,
+                                   int k_dim, long blocks) {
+  const long b = (long)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);  // block (t, s), one wave each
+  if (b >= blocks) return;
+  const int lane = threadIdx.x & 63;
+  const int steps = k_dim >> 5;
+  const long t = b / steps;
+  const int s = (int)(b - t * steps);
+  const long row = t * 16 + (lane & 15);
+  uint4 v = make_uint4(0, 0, 0, 0);
+  if (row < n_out) v = *reinterpret_cast<const uint4*>(w + row * k_dim + s * 32 + (lane >> 4) * 8);
+  *reinterpret_cast<uint4*>(packed + (b * 64 + lane) * 8) = v;
+}
+
+// packed: ceil(n_out / 16) * 16 * k_dim elements.  k_dim must be a multiple of 32.
+extern "C" int mgpt_pack_weight(const void* w, void* packed, int n_out, int k_dim, hipStream_t stream) {
+  if (n_out == 0) return MGPT_OK;
+  if (!w || !packed) return MGPT_ERR_NULL;
+  if (n_out < 0 || k_dim <= 0 || (k_dim % 32) != 0 || ((((size_t)w) | ((size_t)packed)) & 15) != 0)
+    return MGPT_ERR_BAD_SHAPE;
+  const long blocks = (long)((n_out + 15) / 16) * (k_dim / 32);
+  hipLaunchKernelGGL(pack_weight_kernel, dim3((unsigned int)((blocks + 3) / 4)), dim3(256), 0, stream,
+                     (const bf16_t*)w, (bf16_t*)packed, n_out, k_dim, blocks);
+  return mgpt_last_error();
+}

@@ -109,12 +109,15 @@ __global__ __launch_bounds__(256) void linear_decode_kernel(SkinnyArgs a) {
     x0[t] = sd[t] = sq[t] = 0.f;
     if (LN && row_ok[t]) x0[t] = a.x[(long)src[t] * K];
   }
-  const bf16_t* wp = a.w + (long)wo * K + kb + g * 8;
+  // W as it is (a wave's load is sixteen rows' 64 bytes), or packed so that it is 1 KB in one piece
+  const bf16_t* wp = a.w_packed ? a.w_packed + (((long)(o0 >> 4) * (K >> 5) + (kb >> 5)) * 64 + lane) * 8
+                                : a.w + (long)wo * K + kb + g * 8;
+  const int w_step = a.w_packed ? 512 : 32;
   for (int s0 = 0; s0 < steps; s0 += SMAX) {
     bf16x8_t wv[SMAX], av[NT][SMAX];
 #pragma unroll
     for (int i = 0; i < SMAX; ++i)
-      wv[i] = *reinterpret_cast<const bf16x8_t*>(wp + (s0 + i < steps ? s0 + i : 0) * 32);
+      wv[i] = *reinterpret_cast<const bf16x8_t*>(wp + (s0 + i < steps ? s0 + i : 0) * w_step);
     if (LN) {
       float4 lo[NT][SMAX], hi[NT][SMAX];
 #pragma unroll

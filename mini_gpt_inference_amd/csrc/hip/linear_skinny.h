@@ -21,6 +21,7 @@ struct SkinnyArgs {
   const float* colsum;  // S[o] of the folded matrix
   float eps;
   const bf16_t* w;    // [n_out, k_dim] (the folded matrix when x is given)
+  const bf16_t* w_packed;  // the same matrix in fold_norm.hip's packed layout, or null
   const float* bias;  // [n_out] or null (the folded bias when x is given)
   void* out;          // [n_rows, n_out], row stride ldo
   long ldo;

@@ -301,11 +301,12 @@ static int launch_nt(const SkinnyArgs& a, int epi, int out_dtype, dim3 grid, siz
 // a LayerNorm whose gain and bias were folded into w, bias and colsum (fold_norm.hip); otherwise
 // act holds bfloat16 activations.  Refuses (MGPT_ERR_BAD_SHAPE) more than 64 rows and k_dim that
 // is no multiple of 16; the caller then takes the general kernels.  general_only != 0 keeps to this
-// file's kernel also where linear_decode.hip would take the shape.  partials: optional scratch of
+// file's kernel also where linear_decode.hip would take the shape.  w_packed: optional, the
+// same matrix in mgpt_pack_weight's layout (only linear_decode.hip reads it).  partials: optional scratch of
 // mgpt_linear_skinny_partials(...) floats; with it a long inner size with many rows is split over
 // workgroups (two launches).
 extern "C" int mgpt_linear_skinny(const void* act, long lda, const float* x, const int* rows,
-                                  const float* colsum, float eps, const void* w,
+                                  const float* colsum, float eps, const void* w, const void* w_packed,
                                   const float* bias, void* out, int out_dtype, long ldo, int n_rows,
                                   int n_out, int k_dim, int epilogue, void* kpool, void* vpool,
                                   const int* slot_mapping, int q_width, int kv_width, int head_dim,
@@ -341,7 +342,7 @@ extern "C" int mgpt_linear_skinny(const void* act, long lda, const float* x, con
   }
   SkinnyArgs a;
   a.act = (const bf16_t*)act; a.lda = lda; a.x = x; a.rows = rows; a.colsum = colsum; a.eps = eps;
-  a.w = (const bf16_t*)w; a.bias = bias; a.out = out; a.ldo = ldo; a.n_rows = n_rows; a.n_out = n_out;
+  a.w = (const bf16_t*)w; a.w_packed = (const bf16_t*)w_packed; a.bias = bias; a.out = out; a.ldo = ldo; a.n_rows = n_rows; a.n_out = n_out;
   a.k_dim = k_dim; a.ksplit = ks; a.kpool = (bf16_t*)kpool; a.vpool = (bf16_t*)vpool;
   a.slot_mapping = slot_mapping; a.q_width = q_width; a.kv_width = kv_width; a.head_dim = head_dim;
   a.n_kv_head = n_kv_head; a.page_size = page_size;

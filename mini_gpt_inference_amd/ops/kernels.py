@@ -282,15 +282,15 @@ def linear_skinny(a: Optional[torch.Tensor], w: torch.Tensor, bias: Optional[tor
                   n_rows: int, epilogue: int = EPI_NONE, *, ln_x: Optional[torch.Tensor] = None,
                   ln_colsum: Optional[torch.Tensor] = None, ln_eps: float = 0.0,
                   ln_rows: Optional[torch.Tensor] = None, scatter=None, general_only: bool = False,
-                  partials: Optional[torch.Tensor] = None) -> bool:
+                  partials: Optional[torch.Tensor] = None, w_packed: Optional[torch.Tensor] = None) -> bool:
     """bfloat16 MFMA product for at most 64 rows.  With ln_x (the float32 residual stream; ln_rows an
     optional gather) the rows are read through a LayerNorm that fold_layer_norm folded into w, bias
     and ln_colsum.  scatter = (k_pool, v_pool, slot_mapping, q_width, kv_width) also stores the new
     keys and values into their pages.  Up to 16 rows with an inner size that is a multiple of 32 go
     to the kernel laid out for a decode step's latency unless general_only is set.  partials:
     float32 scratch of linear_skinny_partials(...) elements, with which a long inner size under many
-    rows is split over workgroups.  Returns False, having launched nothing, when the kernel does not
-    take the shape."""
+    rows is split over workgroups.  w_packed: pack_weight(w), which the decode kernel reads faster
+    than w itself.  Returns False, having launched nothing, when the kernel does not take the shape."""
     if n_rows > _SKINNY_MAX_ROWS or w.dtype != torch.bfloat16:
         return False
     n_out, k_dim = w.shape
@@ -323,6 +323,11 @@ def linear_skinny(a: Optional[torch.Tensor], w: torch.Tensor, bias: Optional[tor
         if a.stride(0) % 8 != 0 or a.data_ptr() % 16 != 0:
             return False
         lda = a.stride(0)
+    if w_packed is not None:
+        _need_cuda(w_packed)
+        _need(w_packed.dtype == torch.bfloat16 and w_packed.is_contiguous() and k_dim % 32 == 0
+              and w_packed.numel() == -(-n_out // 16) * 16 * k_dim and w_packed.data_ptr() % 16 == 0,
+              "w_packed must be pack_weight(w)")
     if partials is not None:
         _need_cuda(partials)
         _need(partials.dtype == torch.float32 and partials.is_contiguous() and partials.data_ptr() % 16 == 0,
@@ -338,13 +343,27 @@ def linear_skinny(a: Optional[torch.Tensor], w: torch.Tensor, bias: Optional[tor
         _need_i32("slot_mapping", sm, n_rows)
     rc = library.kernels().mgpt_linear_skinny(
         _ptr(a if ln_x is None else None), lda, _ptr(ln_x), _ptr(ln_rows), _ptr(ln_colsum),
-        float(ln_eps), _ptr(w), _ptr(bias), _ptr(out), _dtype_code(out), out.stride(0), n_rows, n_out, k_dim,
-        epilogue, _ptr(kp), _ptr(vp), _ptr(sm), q_width, kv_width, head_dim, n_kv_head, page_size,
+        float(ln_eps), _ptr(w), _ptr(w_packed), _ptr(bias), _ptr(out), _dtype_code(out), out.stride(0), n_rows,
+        n_out, k_dim, epilogue, _ptr(kp), _ptr(vp), _ptr(sm), q_width, kv_width, head_dim, n_kv_head, page_size,
         1 if general_only else 0, _ptr(partials), 0 if partials is None else partials.numel(), _stream())
     if rc == -2:
         return False
     _check(rc, "linear_skinny")
     return True
+
+
+def pack_weight(w: torch.Tensor) -> Optional[torch.Tensor]:
+    """A copy of a bfloat16 matrix [out, in] in the layout the decode step's product loads in 1 KB
+    pieces (blocks of 16 rows x 32 columns in MFMA operand order; rows padded to a multiple of 16
+    with zeros).  None if the inner size is no multiple of 32."""
+    _need_cuda(w)
+    _need(w.dtype == torch.bfloat16 and w.dim() == 2 and w.is_contiguous(), "the matrix must be dense bfloat16")
+    n_out, k_dim = w.shape
+    if k_dim % 32 != 0 or w.data_ptr() % 16 != 0:
+        return None
+    packed = torch.empty(-(-n_out // 16) * 16 * k_dim, dtype=torch.bfloat16, device=w.device)
+    _check(library.kernels().mgpt_pack_weight(_ptr(w), _ptr(packed), n_out, k_dim, _stream()), "pack_weight")
+    return packed
 
 
 def linear_skinny_partials(n_rows: int, n_out: int, k_dim: int, has_ln: bool, epilogue: int) -> int:

@@ -54,7 +54,8 @@ def _declare_optional(lib: ctypes.CDLL) -> None:
     """Signatures of the bfloat16 fast kernels."""
     P, I, L, F = c_void_p, c_int, c_long, c_float
     table = {
-        "mgpt_linear_skinny": [P, L, P, P, P, F, P, P, P, I, L, I, I, I, I, P, P, P, I, I, I, I, I, I, P, L, P],
+        "mgpt_linear_skinny": [P, L, P, P, P, F, P, P, P, P, I, L, I, I, I, I, P, P, P, I, I, I, I, I, I, P, L, P],
+        "mgpt_pack_weight": [P, P, I, I, P],
         "mgpt_linear_skinny_partials": [I, I, I, I, I],
         "mgpt_fold_layernorm": [P, P, P, P, P, P, P, I, I, P],
         "mgpt_paged_attention_split_bf16": [P, L, P, L, P, P, P, I, P, P, P, I, I, I, I, I, F, I, P],

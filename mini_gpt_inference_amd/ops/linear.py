@@ -41,6 +41,19 @@ def folded_layer_norm(norm, w: torch.Tensor, bias: Optional[torch.Tensor]):
     return hit[1:]
 
 
+_packed = {}   # matrix buffer -> (matrix, its packed copy or None)
+
+
+def packed_weight(w: torch.Tensor) -> Optional[torch.Tensor]:
+    """The matrix in the layout the decode kernel reads fastest, made once per matrix (at its first
+    decode step, before any graph is captured)."""
+    hit = _packed.get(w.data_ptr())
+    if hit is None or hit[0] is not w:
+        hit = (w, kernels.pack_weight(w))
+        _packed[w.data_ptr()] = hit
+    return hit[1]
+
+
 def as_tensor(ctx, a: Union[torch.Tensor, LazyNorm]) -> torch.Tensor:
     return a.tensor(ctx) if isinstance(a, LazyNorm) else a
 
@@ -66,13 +79,15 @@ def linear(ctx, a: Union[torch.Tensor, LazyNorm], w: torch.Tensor, bias: Optiona
                 and n_rows <= 32 and w.shape[0] <= 4096):
             wf, colsum, bias_f = folded_layer_norm(a.norm, w, bias)
             if kernels.linear_skinny(None, wf, bias_f, out, n_rows, epi, ln_x=a.x, ln_colsum=colsum,
-                                     ln_eps=a.norm.eps, ln_rows=a.rows, scatter=scatter):
+                                     ln_eps=a.norm.eps, ln_rows=a.rows, scatter=scatter,
+                                     w_packed=packed_weight(wf)):
                 return scatter is not None
         partials = None
         need = kernels.linear_skinny_partials(n_rows, w.shape[0], w.shape[1], False, epi) if n_rows > 16 else 0
         if need:
             partials = ctx.workspace.get("linear_partials", need, 1, torch.float32)
-        if kernels.linear_skinny(as_tensor(ctx, a), w, bias, out, n_rows, epi, scatter=scatter, partials=partials):
+        if kernels.linear_skinny(as_tensor(ctx, a), w, bias, out, n_rows, epi, scatter=scatter, partials=partials,
+                                 w_packed=packed_weight(w)):
             return scatter is not None
     a = as_tensor(ctx, a)
     if fast and scatter is not None and kernels.linear_mfma(a, w, bias, out, n_rows, epilogue, scatter=scatter):

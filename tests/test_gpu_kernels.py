@@ -104,6 +104,12 @@ def test_linear_skinny(n, k, o, epi, o_dt, general):
     prev = rnd(g, n + 2, o, dtype=o_dt)
     out = prev.clone().to(DEV)
     assert kernels.linear_skinny(a.to(DEV), w.to(DEV), bias.to(DEV), out, n, epi, general_only=general)
+    if not general and k % 32 == 0:
+        # the same product from the packed copy of the matrix: the same sums in the same order
+        packed = kernels.pack_weight(w.to(DEV))
+        out_p = prev.clone().to(DEV)
+        assert kernels.linear_skinny(a.to(DEV), w.to(DEV), bias.to(DEV), out_p, n, epi, w_packed=packed)
+        assert torch.equal(out_p, out), "the packed matrix gives another result"
     helpers.assert_close(out[:n], _linear_want(a, w, bias, epi, prev)[:n], "bfloat16", f"skinny {n}x{k}x{o}")
     assert torch.equal(out[n:], prev[n:].to(DEV)), "rows beyond n_rows were written"
     out2 = prev.clone().to(DEV)
@@ -149,6 +155,12 @@ def test_linear_skinny_through_a_folded_layer_norm(n, k, o, ln_bias, gather, gen
     out = torch.empty(n, o, dtype=torch.float32, device=DEV)
     assert kernels.linear_skinny(None, wf, bias_f, out, n, kernels.EPI_NONE, ln_x=x.to(DEV), ln_colsum=colsum,
                                  ln_eps=1e-5, ln_rows=i32(rows) if gather else None, general_only=general)
+    if not general and k % 32 == 0:
+        out_p = torch.empty_like(out)
+        assert kernels.linear_skinny(None, wf, bias_f, out_p, n, kernels.EPI_NONE, ln_x=x.to(DEV), ln_colsum=colsum,
+                                     ln_eps=1e-5, ln_rows=i32(rows) if gather else None,
+                                     w_packed=kernels.pack_weight(wf))
+        assert torch.equal(out_p, out), "the packed matrix gives another result"
     h = P.plain_layer_norm(x.double()[rows], lw.double(), lb.double() if ln_bias else None, 1e-5)
     helpers.assert_close(out, P.plain_linear(h, w.double(), bias.double()), "bfloat16", "LN + skinny")
 
