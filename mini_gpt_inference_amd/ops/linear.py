@@ -27,31 +27,38 @@ class LazyNorm:
         return self._tensor
 
 
-_folded = {}   # (matrix, gain, beta, bias) buffers -> (folded matrix, column sums, folded bias)
+# Derived copies of a matrix (folded with a LayerNorm, packed for the decode kernel) hang on the
+# matrix tensor itself, so they live exactly as long as it does.
+_DERIVED = "_mgpt_derived"
+
+
+def _derived(w: torch.Tensor) -> dict:
+    d = getattr(w, _DERIVED, None)
+    if d is None:
+        d = {}
+        setattr(w, _DERIVED, d)
+    return d
 
 
 def folded_layer_norm(norm, w: torch.Tensor, bias: Optional[torch.Tensor]):
-    """The matrix with the LayerNorm's gain and bias folded in, made once per (norm, matrix) pair."""
-    key = (w.data_ptr(), norm.weight.data_ptr(), 0 if norm.bias is None else norm.bias.data_ptr(),
+    """(folded matrix, column sums, folded bias): the matrix with the LayerNorm's gain and bias
+    folded in, made once per (norm, matrix, bias)."""
+    key = ("folded", norm.weight.data_ptr(), 0 if norm.bias is None else norm.bias.data_ptr(),
            0 if bias is None else bias.data_ptr())
-    hit = _folded.get(key)
-    if hit is None or hit[0] is not w:
-        hit = (w,) + kernels.fold_layer_norm(w, norm.weight, norm.bias, bias)
-        _folded[key] = hit
-    return hit[1:]
-
-
-_packed = {}   # matrix buffer -> (matrix, its packed copy or None)
+    d = _derived(w)
+    hit = d.get(key)
+    if hit is None:
+        hit = d[key] = kernels.fold_layer_norm(w, norm.weight, norm.bias, bias)
+    return hit
 
 
 def packed_weight(w: torch.Tensor) -> Optional[torch.Tensor]:
     """The matrix in the layout the decode kernel reads fastest, made once per matrix (at its first
     decode step, before any graph is captured)."""
-    hit = _packed.get(w.data_ptr())
-    if hit is None or hit[0] is not w:
-        hit = (w, kernels.pack_weight(w))
-        _packed[w.data_ptr()] = hit
-    return hit[1]
+    d = _derived(w)
+    if "packed" not in d:
+        d["packed"] = kernels.pack_weight(w)
+    return d["packed"]
 
 
 def as_tensor(ctx, a: Union[torch.Tensor, LazyNorm]) -> torch.Tensor:
