@@ -33,11 +33,14 @@ _DERIVED = "_mgpt_derived"
 
 
 def _derived(w: torch.Tensor) -> dict:
-    d = getattr(w, _DERIVED, None)
-    if d is None:
-        d = {}
-        setattr(w, _DERIVED, d)
-    return d
+    """The table of w's derived copies.  It hangs on the tensor that owns the memory (a view made
+    afresh at every call would take its table with it when it goes), one table per place and shape."""
+    owner = w._base if w._base is not None else w
+    tables = getattr(owner, _DERIVED, None)
+    if tables is None:
+        tables = {}
+        setattr(owner, _DERIVED, tables)
+    return tables.setdefault((w.data_ptr(), tuple(w.shape), tuple(w.stride())), {})
 
 
 def folded_layer_norm(norm, w: torch.Tensor, bias: Optional[torch.Tensor]):
