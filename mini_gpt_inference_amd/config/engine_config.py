@@ -24,7 +24,8 @@ class EngineConfig:
     mixed_batches: bool = True       # False: a step with admissions runs prompts only,
                                      # as the reference does (scheduler.py:52-56)
     dtype: str = "bfloat16"          # "bfloat16" (serving) or "float32" (true 32-bit path)
-    use_graph: bool = True           # replay decode-only steps from a captured HIP graph
+    use_graph: bool = True           # replay decode-only steps, and other steps whose shape repeats, from
+                                     # captured HIP graphs
     decode_burst: int = 8            # decode steps enqueued back to back when nothing else is pending,
                                      # tokens fed on the device from one to the next; 1 = off
     seed: int = 0                    # engine-wide sampler seed

@@ -106,7 +106,8 @@ class LLMEngine:
         self.cache = CacheManager(geometry, engine_config.max_batch_size)
         self.store = KVStore(layout, geometry, engine_config.max_batch_size, self.dtype, self.device)
         max_positions = model.spec.max_positions
-        self.runner = ModelRunner(model, self.cache, self.store, self.dtype, self.device, max_positions)
+        self.runner = ModelRunner(model, self.cache, self.store, self.dtype, self.device, max_positions,
+                                  graph_steps=engine_config.use_graph)
         self.scheduler = Scheduler(
             self.cache, engine_config.max_batch_size,
             max(engine_config.max_num_batched_tokens, engine_config.max_batch_size),
@@ -190,7 +191,7 @@ class LLMEngine:
         if r == 0:
             return []
         decode_only = n == r
-        use_graph = decode_only and self.engine_config.use_graph and m == r
+        use_graph = decode_only and self.engine_config.use_graph and m == r and self.model.graph_safe
         if use_graph:
             cap = _bucket(r)
             graphed = self._graphs.get(cap)
@@ -268,4 +269,5 @@ class LLMEngine:
             "free_blocks": self.cache.num_free_pages(0),
             "allocated_blocks": self.cache.groups[0].num_pages - self.cache.num_free_pages(0),
             "graph_steps": self.num_graph_steps, "eager_steps": self.num_eager_steps,
+            "replayed_eager_steps": self.runner.num_replayed_steps,
         }

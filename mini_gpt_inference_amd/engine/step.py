@@ -96,17 +96,39 @@ class StepShape:
     slots: List[int]
 
 
+@dataclass
+class _StepGraph:
+    """A step shape seen before: how often, and once captured the graph with what it is bound to."""
+    seen: int = 0
+    graph: Optional[torch.cuda.CUDAGraph] = None
+    arena: Optional[StepArena] = None
+    generation: int = -1
+    logits: Optional[torch.Tensor] = None
+
+
 class ModelRunner:
-    """Owns the device side of stepping: arenas, workspace, the cache's pools, the model."""
+    """Owns the device side of stepping: arenas, workspace, the cache's pools, the model.
+
+    Steps run eagerly, one launch per kernel from Python; for a model whose parts all allow it
+    (Part.graph_safe) a step shape that keeps coming is replayed from a HIP graph captured at its
+    third coming, since the host's launches, not the kernels, bound a step of a few hundred
+    tokens.  A shape is the tuple of the requests' token counts and the number of logit rows;
+    everything else a kernel reads comes from the arena's device arrays."""
+
+    MAX_STEP_GRAPHS = 64
+    CAPTURE_AT = 3     # a shape is captured when it comes for the third time (capturing costs a step's launches again)
 
     def __init__(self, model: DecoderModel, cache: CacheManager, store: KVStore, dtype: torch.dtype,
-                 device: torch.device, max_positions: Optional[int]) -> None:
+                 device: torch.device, max_positions: Optional[int], graph_steps: bool = True) -> None:
         self.model, self.cache, self.store = model, cache, store
         self.dtype, self.device = dtype, device
         self.exact = dtype == torch.float32
         self.max_positions = max_positions
         self.vocab_size = model.spec.vocab_size
         self.workspace = Workspace(device)
+        self.graph_steps = graph_steps and device.type == "cuda" and model.graph_safe
+        self._step_graphs: Dict[Tuple, _StepGraph] = {}
+        self.num_replayed_steps = 0
         self._arenas: Dict[Tuple[int, int, int], StepArena] = {}
         self.n_groups = len(cache.groups)
         self.page_sizes = torch.tensor([g.page_size for g in cache.groups], dtype=torch.int32, device=device)
@@ -192,11 +214,51 @@ class ModelRunner:
             host_state_slots=shape.slots, exact=self.exact)
 
     def run(self, arena: StepArena, shape: StepShape) -> torch.Tensor:
-        """Uploads the arena and runs the model eagerly.  Returns float32 logits [n_logits, vocab]."""
+        """Uploads the arena and runs the model.  Returns float32 logits [n_logits, vocab] (in the
+        workspace: the next step overwrites them)."""
         arena.upload()
+        entry = None
+        if self.graph_steps:
+            key = (tuple(shape.q_lens), shape.n_logits)
+            entry = self._step_graphs.get(key)
+            if entry is None:
+                if len(self._step_graphs) >= self.MAX_STEP_GRAPHS:
+                    self._step_graphs.clear()
+                entry = self._step_graphs[key] = _StepGraph()
+            if (entry.graph is not None and entry.arena is arena
+                    and entry.generation == self.workspace.generation):
+                entry.graph.replay()
+                self.num_replayed_steps += 1
+                return entry.logits
+            entry.graph = None
+            entry.seen += 1
         ctx = self.context(arena, shape, padded=False)
         with kernels.pinned_stream():
-            return self.model.forward(ctx)
+            logits = self.model.forward(ctx)
+        if entry is not None and entry.seen >= self.CAPTURE_AT:
+            self._capture(entry, arena, shape)
+        return logits
+
+    def _capture(self, entry: _StepGraph, arena: StepArena, shape: StepShape) -> None:
+        """Records the step just run (every buffer it needs exists now) for the next of its shape."""
+        graph = torch.cuda.CUDAGraph()
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        self.workspace.frozen = True
+        try:
+            with torch.cuda.stream(side):
+                graph.capture_begin()
+                try:
+                    with kernels.pinned_stream():
+                        logits = self.model.forward(self.context(arena, shape, padded=False))
+                finally:
+                    graph.capture_end()
+        except RuntimeError:
+            return   # a buffer would have had to grow: this shape stays eager
+        finally:
+            self.workspace.frozen = False
+            torch.cuda.current_stream().wait_stream(side)
+        entry.graph, entry.arena, entry.generation, entry.logits = graph, arena, self.workspace.generation, logits
 
     def step(self, slots: Sequence[int], ctx_lens: Sequence[int], q_lens: Sequence[int], tokens: Sequence[int],
              logit_rows: Sequence[int]) -> torch.Tensor:

@@ -51,6 +51,12 @@ class Part:
     """Base of every part.  Subclasses set `category` and implement their forward."""
 
     category = "part"
+    # True if forward() launches the same kernels with the same arguments for every step of the same
+    # shape (the numbers of tokens each request brings and of logit rows), taking all else (positions,
+    # lengths, slots, tables) from the step's device arrays: then a step may be captured in a HIP
+    # graph and replayed.  A part that looks at ctx.host_ctx_lens or ctx.host_state_slots, or that
+    # allocates, is not.
+    graph_safe = False
 
     def weight_requests(self) -> Dict[str, WeightRequest]:
         """Parameter name -> shape and role of every tensor this part needs."""
@@ -128,6 +134,7 @@ class Workspace:
         self.device = device
         self._buffers: Dict[str, torch.Tensor] = {}
         self.frozen = False   # set while a HIP graph owns the addresses
+        self.generation = 0   # counts (re)allocations: a graph captured before one holds stale addresses
 
     def get(self, name: str, rows: int, cols: int, dtype: torch.dtype) -> torch.Tensor:
         buf = self._buffers.get(name)
@@ -137,6 +144,7 @@ class Workspace:
             grow = rows if buf is None else max(rows, buf.shape[0])
             buf = torch.empty((grow, cols), dtype=dtype, device=self.device)
             self._buffers[name] = buf
+            self.generation += 1
         return buf
 
 

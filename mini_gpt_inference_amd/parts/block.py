@@ -23,6 +23,8 @@ class Arrangement(Part):
 class PreNorm(Arrangement):
     """x = x + mixer(norm1(x)); x = x + ff(norm2(x)) (reference: src/minigpt_infer/model.py:112-115)."""
 
+    graph_safe = True
+
     def __init__(self, width: int) -> None:
         self.width = int(width)
 

@@ -17,6 +17,8 @@ class TokenEmbedding(Part):
     """x0[t] = tok_emb[id_t] (+ the position encoding's table row), written to the float32
     residual stream (reference: src/minigpt_infer/model.py:123,183)."""
 
+    graph_safe = True
+
     category = "embedding"
 
     def __init__(self, vocab_size: int, width: int) -> None:
@@ -35,6 +37,8 @@ class LinearHead(Part):
     """logits = h W^T, float32 out, no bias (reference: src/minigpt_infer/model.py:128,187).
     With tied = True the matrix is the token embedding's, one buffer seen twice
     (src/minigpt_infer/model.py:129-130)."""
+
+    graph_safe = True
 
     category = "head"
 

@@ -27,6 +27,8 @@ class DenseMLP(FeedForward):
     (reference: src/minigpt_infer/model.py:96-101; there the hidden size is 4*n_embd, here it is
     a parameter)."""
 
+    graph_safe = True
+
     def __init__(self, width: int, hidden: int, bias: bool, activation: str = "gelu_tanh") -> None:
         if activation not in _ACTIVATIONS:
             raise ValueError(f"activation {activation!r} has no kernel epilogue; known: {sorted(_ACTIVATIONS)}")

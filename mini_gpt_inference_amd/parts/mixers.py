@@ -40,6 +40,8 @@ class PagedCausalAttention(Mixer):
     window, only the last `window` of them); softmax in float32; y = P v; heads concatenated
     head-major; out = y Wproj^T (+ b) (model.py:89-90), added into the residual (model.py:113)."""
 
+    graph_safe = True
+
     def __init__(self, width: int, n_head: int, head_dim: int, bias: bool, n_kv_head: Optional[int] = None,
                  scale: Optional[float] = None, window: int = 0) -> None:
         self.width, self.n_head, self.head_dim = int(width), int(n_head), int(head_dim)

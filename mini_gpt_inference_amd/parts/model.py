@@ -153,6 +153,14 @@ class DecoderModel:
                 bindings.append(CacheBinding("none"))
         return CacheLayout(groups, state_numels, bindings)
 
+    @property
+    def graph_safe(self) -> bool:
+        """Whether every part of the model allows a step to be captured in a HIP graph (Part.graph_safe)."""
+        parts = [self.embedding, self.position, self.final_norm, self.head]
+        for layer in self.layers:
+            parts += [layer.arrangement, layer.norm1, layer.mixer, layer.norm2, layer.feed_forward]
+        return all(getattr(p, "graph_safe", False) for p in parts if p is not None)
+
     # ------------------------------------------------------------------ forward
     def forward(self, ctx: StepContext) -> torch.Tensor:
         """Runs the step's tokens through every run of the order and returns float32 logits

@@ -16,6 +16,8 @@ class LayerNorm(Part):
     float32 (reference: nn.LayerNorm at src/minigpt_infer/model.py:107,109,127; there eps is the
     library default, here it is a parameter)."""
 
+    graph_safe = True
+
     category = "norm"
     fusable_layer_norm = True   # a linear kernel may fold weight and bias into its matrix and apply mean, rstd itself
 

@@ -33,6 +33,8 @@ class LearnedAbsolutePositions(PositionEncoding):
     """x0[t] += pos_emb[pos_t] with pos_t the absolute position, which must be < max_positions
     (reference: src/minigpt_infer/model.py:124,177-183)."""
 
+    graph_safe = True
+
     def __init__(self, max_positions: int, width: int) -> None:
         self.max_positions, self.width = int(max_positions), int(width)
         self.weight: Optional[torch.Tensor] = None
@@ -47,6 +49,8 @@ class LearnedAbsolutePositions(PositionEncoding):
 @register_position("none")
 class NoPositions(PositionEncoding):
     """No position signal at all."""
+
+    graph_safe = True
 
     def __init__(self) -> None:
         pass

@@ -257,3 +257,45 @@ def test_real_family_sizes(tmp_path, shape, dtype):
     for i in range(87, 90):
         got.append(rep.run_step({"step": i, "entries": [{"id": "x", "tokens": ids[i:i + 1], "want": [0]}], "end": []}).clone())
     helpers.assert_close(torch.cat(got), want[[0, 33, 69, 70, 86, 87, 88, 89]], dtype, f"{shape} {dtype}")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_step_shapes_that_repeat_are_replayed_from_a_graph_with_the_same_logits(model_folders, dtype):
+    """Single tokens and portions of four, over and over: from the fourth step of a shape on the
+    step is a graph replay; every replay is checked against the plain implementation, with eager
+    steps of other shapes between them; a larger step in between makes the workspace grow, which
+    retires the graphs captured before it."""
+    cfg = helpers.CONFIGS["B"]
+    rng = np.random.default_rng(5)
+    ids = helpers.random_ids(rng, cfg.vocab_size, 120)
+    other = helpers.random_ids(rng, cfg.vocab_size, 90)
+    pcfg, w = P.read_model_folder(model_folders["B"])
+    want, want_other = P.plain_forward(w, pcfg, ids).numpy(), P.plain_forward(w, pcfg, other).numpy()
+    rep = TraceReplayer(model_folders["B"], dtype, 256, poison=True)
+    assert rep.runner.graph_steps
+    fed, step = 0, 0
+
+    def feed(n, rid="x", seq=ids, ref=want, start=None):
+        nonlocal step
+        s = fed if start is None else start
+        got = rep.run_step({"step": step, "entries": [{"id": rid, "tokens": seq[s:s + n], "want": list(range(n))}],
+                            "end": []}).cpu()
+        step += 1
+        helpers.assert_close(got, ref[s:s + n], dtype, f"step {step}: tokens {s}..{s + n}")
+
+    for _ in range(8):                      # shape (1,): eager, eager, capture, then replays
+        feed(1); fed += 1
+    first = rep.runner.num_replayed_steps
+    assert first >= 4
+    for _ in range(6):                      # shape (4,) between them
+        feed(4); fed += 4
+        feed(1); fed += 1
+    assert rep.runner.num_replayed_steps >= first + 8
+    feed(60, "y", other, want_other, 0)     # a larger step: buffers grow, the graphs are stale
+    before = rep.runner.num_replayed_steps
+    for _ in range(8):
+        feed(1); fed += 1
+        feed(4); fed += 4
+    assert rep.runner.num_replayed_steps >= before + 8   # captured again and replayed again
+    for i in range(60, 64):                 # and the other request goes on where it stood
+        feed(1, "y", other, want_other, i)
