@@ -335,19 +335,21 @@ def test_part_constructors_refuse_what_the_kernels_cannot_do():
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_toy_model_generates_through_the_engine(dtype):
-    """The engine, scheduler, state slots and (for decode steps) graph capture work for a model that
-    no registered architecture describes; eviction resets the toy's state because it starts over."""
+    """The engine, scheduler and state slots work for a model that no registered architecture describes;
+    eviction resets the toy's state because it starts over.  The toy mixer does not declare itself
+    graph_safe (it reads host-side lists), so the engine, asked for graphs, still runs every step eagerly."""
     model = DecoderModel(_spec(ORDER))
     weights = _random_weights(model, 12, scale=0.2)
     _bind(model, weights, dtype)
     prompts = [np.random.default_rng(3).integers(0, V, n).tolist() for n in (6, 11, 3)]
     sp = SamplingParams(max_tokens=8, temperature=0.0)
-    # the toy mixer reads host-side lists, so its steps cannot be replayed from a graph
+    assert not model.graph_safe
     engine = LLMEngine(model, None, EngineConfig(block_size=4, num_blocks=40, max_batch_size=3, dtype=dtype,
-                                                 prefill_chunk=4, use_graph=False))
+                                                 prefill_chunk=4, use_graph=True))
     got = engine.generate(prompts, sp)
+    assert engine.stats()["graph_steps"] == 0 and engine.stats()["replayed_eager_steps"] == 0
     tight = LLMEngine(model, None, EngineConfig(block_size=4, num_blocks=9, max_batch_size=3, dtype=dtype,
-                                                use_graph=False))
+                                                use_graph=True))
     got_tight = tight.generate(prompts, sp)
     assert tight.stats()["num_preemptions"] > 0
     for prompt, tokens, tokens_tight in zip(prompts, got, got_tight):
