@@ -39,8 +39,9 @@ def _dtype_code(t: torch.Tensor) -> int:
     raise KernelError(f"kernels take float32 or bfloat16 buffers, got {t.dtype}")
 
 
-def _ptr(t: Optional[torch.Tensor]) -> ctypes.c_void_p:
-    return ctypes.c_void_p(0 if t is None else t.data_ptr())
+def _ptr(t: Optional[torch.Tensor]) -> Optional[int]:
+    """The address for a pointer argument (ctypes takes an int, or None for null, where argtypes say c_void_p)."""
+    return None if t is None else t.data_ptr()
 
 
 _pinned_stream: Optional[ctypes.c_void_p] = None
