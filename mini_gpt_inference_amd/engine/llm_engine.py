@@ -59,8 +59,17 @@ class _GraphedDecode:
         side.wait_stream(torch.cuda.current_stream())
         with torch.cuda.stream(side):
             graph.capture_begin()
-            for _ in range(times):
-                self._launch(shape)
+            try:
+                for _ in range(times):
+                    self._launch(shape)
+            except BaseException:
+                # never leave the stream capturing: the graph object's destructor synchronizes the
+                # device, which a stream that is still capturing turns into an abort of the process
+                try:
+                    graph.capture_end()
+                except RuntimeError:
+                    pass
+                raise
             graph.capture_end()
         torch.cuda.current_stream().wait_stream(side)
         return graph

@@ -19,7 +19,7 @@ import torch
 from ..cache.kv_store import KVStore
 from ..cache.manager import CacheManager
 from ..ops import kernels
-from ..parts.base import GroupView, StepContext, Workspace
+from ..parts.base import GroupView, StepContext, Workspace, WorkspaceFrozen
 from ..parts.model import DecoderModel
 
 
@@ -251,9 +251,16 @@ class ModelRunner:
                 try:
                     with kernels.pinned_stream():
                         logits = self.model.forward(self.context(arena, shape, padded=False))
-                finally:
-                    graph.capture_end()
-        except RuntimeError:
+                except BaseException:
+                    # never leave the stream capturing (the graph object's destructor synchronizes
+                    # the device); the capture is lost, so what ending it reports is of no interest
+                    try:
+                        graph.capture_end()
+                    except RuntimeError:
+                        pass
+                    raise
+                graph.capture_end()
+        except WorkspaceFrozen:
             return   # a buffer would have had to grow: this shape stays eager
         finally:
             self.workspace.frozen = False

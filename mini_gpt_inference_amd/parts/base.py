@@ -127,23 +127,29 @@ class CacheBinding:
     writes: bool = True  # False: the run reads a cache that an earlier run of this step wrote
 
 
+class WorkspaceFrozen(RuntimeError):
+    """A buffer would have to be (re)allocated while a HIP graph holds the workspace's addresses."""
+
+
 class Workspace:
     """Named scratch buffers that grow on demand and are reused from step to step."""
 
     def __init__(self, device: torch.device) -> None:
         self.device = device
-        self._buffers: Dict[str, torch.Tensor] = {}
+        self._buffers: Dict[tuple, torch.Tensor] = {}
         self.frozen = False   # set while a HIP graph owns the addresses
         self.generation = 0   # counts (re)allocations: a graph captured before one holds stale addresses
 
     def get(self, name: str, rows: int, cols: int, dtype: torch.dtype) -> torch.Tensor:
-        buf = self._buffers.get(name)
-        if buf is None or buf.shape[0] < rows or buf.shape[1] != cols or buf.dtype != dtype:
+        # one buffer per (name, width, dtype): layers of different widths that use the same name
+        # must not take each other's buffer away (a step graph holds the addresses of both)
+        key = (name, cols, dtype)
+        buf = self._buffers.get(key)
+        if buf is None or buf.shape[0] < rows:
             if self.frozen:
-                raise RuntimeError(f"workspace buffer {name!r} would have to grow while a graph holds it")
-            grow = rows if buf is None else max(rows, buf.shape[0])
-            buf = torch.empty((grow, cols), dtype=dtype, device=self.device)
-            self._buffers[name] = buf
+                raise WorkspaceFrozen(f"workspace buffer {name!r} would have to grow while a graph holds it")
+            buf = torch.empty((rows, cols), dtype=dtype, device=self.device)
+            self._buffers[key] = buf
             self.generation += 1
         return buf
 

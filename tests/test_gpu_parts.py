@@ -362,3 +362,230 @@ def test_toy_model_generates_through_the_engine(dtype):
         if dtype == "float32":
             assert tokens_tight == tokens
     assert engine.cache.check() == 0 and engine.cache.num_free_pages(0) == 40 and engine.cache.num_free_pages(1) == 40
+
+
+# ----------------------------------------------------------------------------- two more toy parts
+# A position encoding that acts on queries and keys, and a feed-forward that routes each token to
+# one of several experts: defined and registered here, written with library calls, never part of
+# the product.  They show that the hooks of the parts carry such things without a change to the
+# framework's files.
+from mini_gpt_inference_amd.parts.base import register_feed_forward, register_position  # noqa: E402
+from mini_gpt_inference_amd.parts.feedforward import FeedForward  # noqa: E402
+from mini_gpt_inference_amd.parts.positions import PositionEncoding  # noqa: E402
+
+
+@register_position("toy_pair_rotation")
+class ToyPairRotation(PositionEncoding):
+    """Turns the pair (2i, 2i+1) of every head of q and k by the angle pos * base^(-i / (D/2)), so that
+    q.k depends on the distance of the two positions only.  Everything it does is a device operation on
+    device tensors, so it declares itself safe for graphs."""
+
+    rotates = True
+    graph_safe = True
+
+    def __init__(self, head_dim: int, base: float) -> None:
+        self.head_dim, self.base = int(head_dim), float(base)
+        self._freq = None
+
+    def rotate(self, ctx, q, k, n_tokens):
+        half = self.head_dim // 2
+        if self._freq is None:
+            self._freq = (self.base ** (-torch.arange(half, dtype=torch.float64) / half)).float().to(q.device)
+        ang = ctx.positions[:n_tokens].float()[:, None] * self._freq[None, :]
+        cos, sin = ang.cos()[:, None, :], ang.sin()[:, None, :]
+        for t in (q, k):
+            pairs = t[:n_tokens].float().reshape(n_tokens, -1, half, 2)
+            a, b = pairs[..., 0], pairs[..., 1]
+            turned = torch.stack((a * cos - b * sin, a * sin + b * cos), dim=-1)
+            t[:n_tokens].copy_(turned.reshape(n_tokens, -1))
+
+
+def plain_pair_rotation(x, positions, base):
+    """x: [heads, T, D] float64; positions: [T]."""
+    half = x.shape[-1] // 2
+    freq = base ** (-torch.arange(half, dtype=P.DT) / half)
+    ang = positions.to(P.DT)[:, None] * freq[None, :]
+    out = torch.empty_like(x)
+    out[..., 0::2] = x[..., 0::2] * ang.cos() - x[..., 1::2] * ang.sin()
+    out[..., 1::2] = x[..., 0::2] * ang.sin() + x[..., 1::2] * ang.cos()
+    return out
+
+
+@register_feed_forward("toy_top1_experts")
+class ToyTop1Experts(FeedForward):
+    """r = h Wr^T; e = argmax r; out = softmax(r)[e] * gelu(h Wfc[e]^T) Wproj[e]^T.  Asks the host which rows
+    each expert gets, so it is not safe for graphs and does not say it is."""
+
+    def __init__(self, width: int, hidden: int, n_experts: int) -> None:
+        self.width, self.hidden, self.n_experts = int(width), int(hidden), int(n_experts)
+        self.router_weight = self.fc_weight = self.proj_weight = None
+
+    def weight_requests(self):
+        return {"router_weight": WeightRequest((self.n_experts, self.width), MATRIX),
+                "fc_weight": WeightRequest((self.n_experts * self.hidden, self.width), MATRIX),
+                "proj_weight": WeightRequest((self.n_experts * self.width, self.hidden), MATRIX)}
+
+    def forward_add(self, ctx, h, x):
+        n = ctx.n_tokens
+        hn = as_tensor(ctx, h)[:n].float()
+        prob = torch.softmax(hn @ self.router_weight.float().t(), dim=-1)
+        gate, expert = prob.max(dim=-1)
+        fc = self.fc_weight.float().view(self.n_experts, self.hidden, self.width)
+        proj = self.proj_weight.float().view(self.n_experts, self.width, self.hidden)
+        for e in range(self.n_experts):
+            rows = (expert == e).nonzero().flatten()
+            if rows.numel():
+                u = torch.nn.functional.gelu(hn[rows] @ fc[e].t(), approximate="tanh")
+                x[rows] += gate[rows, None] * (u @ proj[e].t())
+
+
+def plain_top1_experts(h, router, fc, proj, n_experts):
+    """Returns the output and the smallest gap between a token's two largest router logits: where
+    that gap is within rounding, the choice of expert is not a fact to compare."""
+    r = h @ router.t()
+    top2 = r.topk(2, dim=-1).values
+    prob = torch.softmax(r, dim=-1)
+    out = torch.zeros_like(h)
+    hidden = fc.shape[0] // n_experts
+    for t in range(h.shape[0]):
+        e = int(r[t].argmax())
+        u = P.plain_gelu_tanh(h[t] @ fc[e * hidden:(e + 1) * hidden].t())
+        out[t] = prob[t, e] * (u @ proj[e * h.shape[1]:(e + 1) * h.shape[1]].t())
+    return out, float((top2[:, 0] - top2[:, 1]).min())
+
+
+ROT_BASE, N_EXPERTS, EXPERT_HIDDEN = 40.0, 3, 56
+
+
+def _rot_spec(order, routed):
+    first = _attn_layer(0, C, H, HK, D, WINDOW, SCALE, HID, EPS)
+    if routed:
+        first = LayerSpec(first.arrangement, first.norm1, first.mixer, first.norm2,
+                          PartSpec("toy_top1_experts", {"width": C, "hidden": EXPERT_HIDDEN, "n_experts": N_EXPERTS},
+                                   {"router_weight": "L0.router.w", "fc_weight": "L0.experts.fc",
+                                    "proj_weight": "L0.experts.pr"}))
+    layers = (first, _attn_layer(1, C, H, H, D, 0, 1 / math.sqrt(D), HID, EPS))
+    return ModelSpec(width=C, vocab_size=V,
+                     embedding=PartSpec("token_embedding", {"vocab_size": V, "width": C}, {"weight": "emb.w"}),
+                     position=PartSpec("toy_pair_rotation", {"head_dim": D, "base": ROT_BASE}),
+                     layers=layers, order=tuple(order), final_norm=_norm("nf.", C, EPS),
+                     head=PartSpec("linear_head", {"vocab_size": V, "width": C, "tied": True}, {"weight": "emb.w"}),
+                     max_positions=None)
+
+
+ROT_ORDER = (LayerRun(0), LayerRun(1), LayerRun(0))
+
+
+def _plain_rot_model(w, ids, routed, first_position=0):
+    """Returns the logits and the smallest router gap met on the way."""
+    x = P.plain_embed(torch.tensor(ids), w["emb.w"].double(), None)
+    positions = torch.arange(first_position, first_position + len(ids))
+    gap = float("inf")
+    for run in ROT_ORDER:
+        p = f"L{run.layer}."
+        hk, window, scale = (HK, WINDOW, SCALE) if run.layer == 0 else (H, 0, 1 / math.sqrt(D))
+        h = _pl_norm(x, w, p + "n1.", EPS)
+        q, k, v = P.plain_split_heads(P.plain_linear(h, w[p + "qkv.w"].double(), w[p + "qkv.b"].double()), H, hk)
+        q, k = plain_pair_rotation(q, positions, ROT_BASE), plain_pair_rotation(k, positions, ROT_BASE)
+        y = P.plain_causal_attention(q, k, v, scale=scale, window=window)
+        x = x + P.plain_linear(y, w[p + "o.w"].double(), w[p + "o.b"].double())
+        h = _pl_norm(x, w, p + "n2.", EPS)
+        if routed and run.layer == 0:
+            m, g = plain_top1_experts(h, w["L0.router.w"].double(), w["L0.experts.fc"].double(),
+                                      w["L0.experts.pr"].double(), N_EXPERTS)
+            gap = min(gap, g)
+            x = x + m
+        else:
+            x = x + _pl_mlp(h, w, p)
+    return _pl_norm(x, w, "nf.", EPS) @ w["emb.w"].double().t(), gap
+
+
+def test_plain_pair_rotation_counts_distances_only():
+    """What pins the plain rotation: position 0 changes nothing, lengths are kept, the scores q.k depend
+    on the distance alone (so a shift of all positions changes no logit), and a wrong sign in one of the
+    two lines would break that."""
+    g = torch.Generator().manual_seed(4)
+    q, k = torch.randn(2, 9, D, generator=g, dtype=P.DT), torch.randn(2, 9, D, generator=g, dtype=P.DT)
+    pos = torch.arange(9)
+    assert torch.equal(plain_pair_rotation(q[:, :1], pos[:1], ROT_BASE), q[:, :1])
+    assert torch.allclose(plain_pair_rotation(q, pos, ROT_BASE).norm(dim=-1), q.norm(dim=-1), rtol=1e-12)
+    s0 = plain_pair_rotation(q, pos, ROT_BASE) @ plain_pair_rotation(k, pos, ROT_BASE).transpose(1, 2)
+    s7 = plain_pair_rotation(q, pos + 7, ROT_BASE) @ plain_pair_rotation(k, pos + 7, ROT_BASE).transpose(1, 2)
+    assert torch.allclose(s0, s7, atol=1e-12)
+    assert not torch.allclose(s0, q @ k.transpose(1, 2), atol=1e-3)
+    model = DecoderModel(_rot_spec(ROT_ORDER, routed=True))
+    w = _random_weights(model, 21)
+    ids = np.random.default_rng(8).integers(0, V, 17).tolist()
+    a, b = _plain_rot_model(w, ids, True)[0], _plain_rot_model(w, ids, True, first_position=11)[0]
+    assert torch.allclose(a, b, atol=1e-10)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("routed", [False, True])
+def test_toy_rotation_and_toy_experts_whole_and_cut(dtype, routed):
+    model = DecoderModel(_rot_spec(ROT_ORDER, routed))
+    assert model.graph_safe == (not routed)
+    weights = _random_weights(model, 48)      # a seed with which no token's two best experts come close
+    if routed:
+        weights["L0.router.w"] = (weights["L0.router.w"] * 4).to(torch.bfloat16)
+    _bind(model, weights, dtype)
+    rng = np.random.default_rng(6)
+    reqs = [rng.integers(0, V, n).tolist() for n in (29, 12)]
+    plain = [_plain_rot_model(weights, ids, routed) for ids in reqs]
+    want = [p[0].numpy() for p in plain]
+    if routed:      # the inputs are only valid if no token's choice of expert hangs on rounding
+        assert min(p[1] for p in plain) > 0.25, min(p[1] for p in plain)
+
+    runner, cache = _runner(model, dtype)
+    slots = [cache.acquire_slot() for _ in reqs]
+    for s, ids in zip(slots, reqs):
+        assert cache.reserve(s, len(ids))
+    whole = runner.step(slots, [0, 0], [len(r) for r in reqs], sum(reqs, []), list(range(sum(map(len, reqs)))))
+    helpers.assert_close(whole[:29], want[0], dtype, "whole 0")
+    helpers.assert_close(whole[29:], want[1], dtype, "whole 1")
+    for s in slots:
+        cache.free_slot(s)
+
+    slots = [cache.acquire_slot() for _ in reqs]
+    done, got = [0, 0], [[], []]
+    sizes = [[6, 1, 1, 9, 2, 1], [3, 1, 2, 1, 1]]
+    step = 0
+    while any(d < len(r) for d, r in zip(done, reqs)):
+        batch = [(i, min(sizes[i][step % len(sizes[i])], len(reqs[i]) - done[i])) for i in range(2)
+                 if done[i] < len(reqs[i])]
+        step += 1
+        for i, q in batch:
+            assert cache.reserve(slots[i], done[i] + q)
+        toks = sum((reqs[i][done[i]:done[i] + q] for i, q in batch), [])
+        out = runner.step([slots[i] for i, _ in batch], [done[i] for i, _ in batch], [q for _, q in batch], toks,
+                          list(range(len(toks))))
+        o = 0
+        for i, q in batch:
+            got[i].append(out[o:o + q].cpu())
+            o += q
+            done[i] += q
+            cache.release_passed(slots[i], done[i])
+    for i in range(2):
+        helpers.assert_close(torch.cat(got[i]), want[i], dtype, f"cut request {i}")
+    assert cache.check() == 0
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_toy_rotation_decodes_from_graphs(dtype):
+    """A toy part that says it is safe for graphs is captured with the rest: greedy generation through
+    the engine, decode steps replayed from graphs, each token the plain model's choice."""
+    model = DecoderModel(_rot_spec(ROT_ORDER, routed=False))
+    weights = _random_weights(model, 23, scale=0.2)
+    _bind(model, weights, dtype)
+    prompts = [np.random.default_rng(5).integers(0, V, n).tolist() for n in (7, 4)]
+    engine = LLMEngine(model, None, EngineConfig(block_size=4, num_blocks=40, max_batch_size=2, dtype=dtype,
+                                                 use_graph=True))
+    got = engine.generate(prompts, SamplingParams(max_tokens=12, temperature=0.0))
+    assert engine.stats()["graph_steps"] > 0
+    for prompt, tokens in zip(prompts, got):
+        ids = list(prompt)
+        for tok in tokens:
+            logits = _plain_rot_model(weights, ids, False)[0][-1].numpy()
+            margin = 2 * helpers.TOL[dtype] * max(1.0, np.abs(logits).max())
+            assert logits[tok] >= logits.max() - margin
+            ids.append(tok)
