@@ -1,18 +1,32 @@
-// Tiled bfloat16 matrix product on the MFMA units for many rows (prompt portions).
+// Tiled bfloat16 matrix product on the MFMA units for many rows (prompt portions):
+// out[n, o] = sum_k act[n, k] * W[o, k] (+ bias[o]) with an optional GELU-tanh or residual-add
+// epilogue, or one that also stores new keys and values into their cache pages (nn.Linear as in
+// src/minigpt_infer/model.py:43-44,96-101; the cache write of src/minigpt_infer/cache/paged.py:125-137).
 //
-// out[n, o] = sum_k act[n, k] * W[o, k] (+ bias[o]) with an optional GELU-tanh or
-// residual-add epilogue: nn.Linear as in src/minigpt_infer/model.py:43-44,96-101.
+// One kernel template, five tile shapes.  What bounds a tile kernel on this machine is the traffic
+// between LDS and the MFMA units: a wave that owns R x C outputs reads (R + C) * 32 operand values
+// from LDS for R * C * 32 multiply-adds, so a wave's tile is as large as the problem allows while
+// it still gives every compute unit work: 256 x 256 outputs per workgroup (eight waves of
+// 128 x 64) for large problems, down to 32 x 32 (four waves of 16 x 16) for a prompt portion of a
+// hundred tokens.  A step along k is 64 long.
 //
-// A workgroup of four waves owns a 128 x 128 (or, for small problems, 64 x 64)
-// tile of the output; each wave a quarter of it, as 4 x 4 (2 x 2)
-// v_mfma_f32_16x16x32_bf16 accumulators.  Per step of 32 along k the workgroup
-// stages a slice (32 or 64 along k) of the activations and of W
-// in LDS (rows padded by 16 bytes so the 16 rows a MFMA operand reads fall on
-// distinct banks), with the global loads of the next two to four slices in
-// flight while the current one is multiplied.  W is the first MFMA operand, so a lane ends up
-// with four neighbouring output columns of one row and stores them as one
-// vector.
+// The workgroup stages its slice of the activations and of W in LDS twice over.  A row of a slice
+// is 128 bytes, eight chunks of 16; chunk c of row r lies at position c ^ (r & 7) of its row.  With
+// that, the 16 rows x 4 chunks that an MFMA operand read (ds_read_b128) touches are served at the
+// full 256 bytes per clock; rows padded by 16 bytes, the usual remedy, take twice as long on this
+// LDS (measured with SQ_LDS_BANK_CONFLICT), and unpadded rows four times.
+//
+// Two steps' worth of loads are in flight: while step s is multiplied, the chunks of step s + 1
+// (loaded during step s - 1) go into the other LDS buffer and those of step s + 2 are sent for,
+// both spread between the MFMAs, because LDS takes writes at half the rate of reads and all at
+// once they would hold every wave up.  MFMA operands are read from LDS two groups of MFMAs ahead
+// of their use.  W is the first MFMA operand, so a lane ends up with four neighbouring output
+// columns of one row and stores them as one vector.
+//
+// Tiles are numbered so that the workgroups that run at the same time on an XCD (which has an L2
+// of its own) form a block of a few row tiles by a few column tiles, whose operands that L2 holds.
 #include "common.h"
+#include <type_traits>
 
 typedef __attribute__((__vector_size__(8 * sizeof(short)))) short bf16x8_t;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4_t;
@@ -30,265 +44,354 @@ struct MfmaScatter {
   int q_width, kv_width, head_dim, n_kv_head, page_size;
 };
 
-// WT: 16-wide tiles per wave in each direction.  4 -> 128 x 128 per workgroup, 2 -> 64 x 64, 1 -> 32 x 32.
-template <int WT, int EPI, typename OT>
-__global__ __launch_bounds__(256) void linear_mfma_kernel(
+// The bias of the four neighbouring output columns oc..oc+3 a lane holds.
+__device__ __forceinline__ void mfma_bias4(const float* __restrict__ bias, int oc, int n_out, bool vec, float b4[4]) {
+  b4[0] = b4[1] = b4[2] = b4[3] = 0.f;
+  if (!bias) return;
+  if (vec) {
+    const float4 t = *reinterpret_cast<const float4*>(bias + oc);
+    b4[0] = t.x; b4[1] = t.y; b4[2] = t.z; b4[3] = t.w;
+  } else {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) b4[e] = oc + e < n_out ? bias[oc + e] : 0.f;
+  }
+}
+
+// Stores the four columns oc..oc+3 of row n: bias, activation, then a plain store, an add into
+// the residual stream, or a store that also puts key and value columns into their cache pages.
+// `vec`: the four columns can go as one aligned vector.
+template <int EPI, typename OT>
+__device__ __forceinline__ void mfma_store4(const f32x4_t& a, const float b4[4], OT* __restrict__ out, long ldo,
+                                            int n, int oc, int n_out, bool vec, const MfmaScatter& sc) {
+  OT* orow = out + (long)n * ldo;
+  float v[4];
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    v[e] = a[e] + b4[e];
+    if (EPI == MM_EPI_GELU) v[e] = gelu_tanh_fast(v[e]);
+  }
+  if (vec && sizeof(OT) == 4) {
+    float4* dst = reinterpret_cast<float4*>(orow + oc);
+    if (EPI == MM_EPI_RESIDUAL) {
+      const float4 old = *dst;
+      *dst = make_float4(old.x + v[0], old.y + v[1], old.z + v[2], old.w + v[3]);
+    } else {
+      *dst = make_float4(v[0], v[1], v[2], v[3]);
+    }
+  } else if (vec && EPI != MM_EPI_RESIDUAL) {
+    uint2 pk;
+    pk.x = pack_bf16x2(v[0], v[1]);
+    pk.y = pack_bf16x2(v[2], v[3]);
+    *reinterpret_cast<uint2*>(orow + oc) = pk;
+    if (EPI == MM_EPI_QKV && oc >= sc.q_width) {
+      // the four columns lie in one head (the launcher checks that sizes are multiples of 4)
+      const int slot = sc.slot_mapping[n];
+      if (slot >= 0) {
+        const long page = slot / sc.page_size;
+        const int off = slot - (int)page * sc.page_size;
+        const int c = oc - sc.q_width;  // column among keys then values
+        const bool is_v = c >= sc.kv_width;
+        const int cc = is_v ? c - sc.kv_width : c;
+        const int h = cc / sc.head_dim, d = cc - h * sc.head_dim;
+        const long dst = ((page * sc.n_kv_head + h) * sc.page_size + off) * (long)sc.head_dim + d;
+        *reinterpret_cast<uint2*>((is_v ? sc.vpool : sc.kpool) + dst) = pk;
+      }
+    }
+  } else {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const int o = oc + e;
+      if (o >= n_out) continue;
+      if (EPI == MM_EPI_RESIDUAL) {
+        orow[o] = from_float<OT>(to_float<OT>(orow[o]) + v[e]);
+      } else {
+        orow[o] = from_float<OT>(v[e]);
+      }
+    }
+  }
+}
+
+// Deals the workgroup ids out so that an XCD's workgroups (ids that agree modulo 8 go to the same
+// XCD, which has an L2 of its own) are neighbours in tile order.
+__device__ __forceinline__ int mfma_xcd_tile_id(int pid, int total) {
+  const int per_xcd = (total + 7) >> 3, tall = (total & 7) ? (total & 7) : 8;
+  const int xcd = pid & 7, local = pid >> 3;
+  return xcd < tall ? xcd * per_xcd + local : tall * per_xcd + (xcd - tall) * (per_xcd - 1) + local;
+}
+
+namespace {
+
+constexpr int MM_BK = 64;
+constexpr int MM_LD = MM_BK;       // LDS row stride in elements: 128 bytes, eight 16-byte chunks
+constexpr int MM_GROUP = 4;         // row tiles per block of tiles
+
+// WTM x WTN: 16-wide tiles per wave along the rows of the activations and along the rows of W;
+// WVM x WVN: waves in a workgroup along the same.
+template <int WTM, int WTN, int WVM, int WVN, int EPI, typename OT>
+__global__ __launch_bounds__(64 * WVM * WVN) void linear_mfma_kernel(
     const bf16_t* __restrict__ act, long lda, const bf16_t* __restrict__ w,
     const float* __restrict__ bias, OT* __restrict__ out, long ldo, int n_rows, int n_out, int k_dim,
     MfmaScatter sc) {
-  constexpr int TILE = 2 * WT * 16;   // rows and columns of the workgroup's tile
-  constexpr int MM_BK = WT == 4 ? 32 : 64;   // k per step: what fits LDS twice over
-  constexpr int MM_LD = MM_BK + 8;           // LDS row stride in elements (16 bytes of padding)
-  constexpr int TPR = MM_BK / 8;             // threads per staged row (16 bytes each)
-  constexpr int RPP = 256 / TPR;             // rows per staging pass
-  constexpr int PASSES = TILE / RPP;
-  __shared__ __align__(16) bf16_t as[2][TILE * MM_LD];
-  __shared__ __align__(16) bf16_t ws[2][TILE * MM_LD];
+  constexpr int T = 64 * WVM * WVN;
+  constexpr int BM = WVM * WTM * 16, BN = WVN * WTN * 16;
+  constexpr int TPR = MM_BK / 8;  // threads per staged row (16 bytes each)
+  constexpr int RPP = T / TPR;      // rows per staging pass
+  constexpr int PA = BM / RPP, PW = BN / RPP;
+  static_assert(BM % RPP == 0 && BN % RPP == 0 && RPP % 8 == 0 && MM_BK == 64, "tile rows must be whole staging passes");
+  extern __shared__ __align__(16) bf16_t lds[];
+  bf16_t* const as_base = lds;                      // [2][BM * MM_LD]
+  bf16_t* const ws_base = lds + 2 * BM * MM_LD;   // [2][BN * MM_LD]
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  // Workgroups go to the eight XCDs in turn by their id, and each XCD has an L2 of its own.  The ids
-  // are therefore dealt out so that an XCD's workgroups are neighbours in tile order: they walk the
-  // column tiles of the same few row tiles, whose activations then come from memory once instead
-  // of once per XCD.
-  int tile_id;
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int row_tiles = (n_rows + BM - 1) / BM, col_tiles = (n_out + BN - 1) / BN;
+  int row_tile, col_tile;
   {
-    const int total = gridDim.x, pid = blockIdx.x;
-    const int per_xcd = (total + 7) >> 3, tall = (total & 7) ? (total & 7) : 8;
-    const int xcd = pid & 7, local = pid >> 3;
-    tile_id = xcd < tall ? xcd * per_xcd + local : tall * per_xcd + (xcd - tall) * (per_xcd - 1) + local;
+    const int id = mfma_xcd_tile_id(blockIdx.x, gridDim.x);
+    const int per_group = MM_GROUP * col_tiles;
+    const int group = id / per_group, in_group = id - group * per_group;
+    const int first = group * MM_GROUP;
+    const int rows_here = row_tiles - first < MM_GROUP ? row_tiles - first : MM_GROUP;
+    row_tile = first + in_group % rows_here;
+    col_tile = in_group / rows_here;
   }
-  const int col_tiles = (n_out + TILE - 1) / TILE;
-  const int row0 = (tile_id / col_tiles) * TILE, col0 = (tile_id % col_tiles) * TILE;
-  const int wr = (wave >> 1) * (WT * 16), wc = (wave & 1) * (WT * 16);  // this wave's quarter
-  const int lrow = lane & 15, lk = (lane >> 4) * 8;
+  const int row0 = row_tile * BM, col0 = col_tile * BN;
+  const int wr = (wave / WVN) * (WTM * 16), wc = (wave % WVN) * (WTN * 16);
+  const int lrow = lane & 15;
 
-  // staging: thread t copies 16 bytes of rows (t / TPR) + RPP * pass, k offset (t % TPR) * 8
   const int srow = tid / TPR, sk = (tid % TPR) * 8;
+  const int s_lds = srow * MM_LD + (((tid % TPR) ^ (srow & 7)) * 8);  // where this thread's chunk goes (RPP % 8 == 0)
   const bf16x8_t zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
-  // PD slices along k are on their way from memory at any time, each in registers of its own: with
-  // few workgroups on a compute unit the latency of a load is what a step costs, and it is paid
-  // once per PD - 1 steps
-  constexpr int PD = WT == 4 ? 2 : 4;
-  bf16x8_t ga[PD][PASSES], gw[PD][PASSES];
-
-  // Rows past the end are read from the last row (their results are never stored), so that a
-  // load's value is used only when the slice is multiplied: a select on it right after the load
-  // would wait for it and leave nothing in flight.  Only a last, partial slice along k needs zeros.
-  const bf16_t* ap[PASSES];
-  const bf16_t* wp[PASSES];
+  // What a thread stages per step: PA chunks of the activations' slice and PW of W's, each 16 bytes.
+  constexpr int ITEMS = PA + PW;
+  bf16x8_t gv[ITEMS];
+  // rows past the end are read from the last row: their results are never stored
+  const bf16_t* gp[ITEMS];
 #pragma unroll
-  for (int p = 0; p < PASSES; ++p) {
-    const int r = srow + p * RPP;
-    const int an = row0 + r < n_rows ? row0 + r : n_rows - 1;
-    const int wo = col0 + r < n_out ? col0 + r : n_out - 1;
-    ap[p] = act + (long)an * lda + sk;
-    wp[p] = w + (long)wo * k_dim + sk;
+  for (int p = 0; p < PA; ++p) {
+    const int r = row0 + srow + p * RPP;
+    gp[p] = act + (long)(r < n_rows ? r : n_rows - 1) * lda + sk;
   }
-  auto load_global = [&](int set, int k0) {
-    if (k0 + MM_BK <= k_dim) {
 #pragma unroll
-      for (int p = 0; p < PASSES; ++p) {
-        ga[set][p] = *reinterpret_cast<const bf16x8_t*>(ap[p] + k0);
-        gw[set][p] = *reinterpret_cast<const bf16x8_t*>(wp[p] + k0);
-      }
-    } else {
-      const bool k_ok = k0 + sk + 8 <= k_dim;
-#pragma unroll
-      for (int p = 0; p < PASSES; ++p) {
-        const bf16x8_t av = *reinterpret_cast<const bf16x8_t*>(ap[p] + (k_ok ? k0 : 0));
-        const bf16x8_t wv = *reinterpret_cast<const bf16x8_t*>(wp[p] + (k_ok ? k0 : 0));
-        ga[set][p] = k_ok ? av : zero8;
-        gw[set][p] = k_ok ? wv : zero8;
-      }
-    }
+  for (int p = 0; p < PW; ++p) {
+    const int r = col0 + srow + p * RPP;
+    gp[PA + p] = w + (long)(r < n_out ? r : n_out - 1) * k_dim + sk;
+  }
+  // A chunk that lies beyond k_dim (in the last, partial step) is read from the row's start instead
+  // and counts as zero when it is stored: the select then waits for no load.
+  auto load_item = [&](int p, int step) {
+    const int k0 = step * MM_BK;
+    gv[p] = *reinterpret_cast<const bf16x8_t*>(gp[p] + (k0 + sk + 8 <= k_dim ? k0 : 0));
   };
-  auto store_lds = [&](int set, int buf) {
-#pragma unroll
-    for (int p = 0; p < PASSES; ++p) {
-      const int r = srow + p * RPP;
-      *reinterpret_cast<bf16x8_t*>(&as[buf][r * MM_LD + sk]) = ga[set][p];
-      *reinterpret_cast<bf16x8_t*>(&ws[buf][r * MM_LD + sk]) = gw[set][p];
-    }
+  auto store_item = [&](int p, int step, int buf) {
+    bf16_t* dst = p < PA ? as_base + buf * (BM * MM_LD) + p * RPP * MM_LD
+                         : ws_base + buf * (BN * MM_LD) + (p - PA) * RPP * MM_LD;
+    *reinterpret_cast<bf16x8_t*>(dst + s_lds) = step * MM_BK + sk + 8 <= k_dim ? gv[p] : zero8;
   };
 
-  f32x4_t acc[WT][WT];  // [column tile of W][row tile of activations]
+  f32x4_t acc[WTN][WTM];  // [column tile of W][row tile of activations]
 #pragma unroll
-  for (int i = 0; i < WT; ++i)
+  for (int i = 0; i < WTN; ++i)
 #pragma unroll
-    for (int j = 0; j < WT; ++j) acc[i][j] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+    for (int j = 0; j < WTM; ++j) acc[i][j] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
 
   const int k_steps = (k_dim + MM_BK - 1) / MM_BK;
+  const int c0 = ((lane >> 4) ^ (lrow & 7)) * 8;  // this lane's chunk of an operand row, first half of a step
+
+  // One step along k.  Its 2 * WTM groups of MFMAs (one row tile of the activations against the
+  // wave's WTN column tiles, for one half of the step) read their operands from LDS two groups
+  // ahead of their use, so that a read's latency hides behind the MFMAs of the groups before it.
+  // Spread between the groups, the thread puts the next step's chunks (loaded during the step
+  // before this one) into the other LDS buffer and sends for those of the step after: LDS takes
+  // writes at half the rate of reads, and all at once they would hold every wave up.
+  auto k_step = [&](int s, auto store_next, auto load_after) {
+    const int buf = s & 1;
+    const bf16_t* as = as_base + buf * (BM * MM_LD) + (wr + lrow) * MM_LD;
+    const bf16_t* ws = ws_base + buf * (BN * MM_LD) + (wc + lrow) * MM_LD;
+    constexpr int GROUPS = (MM_BK / 32) * WTM;
+    bf16x8_t wf[MM_BK / 32][WTN], af[3];
+    // the second half's chunk is 4 further, which the swizzle turns into a flip of bit 5 of the offset
+    auto read_a = [&](int g) {
+      return *reinterpret_cast<const bf16x8_t*>(as + (g % WTM) * 16 * MM_LD + (c0 ^ ((g / WTM) * 32)));
+    };
 #pragma unroll
-  for (int d = 0; d < PD; ++d)
-    if (d < k_steps) load_global(d, d * MM_BK);
-  store_lds(0, 0);
-  __syncthreads();
-  for (int s0 = 0; s0 < k_steps; s0 += PD) {
+    for (int i = 0; i < WTN; ++i) wf[0][i] = *reinterpret_cast<const bf16x8_t*>(ws + i * 16 * MM_LD + c0);
+    if (WTM == 1) {  // the second half's groups start at once
 #pragma unroll
-    for (int d = 0; d < PD; ++d) {
-      const int s = s0 + d;  // this step's slice sat in register set d and is in LDS buffer s & 1 now
-      if (s < k_steps) {
-        const int buf = s & 1;
-        if (s + PD < k_steps) load_global(d, (s + PD) * MM_BK);
-#pragma unroll
-        for (int kk = 0; kk < MM_BK; kk += 32) {
-          bf16x8_t wf[WT], af[WT];
-#pragma unroll
-          for (int i = 0; i < WT; ++i) {
-            wf[i] = *reinterpret_cast<const bf16x8_t*>(&ws[buf][(wc + i * 16 + lrow) * MM_LD + kk + lk]);
-            af[i] = *reinterpret_cast<const bf16x8_t*>(&as[buf][(wr + i * 16 + lrow) * MM_LD + kk + lk]);
-          }
-#pragma unroll
-          for (int i = 0; i < WT; ++i)
-#pragma unroll
-            for (int j = 0; j < WT; ++j)
-              acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[i], af[j], acc[i][j], 0, 0, 0);
-        }
-        if (s + 1 < k_steps) {
-          store_lds((d + 1) % PD, buf ^ 1);  // the other buffer: its readers finished before the last barrier
-          __syncthreads();
-        }
-      }
+      for (int i = 0; i < WTN; ++i) wf[1][i] = *reinterpret_cast<const bf16x8_t*>(ws + i * 16 * MM_LD + (c0 ^ 32));
     }
+    af[0] = read_a(0);
+    af[1] = read_a(1);
+#pragma unroll
+    for (int g = 0; g < GROUPS; ++g) {
+      if (g + 2 < GROUPS) af[(g + 2) % 3] = read_a(g + 2);
+      if (WTM >= 2 && g % WTM == WTM - 2 && g / WTM + 1 < MM_BK / 32) {
+#pragma unroll
+        for (int i = 0; i < WTN; ++i)
+          wf[g / WTM + 1][i] = *reinterpret_cast<const bf16x8_t*>(ws + i * 16 * MM_LD + (c0 ^ ((g / WTM + 1) * 32)));
+      }
+#pragma unroll
+      for (int p = g * ITEMS / GROUPS; p < (g + 1) * ITEMS / GROUPS; ++p) {
+        if (decltype(store_next)::value) store_item(p, s + 1, buf ^ 1);
+        if (decltype(load_after)::value) load_item(p, s + 2);
+      }
+      // the compiler's scheduler would move each read down to its use again
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int i = 0; i < WTN; ++i)
+        acc[i][g % WTM] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[g / WTM][i], af[g % 3], acc[i][g % WTM], 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    if (decltype(store_next)::value) __syncthreads();  // the other buffer's readers finished before the last barrier
+  };
+  using yes = std::integral_constant<bool, true>;
+  using no = std::integral_constant<bool, false>;
+
+#pragma unroll
+  for (int p = 0; p < ITEMS; ++p) load_item(p, 0);
+#pragma unroll
+  for (int p = 0; p < ITEMS; ++p) store_item(p, 0, 0);
+  if (k_steps > 1) {
+#pragma unroll
+    for (int p = 0; p < ITEMS; ++p) load_item(p, 1);
   }
+  __syncthreads();
+  int s = 0;
+  for (; s + 2 < k_steps; ++s) k_step(s, yes{}, yes{});
+  if (s + 1 < k_steps) k_step(s++, yes{}, no{});
+  k_step(s, no{}, no{});
 
   // lane holds out[row0 + wr + j*16 + (lane & 15)][col0 + wc + i*16 + (lane >> 4)*4 + e], e = 0..3
-  const bool vec = (n_out & 3) == 0 && (ldo & 3) == 0 &&
-                   (((size_t)out | (size_t)bias) & 15) == 0;  // the four columns as one aligned vector
+  const bool vec = (n_out & 3) == 0 && (ldo & 3) == 0 && (((size_t)out | (size_t)bias) & 15) == 0;
 #pragma unroll
-  for (int i = 0; i < WT; ++i) {
+  for (int i = 0; i < WTN; ++i) {
     const int oc = col0 + wc + i * 16 + (lane >> 4) * 4;
     if (oc >= n_out) continue;
-    float b4[4] = {0.f, 0.f, 0.f, 0.f};
-    if (bias) {
-      if (vec) {
-        const float4 t = *reinterpret_cast<const float4*>(bias + oc);
-        b4[0] = t.x; b4[1] = t.y; b4[2] = t.z; b4[3] = t.w;
-      } else {
+    float b4[4];
+    mfma_bias4(bias, oc, n_out, vec, b4);
 #pragma unroll
-        for (int e = 0; e < 4; ++e) b4[e] = oc + e < n_out ? bias[oc + e] : 0.f;
-      }
-    }
-#pragma unroll
-    for (int j = 0; j < WT; ++j) {
+    for (int j = 0; j < WTM; ++j) {
       const int n = row0 + wr + j * 16 + lrow;
       if (n >= n_rows) continue;
-      OT* orow = out + (long)n * ldo;
-      float v[4];
-#pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        v[e] = acc[i][j][e] + b4[e];
-        if (EPI == MM_EPI_GELU) v[e] = gelu_tanh_fast(v[e]);
-      }
-      if (vec && sizeof(OT) == 4) {
-        float4* dst = reinterpret_cast<float4*>(orow + oc);
-        if (EPI == MM_EPI_RESIDUAL) {
-          const float4 old = *dst;
-          *dst = make_float4(old.x + v[0], old.y + v[1], old.z + v[2], old.w + v[3]);
-        } else {
-          *dst = make_float4(v[0], v[1], v[2], v[3]);
-        }
-      } else if (vec && EPI != MM_EPI_RESIDUAL) {
-        uint2 pk;
-        pk.x = pack_bf16x2(v[0], v[1]);
-        pk.y = pack_bf16x2(v[2], v[3]);
-        *reinterpret_cast<uint2*>(orow + oc) = pk;
-        if (EPI == MM_EPI_QKV && oc >= sc.q_width) {
-          // the four columns lie in one head (the launcher checks that sizes are multiples of 4)
-          const int slot = sc.slot_mapping[n];
-          if (slot >= 0) {
-            const long page = slot / sc.page_size;
-            const int off = slot - (int)page * sc.page_size;
-            const int c = oc - sc.q_width;  // column among keys then values
-            const bool is_v = c >= sc.kv_width;
-            const int cc = is_v ? c - sc.kv_width : c;
-            const int h = cc / sc.head_dim, d = cc - h * sc.head_dim;
-            const long dst = ((page * sc.n_kv_head + h) * sc.page_size + off) * (long)sc.head_dim + d;
-            *reinterpret_cast<uint2*>((is_v ? sc.vpool : sc.kpool) + dst) = pk;
-          }
-        }
-      } else {
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          const int o = oc + e;
-          if (o >= n_out) continue;
-          if (EPI == MM_EPI_RESIDUAL) {
-            orow[o] = from_float<OT>(to_float<OT>(orow[o]) + v[e]);
-          } else {
-            orow[o] = from_float<OT>(v[e]);
-          }
-        }
-      }
+      mfma_store4<EPI, OT>(acc[i][j], b4, out, ldo, n, oc, n_out, vec, sc);
     }
   }
 }
 
-template <int WT>
-static int launch_tile(const void* act, long lda, const void* w, const float* bias, void* out, int out_dtype,
-                       long ldo, int n_rows, int n_out, int k_dim, int epilogue, const MfmaScatter& sc,
-                       hipStream_t stream) {
-  constexpr int TILE = 2 * WT * 16;
-  const long tiles = (long)((n_out + TILE - 1) / TILE) * ((n_rows + TILE - 1) / TILE);
+template <int WTM, int WTN, int WVM, int WVN, int EPI, typename OT>
+int launch_one(const void* act, long lda, const void* w, const float* bias, void* out, long ldo, int n_rows,
+               int n_out, int k_dim, const MfmaScatter& sc, hipStream_t stream) {
+  constexpr int BM = WVM * WTM * 16, BN = WVN * WTN * 16;
+  constexpr size_t lds_bytes = 2ul * (BM + BN) * MM_LD * sizeof(bf16_t);
+  auto kernel = linear_mfma_kernel<WTM, WTN, WVM, WVN, EPI, OT>;
+  static bool allowed = false;  // more LDS than a kernel gets without asking
+  if (!allowed) {
+    const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+    if (e != hipSuccess) return (int)e;
+    allowed = true;
+  }
+  const long tiles = (long)((n_rows + BM - 1) / BM) * ((n_out + BN - 1) / BN);
   if (tiles > 0x7fffffffL) return MGPT_ERR_TOO_LARGE;
-  dim3 grid((unsigned int)tiles), block(256);
-#define MM_LAUNCH(E, OT)                                                                               \
-  hipLaunchKernelGGL((linear_mfma_kernel<WT, E, OT>), grid, block, 0, stream, (const bf16_t*)act, lda, \
-                     (const bf16_t*)w, bias, (OT*)out, ldo, n_rows, n_out, k_dim, sc)
-  if (epilogue == MM_EPI_NONE && out_dtype == MGPT_BF16) MM_LAUNCH(MM_EPI_NONE, bf16_t);
-  else if (epilogue == MM_EPI_NONE && out_dtype == MGPT_F32) MM_LAUNCH(MM_EPI_NONE, float);
-  else if (epilogue == MM_EPI_GELU && out_dtype == MGPT_BF16) MM_LAUNCH(MM_EPI_GELU, bf16_t);
-  else if (epilogue == MM_EPI_RESIDUAL && out_dtype == MGPT_F32) MM_LAUNCH(MM_EPI_RESIDUAL, float);
-  else if (epilogue == MM_EPI_QKV && out_dtype == MGPT_BF16) MM_LAUNCH(MM_EPI_QKV, bf16_t);
-  else return MGPT_ERR_BAD_DTYPE;
-#undef MM_LAUNCH
+  hipLaunchKernelGGL(kernel, dim3((unsigned int)tiles), dim3(64 * WVM * WVN), lds_bytes, stream,
+                     (const bf16_t*)act, lda, (const bf16_t*)w, bias, (OT*)out, ldo, n_rows, n_out, k_dim, sc);
   return mgpt_last_error();
 }
 
-// act: [n_rows, k_dim] bfloat16 with row stride lda (a multiple of 8, 16-byte aligned base);
-// w: [n_out, k_dim] dense bfloat16; out: [n_rows, n_out] with row stride ldo.  k_dim must be a
-// multiple of 16.  Refuses other layouts with MGPT_ERR_BAD_SHAPE.
-static int linear_mfma_any(const void* act, long lda, const void* w, const float* bias, void* out,
-                           int out_dtype, long ldo, int n_rows, int n_out, int k_dim, int epilogue,
-                           const MfmaScatter& sc, hipStream_t stream) {
+template <int WTM, int WTN, int WVM, int WVN>
+int launch_shape(const void* act, long lda, const void* w, const float* bias, void* out, int out_dtype, long ldo,
+                 int n_rows, int n_out, int k_dim, int epilogue, const MfmaScatter& sc, hipStream_t stream) {
+#define MM_LAUNCH(E, OT) \
+  return launch_one<WTM, WTN, WVM, WVN, E, OT>(act, lda, w, bias, out, ldo, n_rows, n_out, k_dim, sc, stream)
+  if (epilogue == MM_EPI_NONE && out_dtype == MGPT_BF16) MM_LAUNCH(MM_EPI_NONE, bf16_t);
+  if (epilogue == MM_EPI_NONE && out_dtype == MGPT_F32) MM_LAUNCH(MM_EPI_NONE, float);
+  if (epilogue == MM_EPI_GELU && out_dtype == MGPT_BF16) MM_LAUNCH(MM_EPI_GELU, bf16_t);
+  if (epilogue == MM_EPI_RESIDUAL && out_dtype == MGPT_F32) MM_LAUNCH(MM_EPI_RESIDUAL, float);
+  if (epilogue == MM_EPI_QKV && out_dtype == MGPT_BF16) MM_LAUNCH(MM_EPI_QKV, bf16_t);
+#undef MM_LAUNCH
+  return MGPT_ERR_BAD_DTYPE;
+}
+
+// Tile shapes, largest first: rows x columns of a workgroup's tile, and how many workgroups of it
+// a compute unit holds at a time.
+constexpr int MM_SHAPES = 5;
+constexpr int MM_TILE_ROWS[MM_SHAPES] = {256, 128, 128, 64, 32};
+constexpr int MM_TILE_COLS[MM_SHAPES] = {256, 256, 64, 64, 32};
+
+long tiles_of(int shape, int n_rows, int n_out) {
+  return (long)((n_rows + MM_TILE_ROWS[shape] - 1) / MM_TILE_ROWS[shape]) *
+         ((n_out + MM_TILE_COLS[shape] - 1) / MM_TILE_COLS[shape]);
+}
+
+// The largest tile that still fills the machine's 256 compute units.  The two largest shapes run
+// one workgroup per unit, so what counts for them is also how full their last round is.
+int choose_shape(int n_rows, int n_out) {
+  for (int shape = 0; shape < 2; ++shape) {
+    const long t = tiles_of(shape, n_rows, n_out);
+    const long rounds = (t + 255) / 256;
+    if (t >= (shape == 0 ? 160 : 140) && 10 * t >= 7 * rounds * 256) return shape;
+  }
+  if (tiles_of(2, n_rows, n_out) >= 300) return 2;
+  if (tiles_of(3, n_rows, n_out) >= 192) return 3;
+  return 4;
+}
+
+int launch_any(int shape, const void* act, long lda, const void* w, const float* bias, void* out, int out_dtype,
+               long ldo, int n_rows, int n_out, int k_dim, int epilogue, const MfmaScatter& sc, hipStream_t stream) {
   if (n_rows == 0 || n_out == 0) return MGPT_OK;
   if (!act || !w || !out) return MGPT_ERR_NULL;
   if (n_rows < 0 || n_out < 0 || k_dim <= 0 || (k_dim % 16) != 0 || lda < k_dim || (lda % 8) != 0 ||
       ldo < n_out)
     return MGPT_ERR_BAD_SHAPE;
-  // large tiles reuse operands better, small tiles fill the 256 compute units: take the large
-  // ones only when they alone give every unit several workgroups
-  const long big = (long)((n_out + 127) / 128) * ((n_rows + 127) / 128);
-  if (big >= 384)
-    return launch_tile<4>(act, lda, w, bias, out, out_dtype, ldo, n_rows, n_out, k_dim, epilogue, sc, stream);
-  // and tiles of 32 x 32 where the 64 x 64 ones would leave most of the units idle (a prompt
-  // portion of a few hundred tokens)
-  const long mid = (long)((n_out + 63) / 64) * ((n_rows + 63) / 64);
-  if (mid < 192)
-    return launch_tile<1>(act, lda, w, bias, out, out_dtype, ldo, n_rows, n_out, k_dim, epilogue, sc, stream);
-  return launch_tile<2>(act, lda, w, bias, out, out_dtype, ldo, n_rows, n_out, k_dim, epilogue, sc, stream);
+  if (shape < 0) shape = choose_shape(n_rows, n_out);
+#define MM_ARGS act, lda, w, bias, out, out_dtype, ldo, n_rows, n_out, k_dim, epilogue, sc, stream
+  switch (shape) {
+    case 0: return launch_shape<8, 4, 2, 4>(MM_ARGS);  // 256 x 256, eight waves of 128 x 64
+    case 1: return launch_shape<4, 4, 2, 4>(MM_ARGS);  // 128 x 256, eight waves of 64 x 64
+    case 2: return launch_shape<4, 2, 2, 2>(MM_ARGS);  // 128 x 64, four waves of 64 x 32
+    case 3: return launch_shape<2, 2, 2, 2>(MM_ARGS);  // 64 x 64, four waves of 32 x 32
+    case 4: return launch_shape<1, 1, 2, 2>(MM_ARGS);  // 32 x 32, four waves of 16 x 16
+  }
+#undef MM_ARGS
+  return MGPT_ERR_BAD_SHAPE;
 }
 
+}  // namespace
+
+// act: [n_rows, k_dim] bfloat16 with row stride lda (a multiple of 8, 16-byte aligned base);
+// w: [n_out, k_dim] dense bfloat16; out: [n_rows, n_out] with row stride ldo.  k_dim must be a
+// multiple of 16.  Refuses other layouts with MGPT_ERR_BAD_SHAPE.
 extern "C" int mgpt_linear_mfma(const void* act, long lda, const void* w, const float* bias, void* out,
                                 int out_dtype, long ldo, int n_rows, int n_out, int k_dim, int epilogue,
                                 hipStream_t stream) {
   if (epilogue == MM_EPI_QKV) return MGPT_ERR_BAD_SHAPE;  // mgpt_linear_mfma_qkv brings the pools
   MfmaScatter sc = {};
-  return linear_mfma_any(act, lda, w, bias, out, out_dtype, ldo, n_rows, n_out, k_dim, epilogue, sc, stream);
+  return launch_any(-1, act, lda, w, bias, out, out_dtype, ldo, n_rows, n_out, k_dim, epilogue, sc, stream);
+}
+
+// The same product with the tile shape given (0 = 256 x 256, 1 = 128 x 256, 2 = 128 x 64,
+// 3 = 64 x 64, 4 = 32 x 32) instead of chosen by the size: for tests and measurements of each shape.
+extern "C" int mgpt_linear_mfma_shape(int shape, const void* act, long lda, const void* w, const float* bias,
+                                      void* out, int out_dtype, long ldo, int n_rows, int n_out, int k_dim,
+                                      int epilogue, hipStream_t stream) {
+  if (epilogue == MM_EPI_QKV || shape < 0 || shape >= MM_SHAPES) return MGPT_ERR_BAD_SHAPE;
+  MfmaScatter sc = {};
+  return launch_any(shape, act, lda, w, bias, out, out_dtype, ldo, n_rows, n_out, k_dim, epilogue, sc, stream);
 }
 
 // The fused QKV product of a step with prompt portions: out[n] = act[n] W^T + bias in bfloat16, and
 // the key and value columns (after the first q_width) of every row with a slot also go into the
 // cache pools [pages, n_kv_head, page_size, head_dim].  Refuses (MGPT_ERR_BAD_SHAPE) sizes that
-// are no multiples of 4 and outputs that are not aligned for 8-byte stores.
+// are no multiples of 4 and outputs that are not aligned for 8-byte stores.  shape: as for
+// mgpt_linear_mfma_shape, or negative to have it chosen.
 extern "C" int mgpt_linear_mfma_qkv(const void* act, long lda, const void* w, const float* bias, void* out,
                                     long ldo, int n_rows, int n_out, int k_dim, void* kpool, void* vpool,
                                     const int* slot_mapping, int q_width, int kv_width, int head_dim,
-                                    int n_kv_head, int page_size, hipStream_t stream) {
+                                    int n_kv_head, int page_size, int shape, hipStream_t stream) {
   if (!kpool || !vpool || !slot_mapping) return MGPT_ERR_NULL;
   if (head_dim <= 0 || (head_dim % 4) != 0 || (q_width % 4) != 0 || q_width + 2 * kv_width != n_out ||
       kv_width != n_kv_head * head_dim || page_size <= 0 || (n_out % 4) != 0 || (ldo % 4) != 0 ||
-      (((size_t)out | (size_t)bias) & 15) != 0)
+      (((size_t)out | (size_t)bias) & 15) != 0 || shape >= MM_SHAPES)
     return MGPT_ERR_BAD_SHAPE;
   MfmaScatter sc = {(bf16_t*)kpool, (bf16_t*)vpool, slot_mapping, q_width, kv_width, head_dim, n_kv_head, page_size};
-  return linear_mfma_any(act, lda, w, bias, out, MGPT_BF16, ldo, n_rows, n_out, k_dim, MM_EPI_QKV, sc, stream);
+  return launch_any(shape, act, lda, w, bias, out, MGPT_BF16, ldo, n_rows, n_out, k_dim, MM_EPI_QKV, sc, stream);
 }

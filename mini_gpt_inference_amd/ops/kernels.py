@@ -438,10 +438,11 @@ def paged_attention_decode_bf16(q: torch.Tensor, out: torch.Tensor, k_pool: torc
 
 
 def linear_mfma(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor,
-                n_rows: int, epilogue: int, scatter=None) -> bool:
+                n_rows: int, epilogue: int, scatter=None, shape: Optional[int] = None) -> bool:
     """Tiled bfloat16 MFMA product for many rows.  scatter = (k_pool, v_pool, slot_mapping, q_width,
     kv_width) also stores the new keys and values into their pages (bfloat16 output, no other
-    epilogue).  False when it does not take the shape."""
+    epilogue).  `shape` (0 = 256 x 256 tiles, 1 = 128 x 256, 2 = 128 x 64, 3 = 64 x 64, 4 = 32 x 32) fixes the
+    tile shape that the library otherwise chooses by the size.  False when it does not take the shape."""
     if a.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
         return False
     n_out, k_dim = w.shape
@@ -469,11 +470,15 @@ def linear_mfma(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], 
         _need_i32("slot_mapping", sm, n_rows)
         rc = library.kernels().mgpt_linear_mfma_qkv(
             _ptr(a), a.stride(0), _ptr(w), _ptr(bias), _ptr(out), out.stride(0), n_rows, n_out, k_dim, _ptr(kp),
-            _ptr(vp), _ptr(sm), q_width, kv_width, head_dim, n_kv_head, page_size, _stream())
+            _ptr(vp), _ptr(sm), q_width, kv_width, head_dim, n_kv_head, page_size, -1 if shape is None else int(shape),
+            _stream())
     else:
-        rc = library.kernels().mgpt_linear_mfma(_ptr(a), a.stride(0), _ptr(w), _ptr(bias), _ptr(out),
-                                                _dtype_code(out), out.stride(0), n_rows, n_out, k_dim, epilogue,
-                                                _stream())
+        args = (_ptr(a), a.stride(0), _ptr(w), _ptr(bias), _ptr(out), _dtype_code(out), out.stride(0), n_rows,
+                n_out, k_dim, epilogue, _stream())
+        if shape is None:
+            rc = library.kernels().mgpt_linear_mfma(*args)
+        else:
+            rc = library.kernels().mgpt_linear_mfma_shape(int(shape), *args)
     if rc == -2:
         return False
     _check(rc, "linear_mfma")

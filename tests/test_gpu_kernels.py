@@ -135,6 +135,34 @@ def test_linear_mfma(n, k, o, epi, o_dt):
     helpers.assert_close(out2[:n - 3], _linear_want(a, w, None, epi, prev)[:n - 3], "bfloat16", "mfma partial rows")
 
 
+@pytest.mark.parametrize("n,k,o", [(300, 80, 257), (513, 512, 520), (256, 2048, 256), (1000, 48, 130), (70, 64, 1030)])
+@pytest.mark.parametrize("epi,o_dt", [(kernels.EPI_NONE, "bfloat16"), (kernels.EPI_NONE, "float32"),
+                                      (kernels.EPI_GELU, "bfloat16"), (kernels.EPI_RESIDUAL, "float32")])
+@pytest.mark.parametrize("shape", [0, 1, 2, 3, 4])
+def test_linear_mfma_each_tile_shape(n, k, o, epi, o_dt, shape):
+    """Each tile shape forced at sizes that cut its tiles everywhere: rows and columns past the end, an
+    inner size that ends inside a step, several tiles each way."""
+    g = torch.Generator().manual_seed(16)
+    a, w, bias = rnd(g, n, k, dtype="bfloat16"), rnd(g, o, k, dtype="bfloat16", scale=k ** -0.5), rnd(g, o)
+    prev = rnd(g, n + 2, o, dtype=o_dt)
+    out = prev.clone().to(DEV)
+    assert kernels.linear_mfma(a.to(DEV), w.to(DEV), bias.to(DEV), out, n, epi, shape=shape)
+    helpers.assert_close(out[:n], _linear_want(a, w, bias, epi, prev[:n]), "bfloat16", f"shape {shape} {n}x{k}x{o}")
+    assert torch.equal(out[n:], prev[n:].to(DEV)), "rows beyond n_rows were written"
+
+
+def test_linear_mfma_chooses_the_largest_tiles_for_a_large_problem():
+    """160 tiles of 256 x 256: the library takes that shape by itself, so the result equals the forced one bit by bit."""
+    g = torch.Generator().manual_seed(17)
+    n, k, o = 4096, 320, 2560
+    a, w, bias = rnd(g, n, k, dtype="bfloat16"), rnd(g, o, k, dtype="bfloat16", scale=k ** -0.5), rnd(g, o)
+    out, out_w = (torch.empty(n, o, dtype=torch.bfloat16, device=DEV) for _ in range(2))
+    assert kernels.linear_mfma(a.to(DEV), w.to(DEV), bias.to(DEV), out, n, kernels.EPI_GELU)
+    assert kernels.linear_mfma(a.to(DEV), w.to(DEV), bias.to(DEV), out_w, n, kernels.EPI_GELU, shape=0)
+    assert torch.equal(out, out_w)
+    helpers.assert_close(out, _linear_want(a, w, bias, kernels.EPI_GELU, None), "bfloat16", "large")
+
+
 @pytest.mark.parametrize("general", [False, True])
 @pytest.mark.parametrize("n,k,o,ln_bias,gather", [(8, 512, 1536, True, False), (3, 96, 503, False, True),
                                                   (40, 80, 257, True, True), (64, 2048, 64, False, False), (64, 512, 2048, True, False), (33, 768, 96, True, True),
@@ -220,10 +248,10 @@ def test_linear_skinny_with_the_inner_size_split_over_workgroups(n, k, o, epi, o
     helpers.assert_close(out2[:n], _linear_want(a, w, bias, epi, prev)[:n], "bfloat16", "unsplit")
 
 
-@pytest.mark.parametrize("n", [70, 300, 1100])
-def test_linear_mfma_stores_keys_and_values(n):
-    """The tiled kernel's fused QKV product: all three tile sizes; groups of heads; padded rows (slot -1)
-    leave the pools alone."""
+@pytest.mark.parametrize("n,shape", [(70, None), (300, 3), (1100, 2), (300, 1), (520, 0)])
+def test_linear_mfma_stores_keys_and_values(n, shape):
+    """The tiled kernel's fused QKV product: the tile shape chosen by the size and each larger one forced;
+    groups of heads; padded rows (slot -1) leave the pools alone."""
     g = torch.Generator().manual_seed(15)
     k, h, hk, d, page = 96, 6, 2, 16, 8
     pages = n // page + 3
@@ -236,7 +264,7 @@ def test_linear_mfma_stores_keys_and_values(n):
         slots[t] = -1
     out = torch.empty(n, qw + 2 * kvw, dtype=torch.bfloat16, device=DEV)
     assert kernels.linear_mfma(a.to(DEV), w.to(DEV), bias.to(DEV), out, n, kernels.EPI_NONE,
-                               scatter=(kp, vp, i32(slots), qw, kvw))
+                               scatter=(kp, vp, i32(slots), qw, kvw), shape=shape)
     want = P.plain_linear(a.double(), w.double(), bias.double())
     helpers.assert_close(out, want, "bfloat16", "qkv")
     kflat = kp.float().cpu().permute(0, 2, 1, 3).reshape(pages * page, kvw)
