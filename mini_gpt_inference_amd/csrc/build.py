@@ -27,6 +27,9 @@ HIP_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
     # keep hipcc from forming packed 32-bit float instructions
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    # MFMA results in ordinary registers: left to itself the compiler puts them into the
+    # accumulation registers and copies each one out again for the arithmetic that follows
+    "-mllvm", "-amdgpu-mfma-vgpr-form=1",
 ]
 
 
