@@ -115,7 +115,8 @@ __global__ void layernorm_kernel(const float* __restrict__ x, const float* __res
 
 // The same for widths that are multiples of 4 up to 64 * 4 * LN_VEC with 16-byte aligned rows: every
 // lane loads and stores vectors of four (a row of 512 is two loads per lane instead of eight).
-// LN_VEC is 4 for rows up to 1024 wide and 8 for rows up to 2048.
+// LN_VEC is the number of such vectors a lane holds: the row's width / 256, rounded up to one of
+// 1, 2, 3, 4, 6, 8 (rows up to 2048 wide), so that a row of 512 costs two loads and not four.
 template <typename OT, int LN_VEC>
 __global__ void layernorm_vec_kernel(const float* __restrict__ x, const float* __restrict__ w,
                                      const float* __restrict__ b, OT* __restrict__ out,
@@ -189,13 +190,21 @@ extern "C" int mgpt_layernorm(const float* x, const float* w, const float* b, vo
   dim3 grid((n_rows + rows_per_block - 1) / rows_per_block), block(rows_per_block * MGPT_WAVE);
   const bool vec = (width % 4) == 0 && width <= MGPT_WAVE * 4 * 8 &&
                    ((((size_t)x) | ((size_t)w) | ((size_t)b) | ((size_t)out)) & 15) == 0;
-  const bool narrow = width <= MGPT_WAVE * 4 * 4;
+  const int need = (width / 4 + MGPT_WAVE - 1) / MGPT_WAVE;   // vectors of four per lane
 #define LN_LAUNCH(OT, V) \
   hipLaunchKernelGGL((layernorm_vec_kernel<OT, V>), grid, block, 0, stream, x, w, b, (OT*)out, rows, n_rows, width, eps)
+#define LN_PICK(OT)                    \
+  if (need <= 1) LN_LAUNCH(OT, 1);     \
+  else if (need <= 2) LN_LAUNCH(OT, 2); \
+  else if (need <= 3) LN_LAUNCH(OT, 3); \
+  else if (need <= 4) LN_LAUNCH(OT, 4); \
+  else if (need <= 6) LN_LAUNCH(OT, 6); \
+  else LN_LAUNCH(OT, 8)
   if (vec && out_dtype == MGPT_F32) {
-    if (narrow) LN_LAUNCH(float, 4); else LN_LAUNCH(float, 8);
+    LN_PICK(float);
   } else if (vec && out_dtype == MGPT_BF16) {
-    if (narrow) LN_LAUNCH(bf16_t, 4); else LN_LAUNCH(bf16_t, 8);
+    LN_PICK(bf16_t);
+#undef LN_PICK
 #undef LN_LAUNCH
   } else if (out_dtype == MGPT_F32) {
     hipLaunchKernelGGL(layernorm_kernel<float>, grid, block, 0, stream, x, w, b, (float*)out, rows,

@@ -58,11 +58,12 @@ __device__ __forceinline__ void mfma_bias4(const float* __restrict__ bias, int o
 }
 
 // Stores the four columns oc..oc+3 of row n: bias, activation, then a plain store, an add into
-// the residual stream, or a store that also puts key and value columns into their cache pages.
+// the residual stream, or a store that also puts the four values at cache_dst (a key's or value's
+// place in its cache page; null for query columns and rows without a slot).
 // `vec`: the four columns can go as one aligned vector.
 template <int EPI, typename OT>
 __device__ __forceinline__ void mfma_store4(const f32x4_t& a, const float b4[4], OT* __restrict__ out, long ldo,
-                                            int n, int oc, int n_out, bool vec, const MfmaScatter& sc) {
+                                            int n, int oc, int n_out, bool vec, bf16_t* cache_dst) {
   OT* orow = out + (long)n * ldo;
   float v[4];
 #pragma unroll
@@ -83,20 +84,8 @@ __device__ __forceinline__ void mfma_store4(const f32x4_t& a, const float b4[4],
     pk.x = pack_bf16x2(v[0], v[1]);
     pk.y = pack_bf16x2(v[2], v[3]);
     *reinterpret_cast<uint2*>(orow + oc) = pk;
-    if (EPI == MM_EPI_QKV && oc >= sc.q_width) {
-      // the four columns lie in one head (the launcher checks that sizes are multiples of 4)
-      const int slot = sc.slot_mapping[n];
-      if (slot >= 0) {
-        const long page = slot / sc.page_size;
-        const int off = slot - (int)page * sc.page_size;
-        const int c = oc - sc.q_width;  // column among keys then values
-        const bool is_v = c >= sc.kv_width;
-        const int cc = is_v ? c - sc.kv_width : c;
-        const int h = cc / sc.head_dim, d = cc - h * sc.head_dim;
-        const long dst = ((page * sc.n_kv_head + h) * sc.page_size + off) * (long)sc.head_dim + d;
-        *reinterpret_cast<uint2*>((is_v ? sc.vpool : sc.kpool) + dst) = pk;
-      }
-    }
+    // the four columns lie in one head (the launcher checks that sizes are multiples of 4)
+    if (EPI == MM_EPI_QKV && cache_dst) *reinterpret_cast<uint2*>(cache_dst) = pk;
   } else {
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
@@ -262,17 +251,40 @@ __global__ __launch_bounds__(64 * WVM * WVN) void linear_mfma_kernel(
 
   // lane holds out[row0 + wr + j*16 + (lane & 15)][col0 + wc + i*16 + (lane >> 4)*4 + e], e = 0..3
   const bool vec = (n_out & 3) == 0 && (ldo & 3) == 0 && (((size_t)out | (size_t)bias) & 15) == 0;
+  // A key or value at (row n, column c of head hh, channel d) goes to
+  // ((page * n_kv_head + hh) * page_size + offset) * head_dim + d of its pool, page and offset from
+  // the row's slot: the row's part and the column's part of that are worked out once each.
+  long cache_row[WTM];
+  if (EPI == MM_EPI_QKV) {
+#pragma unroll
+    for (int j = 0; j < WTM; ++j) {
+      const int n = row0 + wr + j * 16 + lrow;
+      const int slot = n < n_rows ? sc.slot_mapping[n] : -1;
+      const int page = slot / sc.page_size, off = slot - page * sc.page_size;
+      cache_row[j] = slot < 0 ? -1 : ((long)page * sc.n_kv_head * sc.page_size + off) * sc.head_dim;
+    }
+  }
 #pragma unroll
   for (int i = 0; i < WTN; ++i) {
     const int oc = col0 + wc + i * 16 + (lane >> 4) * 4;
     if (oc >= n_out) continue;
     float b4[4];
     mfma_bias4(bias, oc, n_out, vec, b4);
+    bf16_t* cache_col = nullptr;
+    if (EPI == MM_EPI_QKV && oc >= sc.q_width) {
+      const int c = oc - sc.q_width;  // column among keys then values
+      const bool is_v = c >= sc.kv_width;
+      const int cc = is_v ? c - sc.kv_width : c;
+      const int hh = cc / sc.head_dim, d = cc - hh * sc.head_dim;
+      cache_col = (is_v ? sc.vpool : sc.kpool) + (long)hh * sc.page_size * sc.head_dim + d;
+    }
 #pragma unroll
     for (int j = 0; j < WTM; ++j) {
       const int n = row0 + wr + j * 16 + lrow;
       if (n >= n_rows) continue;
-      mfma_store4<EPI, OT>(acc[i][j], b4, out, ldo, n, oc, n_out, vec, sc);
+      bf16_t* cache_dst = nullptr;
+      if (EPI == MM_EPI_QKV && cache_col && cache_row[j] >= 0) cache_dst = cache_col + cache_row[j];
+      mfma_store4<EPI, OT>(acc[i][j], b4, out, ldo, n, oc, n_out, vec, cache_dst);
     }
   }
 }

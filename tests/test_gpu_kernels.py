@@ -40,7 +40,9 @@ def test_embed(dtype, with_pos):
 
 @pytest.mark.parametrize("out_dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("width,bias,eps", [(80, True, 1e-5), (1000, False, 1e-2), (48, True, 1e-6), (75, True, 1e-5),
-                                            (1030, False, 1e-5), (1600, True, 1e-5), (512, True, 1e-5), (2052, True, 1e-5)])
+                                            (1030, False, 1e-5), (1600, True, 1e-5), (512, True, 1e-5), (2052, True, 1e-5),
+                                            (256, True, 1e-5), (768, False, 1e-5), (1024, True, 1e-5), (1280, True, 1e-5),
+                                            (2048, False, 1e-5)])
 def test_layer_norm(out_dtype, width, bias, eps):
     g = torch.Generator().manual_seed(1)
     x = rnd(g, 9, width, scale=3.0) + 2.0
