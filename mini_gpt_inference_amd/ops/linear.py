@@ -72,7 +72,7 @@ def linear(ctx, a: Union[torch.Tensor, LazyNorm], w: torch.Tensor, bias: Optiona
            out: torch.Tensor, n_rows: int, epilogue: int = kernels.EPI_NONE, scatter=None) -> bool:
     """out[:n_rows] = a[:n_rows] @ w.T (+ bias) with the epilogue.
 
-    On the bfloat16 path up to 64 rows go to the decode step's MFMA kernels (reading the residual
+    On the bfloat16 path up to 64 rows (16 for a very wide output) go to the decode step's MFMA kernels (reading the residual
     stream through the folded LayerNorm when `a` is a LazyNorm of a fusable norm and the rows are
     few; splitting a long inner size over workgroups when the rows are many) and more rows to the
     tiled MFMA kernel; the 32-bit path, and every shape those refuse, go to the 32-bit FMA kernel.  `scatter` = (k_pool, v_pool,
@@ -81,7 +81,11 @@ def linear(ctx, a: Union[torch.Tensor, LazyNorm], w: torch.Tensor, bias: Optiona
     if n_rows == 0:
         return scatter is not None
     fast = w.dtype == torch.bfloat16 and not ctx.exact and ctx.dtype == torch.bfloat16
-    if fast and n_rows <= 64:
+    # A very wide output (the head) with more than a few rows: the tiled kernel streams the matrix
+    # at the same rate whatever the rows, the decode kernel slows down with every row it adds
+    # (measured at 50k outputs: even at 16 rows, 1.8 times slower at 64).
+    wide_out = n_rows > 16 and w.shape[0] >= 8192
+    if fast and n_rows <= 64 and not wide_out:
         epi = kernels.SK_EPI_QKV if scatter is not None else epilogue
         # every column tile converts the residual rows it multiplies: beyond 32 rows, or for a very
         # wide output (the head), that costs more than a LayerNorm kernel of its own
