@@ -120,7 +120,7 @@ template <int WTM, int WTN, int WVM, int WVN, int EPI, typename OT>
 __global__ __launch_bounds__(64 * WVM * WVN) void linear_mfma_kernel(
     const bf16_t* __restrict__ act, long lda, const bf16_t* __restrict__ w,
     const float* __restrict__ bias, OT* __restrict__ out, long ldo, int n_rows, int n_out, int k_dim,
-    MfmaScatter sc) {
+    int k_parts, long part_stride, MfmaScatter sc) {
   constexpr int T = 64 * WVM * WVN;
   constexpr int BM = WVM * WTM * 16, BN = WVN * WTN * 16;
   constexpr int TPR = MM_BK / 8;  // threads per staged row (16 bytes each)
@@ -133,9 +133,13 @@ __global__ __launch_bounds__(64 * WVM * WVN) void linear_mfma_kernel(
 
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int row_tiles = (n_rows + BM - 1) / BM, col_tiles = (n_out + BN - 1) / BN;
-  int row_tile, col_tile;
+  int row_tile, col_tile, part;
   {
-    const int id = mfma_xcd_tile_id(blockIdx.x, gridDim.x);
+    // with the inner size split into k_parts, part p of every tile comes before part p + 1 of any
+    const int tiles = row_tiles * col_tiles;
+    const int wid = mfma_xcd_tile_id(blockIdx.x, gridDim.x);
+    part = wid / tiles;
+    const int id = wid - part * tiles;
     const int per_group = MM_GROUP * col_tiles;
     const int group = id / per_group, in_group = id - group * per_group;
     const int first = group * MM_GROUP;
@@ -144,6 +148,11 @@ __global__ __launch_bounds__(64 * WVM * WVN) void linear_mfma_kernel(
     col_tile = in_group / rows_here;
   }
   const int row0 = row_tile * BM, col0 = col_tile * BN;
+  // this workgroup's stretch of the inner size (all of it unless the product is split), in whole steps
+  const int k_per = (((k_dim + MM_BK - 1) / MM_BK + k_parts - 1) / k_parts) * MM_BK;
+  const int k_begin = part * k_per;
+  const int k_len = k_dim - k_begin < k_per ? k_dim - k_begin : k_per;
+  out += part * part_stride;
   const int wr = (wave / WVN) * (WTM * 16), wc = (wave % WVN) * (WTN * 16);
   const int lrow = lane & 15;
 
@@ -158,23 +167,23 @@ __global__ __launch_bounds__(64 * WVM * WVN) void linear_mfma_kernel(
 #pragma unroll
   for (int p = 0; p < PA; ++p) {
     const int r = row0 + srow + p * RPP;
-    gp[p] = act + (long)(r < n_rows ? r : n_rows - 1) * lda + sk;
+    gp[p] = act + (long)(r < n_rows ? r : n_rows - 1) * lda + k_begin + sk;
   }
 #pragma unroll
   for (int p = 0; p < PW; ++p) {
     const int r = col0 + srow + p * RPP;
-    gp[PA + p] = w + (long)(r < n_out ? r : n_out - 1) * k_dim + sk;
+    gp[PA + p] = w + (long)(r < n_out ? r : n_out - 1) * k_dim + k_begin + sk;
   }
-  // A chunk that lies beyond k_dim (in the last, partial step) is read from the row's start instead
+  // A chunk that lies beyond the stretch's end (in its last, partial step) is read from the row's start instead
   // and counts as zero when it is stored: the select then waits for no load.
   auto load_item = [&](int p, int step) {
     const int k0 = step * MM_BK;
-    gv[p] = *reinterpret_cast<const bf16x8_t*>(gp[p] + (k0 + sk + 8 <= k_dim ? k0 : 0));
+    gv[p] = *reinterpret_cast<const bf16x8_t*>(gp[p] + (k0 + sk + 8 <= k_len ? k0 : 0));
   };
   auto store_item = [&](int p, int step, int buf) {
     bf16_t* dst = p < PA ? as_base + buf * (BM * MM_LD) + p * RPP * MM_LD
                          : ws_base + buf * (BN * MM_LD) + (p - PA) * RPP * MM_LD;
-    *reinterpret_cast<bf16x8_t*>(dst + s_lds) = step * MM_BK + sk + 8 <= k_dim ? gv[p] : zero8;
+    *reinterpret_cast<bf16x8_t*>(dst + s_lds) = step * MM_BK + sk + 8 <= k_len ? gv[p] : zero8;
   };
 
   f32x4_t acc[WTN][WTM];  // [column tile of W][row tile of activations]
@@ -183,7 +192,7 @@ __global__ __launch_bounds__(64 * WVM * WVN) void linear_mfma_kernel(
 #pragma unroll
     for (int j = 0; j < WTM; ++j) acc[i][j] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
 
-  const int k_steps = (k_dim + MM_BK - 1) / MM_BK;
+  const int k_steps = (k_len + MM_BK - 1) / MM_BK;
   const int c0 = ((lane >> 4) ^ (lrow & 7)) * 8;  // this lane's chunk of an operand row, first half of a step
 
   // One step along k.  Its 2 * WTM groups of MFMAs (one row tile of the activations against the
@@ -291,7 +300,7 @@ __global__ __launch_bounds__(64 * WVM * WVN) void linear_mfma_kernel(
 
 template <int WTM, int WTN, int WVM, int WVN, int EPI, typename OT>
 int launch_one(const void* act, long lda, const void* w, const float* bias, void* out, long ldo, int n_rows,
-               int n_out, int k_dim, const MfmaScatter& sc, hipStream_t stream) {
+               int n_out, int k_dim, int k_parts, long part_stride, const MfmaScatter& sc, hipStream_t stream) {
   constexpr int BM = WVM * WTM * 16, BN = WVN * WTN * 16;
   constexpr size_t lds_bytes = 2ul * (BM + BN) * MM_LD * sizeof(bf16_t);
   auto kernel = linear_mfma_kernel<WTM, WTN, WVM, WVN, EPI, OT>;
@@ -302,18 +311,21 @@ int launch_one(const void* act, long lda, const void* w, const float* bias, void
     if (e != hipSuccess) return (int)e;
     allowed = true;
   }
-  const long tiles = (long)((n_rows + BM - 1) / BM) * ((n_out + BN - 1) / BN);
+  const long tiles = (long)((n_rows + BM - 1) / BM) * ((n_out + BN - 1) / BN) * k_parts;
   if (tiles > 0x7fffffffL) return MGPT_ERR_TOO_LARGE;
   hipLaunchKernelGGL(kernel, dim3((unsigned int)tiles), dim3(64 * WVM * WVN), lds_bytes, stream,
-                     (const bf16_t*)act, lda, (const bf16_t*)w, bias, (OT*)out, ldo, n_rows, n_out, k_dim, sc);
+                     (const bf16_t*)act, lda, (const bf16_t*)w, bias, (OT*)out, ldo, n_rows, n_out, k_dim, k_parts,
+                     part_stride, sc);
   return mgpt_last_error();
 }
 
 template <int WTM, int WTN, int WVM, int WVN>
 int launch_shape(const void* act, long lda, const void* w, const float* bias, void* out, int out_dtype, long ldo,
-                 int n_rows, int n_out, int k_dim, int epilogue, const MfmaScatter& sc, hipStream_t stream) {
-#define MM_LAUNCH(E, OT) \
-  return launch_one<WTM, WTN, WVM, WVN, E, OT>(act, lda, w, bias, out, ldo, n_rows, n_out, k_dim, sc, stream)
+                 int n_rows, int n_out, int k_dim, int epilogue, int k_parts, long part_stride,
+                 const MfmaScatter& sc, hipStream_t stream) {
+#define MM_LAUNCH(E, OT)                                                                                     \
+  return launch_one<WTM, WTN, WVM, WVN, E, OT>(act, lda, w, bias, out, ldo, n_rows, n_out, k_dim, k_parts, \
+                                               part_stride, sc, stream)
   if (epilogue == MM_EPI_NONE && out_dtype == MGPT_BF16) MM_LAUNCH(MM_EPI_NONE, bf16_t);
   if (epilogue == MM_EPI_NONE && out_dtype == MGPT_F32) MM_LAUNCH(MM_EPI_NONE, float);
   if (epilogue == MM_EPI_GELU && out_dtype == MGPT_BF16) MM_LAUNCH(MM_EPI_GELU, bf16_t);
@@ -323,11 +335,11 @@ int launch_shape(const void* act, long lda, const void* w, const float* bias, vo
   return MGPT_ERR_BAD_DTYPE;
 }
 
-// Tile shapes, largest first: rows x columns of a workgroup's tile, and how many workgroups of it
-// a compute unit holds at a time.
+// Tile shapes, largest first: rows x columns of a workgroup's tile.
 constexpr int MM_SHAPES = 5;
 constexpr int MM_TILE_ROWS[MM_SHAPES] = {256, 128, 128, 64, 32};
 constexpr int MM_TILE_COLS[MM_SHAPES] = {256, 256, 64, 64, 32};
+constexpr int MM_MAX_PARTS = 8;
 
 long tiles_of(int shape, int n_rows, int n_out) {
   return (long)((n_rows + MM_TILE_ROWS[shape] - 1) / MM_TILE_ROWS[shape]) *
@@ -347,47 +359,181 @@ int choose_shape(int n_rows, int n_out) {
   return 4;
 }
 
-int launch_any(int shape, const void* act, long lda, const void* w, const float* bias, void* out, int out_dtype,
-               long ldo, int n_rows, int n_out, int k_dim, int epilogue, const MfmaScatter& sc, hipStream_t stream) {
+// Whether the inner size is split into stretches, and then with which tile shape and into how many
+// (parts == 1: not at all, and the shape is the one chosen by the tiles alone).  A long inner size
+// with few tiles leaves most compute units idle for a long time: then several workgroups share a
+// tile, each writes the sum over its stretch to the caller's buffer, and a second kernel adds the
+// sums in the order of k (so the result does not depend on which workgroup ran when) and applies
+// the epilogue.  That costs a pass over parts x the output, so it is done only for an inner size of
+// at least 32 steps whose unsplit product would not fill the compute units; every stretch is at
+// least 8 steps long; 64 x 64 tiles if they and the stretches together fill the units, else 32 x 32.
+// The QKV epilogue is never split.
+void choose_split(int n_rows, int n_out, int k_dim, int epilogue, int* shape, int* parts) {
+  *shape = choose_shape(n_rows, n_out);
+  *parts = 1;
+  const int steps = (k_dim + MM_BK - 1) / MM_BK;
+  // "would not fill the units": counted in 64 x 64 tiles for a very long inner size, where the many
+  // 32 x 32 tiles that would fill them take far longer than 64 x 64 tiles with stretches
+  if (epilogue == MM_EPI_QKV || (n_out & 3) != 0 || steps < 32 || tiles_of(steps >= 64 ? 3 : 4, n_rows, n_out) >= 256)
+    return;
+  for (int sh = 3; sh <= 4; ++sh) {
+    const long t = tiles_of(sh, n_rows, n_out);
+    int p = 1;
+    while (p < MM_MAX_PARTS && t * p * 2 <= 640 && steps / (p * 2) >= 8) p *= 2;
+    if (p > 1 && (t * p >= 256 || sh == 4)) {
+      *shape = sh;
+      *parts = p;
+      return;
+    }
+  }
+}
+
+// drops stretches that would be empty (the stretch length is rounded up to whole steps)
+int used_parts(int k_dim, int parts) {
+  const int steps = (k_dim + MM_BK - 1) / MM_BK;
+  const int per = (steps + parts - 1) / parts;
+  return (steps + per - 1) / per;
+}
+
+// out[n, o] = sum over the stretches' sums, in their order, + bias, with the epilogue
+template <int EPI, typename OT>
+__global__ __launch_bounds__(256) void linear_mfma_join_kernel(const float* __restrict__ partials, int k_parts,
+                                                               const float* __restrict__ bias, OT* __restrict__ out,
+                                                               long ldo, int n_rows, int n_out) {
+  const int quads = n_out >> 2;
+  const long idx = (long)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= (long)n_rows * quads) return;
+  const int row = (int)(idx / quads), oc = (int)(idx - (long)row * quads) * 4;
+  const float* p = partials + (long)row * n_out + oc;
+  const long part_stride = (long)n_rows * n_out;
+  float4 v = *reinterpret_cast<const float4*>(p);
+  for (int s = 1; s < k_parts; ++s) {
+    const float4 t = *reinterpret_cast<const float4*>(p + s * part_stride);
+    v.x += t.x; v.y += t.y; v.z += t.z; v.w += t.w;
+  }
+  if (bias) {
+    const bool al = (((size_t)bias) & 15) == 0;
+    if (al) {
+      const float4 b4 = *reinterpret_cast<const float4*>(bias + oc);
+      v.x += b4.x; v.y += b4.y; v.z += b4.z; v.w += b4.w;
+    } else {
+      v.x += bias[oc]; v.y += bias[oc + 1]; v.z += bias[oc + 2]; v.w += bias[oc + 3];
+    }
+  }
+  if (EPI == MM_EPI_GELU) {
+    v.x = gelu_tanh_fast(v.x); v.y = gelu_tanh_fast(v.y); v.z = gelu_tanh_fast(v.z); v.w = gelu_tanh_fast(v.w);
+  }
+  OT* orow = out + (long)row * ldo + oc;
+  const float r[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    if (EPI == MM_EPI_RESIDUAL) orow[e] = from_float<OT>(to_float<OT>(orow[e]) + r[e]);
+    else orow[e] = from_float<OT>(r[e]);
+  }
+}
+
+int launch_join(const float* partials, int k_parts, const float* bias, void* out, int out_dtype, long ldo,
+                int n_rows, int n_out, int epilogue, hipStream_t stream) {
+  const long work = (long)n_rows * (n_out >> 2);
+  dim3 grid((unsigned int)((work + 255) / 256));
+#define MM_JOIN(E, OT)                                                                                  \
+  hipLaunchKernelGGL((linear_mfma_join_kernel<E, OT>), grid, dim3(256), 0, stream, partials, k_parts, \
+                     bias, (OT*)out, ldo, n_rows, n_out)
+  if (epilogue == MM_EPI_NONE && out_dtype == MGPT_BF16) MM_JOIN(MM_EPI_NONE, bf16_t);
+  else if (epilogue == MM_EPI_NONE && out_dtype == MGPT_F32) MM_JOIN(MM_EPI_NONE, float);
+  else if (epilogue == MM_EPI_GELU && out_dtype == MGPT_BF16) MM_JOIN(MM_EPI_GELU, bf16_t);
+  else if (epilogue == MM_EPI_RESIDUAL && out_dtype == MGPT_F32) MM_JOIN(MM_EPI_RESIDUAL, float);
+  else return MGPT_ERR_BAD_DTYPE;
+#undef MM_JOIN
+  return mgpt_last_error();
+}
+
+bool shapes_ok(const void* act, long lda, const void* w, const void* out, long ldo, int n_rows, int n_out, int k_dim) {
+  return act && w && out && n_rows >= 0 && n_out >= 0 && k_dim > 0 && (k_dim % 16) == 0 && lda >= k_dim &&
+         (lda % 8) == 0 && ldo >= n_out;
+}
+
+// shape < 0: chosen by the size.  k_parts: 0 = chosen by the size, together with the shape, if
+// `partials` holds enough floats (else unsplit; with a given shape unsplit too), 1 = unsplit,
+// more = that many stretches (refused if the buffer is too small).
+int launch_any(int shape, int k_parts, const void* act, long lda, const void* w, const float* bias, void* out,
+               int out_dtype, long ldo, int n_rows, int n_out, int k_dim, int epilogue, float* partials,
+               long partials_floats, const MfmaScatter& sc, hipStream_t stream) {
   if (n_rows == 0 || n_out == 0) return MGPT_OK;
   if (!act || !w || !out) return MGPT_ERR_NULL;
-  if (n_rows < 0 || n_out < 0 || k_dim <= 0 || (k_dim % 16) != 0 || lda < k_dim || (lda % 8) != 0 ||
-      ldo < n_out)
-    return MGPT_ERR_BAD_SHAPE;
+  if (!shapes_ok(act, lda, w, out, ldo, n_rows, n_out, k_dim)) return MGPT_ERR_BAD_SHAPE;
+  const bool forced = k_parts > 1;
+  if (shape < 0 && k_parts == 0 && partials) {
+    choose_split(n_rows, n_out, k_dim, epilogue, &shape, &k_parts);
+    if (k_parts > 1 && (long)used_parts(k_dim, k_parts) * n_rows * n_out > partials_floats) shape = -1, k_parts = 1;
+  }
   if (shape < 0) shape = choose_shape(n_rows, n_out);
-#define MM_ARGS act, lda, w, bias, out, out_dtype, ldo, n_rows, n_out, k_dim, epilogue, sc, stream
+  if (shape >= MM_SHAPES) return MGPT_ERR_BAD_SHAPE;
+  if (k_parts == 0) k_parts = 1;
+  if (k_parts > 1) {
+    k_parts = used_parts(k_dim, k_parts > MM_MAX_PARTS ? MM_MAX_PARTS : k_parts);
+    const bool fits = partials && (long)k_parts * n_rows * n_out <= partials_floats &&
+                      (((size_t)partials) & 15) == 0 && (n_out & 3) == 0 && epilogue != MM_EPI_QKV;
+    if (!fits) {
+      if (forced) return MGPT_ERR_BAD_SHAPE;
+      k_parts = 1;
+    }
+  }
+  const bool split = k_parts > 1;
+  void* dst = split ? (void*)partials : out;
+  const float* b = split ? nullptr : bias;
+  const int dt = split ? MGPT_F32 : out_dtype, epi = split ? MM_EPI_NONE : epilogue;
+  const long ld = split ? n_out : ldo, stride = split ? (long)n_rows * n_out : 0;
+#define MM_ARGS act, lda, w, b, dst, dt, ld, n_rows, n_out, k_dim, epi, k_parts, stride, sc, stream
+  int rc = MGPT_ERR_BAD_SHAPE;
   switch (shape) {
-    case 0: return launch_shape<8, 4, 2, 4>(MM_ARGS);  // 256 x 256, eight waves of 128 x 64
-    case 1: return launch_shape<4, 4, 2, 4>(MM_ARGS);  // 128 x 256, eight waves of 64 x 64
-    case 2: return launch_shape<4, 2, 2, 2>(MM_ARGS);  // 128 x 64, four waves of 64 x 32
-    case 3: return launch_shape<2, 2, 2, 2>(MM_ARGS);  // 64 x 64, four waves of 32 x 32
-    case 4: return launch_shape<1, 1, 2, 2>(MM_ARGS);  // 32 x 32, four waves of 16 x 16
+    case 0: rc = launch_shape<8, 4, 2, 4>(MM_ARGS); break;  // 256 x 256, eight waves of 128 x 64
+    case 1: rc = launch_shape<4, 4, 2, 4>(MM_ARGS); break;  // 128 x 256, eight waves of 64 x 64
+    case 2: rc = launch_shape<4, 2, 2, 2>(MM_ARGS); break;  // 128 x 64, four waves of 64 x 32
+    case 3: rc = launch_shape<2, 2, 2, 2>(MM_ARGS); break;  // 64 x 64, four waves of 32 x 32
+    case 4: rc = launch_shape<1, 1, 2, 2>(MM_ARGS); break;  // 32 x 32, four waves of 16 x 16
   }
 #undef MM_ARGS
-  return MGPT_ERR_BAD_SHAPE;
+  if (rc != MGPT_OK || !split) return rc;
+  return launch_join(partials, k_parts, bias, out, out_dtype, ldo, n_rows, n_out, epilogue, stream);
 }
 
 }  // namespace
 
+// How many floats of scratch the product would use if it were split along its inner size (0: it
+// would not be split).  The caller brings that buffer to mgpt_linear_mfma.
+extern "C" long mgpt_linear_mfma_partials(int n_rows, int n_out, int k_dim, int epilogue) {
+  if (n_rows <= 0 || n_out <= 0 || k_dim <= 0) return 0;
+  int shape, parts;
+  choose_split(n_rows, n_out, k_dim, epilogue, &shape, &parts);
+  return parts > 1 ? (long)used_parts(k_dim, parts) * n_rows * n_out : 0;
+}
+
 // act: [n_rows, k_dim] bfloat16 with row stride lda (a multiple of 8, 16-byte aligned base);
 // w: [n_out, k_dim] dense bfloat16; out: [n_rows, n_out] with row stride ldo.  k_dim must be a
-// multiple of 16.  Refuses other layouts with MGPT_ERR_BAD_SHAPE.
+// multiple of 16.  partials: scratch of partials_floats floats (16-byte aligned) or null; with it
+// a long inner size over few tiles is split (mgpt_linear_mfma_partials says how much that needs).
+// Refuses other layouts with MGPT_ERR_BAD_SHAPE.
 extern "C" int mgpt_linear_mfma(const void* act, long lda, const void* w, const float* bias, void* out,
                                 int out_dtype, long ldo, int n_rows, int n_out, int k_dim, int epilogue,
-                                hipStream_t stream) {
+                                float* partials, long partials_floats, hipStream_t stream) {
   if (epilogue == MM_EPI_QKV) return MGPT_ERR_BAD_SHAPE;  // mgpt_linear_mfma_qkv brings the pools
   MfmaScatter sc = {};
-  return launch_any(-1, act, lda, w, bias, out, out_dtype, ldo, n_rows, n_out, k_dim, epilogue, sc, stream);
+  return launch_any(-1, 0, act, lda, w, bias, out, out_dtype, ldo, n_rows, n_out, k_dim, epilogue, partials,
+                    partials_floats, sc, stream);
 }
 
 // The same product with the tile shape given (0 = 256 x 256, 1 = 128 x 256, 2 = 128 x 64,
-// 3 = 64 x 64, 4 = 32 x 32) instead of chosen by the size: for tests and measurements of each shape.
-extern "C" int mgpt_linear_mfma_shape(int shape, const void* act, long lda, const void* w, const float* bias,
-                                      void* out, int out_dtype, long ldo, int n_rows, int n_out, int k_dim,
-                                      int epilogue, hipStream_t stream) {
-  if (epilogue == MM_EPI_QKV || shape < 0 || shape >= MM_SHAPES) return MGPT_ERR_BAD_SHAPE;
+// 3 = 64 x 64, 4 = 32 x 32; negative: chosen) and the number of stretches of the inner size given
+// (k_parts as for launch_any above), instead of chosen by the size: for tests and measurements.
+extern "C" int mgpt_linear_mfma_shape(int shape, int k_parts, const void* act, long lda, const void* w,
+                                      const float* bias, void* out, int out_dtype, long ldo, int n_rows,
+                                      int n_out, int k_dim, int epilogue, float* partials, long partials_floats,
+                                      hipStream_t stream) {
+  if (epilogue == MM_EPI_QKV || shape >= MM_SHAPES || k_parts < 0) return MGPT_ERR_BAD_SHAPE;
   MfmaScatter sc = {};
-  return launch_any(shape, act, lda, w, bias, out, out_dtype, ldo, n_rows, n_out, k_dim, epilogue, sc, stream);
+  return launch_any(shape, k_parts, act, lda, w, bias, out, out_dtype, ldo, n_rows, n_out, k_dim, epilogue,
+                    partials, partials_floats, sc, stream);
 }
 
 // The fused QKV product of a step with prompt portions: out[n] = act[n] W^T + bias in bfloat16, and
@@ -405,5 +551,6 @@ extern "C" int mgpt_linear_mfma_qkv(const void* act, long lda, const void* w, co
       (((size_t)out | (size_t)bias) & 15) != 0 || shape >= MM_SHAPES)
     return MGPT_ERR_BAD_SHAPE;
   MfmaScatter sc = {(bf16_t*)kpool, (bf16_t*)vpool, slot_mapping, q_width, kv_width, head_dim, n_kv_head, page_size};
-  return launch_any(shape, act, lda, w, bias, out, MGPT_BF16, ldo, n_rows, n_out, k_dim, MM_EPI_QKV, sc, stream);
+  return launch_any(shape, 1, act, lda, w, bias, out, MGPT_BF16, ldo, n_rows, n_out, k_dim, MM_EPI_QKV, nullptr, 0, sc,
+                    stream);
 }

@@ -437,12 +437,21 @@ def paged_attention_decode_bf16(q: torch.Tensor, out: torch.Tensor, k_pool: torc
     return True
 
 
+def linear_mfma_partials(n_rows: int, n_out: int, k_dim: int, epilogue: int) -> int:
+    """Floats of scratch that linear_mfma would use to split this product along its inner size
+    (0: it would not split it)."""
+    return int(library.kernels().mgpt_linear_mfma_partials(n_rows, n_out, k_dim, epilogue))
+
+
 def linear_mfma(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor,
-                n_rows: int, epilogue: int, scatter=None, shape: Optional[int] = None) -> bool:
+                n_rows: int, epilogue: int, scatter=None, shape: Optional[int] = None,
+                partials: Optional[torch.Tensor] = None, k_parts: Optional[int] = None) -> bool:
     """Tiled bfloat16 MFMA product for many rows.  scatter = (k_pool, v_pool, slot_mapping, q_width,
     kv_width) also stores the new keys and values into their pages (bfloat16 output, no other
-    epilogue).  `shape` (0 = 256 x 256 tiles, 1 = 128 x 256, 2 = 128 x 64, 3 = 64 x 64, 4 = 32 x 32) fixes the
-    tile shape that the library otherwise chooses by the size.  False when it does not take the shape."""
+    epilogue).  `partials`: float32 scratch with which a long inner size over few tiles is split
+    among workgroups (linear_mfma_partials says how much it takes).  `shape` (0 = 256 x 256 tiles,
+    1 = 128 x 256, 2 = 128 x 64, 3 = 64 x 64, 4 = 32 x 32) and `k_parts` fix what the library otherwise
+    chooses by the size.  False when it does not take the shape."""
     if a.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
         return False
     n_out, k_dim = w.shape
@@ -473,12 +482,16 @@ def linear_mfma(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], 
             _ptr(vp), _ptr(sm), q_width, kv_width, head_dim, n_kv_head, page_size, -1 if shape is None else int(shape),
             _stream())
     else:
+        if partials is not None:
+            _need_cuda(partials)
+            _need(partials.dtype == torch.float32 and partials.is_contiguous(), "partials must be dense float32")
         args = (_ptr(a), a.stride(0), _ptr(w), _ptr(bias), _ptr(out), _dtype_code(out), out.stride(0), n_rows,
-                n_out, k_dim, epilogue, _stream())
-        if shape is None:
+                n_out, k_dim, epilogue, _ptr(partials), 0 if partials is None else partials.numel(), _stream())
+        if shape is None and k_parts is None:
             rc = library.kernels().mgpt_linear_mfma(*args)
         else:
-            rc = library.kernels().mgpt_linear_mfma_shape(int(shape), *args)
+            rc = library.kernels().mgpt_linear_mfma_shape(-1 if shape is None else int(shape),
+                                                          0 if k_parts is None else int(k_parts), *args)
     if rc == -2:
         return False
     _check(rc, "linear_mfma")

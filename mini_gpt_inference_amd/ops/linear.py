@@ -75,7 +75,7 @@ def linear(ctx, a: Union[torch.Tensor, LazyNorm], w: torch.Tensor, bias: Optiona
     On the bfloat16 path up to 64 rows (16 for a very wide output) go to the decode step's MFMA kernels (reading the residual
     stream through the folded LayerNorm when `a` is a LazyNorm of a fusable norm and the rows are
     few; splitting a long inner size over workgroups when the rows are many) and more rows to the
-    tiled MFMA kernel; the 32-bit path, and every shape those refuse, go to the 32-bit FMA kernel.  `scatter` = (k_pool, v_pool,
+    tiled MFMA kernel (which also splits a long inner size when its tiles are few); the 32-bit path, and every shape those refuse, go to the 32-bit FMA kernel.  `scatter` = (k_pool, v_pool,
     slot_mapping, q_width, kv_width) asks for the new keys and values to be stored into their
     pages by the same kernel; the return value says whether that was done."""
     if n_rows == 0:
@@ -106,7 +106,10 @@ def linear(ctx, a: Union[torch.Tensor, LazyNorm], w: torch.Tensor, bias: Optiona
     a = as_tensor(ctx, a)
     if fast and scatter is not None and kernels.linear_mfma(a, w, bias, out, n_rows, epilogue, scatter=scatter):
         return True
-    if fast and kernels.linear_mfma(a, w, bias, out, n_rows, epilogue):
-        return False
+    if fast:
+        need = kernels.linear_mfma_partials(n_rows, w.shape[0], w.shape[1], epilogue)
+        partials = ctx.workspace.get("linear_partials", need, 1, torch.float32) if need else None
+        if kernels.linear_mfma(a, w, bias, out, n_rows, epilogue, partials=partials):
+            return False
     kernels.linear_generic(a, w, bias, out, n_rows, epilogue)
     return False

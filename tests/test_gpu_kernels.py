@@ -153,6 +153,50 @@ def test_linear_mfma_each_tile_shape(n, k, o, epi, o_dt, shape):
     assert torch.equal(out[n:], prev[n:].to(DEV)), "rows beyond n_rows were written"
 
 
+@pytest.mark.parametrize("n,k,o,shape,parts", [(100, 2048, 96, 4, 4), (70, 1040, 132, 3, 2), (300, 6400, 64, 3, 8),
+                                                (33, 576, 40, 4, 3), (130, 1600, 260, 2, 4)])
+@pytest.mark.parametrize("epi,o_dt", [(kernels.EPI_NONE, "bfloat16"), (kernels.EPI_NONE, "float32"),
+                                      (kernels.EPI_GELU, "bfloat16"), (kernels.EPI_RESIDUAL, "float32")])
+def test_linear_mfma_split_along_the_inner_size(n, k, o, shape, parts, epi, o_dt):
+    """Several workgroups per tile, each with a stretch of the inner size (also one that ends inside a step
+    and a number of stretches that leaves the last one short), their sums joined by the second kernel."""
+    g = torch.Generator().manual_seed(18)
+    a, w, bias = rnd(g, n, k, dtype="bfloat16"), rnd(g, o, k, dtype="bfloat16", scale=k ** -0.5), rnd(g, o)
+    prev = rnd(g, n + 2, o, dtype=o_dt)
+    out = prev.clone().to(DEV)
+    scratch = torch.full((parts * n * o + 8,), float("nan"), device=DEV)
+    assert kernels.linear_mfma(a.to(DEV), w.to(DEV), bias.to(DEV), out, n, epi, shape=shape, k_parts=parts,
+                               partials=scratch)
+    helpers.assert_close(out[:n], _linear_want(a, w, bias, epi, prev[:n]), "bfloat16", f"split {parts} of {k}")
+    assert torch.equal(out[n:], prev[n:].to(DEV)), "rows beyond n_rows were written"
+    # twice the same: the sums are joined in a fixed order
+    out2 = prev.clone().to(DEV)
+    assert kernels.linear_mfma(a.to(DEV), w.to(DEV), bias.to(DEV), out2, n, epi, shape=shape, k_parts=parts,
+                               partials=scratch)
+    assert torch.equal(out, out2)
+    # a buffer that is too small is refused when the split is forced, and not used when it is not
+    assert not kernels.linear_mfma(a.to(DEV), w.to(DEV), bias.to(DEV), out2, n, epi, shape=shape, k_parts=parts,
+                                   partials=scratch[:16])
+
+
+def test_linear_mfma_splits_by_itself_when_tiles_are_few_and_the_inner_size_long():
+    g = torch.Generator().manual_seed(19)
+    n, k, o = 140, 6400, 1600
+    need = kernels.linear_mfma_partials(n, o, k, kernels.EPI_RESIDUAL)
+    assert need > 0 and need % (n * o) == 0
+    assert kernels.linear_mfma_partials(2048, 2048, 512, kernels.EPI_GELU) == 0
+    a, w, bias = rnd(g, n, k, dtype="bfloat16"), rnd(g, o, k, dtype="bfloat16", scale=k ** -0.5), rnd(g, o)
+    prev = rnd(g, n, o)
+    out, out1 = prev.clone().to(DEV), prev.clone().to(DEV)
+    assert kernels.linear_mfma(a.to(DEV), w.to(DEV), bias.to(DEV), out, n, kernels.EPI_RESIDUAL,
+                               partials=torch.empty(need, device=DEV))
+    assert kernels.linear_mfma(a.to(DEV), w.to(DEV), bias.to(DEV), out1, n, kernels.EPI_RESIDUAL)   # unsplit
+    want = _linear_want(a, w, bias, kernels.EPI_RESIDUAL, prev)
+    helpers.assert_close(out, want, "bfloat16", "split by itself")
+    helpers.assert_close(out1, want, "bfloat16", "unsplit")
+    assert not torch.equal(out, out1)      # another order of summation: it did split
+
+
 def test_linear_mfma_chooses_the_largest_tiles_for_a_large_problem():
     """160 tiles of 256 x 256: the library takes that shape by itself, so the result equals the forced one bit by bit."""
     g = torch.Generator().manual_seed(17)
