@@ -172,7 +172,8 @@ def serve_run(args, name):
             "seconds": round(elapsed, 3), "requests": len(requests), "generated_tokens": produced,
             "prompt_tokens": sum(len(p) for p, _ in requests), "n_layer": cfg.n_layer, "n_embd": cfg.n_embd,
             "n_head": cfg.n_head, "vocab_size": cfg.vocab_size, "pages": pages, "page_demand": demand,
-            "steps": stats["num_steps"], "preemptions": stats["num_preemptions"],
+            "steps": stats["num_steps"], "decode_graph_steps": stats["graph_steps"],
+            "other_steps_replayed": stats["replayed_eager_steps"], "preemptions": stats["num_preemptions"],
             "prompt_tokens_computed": stats["num_prompt_tokens"], "dtype": args.dtype, "weights": "random"}
 
 

@@ -67,8 +67,8 @@ __global__ __launch_bounds__(AW_WAVES * 64) void paged_attention_decode_kernel(
     const bf16_t* __restrict__ q, long ldq, bf16_t* __restrict__ out, long ldo,
     const bf16_t* __restrict__ kpool, const bf16_t* __restrict__ vpool,
     const int* __restrict__ block_tables, int max_blocks, const int* __restrict__ positions,
-    const int* __restrict__ q_req, int n_head, int n_kv_head, int page_shift, int num_pages,
-    unsigned int page_bytes, float scale_log2e, int window) {
+    const int* __restrict__ q_req, const int* __restrict__ cu_q, int n_head, int n_kv_head, int page_shift,
+    int num_pages, unsigned int page_bytes, float scale_log2e, int window) {
   constexpr int LPK = D / 8;     // lanes per key
   constexpr int KPI = 64 / LPK;  // keys per load instruction
   constexpr int ROWS = AW_WAVES * KPI;      // partial results: one per (key subgroup, wave)
@@ -87,11 +87,15 @@ __global__ __launch_bounds__(AW_WAVES * 64) void paged_attention_decode_kernel(
 
   // ---- first round trip: the token's request and position, its query, and (decode-only steps)
   // the block table entries of the first pass
-  const int qr = q_req[n];
+  int qr = q_req[n];
   const int qpos = positions[n];
   uint4 qraw = *reinterpret_cast<const uint4*>(q + (long)n * ldq + (long)h * D + dg * 8);
   int r = n;
-  if (!IDENT) r = qr < 0 ? 0 : qr;  // waits for qr
+  if (!IDENT) {
+    r = qr < 0 ? 0 : qr;  // waits for qr
+    // a step that also holds prompt portions: their tokens are another kernel's, and count as padding here
+    if (cu_q && cu_q[r + 1] - cu_q[r] != 1) qr = -1;
+  }
   int first_chunk = 0;
   if (window > 0) first_chunk = (qpos - window + 1 > 0 ? qpos - window + 1 : 0) / 64;  // waits for qpos
   const int* bt = block_tables + (long)r * max_blocks;
@@ -214,18 +218,20 @@ __global__ __launch_bounds__(AW_WAVES * 64) void paged_attention_decode_kernel(
 }
 
 // positions[n]: absolute position of token n; q_req[n]: its request (block table row), -1 for a
-// padded token.  identity != 0 promises q_req[n] is n or -1 (a decode-only step).  Refuses
+// padded token.  identity != 0 promises q_req[n] is n or -1 (a decode-only step).  cu_q (optional,
+// without identity): the requests' token offsets; tokens of requests that bring more than one token
+// are then left to another kernel.  Refuses
 // (MGPT_ERR_BAD_SHAPE) other head sizes than 16, 32, 64, 128, page sizes that are no power of two
 // and pools of 4 GiB or more.
 extern "C" int mgpt_paged_attention_decode_bf16(
     const void* q, long ldq, void* out, long ldo, const void* kpool, const void* vpool,
-    const int* block_tables, int max_blocks, const int* positions, const int* q_req, int n_tokens,
-    int n_head, int n_kv_head, int head_dim, int page_size, int num_pages, float scale, int window,
+    const int* block_tables, int max_blocks, const int* positions, const int* q_req, const int* cu_q,
+    int n_tokens, int n_head, int n_kv_head, int head_dim, int page_size, int num_pages, float scale, int window,
     int identity, hipStream_t stream) {
   if (n_tokens == 0) return MGPT_OK;
   if (!q || !out || !kpool || !vpool || !block_tables || !positions || !q_req) return MGPT_ERR_NULL;
   if (n_tokens < 0 || n_head <= 0 || n_kv_head <= 0 || (n_head % n_kv_head) != 0 || page_size <= 0 ||
-      max_blocks <= 0 || num_pages <= 0 || window < 0 || (ldq % 8) != 0)
+      max_blocks <= 0 || num_pages <= 0 || window < 0 || (ldq % 8) != 0 || (identity && cu_q))
     return MGPT_ERR_BAD_SHAPE;
   if (n_head > 65535) return MGPT_ERR_TOO_LARGE;
   int page_shift = -1;
@@ -241,7 +247,7 @@ extern "C" int mgpt_paged_attention_decode_bf16(
 #define AW_LAUNCH2(DD, ID)                                                                                 \
   hipLaunchKernelGGL((paged_attention_decode_kernel<DD, ID>), grid, block, 0, stream, (const bf16_t*)q, ldq, \
                      (bf16_t*)out, ldo, (const bf16_t*)kpool, (const bf16_t*)vpool, block_tables,          \
-                     max_blocks, positions, q_req, n_head, n_kv_head, page_shift, num_pages, page_bytes,  \
+                     max_blocks, positions, q_req, cu_q, n_head, n_kv_head, page_shift, num_pages, page_bytes, \
                      scale_log2e, window)
 #define AW_LAUNCH(DD)              \
   do {                             \

@@ -65,7 +65,8 @@ __global__ __launch_bounds__(256 * G) void prefill_attention_kernel(
     const bf16_t* __restrict__ q, long ldq, bf16_t* __restrict__ out, long ldo,
     const bf16_t* __restrict__ kpool, const bf16_t* __restrict__ vpool,
     const int* __restrict__ block_tables, int max_blocks, const int* __restrict__ cu_q,
-    const int* __restrict__ seq_lens, int n_head, int n_kv_head, int page_size, float scale, int window) {
+    const int* __restrict__ seq_lens, int n_head, int n_kv_head, int page_size, float scale, int window,
+    int single_below) {
   constexpr int THREADS = 256 * G;
   constexpr int SB = PF_KT * G;    // keys staged per step
   constexpr int KLD = D + 8;       // key rows in LDS
@@ -81,7 +82,7 @@ __global__ __launch_bounds__(256 * G) void prefill_attention_kernel(
   const int r = blockIdx.y, h = blockIdx.z;
   const int q_start = cu_q[r], q_len = cu_q[r + 1] - q_start;
   const int q0 = (int)blockIdx.x * PF_QT;
-  if (q0 >= q_len) return;
+  if (q0 >= q_len || (q_len == 1 && q_start < single_below)) return;   // the same for the whole workgroup
   const int seq_len = seq_lens[r];
   const int ctx = seq_len - q_len;
   const int tid = threadIdx.x, lane = tid & 63;
@@ -310,13 +311,15 @@ __global__ __launch_bounds__(256 * G) void prefill_attention_kernel(
 }
 
 // One workgroup per (64-query tile, request, head); max_q_len sizes the grid and is the host's
-// upper bound on the tokens any request brings.  Head sizes 32, 64, 96, 128 and a positive scale;
-// others are refused.
+// upper bound on the tokens any request brings (a request may bring none: its workgroups leave at
+// once).  single_below: requests that bring exactly one token, and that as one of the step's first
+// single_below tokens, are left to another kernel.  Head
+// sizes 32, 64, 96, 128 and a positive scale; others are refused.
 extern "C" int mgpt_prefill_attention_bf16(
     const void* q, long ldq, void* out, long ldo, const void* kpool, const void* vpool,
     const int* block_tables, int max_blocks, const int* cu_q, const int* seq_lens, int n_req,
     int max_q_len, int n_head, int n_kv_head, int head_dim, int page_size, float scale, int window,
-    hipStream_t stream) {
+    int single_below, hipStream_t stream) {
   if (n_req == 0 || max_q_len == 0) return MGPT_OK;
   if (!q || !out || !kpool || !vpool || !block_tables || !cu_q || !seq_lens) return MGPT_ERR_NULL;
   if (n_req < 0 || max_q_len < 0 || n_head <= 0 || n_kv_head <= 0 || (n_head % n_kv_head) != 0 ||
@@ -337,7 +340,8 @@ extern "C" int mgpt_prefill_attention_bf16(
     }                                                                                                           \
     hipLaunchKernelGGL((prefill_attention_kernel<DD, GG>), grid, dim3(256 * GG), lds_bytes, stream,             \
                        (const bf16_t*)q, ldq, (bf16_t*)out, ldo, (const bf16_t*)kpool, (const bf16_t*)vpool,    \
-                       block_tables, max_blocks, cu_q, seq_lens, n_head, n_kv_head, page_size, scale, window);  \
+                       block_tables, max_blocks, cu_q, seq_lens, n_head, n_kv_head, page_size, scale, window,   \
+                       single_below);                                                                          \
   }
   // Two wave groups halve the walk of a tile over its keys; one group leaves LDS for a second
   // workgroup on the compute unit.  The first serves a step with few tiles, the second one with many.

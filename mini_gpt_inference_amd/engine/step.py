@@ -35,6 +35,16 @@ def _bucket(n: int) -> int:
     return b
 
 
+def _bucket_tokens(n: int) -> int:
+    """The token capacity of a step of n tokens.  A graph made for a capacity runs every kernel over
+    all of it, so beyond 64 the capacities lie closer than powers of two: a quarter of the power of
+    two below n apart (at most 25 % of padding)."""
+    if n <= 64:
+        return _bucket(n)
+    step = _bucket(n) // 8
+    return -(-n // step) * step
+
+
 class StepArena:
     """Pinned host arrays and their device mirror for steps of up to (n_cap tokens, r_cap requests,
     m_cap logit rows)."""
@@ -127,7 +137,8 @@ class ModelRunner:
         self.vocab_size = model.spec.vocab_size
         self.workspace = Workspace(device)
         self.graph_steps = graph_steps and device.type == "cuda" and model.graph_safe
-        self._step_graphs: Dict[Tuple, _StepGraph] = {}
+        self._step_graphs: Dict[Tuple, _StepGraph] = {}     # by exact shape; emptied when it has MAX_STEP_GRAPHS
+        self._bucket_graphs: Dict[Tuple, _StepGraph] = {}   # by capacities: as many as there are buckets
         self.num_replayed_steps = 0
         self._arenas: Dict[Tuple[int, int, int], StepArena] = {}
         self.n_groups = len(cache.groups)
@@ -140,7 +151,7 @@ class ModelRunner:
 
     # ------------------------------------------------------------------ arenas
     def arena(self, n_tokens: int, n_req: int, n_logits: int) -> StepArena:
-        key = (_bucket(max(n_tokens, 1)), _bucket(max(n_req, 1)), _bucket(max(n_logits, 1)))
+        key = (_bucket_tokens(max(n_tokens, 1)), _bucket(max(n_req, 1)), _bucket(max(n_logits, 1)))
         a = self._arenas.get(key)
         if a is None:
             a = StepArena(*key, self.n_groups, self.max_blocks, self.device)
@@ -191,8 +202,12 @@ class ModelRunner:
         return StepShape(n, r, m, max(q_lens, default=0), max_seq, q_lens, ctx_lens, slots)
 
     # ------------------------------------------------------------------ running
-    def context(self, arena: StepArena, shape: StepShape, padded: bool, workspace: Optional[Workspace] = None
-                ) -> StepContext:
+    def context(self, arena: StepArena, shape: StepShape, padded: bool, workspace: Optional[Workspace] = None,
+                lead_cap: Optional[int] = None) -> StepContext:
+        """What the parts see of the step.  padded: every kernel runs over the arena's capacities (rows,
+        requests, logit rows) instead of the step's own counts.  lead_cap (with padded): the context
+        of a bucket of steps with prompt portions, in which nothing may depend on the step at hand
+        but the capacities and lead_cap."""
         d = arena.d
         groups = []
         for g, geo in enumerate(self.cache.groups):
@@ -203,44 +218,80 @@ class ModelRunner:
                                                (g + 1) * arena.r_cap * arena.max_blocks]
                 .view(arena.r_cap, arena.max_blocks),
                 k_pools=self.store.k_pools(g), v_pools=self.store.v_pools(g)))
+        bucket = padded and lead_cap is not None
         return StepContext(
             n_tokens=shape.n_tokens, n_rows=arena.n_cap if padded else shape.n_tokens,
             n_req=shape.n_req, n_logits=shape.n_logits, m_rows=arena.m_cap if padded else shape.n_logits,
             token_ids=d["token_ids"], positions=d["positions"], q_req=d["q_req"], cu_q=d["cu_q"],
             seq_lens=d["seq_lens"], state_slots=d["state_slots"], logit_rows=d["logit_rows"],
             groups=groups, state_pools=self.store.state_pools, dtype=self.dtype,
-            workspace=workspace or self.workspace, max_q_len=shape.max_q_len, max_seq_len=shape.max_seq_len,
-            decode_only=shape.max_q_len <= 1, host_q_lens=shape.q_lens, host_ctx_lens=shape.ctx_lens,
-            host_state_slots=shape.slots, exact=self.exact)
+            workspace=workspace or self.workspace,
+            max_q_len=arena.n_cap if bucket else shape.max_q_len, max_seq_len=shape.max_seq_len,
+            decode_only=False if bucket else shape.max_q_len <= 1,
+            host_q_lens=None if bucket else shape.q_lens, host_ctx_lens=None if bucket else shape.ctx_lens,
+            host_state_slots=None if bucket else shape.slots, exact=self.exact, padded=padded,
+            lead_cap=lead_cap or 0)
 
     def run(self, arena: StepArena, shape: StepShape) -> torch.Tensor:
         """Uploads the arena and runs the model.  Returns float32 logits [n_logits, vocab] (in the
-        workspace: the next step overwrites them)."""
+        workspace: the next step overwrites them).
+
+        Two kinds of graphs, both made when what they stand for has come CAPTURE_AT times: one for an
+        exact shape (the requests' token counts and the number of logit rows), which runs only the
+        step's own rows; and one for a bucket (the arena's capacities and how many tokens the leading
+        single-token requests may take), padded to those, which serves every step of the bucket
+        whatever its requests bring."""
         arena.upload()
-        entry = None
-        if self.graph_steps:
-            key = (tuple(shape.q_lens), shape.n_logits)
-            entry = self._step_graphs.get(key)
-            if entry is None:
-                if len(self._step_graphs) >= self.MAX_STEP_GRAPHS:
-                    self._step_graphs.clear()
-                entry = self._step_graphs[key] = _StepGraph()
-            if (entry.graph is not None and entry.arena is arena
-                    and entry.generation == self.workspace.generation):
-                entry.graph.replay()
-                self.num_replayed_steps += 1
-                return entry.logits
-            entry.graph = None
-            entry.seen += 1
-        ctx = self.context(arena, shape, padded=False)
+        if not self.graph_steps:
+            with kernels.pinned_stream():
+                return self.model.forward(self.context(arena, shape, padded=False))
+        exact = self._entry((tuple(shape.q_lens), shape.n_logits))
+        if self._live(exact, arena):
+            exact.graph.replay()
+            self.num_replayed_steps += 1
+            return exact.logits
+        lead = 0
+        while lead < shape.n_req and shape.q_lens[lead] == 1:
+            lead += 1
+        lead_cap = min(-(-lead // 16) * 16, arena.n_cap)
+        bucket = self._bucket_graphs.setdefault((arena.n_cap, arena.r_cap, arena.m_cap, lead_cap), _StepGraph())
+        exact.seen += 1
+        bucket.seen += 1
+        if exact.seen < self.CAPTURE_AT and self._live(bucket, arena):
+            bucket.graph.replay()
+            self.num_replayed_steps += 1
+            return bucket.logits[:shape.n_logits]
         with kernels.pinned_stream():
-            logits = self.model.forward(ctx)
-        if entry is not None and entry.seen >= self.CAPTURE_AT:
-            self._capture(entry, arena, shape)
+            logits = self.model.forward(self.context(arena, shape, padded=False))
+        if exact.seen >= self.CAPTURE_AT:
+            self._capture(exact, arena, shape, None)
+        elif bucket.seen >= self.CAPTURE_AT and not self._live(bucket, arena):
+            self._capture(bucket, arena, shape, lead_cap)
         return logits
 
-    def _capture(self, entry: _StepGraph, arena: StepArena, shape: StepShape) -> None:
-        """Records the step just run (every buffer it needs exists now) for the next of its shape."""
+    def _entry(self, key: Tuple) -> _StepGraph:
+        entry = self._step_graphs.get(key)
+        if entry is None:
+            if len(self._step_graphs) >= self.MAX_STEP_GRAPHS:
+                self._step_graphs.clear()
+            entry = self._step_graphs[key] = _StepGraph()
+        return entry
+
+    def _live(self, entry: _StepGraph, arena: StepArena) -> bool:
+        return (entry.graph is not None and entry.arena is arena
+                and entry.generation == self.workspace.generation)
+
+    def _capture(self, entry: _StepGraph, arena: StepArena, shape: StepShape, lead_cap: Optional[int]) -> None:
+        """Records the step that the arena holds for the next of its shape (lead_cap None) or of its
+        bucket.  A bucket's graph runs over more rows than the eager step before it did, so it runs
+        once eagerly first: every buffer it needs exists then."""
+        def forward():
+            ctx = self.context(arena, shape, padded=lead_cap is not None, lead_cap=lead_cap)
+            with kernels.pinned_stream():
+                return self.model.forward(ctx)
+        entry.graph = None
+        if lead_cap is not None:
+            forward()
         graph = torch.cuda.CUDAGraph()
         side = torch.cuda.Stream()
         side.wait_stream(torch.cuda.current_stream())
@@ -249,8 +300,7 @@ class ModelRunner:
             with torch.cuda.stream(side):
                 graph.capture_begin()
                 try:
-                    with kernels.pinned_stream():
-                        logits = self.model.forward(self.context(arena, shape, padded=False))
+                    logits = forward()
                 except BaseException:
                     # never leave the stream capturing (the graph object's destructor synchronizes
                     # the device); the capture is lost, so what ending it reports is of no interest

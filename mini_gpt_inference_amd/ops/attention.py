@@ -31,6 +31,22 @@ def _mixed_step(ctx, q, out, k_pool, v_pool, group, n_head: int, scale: float, w
                                           ctx.n_req, ctx.max_q_len, n_head, scale, window)
 
 
+def _padded_mixed_step(ctx, q, out, k_pool, v_pool, group, n_head: int, scale: float, window: int) -> bool:
+    """A step with prompt portions that is padded to its bucket's sizes (a graph replays it for every
+    step of the bucket): which request brings how many tokens is known on the device only.  The
+    decode kernel goes over the step's first `ctx.lead_cap` tokens (decoding requests lead a step)
+    and leaves out those of requests with several tokens; the tile kernel goes over all requests and
+    leaves out those whose one token the decode kernel had; requests and tokens of the padding have
+    neither.  False if the tile kernel refuses (the caller's general kernel then does all tokens again)."""
+    r = ctx.cu_q.numel() - 1
+    lead = min(ctx.lead_cap, ctx.n_rows)
+    singles = lead > 0 and kernels.paged_attention_decode_bf16(
+        q, out, k_pool, v_pool, group.block_tables, ctx.positions, ctx.q_req, lead, n_head, scale, window,
+        cu_q=ctx.cu_q)
+    return kernels.prefill_attention_bf16(q, out, k_pool, v_pool, group.block_tables, ctx.cu_q, ctx.seq_lens, r,
+                                          ctx.n_rows, n_head, scale, window, single_below=lead if singles else 0)
+
+
 def paged_attention(ctx, q: torch.Tensor, out: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor,
                     group, n_head: int, scale: float, window: int) -> None:
     """Attention of the step's tokens (rows of q) over their requests' pages.
@@ -45,8 +61,11 @@ def paged_attention(ctx, q: torch.Tensor, out: torch.Tensor, k_pool: torch.Tenso
                 q, out, k_pool, v_pool, group.block_tables, ctx.positions, ctx.q_req, n, n_head, scale, window,
                 identity=True):
             return
-        if not ctx.decode_only and ctx.n_rows == ctx.n_tokens and _mixed_step(ctx, q, out, k_pool, v_pool, group,
-                                                                               n_head, scale, window):
+        if not ctx.decode_only and not ctx.padded and _mixed_step(ctx, q, out, k_pool, v_pool, group, n_head, scale,
+                                                                  window):
+            return
+        if not ctx.decode_only and ctx.padded and _padded_mixed_step(ctx, q, out, k_pool, v_pool, group, n_head,
+                                                                     scale, window):
             return
         if kernels.paged_attention_split_bf16(q, out, k_pool, v_pool, group.block_tables, ctx.cu_q, ctx.seq_lens,
                                               ctx.q_req, n, r, n_head, scale, window):

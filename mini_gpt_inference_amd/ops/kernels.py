@@ -401,11 +401,12 @@ def paged_attention_split_bf16(q: torch.Tensor, out: torch.Tensor, k_pool: torch
 def paged_attention_decode_bf16(q: torch.Tensor, out: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor,
                                 block_tables: torch.Tensor, positions: torch.Tensor, q_req: torch.Tensor,
                                 n_tokens: int, n_head: int, scale: float, window: int = 0,
-                                identity: bool = False) -> bool:
+                                identity: bool = False, cu_q: Optional[torch.Tensor] = None) -> bool:
     """bfloat16 attention for single tokens (one query per request and step), keys split over eight
     waves.  positions[n] is token n's absolute position, q_req[n] its block table row or -1 for a
-    padded token; identity=True promises q_req[n] in (n, -1).  False if refused (other head sizes
-    than 16, 32, 64, 128)."""
+    padded token; identity=True promises q_req[n] in (n, -1).  With cu_q (the requests' token offsets;
+    not with identity) tokens of requests that bring more than one token are skipped.  False if
+    refused (other head sizes than 16, 32, 64, 128)."""
     if q.dtype != torch.bfloat16:
         return False
     _need_cuda(q, out, k_pool, v_pool, block_tables, positions, q_req)
@@ -427,9 +428,13 @@ def paged_attention_decode_bf16(q: torch.Tensor, out: torch.Tensor, k_pool: torc
     _need_i32("q_req", q_req, n_tokens)
     if identity:
         _need(block_tables.shape[0] >= n_tokens, "a decode-only step needs a block table row per token")
+        _need(cu_q is None, "cu_q is for steps that are not decode-only")
+    if cu_q is not None:
+        _need_cuda(cu_q)
+        _need_i32("cu_q", cu_q, block_tables.shape[0] + 1)
     rc = library.kernels().mgpt_paged_attention_decode_bf16(
         _ptr(q), q.stride(0), _ptr(out), out.stride(0), _ptr(k_pool), _ptr(v_pool), _ptr(block_tables),
-        block_tables.shape[1], _ptr(positions), _ptr(q_req), n_tokens, n_head, n_kv_head, head_dim, page_size,
+        block_tables.shape[1], _ptr(positions), _ptr(q_req), _ptr(cu_q), n_tokens, n_head, n_kv_head, head_dim, page_size,
         num_pages, float(scale), int(window), 1 if identity else 0, _stream())
     if rc == -2:
         return False
@@ -437,10 +442,19 @@ def paged_attention_decode_bf16(q: torch.Tensor, out: torch.Tensor, k_pool: torc
     return True
 
 
+_MFMA_PARTIALS: dict = {}   # the library's answer per size: asked at every product of every step
+
+
 def linear_mfma_partials(n_rows: int, n_out: int, k_dim: int, epilogue: int) -> int:
     """Floats of scratch that linear_mfma would use to split this product along its inner size
     (0: it would not split it)."""
-    return int(library.kernels().mgpt_linear_mfma_partials(n_rows, n_out, k_dim, epilogue))
+    key = (n_rows, n_out, k_dim, epilogue)
+    hit = _MFMA_PARTIALS.get(key)
+    if hit is None:
+        if len(_MFMA_PARTIALS) > 4096:
+            _MFMA_PARTIALS.clear()
+        hit = _MFMA_PARTIALS[key] = int(library.kernels().mgpt_linear_mfma_partials(n_rows, n_out, k_dim, epilogue))
+    return hit
 
 
 def linear_mfma(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor,
@@ -500,9 +514,12 @@ def linear_mfma(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], 
 
 def prefill_attention_bf16(q: torch.Tensor, out: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor,
                            block_tables: torch.Tensor, cu_q: torch.Tensor, seq_lens: torch.Tensor, n_req: int,
-                           max_q_len: int, n_head: int, scale: float, window: int = 0) -> bool:
+                           max_q_len: int, n_head: int, scale: float, window: int = 0,
+                           single_below: int = 0) -> bool:
     """MFMA tile attention for steps with prompt portions (every request's tokens are consecutive
-    rows of q from cu_q).  False when it does not take the case."""
+    rows of q from cu_q; a request may bring none).  Requests that bring exactly one token, and that
+    among the step's first `single_below` tokens, are left to another kernel.  False when it does
+    not take the case."""
     if q.dtype != torch.bfloat16:
         return False
     _need_cuda(q, out, k_pool, v_pool, block_tables, cu_q, seq_lens)
@@ -524,7 +541,7 @@ def prefill_attention_bf16(q: torch.Tensor, out: torch.Tensor, k_pool: torch.Ten
     rc = library.kernels().mgpt_prefill_attention_bf16(
         _ptr(q), q.stride(0), _ptr(out), out.stride(0), _ptr(k_pool), _ptr(v_pool), _ptr(block_tables),
         block_tables.shape[1], _ptr(cu_q), _ptr(seq_lens), n_req, max_q_len, n_head, n_kv_head, head_dim,
-        page_size, float(scale), int(window), _stream())
+        page_size, float(scale), int(window), int(single_below), _stream())
     if rc == -2:
         return False
     _check(rc, "prefill_attention_bf16")

@@ -60,12 +60,12 @@ def _declare_optional(lib: ctypes.CDLL) -> None:
         "mgpt_fold_layernorm": [P, P, P, P, P, P, P, I, I, P],
         "mgpt_paged_attention_split_bf16": [P, L, P, L, P, P, P, I, P, P, P, I, I, I, I, I, F, I, P],
         "mgpt_paged_attention_split_fast_bf16": [P, L, P, L, P, P, P, I, P, P, P, I, I, I, I, I, F, I, P],
-        "mgpt_paged_attention_decode_bf16": [P, L, P, L, P, P, P, I, P, P, I, I, I, I, I, I, F, I, I, P],
+        "mgpt_paged_attention_decode_bf16": [P, L, P, L, P, P, P, I, P, P, P, I, I, I, I, I, I, F, I, I, P],
         "mgpt_linear_mfma": [P, L, P, P, P, I, L, I, I, I, I, P, L, P],
         "mgpt_linear_mfma_shape": [I, I, P, L, P, P, P, I, L, I, I, I, I, P, L, P],
         "mgpt_linear_mfma_partials": [I, I, I, I],
         "mgpt_linear_mfma_qkv": [P, L, P, P, P, L, I, I, I, P, P, P, I, I, I, I, I, I, P],
-        "mgpt_prefill_attention_bf16": [P, L, P, L, P, P, P, I, P, P, I, I, I, I, I, I, F, I, P],
+        "mgpt_prefill_attention_bf16": [P, L, P, L, P, P, P, I, P, P, I, I, I, I, I, I, F, I, I, P],
     }
     for name, argtypes in table.items():
         fn = getattr(lib, name, None)

@@ -184,3 +184,6 @@ class StepContext:
     host_ctx_lens: Optional[List[int]] = None
     host_state_slots: Optional[List[int]] = None
     exact: bool = False          # true 32-bit path: no fast-math intrinsics
+    padded: bool = False         # rows and requests are padded to a bucket's sizes (n_rows, cu_q.numel() - 1):
+                                 # the host values above then describe the bucket, not the step
+    lead_cap: int = 0            # padded steps: the decoding requests' tokens lie among the first lead_cap

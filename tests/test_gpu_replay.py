@@ -299,3 +299,53 @@ def test_step_shapes_that_repeat_are_replayed_from_a_graph_with_the_same_logits(
     assert rep.runner.num_replayed_steps >= before + 8   # captured again and replayed again
     for i in range(60, 64):                 # and the other request goes on where it stood
         feed(1, "y", other, want_other, i)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_steps_of_a_bucket_are_replayed_from_one_padded_graph(model_folders, dtype, name):
+    """Steps whose shapes never repeat but fall into one bucket of capacities (tokens, requests, logit
+    rows, leading single tokens): the third one makes the bucket's padded graph, the later ones are
+    replays of it with other requests, other cuts and other numbers of single tokens, each checked
+    against the plain implementation; eager steps of another bucket come between them."""
+    cfg = helpers.CONFIGS[name]
+    rng = np.random.default_rng(9)
+    limit = cfg.block_size
+    seqs = {rid: helpers.random_ids(rng, cfg.vocab_size, min(limit, n)) for rid, n in
+            (("a", 60), ("b", 64), ("c", 58), ("d", 40))}
+    pcfg, w = P.read_model_folder(model_folders[name])
+    want = {rid: P.plain_forward(w, pcfg, s).numpy() for rid, s in seqs.items()}
+    rep = TraceReplayer(model_folders[name], dtype, 512, poison=True)
+    assert rep.runner.graph_steps
+    fed = {rid: 0 for rid in seqs}
+    step = 0
+
+    def run(parts):
+        """parts: [(request, tokens to feed)], single tokens first as a scheduler would put them."""
+        nonlocal step
+        entries = []
+        for rid, n in parts:
+            s = fed[rid]
+            entries.append({"id": rid, "tokens": seqs[rid][s:s + n], "want": [n - 1]})
+        got = rep.run_step({"step": step, "entries": entries, "end": []}).cpu()
+        for row, (rid, n) in enumerate(parts):
+            helpers.assert_close(got[row], want[rid][fed[rid] + n - 1], dtype, f"step {step}: {rid} +{n}")
+            fed[rid] += n
+        step += 1
+
+    run([("a", 9), ("b", 3)])           # everyone has a context before the single tokens start
+    run([("c", 2), ("d", 5)])
+    # the bucket: 17..20 tokens, 3..4 requests and logit rows, 1..16 leading single tokens
+    plan = [[("a", 1), ("b", 1), ("c", 15), ("d", 2)],
+            [("d", 1), ("a", 1), ("b", 16)],
+            [("c", 1), ("a", 2), ("b", 14), ("d", 3)],      # third step of the bucket: captured here
+            [("b", 1), ("c", 1), ("d", 1), ("a", 14)],
+            [("a", 1), ("d", 1), ("c", 17)],
+            [("d", 1), ("b", 1), ("a", 1), ("c", 15)],
+            [("c", 1), ("a", 17), ("d", 2)]]
+    before = rep.runner.num_replayed_steps
+    for i, parts in enumerate(plan):
+        run(parts)
+        if i == 3:
+            run([("b", 2)])             # another bucket in between, eagerly
+    assert rep.runner.num_replayed_steps >= before + 4
