@@ -260,6 +260,66 @@ __global__ __launch_bounds__(64 * WVM * WVN) void linear_mfma_kernel(
 
   // lane holds out[row0 + wr + j*16 + (lane & 15)][col0 + wc + i*16 + (lane >> 4)*4 + e], e = 0..3
   const bool vec = (n_out & 3) == 0 && (ldo & 3) == 0 && (((size_t)out | (size_t)bias) & 15) == 0;
+  // bfloat16 outputs go through LDS (the staged operands are done with): a lane's four columns of
+  // sixteen different rows would be sixteen 8-byte pieces per store; from LDS a thread stores 16
+  // bytes and a row's threads a whole stretch of the row, and a key's or value's eight channels
+  // go to their cache page the same way.
+  constexpr int LDT = BN + 8;   // row stride of the tile in LDS
+  constexpr int LDS_ELEMS = 2 * (BM + BN) * MM_LD;
+  // the whole tile at once if it fits, else the rows of one row of waves at a time
+  constexpr int STAGE_ROWS = BM * LDT <= LDS_ELEMS ? BM : BM / WVM;
+  constexpr bool CAN_STAGE = sizeof(OT) == 2 && STAGE_ROWS * LDT <= LDS_ELEMS;
+  if (CAN_STAGE && EPI != MM_EPI_RESIDUAL && (n_out & 7) == 0 && (ldo & 7) == 0 && (((size_t)out) & 15) == 0 &&
+      (EPI != MM_EPI_QKV || ((sc.q_width | sc.kv_width | sc.head_dim) & 7) == 0)) {
+    bf16_t* tile = lds;
+    for (int part = 0; part < BM / STAGE_ROWS; ++part) {
+      __syncthreads();   // the staged operands, or the part before this one, are done with
+      if (wr / STAGE_ROWS == part) {
+#pragma unroll
+        for (int i = 0; i < WTN; ++i) {
+          const int tc = wc + i * 16 + (lane >> 4) * 4, oc = col0 + tc;
+          float b4[4];
+          mfma_bias4(bias, oc < n_out ? oc : 0, n_out, (((size_t)bias) & 15) == 0, b4);
+#pragma unroll
+          for (int j = 0; j < WTM; ++j) {
+            float v[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              v[e] = acc[i][j][e] + b4[e];
+              if (EPI == MM_EPI_GELU) v[e] = gelu_tanh_fast(v[e]);
+            }
+            uint2 pk;
+            pk.x = pack_bf16x2(v[0], v[1]);
+            pk.y = pack_bf16x2(v[2], v[3]);
+            *reinterpret_cast<uint2*>(&tile[(wr - part * STAGE_ROWS + j * 16 + lrow) * LDT + tc]) = pk;
+          }
+        }
+      }
+      __syncthreads();
+      constexpr int CPR = BN / 8;   // 16-byte chunks per tile row
+      for (int c = tid; c < STAGE_ROWS * CPR; c += T) {
+        const int row = c / CPR, tc = (c % CPR) * 8;
+        const int n = row0 + part * STAGE_ROWS + row, oc = col0 + tc;
+        if (n >= n_rows || oc >= n_out) continue;
+        const uint4 v8 = *reinterpret_cast<const uint4*>(&tile[row * LDT + tc]);
+        *reinterpret_cast<uint4*>(reinterpret_cast<bf16_t*>(out) + (long)n * ldo + oc) = v8;
+        if (EPI == MM_EPI_QKV && oc >= sc.q_width) {
+          // the chunk's eight columns lie in one head
+          const int slot = sc.slot_mapping[n];
+          if (slot >= 0) {
+            const int page = slot / sc.page_size, off = slot - page * sc.page_size;
+            const int cq = oc - sc.q_width;  // column among keys then values
+            const bool is_v = cq >= sc.kv_width;
+            const int cc = is_v ? cq - sc.kv_width : cq;
+            const int hh = cc / sc.head_dim, d = cc - hh * sc.head_dim;
+            const long dst = (((long)page * sc.n_kv_head + hh) * sc.page_size + off) * sc.head_dim + d;
+            *reinterpret_cast<uint4*>((is_v ? sc.vpool : sc.kpool) + dst) = v8;
+          }
+        }
+      }
+    }
+    return;
+  }
   // A key or value at (row n, column c of head hh, channel d) goes to
   // ((page * n_kv_head + hh) * page_size + offset) * head_dim + d of its pool, page and offset from
   // the row's slot: the row's part and the column's part of that are worked out once each.
