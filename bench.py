@@ -96,7 +96,7 @@ def prefill_run(args, dtype, reps=5):
     runner, cache = engine.runner, engine.cache
     t_len = min(1024, cfg.block_size)
     rng = np.random.default_rng(1)
-    tokens = rng.integers(0, cfg.vocab_size, 2 * t_len).tolist()
+    tokens = rng.integers(0, cfg.vocab_size, 2 * t_len).astype(np.int32)   # prompts held as arrays, not lists
     times = []
     for rep in range(reps + 2):
         slots = [cache.acquire_slot(), cache.acquire_slot()]
