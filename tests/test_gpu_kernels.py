@@ -416,6 +416,59 @@ def test_paged_attention(kernel, case, window):
     helpers.assert_close(out, c.want(scale, window), dtype, f"{kernel} case {case} window {window}")
 
 
+@pytest.mark.parametrize("window", [0, 33])
+@pytest.mark.parametrize("d", [32, 64])
+def test_prefill_attention_with_many_tiles(d, window):
+    """More than 320 query tiles in the step: the tile kernel then runs with one wave group and two
+    workgroups on a compute unit instead of two wave groups that split the keys."""
+    lens = [130 + 7 * i for i in range(11)]
+    c = PagedCase(seq_lens=lens, q_lens=[70 + (i % 3) for i in range(11)], h=16, hk=4, d=d, page=16,
+                  dtype="bfloat16", seed=d)
+    assert 11 * 2 * 16 > 320
+    out = torch.full((c.n, c.h * c.d), float("nan"), dtype=torch.bfloat16, device=DEV)
+    scale = 1.0 / math.sqrt(d)
+    assert kernels.prefill_attention_bf16(c.q_flat, out, c.kp, c.vp, c.bt, c.cu, c.sl, len(lens), max(c.q_lens),
+                                          c.h, scale, window)
+    helpers.assert_close(out, c.want(scale, window), "bfloat16", f"many tiles, head size {d}")
+
+
+@pytest.mark.parametrize("window", [0, 20])
+def test_single_tokens_and_portions_told_apart_on_the_device(window):
+    """What a padded graph of a step with prompt portions launches: the decode kernel over the first 16
+    tokens, leaving out those of requests with several tokens; the tile kernel over all requests
+    (padded to 8, the padding bringing no tokens), leaving out the single tokens among the first 16.
+    Together they write every token's row once: single tokens before and after the 16th, portions
+    that start before it."""
+    q_lens = [1, 1, 1, 9, 1, 1, 30]            # tokens 0, 1, 2 | 3..11 | 12 | 13 | 14..43: token 13 < 16 <= 14 + 30
+    seq_lens = [50, 1, 77, 40, 200, 18, 64]
+    c = PagedCase(seq_lens=seq_lens, q_lens=q_lens, h=4, hk=2, d=64, page=16, dtype="bfloat16", seed=3)
+    scale = 0.125
+    r_cap, n_cap = 8, 48
+    cu = torch.full((r_cap + 1,), c.n, dtype=torch.int32)
+    cu[:len(q_lens) + 1] = c.cu.cpu()
+    sl = torch.zeros(r_cap, dtype=torch.int32)
+    sl[:len(q_lens)] = c.sl.cpu()
+    bt = torch.full((r_cap, c.bt.shape[1]), -1, dtype=torch.int32)
+    bt[:len(q_lens)] = c.bt.cpu()
+    q_req = torch.full((n_cap,), -1, dtype=torch.int32)
+    q_req[:c.n] = c.q_req.cpu()
+    pos = torch.zeros(n_cap, dtype=torch.int32)
+    pos[:c.n] = torch.tensor([s - ql + j for s, ql in zip(seq_lens, q_lens) for j in range(ql)], dtype=torch.int32)
+    qp = torch.zeros(n_cap, c.q_flat.shape[1], dtype=torch.bfloat16, device=DEV)
+    qp[:c.n] = c.q_flat
+    out = torch.full((n_cap, c.h * c.d), float("nan"), dtype=torch.bfloat16, device=DEV)
+    cu, sl, bt, q_req, pos = (t.to(DEV) for t in (cu, sl, bt, q_req, pos))
+    assert kernels.paged_attention_decode_bf16(qp, out, c.kp, c.vp, bt, pos, q_req, 16, c.h, scale, window, cu_q=cu)
+    singles = [0, 1, 2, 12, 13]
+    others = [t for t in range(c.n) if t not in singles]
+    assert torch.isnan(out[others].float()).all(), "the decode kernel wrote a portion's token"
+    assert not torch.isnan(out[singles].float()).any()
+    assert kernels.prefill_attention_bf16(qp, out, c.kp, c.vp, bt, cu, sl, r_cap, n_cap, c.h, scale, window,
+                                          single_below=16)
+    helpers.assert_close(out[:c.n], c.want(scale, window), "bfloat16", "single tokens and portions together")
+    assert torch.isnan(out[c.n:].float()).all(), "a padded row was written"
+
+
 DECODE_CASES = [
     dict(seq_lens=[600, 1, 64, 65, 513, 300], q_lens=[1] * 6, h=4, hk=2, d=64, page=16),
     dict(seq_lens=[130, 1030, 7], q_lens=[1] * 3, h=3, hk=3, d=128, page=32),
