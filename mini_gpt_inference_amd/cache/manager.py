@@ -23,9 +23,13 @@ class CacheError(RuntimeError):
     pass
 
 
-def _ip(a: np.ndarray):
+def _ip(a):
+    """The address of an int32 array for the library; an address (int) passes through, which lets a
+    caller that fills the same arrays at every step look them up once."""
+    if isinstance(a, int):
+        return a
     assert a.dtype == np.int32 and a.flags["C_CONTIGUOUS"]
-    return a.ctypes.data_as(ctypes.c_void_p)
+    return a.ctypes.data
 
 
 class CacheManager:
@@ -99,15 +103,18 @@ class CacheManager:
     def build_step(self, slots: Sequence[int], ctx_lens: Sequence[int], q_lens: Sequence[int], n_stride: int,
                    r_stride: int, max_blocks: int, positions: np.ndarray, q_req: np.ndarray, cu_q: np.ndarray,
                    seq_lens: np.ndarray, slot_mapping: np.ndarray, block_tables: np.ndarray) -> int:
+        """Fills the step's per-token and per-request arrays (int32 arrays of the strides' sizes, or
+        their addresses, all six alike) and returns the number of tokens."""
         r = len(slots)
         mk = lambda v: np.ascontiguousarray(np.asarray(v, dtype=np.int32).reshape(-1))
         s, c, q = mk(slots), mk(ctx_lens), mk(q_lens)
         if r == 0:
             s = c = q = np.zeros(1, dtype=np.int32)
         g = len(self.groups)
-        assert positions.size >= n_stride and q_req.size >= n_stride and cu_q.size >= r_stride + 1
-        assert seq_lens.size >= r_stride and slot_mapping.size >= g * n_stride
-        assert block_tables.size >= g * r_stride * max_blocks
+        if not isinstance(positions, int):
+            assert positions.size >= n_stride and q_req.size >= n_stride and cu_q.size >= r_stride + 1
+            assert seq_lens.size >= r_stride and slot_mapping.size >= g * n_stride
+            assert block_tables.size >= g * r_stride * max_blocks
         n = self._lib.mgpt_cache_build_step(self._h, r, _ip(s), _ip(c), _ip(q), n_stride, r_stride, max_blocks,
                                             _ip(positions), _ip(q_req), _ip(cu_q), _ip(seq_lens),
                                             _ip(slot_mapping), _ip(block_tables))

@@ -5,8 +5,8 @@
 // with ctx > 0 is the offset-causal case of src/minigpt_infer/batch.py:202-227), scores scaled,
 // softmax and all sums in float32 (src/minigpt_infer/model.py:61-87).
 //
-// A workgroup of four waves takes 64 consecutive queries of one request and one head, 16 per
-// wave.  It walks the keys in blocks of 128 (aligned to multiples of 128 of the key position):
+// A workgroup takes 64 consecutive queries of one request and one head, 16 per wave (four waves,
+// or eight in two groups that share the keys between them, see the kernel).  It walks the keys in blocks of 128 (aligned to multiples of 128 of the key position):
 // the block's key and value rows go to LDS as they are, gathered row by row through the block
 // table, so any page size works and nothing outside [begin, end) is loaded.  LDS holds two
 // blocks: while one is multiplied, the next (fetched from memory into registers a block earlier)
@@ -18,8 +18,7 @@
 // probabilities never leave their registers.  The transposing LDS read of this chip
 // (ds_read_b64_tr_b16) does that: the 16 lanes of a block point at 4 rows x 4 chunks of 4
 // channels, row j / 4 and chunk j % 4 for lane j, and lane i comes back with channel i of the
-// four rows.  Running max, sum and rescaling per query are the
-// usual online softmax, kept short because at head size 64 it, not the MFMAs, is what a block
+// four rows.  Running max, sum and rescaling per query are the usual online softmax, kept short because at head size 64 it, not the MFMAs, is what a block
 // costs: exp2(score * scale' - max) is one fused multiply-add and one v_exp_f32 (scale' holds
 // log2 e), the maximum over the four lanes that share a query goes through two lane swaps
 // instead of LDS, and the row sum stays split over those lanes until the end.
@@ -29,7 +28,6 @@ typedef __attribute__((__vector_size__(8 * sizeof(short)))) short bf16x8_t;
 typedef __attribute__((__vector_size__(4 * sizeof(short)))) short bf16x4_t;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4_t;
 typedef __attribute__((__vector_size__(4 * sizeof(unsigned int)))) unsigned int u32x4_t;
-typedef __attribute__((__vector_size__(2 * sizeof(unsigned int)))) unsigned int u32x2_t;
 
 #define PF_QT 64   // queries per workgroup
 #define PF_KT 128  // keys per block

@@ -74,6 +74,9 @@ class StepArena:
             dv = self.dev_t[off:off + n]
             self.d[name] = dv.view(torch.float32) if typ is np.float32 else dv
             off += _round_up(n, 4)
+        # the addresses of the arrays that the cache manager fills at every step
+        self.h_addr: Dict[str, int] = {name: int(self.h[name].ctypes.data) for name in
+                                       ("positions", "q_req", "cu_q", "seq_lens", "slot_mapping", "block_tables")}
         self.h["seeds"] = self.h["seeds"].view(np.uint64)
         self.d["seeds"] = self.d["seeds"].view(torch.int64)
         self.tokens_out = torch.zeros(m_cap, dtype=torch.int32, device=device)
@@ -164,24 +167,29 @@ class ModelRunner:
         """Fills the arena for requests given by their cache slots: request i brings q_lens[i] tokens
         (its part of the flat `tokens`) on top of ctx_lens[i] cached ones.  logit_rows index `tokens`."""
         arena.host_ready()
-        h = arena.h
-        self.check_positions(ctx_lens, q_lens)
+        h, a = arena.h, arena.h_addr
+        max_seq = self.check_positions(ctx_lens, q_lens)
         n = self.cache.build_step(slots, ctx_lens, q_lens, arena.n_cap, arena.r_cap, arena.max_blocks,
-                                  h["positions"], h["q_req"], h["cu_q"], h["seq_lens"], h["slot_mapping"],
-                                  h["block_tables"])
+                                  a["positions"], a["q_req"], a["cu_q"], a["seq_lens"], a["slot_mapping"],
+                                  a["block_tables"])
         if n != len(tokens):
             raise ValueError(f"the step's requests bring {n} tokens, but {len(tokens)} token ids were given")
-        h["token_ids"][:n] = np.asarray(tokens, dtype=np.int32)
-        h["token_ids"][n:] = 0
+        ids = h["token_ids"]
+        ids[:n] = tokens          # a list or an array
+        ids[n:] = 0
+        # one comparison for both ends: a negative id is a huge unsigned one
+        if n and int(ids[:n].view(np.uint32).max()) >= self.vocab_size:
+            raise ValueError(f"token id outside 0..{self.vocab_size - 1}")
         r, m = len(slots), len(logit_rows)
-        h["state_slots"][:r] = np.asarray(slots, dtype=np.int32)
+        h["state_slots"][:r] = slots
         h["state_slots"][r:] = -1
         rows = np.asarray(logit_rows, dtype=np.int32)
         if m and (rows.min() < 0 or rows.max() >= n):
             raise ValueError("a wanted logit row lies outside the step's tokens")
         h["logit_rows"][:m] = rows
         h["logit_rows"][m:] = 0
-        return self.shape_of(arena, n, r, m, list(q_lens), list(ctx_lens), list(slots))
+        q_lens = list(q_lens)
+        return StepShape(n, r, m, max(q_lens, default=0), max_seq, q_lens, list(ctx_lens), list(slots))
 
     def check_positions(self, ctx_lens: Sequence[int], q_lens: Sequence[int]) -> int:
         """The longest sequence after the step; refuses positions the model does not have
