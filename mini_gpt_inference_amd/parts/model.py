@@ -175,7 +175,10 @@ class DecoderModel:
             layer.arrangement.run(ctx, x, layer.norm1, layer.mixer, layer.norm2, layer.feed_forward, binding,
                                   self.position)
         m = ctx.m_rows
-        logits = ws.get("logits", m, self.spec.vocab_size, torch.float32)
+        # rows start 16 bytes apart at least: the sampling kernel then reads them four floats at a time
+        # whatever the vocabulary's size (50257 is odd)
+        vocab = self.spec.vocab_size
+        logits = ws.get("logits", m, -(-vocab // 4) * 4, torch.float32)[:, :vocab]
         if m:
             self.head.forward(ctx, LazyNorm(self.final_norm, x, m, rows=ctx.logit_rows, buffer="final_normed"),
                               logits, m)
