@@ -64,6 +64,8 @@ def model_spec(cfg: GPTConfig) -> ModelSpec:
         head=PartSpec("linear_head", {"vocab_size": cfg.vocab_size, "width": c, "tied": True},
                       {"weight": "tok_emb.weight"}),
         max_positions=cfg.block_size,
+        # a torch state dict lists the tied head a second time (model.py:128-130)
+        tied_aliases=(("lm_head.weight", "tok_emb.weight"),),
     )
 
 

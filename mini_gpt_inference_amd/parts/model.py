@@ -50,6 +50,8 @@ class ModelSpec:
     final_norm: PartSpec
     head: PartSpec
     max_positions: Optional[int] = None
+    # (duplicate name, tensor it must equal): names a checkpoint may carry beside the tensor they alias
+    tied_aliases: Tuple[Tuple[str, str], ...] = ()
 
 
 @dataclass(frozen=True)

@@ -102,6 +102,6 @@ def load_model(model_dir: str, dtype: str, device: str = "cuda"):
     model = DecoderModel(arch.model_spec(config))
     compute = {"bfloat16": torch.bfloat16, "float32": torch.float32}[dtype]
     tensors = load_tensors(model_dir, model.weight_requests(), compute, torch.device(device),
-                           tied={"lm_head.weight": "tok_emb.weight"})
+                           tied=dict(model.spec.tied_aliases))
     model.bind(tensors)
     return model, config, arch
