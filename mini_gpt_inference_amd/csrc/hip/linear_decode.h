@@ -40,9 +40,11 @@ __global__ __launch_bounds__(256) void linear_decode_kernel(SkinnyArgs a) {
   const int o0 = (SPLIT ? (int)(blockIdx.x / a.k_parts) : (int)blockIdx.x) * 16;
   const int wo = min(o0 + lrow, a.n_out - 1);  // a column past the end reads the last row; never stored
   const int oc = o0 + g * 4;  // this lane's four output columns, of rows lrow + 16 t
+  // rows of this workgroup: with gridDim.y > 1 the rows are dealt out in groups of NT * 16
+  const int r0 = (int)blockIdx.y * (NT * 16) + lrow;
   bool row_ok[NT];
 #pragma unroll
-  for (int t = 0; t < NT; ++t) row_ok[t] = t * 16 + lrow < a.n_rows;
+  for (int t = 0; t < NT; ++t) row_ok[t] = r0 + t * 16 < a.n_rows;
 
   // ---- every load this lane will need, issued before anything waits.  Loads are unconditional
   // within a row (a k step past this wave's range reads the range's first step again and is not
@@ -50,8 +52,8 @@ __global__ __launch_bounds__(256) void linear_decode_kernel(SkinnyArgs a) {
   int src[NT];
 #pragma unroll
   for (int t = 0; t < NT; ++t) {
-    src[t] = t * 16 + lrow;
-    if (LN && a.rows != nullptr && row_ok[t]) src[t] = a.rows[t * 16 + lrow];
+    src[t] = r0 + t * 16;
+    if (LN && a.rows != nullptr && row_ok[t]) src[t] = a.rows[r0 + t * 16];
   }
   // the epilogue's inputs (first wave only)
   const bool col_writer = wave == 0 && oc < a.n_out;
@@ -86,7 +88,7 @@ __global__ __launch_bounds__(256) void linear_decode_kernel(SkinnyArgs a) {
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
       if (!row_ok[t]) continue;
-      const OT* orow = out + (long)(t * 16 + lrow) * a.ldo;
+      const OT* orow = out + (long)(r0 + t * 16) * a.ldo;
       if (EPI == SK_EPI_RESIDUAL) {
         if (VEC) {
           const float4 o4 = *reinterpret_cast<const float4*>(orow + oc);
@@ -96,7 +98,7 @@ __global__ __launch_bounds__(256) void linear_decode_kernel(SkinnyArgs a) {
           for (int i = 0; i < 4; ++i) old4[t][i] = to_float<OT>(orow[min(oc + i, a.n_out - 1)]);
         }
       }
-      if (EPI == SK_EPI_QKV) slot[t] = a.slot_mapping[t * 16 + lrow];
+      if (EPI == SK_EPI_QKV) slot[t] = a.slot_mapping[r0 + t * 16];
     }
   }
 
@@ -160,7 +162,7 @@ __global__ __launch_bounds__(256) void linear_decode_kernel(SkinnyArgs a) {
 #pragma unroll
         for (int i = 0; i < SMAX; ++i) av[t][i] = zero8;
         if (row_ok[t]) {
-          const bf16_t* ap = a.act + (long)(t * 16 + lrow) * a.lda + kb + g * 8;
+          const bf16_t* ap = a.act + (long)(r0 + t * 16) * a.lda + kb + g * 8;
 #pragma unroll
           for (int i = 0; i < SMAX; ++i)
             av[t][i] = *reinterpret_cast<const bf16x8_t*>(ap + (s0 + i < steps ? s0 + i : 0) * 32);
@@ -215,12 +217,12 @@ __global__ __launch_bounds__(256) void linear_decode_kernel(SkinnyArgs a) {
     }
   }
 
-  // ---- epilogue: lane holds out[t * 16 + lrow][oc + i], i = 0..3
+  // ---- epilogue: lane holds out[r0 + t * 16][oc + i], i = 0..3
   if (SPLIT) {
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
       if (!row_ok[t]) continue;
-      float* prow = a.partials + ((long)part * a.n_rows + t * 16 + lrow) * a.n_out + oc;
+      float* prow = a.partials + ((long)part * a.n_rows + r0 + t * 16) * a.n_out + oc;
       *reinterpret_cast<float4*>(prow) = make_float4(acc[t][0], acc[t][1], acc[t][2], acc[t][3]);
     }
     return;
@@ -228,7 +230,7 @@ __global__ __launch_bounds__(256) void linear_decode_kernel(SkinnyArgs a) {
 #pragma unroll
   for (int t = 0; t < NT; ++t) {
     if (!row_ok[t]) continue;
-    OT* orow = out + (long)(t * 16 + lrow) * a.ldo;
+    OT* orow = out + (long)(r0 + t * 16) * a.ldo;
     float v[4];
     float mean = 0.f, rstd = 1.f;
     if (LN) {

@@ -3,6 +3,9 @@
 
 int mgpt_launch_linear_decode_rows(const SkinnyArgs& a, int epilogue, int out_dtype, hipStream_t stream);
 
+#define SK_ROW_GROUPS_MAX_BYTES (6L << 20)
+#define SK_ROW_GROUPS_MAX_K 2048
+
 template <int SMAX>
 static int launch_one_tile(const SkinnyArgs& a, int epilogue, int out_dtype, dim3 grid, hipStream_t s) {
   const bool ln = a.x != nullptr;
@@ -13,6 +16,22 @@ static int launch_one_tile(const SkinnyArgs& a, int epilogue, int out_dtype, dim
             : launch_decode_epi<1, SMAX, false, false>(a, epilogue, out_dtype, grid, s);
 }
 
+// More than 16 rows: the rows either share the W that a workgroup loads (two to four tiles of 16
+// rows per workgroup, linear_decode_rows.hip), or are dealt out in groups of 16 to workgroups of
+// their own, which then are the 16-row kernel at its own pace: the matrix is read once per group,
+// and a small matrix comes out of the L2 (the groups of a column tile run on one XCD when the number
+// of column tiles is a multiple of 8).  The second is faster while the matrix is small and its
+// inner size not long (measured on layer matrices of 0.5 to 19 MB at 17 to 64 rows: at 64 rows
+// [1536 x 512] takes 4.6 us against 6.9 with the LayerNorm kernel that the first way needs,
+// [512 x 2048] 4.6 against 6.3 with its split, [768 x 3072] at 17 rows 6.8 against 5.5,
+// [6400 x 1600] at 64 rows 31.7 against 22.2).
+bool mgpt_linear_decode_row_groups(int n_rows, int n_out, int k_dim, int rows_mode) {
+  if (n_rows <= 16 || n_rows > 64 || (k_dim % 32) != 0) return false;
+  if (rows_mode == SK_ROWS_GROUPS) return true;
+  if (rows_mode == SK_ROWS_SHARE_W) return false;
+  return k_dim <= SK_ROW_GROUPS_MAX_K && (long)n_out * k_dim * (long)sizeof(bf16_t) <= SK_ROW_GROUPS_MAX_BYTES;
+}
+
 // The caller (mgpt_linear_skinny) has checked pointers, strides and the scatter's sizes.  Takes up
 // to 64 rows and any k_dim that is a multiple of 32; more than 16 rows only with an epilogue that
 // can use vectors of four.
@@ -21,9 +40,10 @@ int mgpt_launch_linear_decode(const SkinnyArgs& a, int epilogue, int out_dtype, 
   // the scatter stores four neighbouring columns of a head at once
   if (epilogue == SK_EPI_QKV && ((a.n_out % 16) != 0 || (a.ldo % 4) != 0 || (((size_t)a.out) & 15) != 0))
     return MGPT_ERR_BAD_SHAPE;
-  if (a.n_rows > 16) return mgpt_launch_linear_decode_rows(a, epilogue, out_dtype, stream);
+  if (a.n_rows > 16 && !mgpt_linear_decode_row_groups(a.n_rows, a.n_out, a.k_dim, a.rows_mode))
+    return mgpt_launch_linear_decode_rows(a, epilogue, out_dtype, stream);
   const int per = (a.k_dim / 32 + 3) / 4;  // k steps of the first waves
-  dim3 grid((a.n_out + 15) / 16);
+  dim3 grid((a.n_out + 15) / 16, (a.n_rows + 15) / 16);
   if (per <= 4) return launch_one_tile<4>(a, epilogue, out_dtype, grid, stream);
   if (per <= 8) return launch_one_tile<8>(a, epilogue, out_dtype, grid, stream);
   return launch_one_tile<16>(a, epilogue, out_dtype, grid, stream);  // longer ranges: several passes

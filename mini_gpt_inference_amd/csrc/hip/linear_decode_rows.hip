@@ -37,8 +37,9 @@ static int launch_tiles_unaligned_head(const SkinnyArgs& a, hipStream_t s) {
 // order and applies bias, GELU or the residual add.
 #define LDR_PARTS 4
 
-long mgpt_linear_decode_partials(int n_rows, int n_out, int k_dim, bool ln, int epilogue) {
+long mgpt_linear_decode_partials(int n_rows, int n_out, int k_dim, bool ln, int epilogue, int rows_mode) {
   if (ln || epilogue == SK_EPI_QKV || n_rows <= 16 || n_rows > 64) return 0;
+  if (mgpt_linear_decode_row_groups(n_rows, n_out, k_dim, rows_mode)) return 0;
   if (k_dim < 1024 || (k_dim % (32 * LDR_PARTS)) != 0 || (n_out % 16) != 0 || n_out / 16 >= 128) return 0;
   return (long)LDR_PARTS * n_rows * n_out;
 }
@@ -106,7 +107,7 @@ static int launch_split(const SkinnyArgs& a0, int epilogue, int out_dtype, hipSt
 int mgpt_launch_linear_decode_rows(const SkinnyArgs& a, int epilogue, int out_dtype, hipStream_t stream) {
   const int nt = (a.n_rows + 15) / 16;
   if (a.partials != nullptr && decode_vec_ok(a) &&
-      mgpt_linear_decode_partials(a.n_rows, a.n_out, a.k_dim, a.x != nullptr, epilogue) > 0) {
+      mgpt_linear_decode_partials(a.n_rows, a.n_out, a.k_dim, a.x != nullptr, epilogue, a.rows_mode) > 0) {
     switch (nt) {
       case 2: return launch_split<2>(a, epilogue, out_dtype, stream);
       case 3: return launch_split<3>(a, epilogue, out_dtype, stream);

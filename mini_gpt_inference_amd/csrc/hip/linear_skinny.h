@@ -10,6 +10,9 @@ typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4_t;
 #define SK_EPI_RESIDUAL 2
 #define SK_EPI_QKV 3
 
+#define SK_ROWS_SHARE_W 2
+#define SK_ROWS_GROUPS 3
+
 #define SK_WAVES 4        // waves of a workgroup without a prologue
 #define SK_LN_WAVES 16    // waves of a workgroup with the LayerNorm prologue: one row each
 
@@ -31,6 +34,9 @@ struct SkinnyArgs {
   // partials[part][row][column] and a second kernel adds them and applies the epilogue
   float* partials;
   int k_parts;
+  // more than 16 rows in linear_decode.hip: 0 = the launcher chooses, SK_ROWS_SHARE_W = one workgroup
+  // per column tile takes all rows, SK_ROWS_GROUPS = one workgroup per column tile and 16 rows
+  int rows_mode;
   // key/value scatter (SK_EPI_QKV)
   bf16_t* kpool;
   bf16_t* vpool;
@@ -42,4 +48,6 @@ struct SkinnyArgs {
 // MGPT_ERR_BAD_SHAPE for what it does not take (the general kernel then runs).
 int mgpt_launch_linear_decode(const SkinnyArgs& a, int epilogue, int out_dtype, hipStream_t stream);
 // floats of partial sums the split over workgroups needs for this shape; 0: no split
-long mgpt_linear_decode_partials(int n_rows, int n_out, int k_dim, bool ln, int epilogue);
+long mgpt_linear_decode_partials(int n_rows, int n_out, int k_dim, bool ln, int epilogue, int rows_mode);
+// whether 17 to 64 rows of this shape go to one workgroup per column tile and 16 rows
+bool mgpt_linear_decode_row_groups(int n_rows, int n_out, int k_dim, int rows_mode);

@@ -300,8 +300,9 @@ static int launch_nt(const SkinnyArgs& a, int epi, int out_dtype, dim3 grid, siz
 // With x given (then act is ignored) the rows are read from the float32 residual stream through
 // a LayerNorm whose gain and bias were folded into w, bias and colsum (fold_norm.hip); otherwise
 // act holds bfloat16 activations.  Refuses (MGPT_ERR_BAD_SHAPE) more than 64 rows and k_dim that
-// is no multiple of 16; the caller then takes the general kernels.  general_only != 0 keeps to this
-// file's kernel also where linear_decode.hip would take the shape.  w_packed: optional, the
+// is no multiple of 16; the caller then takes the general kernels.  mode: 0 = the launcher chooses;
+// 1 keeps to this file's kernel also where linear_decode.hip would take the shape; SK_ROWS_SHARE_W
+// and SK_ROWS_GROUPS say how linear_decode.hip treats more than 16 rows (see there).  w_packed: optional, the
 // same matrix in mgpt_pack_weight's layout (only linear_decode.hip reads it).  partials: optional scratch of
 // mgpt_linear_skinny_partials(...) floats; with it a long inner size with many rows is split over
 // workgroups (two launches).
@@ -310,7 +311,7 @@ extern "C" int mgpt_linear_skinny(const void* act, long lda, const float* x, con
                                   const float* bias, void* out, int out_dtype, long ldo, int n_rows,
                                   int n_out, int k_dim, int epilogue, void* kpool, void* vpool,
                                   const int* slot_mapping, int q_width, int kv_width, int head_dim,
-                                  int n_kv_head, int page_size, int general_only, float* partials,
+                                  int n_kv_head, int page_size, int mode, float* partials,
                                   long partials_floats, hipStream_t stream) {
   if (n_rows == 0 || n_out == 0) return MGPT_OK;
   if (!w || !out || (!act && !x)) return MGPT_ERR_NULL;
@@ -348,9 +349,11 @@ extern "C" int mgpt_linear_skinny(const void* act, long lda, const float* x, con
   a.n_kv_head = n_kv_head; a.page_size = page_size;
   // room for the parts of a split over workgroups, if the caller brought enough of it
   a.k_parts = 1;
-  a.partials = (partials && partials_floats >= mgpt_linear_decode_partials(n_rows, n_out, k_dim, ln, epilogue))
+  a.rows_mode = (mode == SK_ROWS_SHARE_W || mode == SK_ROWS_GROUPS) ? mode : 0;
+  a.partials = (partials && partials_floats >= mgpt_linear_decode_partials(n_rows, n_out, k_dim, ln, epilogue,
+                                                                           a.rows_mode))
                    ? partials : nullptr;
-  if (!general_only) {
+  if (mode != 1) {
     // the rows of a decode step: the kernel laid out for latency, where it takes the shape
     const int rc = mgpt_launch_linear_decode(a, epilogue, out_dtype, stream);
     if (rc != MGPT_ERR_BAD_SHAPE) return rc;
@@ -377,5 +380,11 @@ extern "C" int mgpt_linear_skinny(const void* act, long lda, const float* x, con
 
 // floats of scratch with which mgpt_linear_skinny splits this shape's inner size over workgroups; 0: it would not
 extern "C" long mgpt_linear_skinny_partials(int n_rows, int n_out, int k_dim, int has_ln, int epilogue) {
-  return mgpt_linear_decode_partials(n_rows, n_out, k_dim, has_ln != 0, epilogue);
+  return mgpt_linear_decode_partials(n_rows, n_out, k_dim, has_ln != 0, epilogue, 0);
+}
+
+// 1 if mgpt_linear_skinny, left to choose, deals the rows of this shape out in groups of 16 (then a
+// folded LayerNorm costs a workgroup no more than at 16 rows)
+extern "C" int mgpt_linear_skinny_row_groups(int n_rows, int n_out, int k_dim) {
+  return mgpt_linear_decode_row_groups(n_rows, n_out, k_dim, 0) ? 1 : 0;
 }

@@ -283,7 +283,8 @@ def linear_skinny(a: Optional[torch.Tensor], w: torch.Tensor, bias: Optional[tor
                   n_rows: int, epilogue: int = EPI_NONE, *, ln_x: Optional[torch.Tensor] = None,
                   ln_colsum: Optional[torch.Tensor] = None, ln_eps: float = 0.0,
                   ln_rows: Optional[torch.Tensor] = None, scatter=None, general_only: bool = False,
-                  partials: Optional[torch.Tensor] = None, w_packed: Optional[torch.Tensor] = None) -> bool:
+                  partials: Optional[torch.Tensor] = None, w_packed: Optional[torch.Tensor] = None,
+                  rows_mode: int = 0) -> bool:
     """bfloat16 MFMA product for at most 64 rows.  With ln_x (the float32 residual stream; ln_rows an
     optional gather) the rows are read through a LayerNorm that fold_layer_norm folded into w, bias
     and ln_colsum.  scatter = (k_pool, v_pool, slot_mapping, q_width, kv_width) also stores the new
@@ -291,7 +292,8 @@ def linear_skinny(a: Optional[torch.Tensor], w: torch.Tensor, bias: Optional[tor
     to the kernel laid out for a decode step's latency unless general_only is set.  partials:
     float32 scratch of linear_skinny_partials(...) elements, with which a long inner size under many
     rows is split over workgroups.  w_packed: pack_weight(w), which the decode kernel reads faster
-    than w itself.  Returns False, having launched nothing, when the kernel does not take the shape."""
+    than w itself.  rows_mode: how the decode kernel treats 17 to 64 rows (0: it chooses, ROWS_SHARE_W:
+    one workgroup per column tile takes all rows, ROWS_GROUPS: one per column tile and 16 rows).  Returns False, having launched nothing, when the kernel does not take the shape."""
     if n_rows > _SKINNY_MAX_ROWS or w.dtype != torch.bfloat16:
         return False
     n_out, k_dim = w.shape
@@ -346,7 +348,7 @@ def linear_skinny(a: Optional[torch.Tensor], w: torch.Tensor, bias: Optional[tor
         _ptr(a if ln_x is None else None), lda, _ptr(ln_x), _ptr(ln_rows), _ptr(ln_colsum),
         float(ln_eps), _ptr(w), _ptr(w_packed), _ptr(bias), _ptr(out), _dtype_code(out), out.stride(0), n_rows,
         n_out, k_dim, epilogue, _ptr(kp), _ptr(vp), _ptr(sm), q_width, kv_width, head_dim, n_kv_head, page_size,
-        1 if general_only else 0, _ptr(partials), 0 if partials is None else partials.numel(), _stream())
+        1 if general_only else rows_mode, _ptr(partials), 0 if partials is None else partials.numel(), _stream())
     if rc == -2:
         return False
     _check(rc, "linear_skinny")
@@ -365,6 +367,15 @@ def pack_weight(w: torch.Tensor) -> Optional[torch.Tensor]:
     packed = torch.empty(-(-n_out // 16) * 16 * k_dim, dtype=torch.bfloat16, device=w.device)
     _check(library.kernels().mgpt_pack_weight(_ptr(w), _ptr(packed), n_out, k_dim, _stream()), "pack_weight")
     return packed
+
+
+ROWS_SHARE_W, ROWS_GROUPS = 2, 3
+
+
+def linear_skinny_row_groups(n_rows: int, n_out: int, k_dim: int) -> bool:
+    """Whether linear_skinny, left to choose, gives every 16 of these rows workgroups of their own
+    (a folded LayerNorm then costs a workgroup what it costs at 16 rows)."""
+    return bool(library.kernels().mgpt_linear_skinny_row_groups(n_rows, n_out, k_dim))
 
 
 def linear_skinny_partials(n_rows: int, n_out: int, k_dim: int, has_ln: bool, epilogue: int) -> int:

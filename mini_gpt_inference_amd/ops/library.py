@@ -57,6 +57,7 @@ def _declare_optional(lib: ctypes.CDLL) -> None:
         "mgpt_linear_skinny": [P, L, P, P, P, F, P, P, P, P, I, L, I, I, I, I, P, P, P, I, I, I, I, I, I, P, L, P],
         "mgpt_pack_weight": [P, P, I, I, P],
         "mgpt_linear_skinny_partials": [I, I, I, I, I],
+        "mgpt_linear_skinny_row_groups": [I, I, I],
         "mgpt_fold_layernorm": [P, P, P, P, P, P, P, I, I, P],
         "mgpt_paged_attention_split_bf16": [P, L, P, L, P, P, P, I, P, P, P, I, I, I, I, I, F, I, P],
         "mgpt_paged_attention_split_fast_bf16": [P, L, P, L, P, P, P, I, P, P, P, I, I, I, I, I, F, I, P],

@@ -64,6 +64,17 @@ def packed_weight(w: torch.Tensor) -> Optional[torch.Tensor]:
     return d["packed"]
 
 
+# A LayerNorm is folded into the product that reads it only for this many rows and for outputs this
+# wide at most: every column tile converts the float32 residual rows it multiplies, which beyond
+# these costs more than a LayerNorm kernel of its own.
+FOLD_MAX_ROWS = 32
+FOLD_MAX_OUT = 4096
+# A very wide output (the head) goes to the decode kernel up to this many rows, and a long inner size
+# is split over workgroups (a second kernel then adds the parts) from more than this many rows on.
+WIDE_OUT_DECODE_ROWS = 16
+SPLIT_MIN_ROWS = 16
+
+
 def as_tensor(ctx, a: Union[torch.Tensor, LazyNorm]) -> torch.Tensor:
     return a.tensor(ctx) if isinstance(a, LazyNorm) else a
 
@@ -84,20 +95,20 @@ def linear(ctx, a: Union[torch.Tensor, LazyNorm], w: torch.Tensor, bias: Optiona
     # A very wide output (the head) with more than a few rows: the tiled kernel streams the matrix
     # at the same rate whatever the rows, the decode kernel slows down with every row it adds
     # (measured at 50k outputs: even at 16 rows, 1.8 times slower at 64).
-    wide_out = n_rows > 16 and w.shape[0] >= 8192
+    wide_out = n_rows > WIDE_OUT_DECODE_ROWS and w.shape[0] >= 8192
     if fast and n_rows <= 64 and not wide_out:
         epi = kernels.SK_EPI_QKV if scatter is not None else epilogue
-        # every column tile converts the residual rows it multiplies: beyond 32 rows, or for a very
-        # wide output (the head), that costs more than a LayerNorm kernel of its own
         if (isinstance(a, LazyNorm) and getattr(a.norm, "fusable_layer_norm", False) and a._tensor is None
-                and n_rows <= 32 and w.shape[0] <= 4096):
+                and w.shape[0] <= FOLD_MAX_OUT
+                and (n_rows <= FOLD_MAX_ROWS or kernels.linear_skinny_row_groups(n_rows, w.shape[0], w.shape[1]))):
             wf, colsum, bias_f = folded_layer_norm(a.norm, w, bias)
             if kernels.linear_skinny(None, wf, bias_f, out, n_rows, epi, ln_x=a.x, ln_colsum=colsum,
                                      ln_eps=a.norm.eps, ln_rows=a.rows, scatter=scatter,
                                      w_packed=packed_weight(wf)):
                 return scatter is not None
         partials = None
-        need = kernels.linear_skinny_partials(n_rows, w.shape[0], w.shape[1], False, epi) if n_rows > 16 else 0
+        need = kernels.linear_skinny_partials(n_rows, w.shape[0], w.shape[1], False, epi) \
+            if n_rows > SPLIT_MIN_ROWS else 0
         if need:
             partials = ctx.workspace.get("linear_partials", need, 1, torch.float32)
         if kernels.linear_skinny(as_tensor(ctx, a), w, bias, out, n_rows, epi, scatter=scatter, partials=partials,

@@ -112,6 +112,13 @@ def test_linear_skinny(n, k, o, epi, o_dt, general):
         out_p = prev.clone().to(DEV)
         assert kernels.linear_skinny(a.to(DEV), w.to(DEV), bias.to(DEV), out_p, n, epi, w_packed=packed)
         assert torch.equal(out_p, out), "the packed matrix gives another result"
+        # more than 16 rows: all rows in one workgroup per column tile, or 16 rows to a workgroup
+        for mode in (kernels.ROWS_SHARE_W, kernels.ROWS_GROUPS):
+            out_m = prev.clone().to(DEV)
+            assert kernels.linear_skinny(a.to(DEV), w.to(DEV), bias.to(DEV), out_m, n, epi, w_packed=packed,
+                                         rows_mode=mode)
+            helpers.assert_close(out_m[:n], _linear_want(a, w, bias, epi, prev)[:n], "bfloat16", f"rows mode {mode}")
+            assert torch.equal(out_m[n:], prev[n:].to(DEV)), "rows beyond n_rows were written"
     helpers.assert_close(out[:n], _linear_want(a, w, bias, epi, prev)[:n], "bfloat16", f"skinny {n}x{k}x{o}")
     assert torch.equal(out[n:], prev[n:].to(DEV)), "rows beyond n_rows were written"
     out2 = prev.clone().to(DEV)
@@ -237,20 +244,34 @@ def test_linear_skinny_through_a_folded_layer_norm(n, k, o, ln_bias, gather, gen
         assert torch.equal(out_p, out), "the packed matrix gives another result"
     h = P.plain_layer_norm(x.double()[rows], lw.double(), lb.double() if ln_bias else None, 1e-5)
     helpers.assert_close(out, P.plain_linear(h, w.double(), bias.double()), "bfloat16", "LN + skinny")
+    if not general and k % 32 == 0:
+        for mode in (kernels.ROWS_SHARE_W, kernels.ROWS_GROUPS):
+            out_m = torch.full((n + 1, o), float("nan"), dtype=torch.float32, device=DEV)
+            assert kernels.linear_skinny(None, wf, bias_f, out_m, n, kernels.EPI_NONE, ln_x=x.to(DEV),
+                                         ln_colsum=colsum, ln_eps=1e-5, ln_rows=i32(rows) if gather else None,
+                                         rows_mode=mode)
+            helpers.assert_close(out_m[:n], P.plain_linear(h, w.double(), bias.double()), "bfloat16",
+                                 f"LN + skinny, rows mode {mode}")
+            assert torch.isnan(out_m[n:]).all(), "rows beyond n_rows were written"
 
 
-@pytest.mark.parametrize("general", [False, True])
-def test_linear_skinny_stores_keys_and_values(general):
+@pytest.mark.parametrize("general,n,rows_mode", [(False, 6, 0), (True, 6, 0), (True, 40, 0),
+                                                 (False, 40, kernels.ROWS_SHARE_W), (False, 40, kernels.ROWS_GROUPS),
+                                                 (False, 64, kernels.ROWS_GROUPS)])
+def test_linear_skinny_stores_keys_and_values(general, n, rows_mode):
     g = torch.Generator().manual_seed(5)
-    n, k, h, hk, d, page, pages = 6, 64, 4, 2, 16, 4, 9
+    k, h, hk, d, page, pages = 64, 4, 2, 16, 4, 23
     qw, kvw = h * d, hk * d
     a, w, bias = rnd(g, n, k, dtype="bfloat16"), rnd(g, qw + 2 * kvw, k, dtype="bfloat16", scale=0.2), rnd(g, qw + 2 * kvw)
     kp = torch.full((pages, hk, page, d), float("nan"), dtype=torch.bfloat16, device=DEV)
     vp = kp.clone()
     slots = [4 * 8 + 3, 0, 7, -1, 4 * 2 + 1, 4 * 8 + 0]
+    if n > 6:   # distinct slots all over the pool, a padded token now and then
+        slots = torch.randperm(pages * page, generator=g)[:n].tolist()
+        slots = [-1 if t % 9 == 4 else s for t, s in enumerate(slots)]
     out = torch.empty(n, qw + 2 * kvw, dtype=torch.bfloat16, device=DEV)
     assert kernels.linear_skinny(a.to(DEV), w.to(DEV), bias.to(DEV), out, n, kernels.SK_EPI_QKV,
-                                 scatter=(kp, vp, i32(slots), qw, kvw), general_only=general)
+                                 scatter=(kp, vp, i32(slots), qw, kvw), general_only=general, rows_mode=rows_mode)
     want = P.plain_linear(a.double(), w.double(), bias.double())
     helpers.assert_close(out, want, "bfloat16", "qkv")
     written = torch.zeros(pages * page, dtype=torch.bool)
@@ -271,11 +292,15 @@ def test_linear_skinny_stores_keys_and_values(general):
 @pytest.mark.parametrize("epi,o_dt", [(kernels.EPI_NONE, "bfloat16"), (kernels.EPI_NONE, "float32"),
                                       (kernels.EPI_GELU, "bfloat16"), (kernels.EPI_RESIDUAL, "float32")])
 def test_linear_skinny_with_the_inner_size_split_over_workgroups(n, k, o, epi, o_dt):
-    """With scratch for the parts, a long inner size under more than 16 rows runs as two launches; the
-    result is the unsplit kernel's up to the order of four sums."""
+    """With scratch for the parts, a long inner size under more than 16 rows whose rows stay in one
+    workgroup per column tile runs as two launches; the result is the unsplit kernel's up to the order
+    of four sums.  Left to choose, the launcher splits only what it does not deal out in groups of
+    16 rows (a small matrix with an inner size up to 2048)."""
     g = torch.Generator().manual_seed(16)
-    need = kernels.linear_skinny_partials(n, o, k, False, epi)
-    assert need == 4 * n * o
+    need = 4 * n * o
+    groups = kernels.linear_skinny_row_groups(n, o, k)
+    assert groups == (k <= 2048 and o * k * 2 <= 6 << 20)
+    assert kernels.linear_skinny_partials(n, o, k, False, epi) == (0 if groups else need)
     assert kernels.linear_skinny_partials(16, o, k, False, epi) == 0          # few rows: one launch is as fast
     assert kernels.linear_skinny_partials(n, o, 512, False, epi) == 0         # a short inner size
     assert kernels.linear_skinny_partials(n, o, k, True, epi) == 0            # not through a folded LayerNorm
@@ -285,12 +310,16 @@ def test_linear_skinny_with_the_inner_size_split_over_workgroups(n, k, o, epi, o
     for b in (bias, None):
         out = prev.clone().to(DEV)
         assert kernels.linear_skinny(a.to(DEV), w.to(DEV), None if b is None else b.to(DEV), out, n, epi,
-                                     partials=partials)
+                                     partials=partials, rows_mode=kernels.ROWS_SHARE_W)
+        assert not torch.isnan(partials[:need]).any(), "the parts were not written: no split happened"
+        partials.fill_(float("nan"))
         helpers.assert_close(out[:n], _linear_want(a, w, b, epi, prev)[:n], "bfloat16", f"split {n}x{k}x{o}")
         assert torch.equal(out[n:], prev[n:].to(DEV)), "rows beyond n_rows were written"
     # too little scratch: the unsplit kernel, same result
     out2 = prev.clone().to(DEV)
-    assert kernels.linear_skinny(a.to(DEV), w.to(DEV), bias.to(DEV), out2, n, epi, partials=partials[:need // 2])
+    assert kernels.linear_skinny(a.to(DEV), w.to(DEV), bias.to(DEV), out2, n, epi, partials=partials[:need // 2],
+                                 rows_mode=kernels.ROWS_SHARE_W)
+    assert torch.isnan(partials).all(), "too little scratch was written to"
     helpers.assert_close(out2[:n], _linear_want(a, w, bias, epi, prev)[:n], "bfloat16", "unsplit")
 
 

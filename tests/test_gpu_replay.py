@@ -172,6 +172,35 @@ def test_long_decoding_and_first_tokens(model_folders, dtype):
         rep.run_step({"step": 999, "entries": [{"id": "x", "tokens": [1], "want": [0]}], "end": []})
 
 
+@pytest.mark.parametrize("n_req", [17, 40, 64])
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_many_requests_decoding_together(model_folders, name, dtype, n_req):
+    """Decode steps of 17 to 64 requests (where the products deal the rows out in groups of 16, or
+    share the matrix between them): prompts of different lengths enter a few at a time, then all
+    requests bring one token a step."""
+    cfg = helpers.CONFIGS[name]
+    rng = np.random.default_rng(21)
+    n_dec = 6
+    reqs = {f"r{i}": helpers.random_ids(rng, cfg.vocab_size, int(rng.integers(1, cfg.block_size - n_dec)) + n_dec)
+            for i in range(n_req)}
+    pcfg, w = P.read_model_folder(model_folders[name])
+    want = {rid: P.plain_forward(w, pcfg, ids).numpy() for rid, ids in reqs.items()}
+    plan = helpers.TracePlan()
+    rids = list(reqs)
+    for i in range(0, n_req, 5):       # prompts, five requests a step
+        plan.add_step([(r, reqs[r][:-n_dec], len(reqs[r])) for r in rids[i:i + 5]])
+    for j in range(n_dec, 0, -1):      # then every request's next token, all in one step
+        plan.add_step([(r, reqs[r][len(reqs[r]) - j:len(reqs[r]) - j + 1], len(reqs[r])) for r in rids],
+                      end=rids if j == 1 else [])
+    replayer = TraceReplayer(model_folders[name], dtype, plan.tight_tokens(16), max_live=n_req, poison=True)
+    got = plan.assemble(helpers.run_plan_in_process(replayer, plan), {r: len(t) for r, t in reqs.items()},
+                        cfg.vocab_size)
+    for rid in reqs:
+        helpers.assert_close(got[rid], want[rid], dtype, f"{name} {dtype} {n_req} requests, {rid}")
+    assert replayer.cache.check() == 0 and replayer.cache.num_free_pages() == replayer.num_pages
+
+
 def _far_key_edit(tensors):
     """Makes the last query of the LONG model look mostly at one far key whose value is the
     opposite of its own.  Queries and keys share one enlarged projection that reads the first 40
