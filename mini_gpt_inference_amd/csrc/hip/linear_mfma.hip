@@ -418,6 +418,14 @@ long tiles_of(int shape, int n_rows, int n_out) {
 // The largest tile that still fills the machine's 256 compute units.  The two largest shapes run
 // one workgroup per unit, so what counts for them is also how full their last round is.
 int choose_shape(int n_rows, int n_out) {
+  // Few rows under a wide output (the head of a decode step, 50k columns): the product is a pass over
+  // the matrix, and a tile taller than the rows only makes each workgroup's share of that pass
+  // larger.  Measured at 50304 x 512 (and alike at inner sizes 768 and 1600): 32 rows take 11.4 us
+  // with 32 x 32 tiles and 17.9 with 256 x 256, 64 rows 13.9 with 64 x 64 and 19.3, 128 rows 17.5
+  // with 128 x 256 and 22.4; from 256 rows on the largest tile is the fastest again.
+  if (n_rows <= 32 && tiles_of(4, n_rows, n_out) >= 256) return 4;
+  if (n_rows <= 64 && tiles_of(3, n_rows, n_out) >= 256) return 3;
+  if (n_rows <= 128 && tiles_of(1, n_rows, n_out) >= 160) return 1;
   for (int shape = 0; shape < 2; ++shape) {
     const long t = tiles_of(shape, n_rows, n_out);
     const long rounds = (t + 255) / 256;

@@ -64,14 +64,22 @@ def packed_weight(w: torch.Tensor) -> Optional[torch.Tensor]:
     return d["packed"]
 
 
-# A LayerNorm is folded into the product that reads it only for this many rows and for outputs this
-# wide at most: every column tile converts the float32 residual rows it multiplies, which beyond
-# these costs more than a LayerNorm kernel of its own.
+# A LayerNorm is folded into the product that reads it only for outputs this wide at most, and for
+# this many rows unless the decode kernel deals the rows out in groups of 16: every workgroup
+# converts the float32 residual rows it multiplies, which beyond these costs more than a LayerNorm
+# kernel of its own (at 64 rows in one workgroup the decode step of the 50.9M model took 0.397 ms
+# with the fold and 0.375 ms without).
 FOLD_MAX_ROWS = 32
 FOLD_MAX_OUT = 4096
-# A very wide output (the head) goes to the decode kernel up to this many rows, and a long inner size
-# is split over workgroups (a second kernel then adds the parts) from more than this many rows on.
-WIDE_OUT_DECODE_ROWS = 16
+# A very wide output (the head, 8192 columns and more) goes to the decode kernel while rows x inner
+# size stays within this, and to the tiled kernel beyond: that one streams the matrix at nearly the
+# same rate whatever the rows (50304 x 512: 10.2 us at 1 row, 11.4 at 32, 14.0 at 64), the decode
+# kernel is ahead by up to a microsecond at few rows and a short inner size and slows down with every
+# row (9.4, 16.4, 28.5 us; at an inner size of 1600 it is behind from 4 rows on).
+WIDE_OUT = 8192
+WIDE_OUT_DECODE_WORK = 8192
+# A long inner size is split over workgroups (a second kernel then adds the parts) from more than
+# this many rows on.
 SPLIT_MIN_ROWS = 16
 
 
@@ -83,7 +91,7 @@ def linear(ctx, a: Union[torch.Tensor, LazyNorm], w: torch.Tensor, bias: Optiona
            out: torch.Tensor, n_rows: int, epilogue: int = kernels.EPI_NONE, scatter=None) -> bool:
     """out[:n_rows] = a[:n_rows] @ w.T (+ bias) with the epilogue.
 
-    On the bfloat16 path up to 64 rows (16 for a very wide output) go to the decode step's MFMA kernels (reading the residual
+    On the bfloat16 path up to 64 rows (fewer for a very wide output) go to the decode step's MFMA kernels (reading the residual
     stream through the folded LayerNorm when `a` is a LazyNorm of a fusable norm and the rows are
     few; splitting a long inner size over workgroups when the rows are many) and more rows to the
     tiled MFMA kernel (which also splits a long inner size when its tiles are few); the 32-bit path, and every shape those refuse, go to the 32-bit FMA kernel.  `scatter` = (k_pool, v_pool,
@@ -92,10 +100,7 @@ def linear(ctx, a: Union[torch.Tensor, LazyNorm], w: torch.Tensor, bias: Optiona
     if n_rows == 0:
         return scatter is not None
     fast = w.dtype == torch.bfloat16 and not ctx.exact and ctx.dtype == torch.bfloat16
-    # A very wide output (the head) with more than a few rows: the tiled kernel streams the matrix
-    # at the same rate whatever the rows, the decode kernel slows down with every row it adds
-    # (measured at 50k outputs: even at 16 rows, 1.8 times slower at 64).
-    wide_out = n_rows > WIDE_OUT_DECODE_ROWS and w.shape[0] >= 8192
+    wide_out = w.shape[0] >= WIDE_OUT and n_rows * w.shape[1] > WIDE_OUT_DECODE_WORK
     if fast and n_rows <= 64 and not wide_out:
         epi = kernels.SK_EPI_QKV if scatter is not None else epilogue
         if (isinstance(a, LazyNorm) and getattr(a.norm, "fusable_layer_norm", False) and a._tensor is None
