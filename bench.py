@@ -36,7 +36,7 @@ def build_engine(args, batch, dtype):
     pages = batch * (-(-args.positions // args.kv_block)) + 8
     ecfg = EngineConfig(block_size=args.kv_block, num_blocks=pages, max_batch_size=max(batch, 2),
                         max_num_batched_tokens=max(4096, batch * args.prompt), dtype=dtype,
-                        use_graph=not args.no_graph, decode_burst=args.burst)
+                        use_graph=not args.no_graph, decode_burst=args.burst, decode_chain=args.chain)
     return LLMEngine.from_random(cfg, seed=0, engine_config=ecfg), cfg
 
 
@@ -49,7 +49,7 @@ def decode_run(args, batch, steps, warmup, dtype):
 
     engine, cfg = build_engine(args, batch, dtype)
     rng = np.random.default_rng(0)
-    budget = steps + warmup + 2 * args.burst + 2
+    budget = steps + warmup + 2 * args.burst * args.chain + 2
     assert args.prompt + budget <= cfg.block_size, "prompt + decode steps exceed the model's positions"
     for i in range(batch):
         engine.add_request(Request(f"b{i}", rng.integers(0, cfg.vocab_size, args.prompt).tolist(),
@@ -62,7 +62,7 @@ def decode_run(args, batch, steps, warmup, dtype):
         """engine.step() until exactly n more decode steps have run (a call may run a burst of them)."""
         first, tokens = sched.num_steps, sched.num_decode_tokens
         while sched.num_steps - first < n:
-            engine.step()
+            engine.step(max_decode_steps=n - (sched.num_steps - first))
         assert sched.num_steps - first == n, "the decode bursts do not divide the number of steps"
         assert sched.num_decode_tokens - tokens == n * batch, "a request dropped out of the decode steps"
 
@@ -154,7 +154,7 @@ def serve_run(args, name):
     pages = max(int(demand * w["pool_frac"]), -(-cfg.block_size // args.kv_block) + 1)
     ecfg = EngineConfig(block_size=args.kv_block, num_blocks=pages, max_batch_size=w["requests"],
                         max_num_batched_tokens=4096, prefill_chunk=w["prefill_chunk"], dtype=args.dtype,
-                        use_graph=not args.no_graph, decode_burst=args.burst)
+                        use_graph=not args.no_graph, decode_burst=args.burst, decode_chain=args.chain)
     engine = LLMEngine.from_random(cfg, seed=0, engine_config=ecfg)
     for i, (p, o) in enumerate(requests):
         engine.add_request(Request(f"r{i}", p, SamplingParams(max_tokens=o, temperature=0.0)))
@@ -192,7 +192,8 @@ def main() -> int:
     ap.add_argument("--prompt", type=int, default=128)
     ap.add_argument("--kv-block", type=int, default=16)
     ap.add_argument("--no-graph", action="store_true")
-    ap.add_argument("--burst", type=int, default=8, help="decode steps enqueued back to back (1 = off)")
+    ap.add_argument("--burst", type=int, default=8, help="decode steps captured as one graph (1 = off)")
+    ap.add_argument("--chain", type=int, default=4, help="such graphs enqueued before the host waits")
     ap.add_argument("--no-extras", action="store_true", help="skip prefill and the batch 1 / 64 points")
     ap.add_argument("--workload", choices=sorted(WORKLOADS), default=None,
                     help="instead of the decode measurement: a whole continuous-batching run with the shape "
@@ -232,7 +233,8 @@ def main() -> int:
             "vocab_size": cfg.vocab_size, "block_size": cfg.block_size, "bias": True,
             "global_batch": args.batch, "seq_len": cfg.block_size, "prompt_len": args.prompt,
             "mean_context": round(mean_ctx, 1), "kv_block": args.kv_block, "weights": "random",
-            "hip_graph": bool(stats["graph_steps"]), "decode_burst": args.burst, "parallelism": "single-gpu",
+            "hip_graph": bool(stats["graph_steps"]), "decode_burst": args.burst, "decode_chain": args.chain,
+            "parallelism": "single-gpu",
         },
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 5)},

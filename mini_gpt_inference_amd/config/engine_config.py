@@ -26,8 +26,12 @@ class EngineConfig:
     dtype: str = "bfloat16"          # "bfloat16" (serving) or "float32" (true 32-bit path)
     use_graph: bool = True           # replay decode-only steps, and other steps whose shape repeats, from
                                      # captured HIP graphs
-    decode_burst: int = 8            # decode steps enqueued back to back when nothing else is pending,
-                                     # tokens fed on the device from one to the next; 1 = off
+    decode_burst: int = 8            # decode steps captured as one graph and enqueued back to back when
+                                     # nothing else is pending, tokens fed on the device from one to the
+                                     # next; 1 = off
+    decode_chain: int = 4            # such graphs enqueued one behind the other before the host waits: it
+                                     # launches the next and takes in the tokens of the last while the
+                                     # device is at work
     seed: int = 0                    # engine-wide sampler seed
     real_vocab_size: Optional[int] = None  # ids at or above it are never sampled
                                            # (src/minigpt_infer/tokenizer.py:37-46)
@@ -37,6 +41,8 @@ class EngineConfig:
             raise ValueError("block_size, num_blocks and max_batch_size must be positive")
         if self.max_num_batched_tokens <= 0:
             raise ValueError("max_num_batched_tokens must be positive")
+        if self.decode_burst < 1 or self.decode_chain < 1:
+            raise ValueError("decode_burst and decode_chain must be at least 1")
         if self.prefill_chunk < 0:
             raise ValueError("prefill_chunk must be >= 0")
         if self.dtype in ("bf16",):

@@ -209,10 +209,10 @@ int mgpt_sched_plan_burst(void* s, int max_k) {
   GUARD_END(-100)
 }
 
-int mgpt_sched_commit_burst(void* s, const int* tokens, int k, int* out_ids, int* out_tokens, int* out_finished,
-                            int* out_reason, int cap) {
+int mgpt_sched_commit_burst(void* s, const int* tokens, int k, int last, int* out_ids, int* out_tokens,
+                            int* out_finished, int* out_reason, int cap) {
   GUARD_BEGIN
-  const auto& o = static_cast<Scheduler*>(s)->commit_burst(tokens, k);
+  const auto& o = static_cast<Scheduler*>(s)->commit_burst(tokens, k, last != 0);
   if ((int)o.size() > cap) return -1;
   for (size_t i = 0; i < o.size(); ++i) {
     out_ids[i] = o[i].id;

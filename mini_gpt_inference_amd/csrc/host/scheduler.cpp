@@ -231,7 +231,7 @@ int Scheduler::plan_burst(int max_k) {
   return k;
 }
 
-const std::vector<StepOutput>& Scheduler::commit_burst(const int* tokens, int k) {
+const std::vector<StepOutput>& Scheduler::commit_burst(const int* tokens, int k, bool last) {
   outputs_.clear();
   const std::vector<StepEntry> entries = entries_;
   const int n = (int)entries.size();
@@ -250,7 +250,7 @@ const std::vector<StepOutput>& Scheduler::commit_burst(const int* tokens, int k)
       outputs_.push_back({r.id, token, why != NOT_FINISHED, (int)why});
     }
   }
-  entries_.clear();
+  if (last) entries_.clear();
   return outputs_;
 }
 

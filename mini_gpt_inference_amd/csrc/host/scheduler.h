@@ -95,8 +95,10 @@ class Scheduler {
   // (then nothing has changed).  Step j of a burst feeds position ctx + j.
   int plan_burst(int max_k);
   // tokens[j * n_entries + i]: what entry i sampled in step j.  A request that meets its end token
-  // in step j ends there; what the device computed for it afterwards is dropped.
-  const std::vector<StepOutput>& commit_burst(const int* tokens, int k);
+  // in step j ends there; what the device computed for it afterwards is dropped.  A burst may be
+  // handed in in several stretches of steps, in order (the device is then still at work on the later
+  // ones: pages that a request's end frees are given to nobody before the next plan); `last` ends it.
+  const std::vector<StepOutput>& commit_burst(const int* tokens, int k, bool last = true);
 
   const Request* request(int id) const;
   const std::deque<int>& waiting() const { return waiting_; }

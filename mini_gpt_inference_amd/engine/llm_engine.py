@@ -35,12 +35,14 @@ class _GraphedDecode:
     and appends the tokens to `history`, so that steps can follow each other with no copy between
     them: `burst` of them are captured as one graph as well."""
 
-    def __init__(self, runner: ModelRunner, sampler: Sampler, cap: int, burst: int) -> None:
+    def __init__(self, runner: ModelRunner, sampler: Sampler, cap: int, burst: int, chain: int = 1) -> None:
         self.runner, self.sampler, self.cap, self.burst = runner, sampler, cap, max(burst, 1)
+        self.max_steps = self.burst * max(chain, 1)      # most steps enqueued from one upload
         self.arena = StepArena(cap, cap, cap, runner.n_groups, runner.max_blocks, runner.device)
         self.workspace = Workspace(runner.device)
-        self.history = torch.zeros(self.burst, cap, dtype=torch.int32, device=runner.device)
-        self.history_host = torch.zeros(self.burst, cap, dtype=torch.int32, pin_memory=runner.device.type == "cuda")
+        self.history = torch.zeros(self.max_steps, cap, dtype=torch.int32, device=runner.device)
+        self.history_host = torch.zeros(self.max_steps, cap, dtype=torch.int32,
+                                        pin_memory=runner.device.type == "cuda")
         self.graph: Optional[torch.cuda.CUDAGraph] = None
         self.burst_graph: Optional[torch.cuda.CUDAGraph] = None
         self.shape: Optional[StepShape] = None   # of the last single step; launch geometry for captures
@@ -89,19 +91,35 @@ class _GraphedDecode:
         self.shape = shape
         self.graph.replay()
 
-    def run_burst(self, k: int) -> None:
-        """k steps from the uploaded arena, each feeding the next on the device; their tokens are in
-        history[:k] afterwards."""
+    def run_burst(self, k: int):
+        """k steps from the uploaded arena, each feeding the next on the device.  They are enqueued in
+        stretches (whole captured bursts, then single steps); behind each stretch its rows of the
+        history are copied to the host and an event is recorded.  Returns [(first step, end step,
+        event)]: once a stretch's event has passed, history_host[first:end] holds its tokens, while
+        the device is at work on the stretches behind it."""
         if self.graph is None:
             raise RuntimeError("a burst needs the single step's graph, which the first decode step captures")
+        if k > self.max_steps:
+            raise ValueError(f"{k} steps asked for, the history holds {self.max_steps}")
         self.arena.upload()
-        if k == self.burst:
-            if self.burst_graph is None:
-                self.burst_graph = self._capture(self.shape, k)
-            self.burst_graph.replay()
-        else:
-            for _ in range(k):
-                self.graph.replay()
+        stretches, done = [], 0
+        while done < k:
+            if k - done >= self.burst > 1:
+                if self.burst_graph is None:
+                    self.burst_graph = self._capture(self.shape, self.burst)
+                self.burst_graph.replay()
+                end = done + self.burst
+            else:
+                end = done
+                while end < k:      # the rest: single steps one behind the other, one copy and one event
+                    self.graph.replay()
+                    end += 1
+            self.history_host[done:end].copy_(self.history[done:end], non_blocking=True)
+            event = torch.cuda.Event()
+            event.record()
+            stretches.append((done, end, event))
+            done = end
+        return stretches
 
 
 class LLMEngine:
@@ -170,9 +188,10 @@ class LLMEngine:
         return False if sid is None else self.scheduler.cancel(sid)
 
     # ------------------------------------------------------------------ stepping
-    def _try_burst(self) -> Optional[List[RequestOutput]]:
+    def _try_burst(self, max_steps: Optional[int] = None) -> Optional[List[RequestOutput]]:
         """Several decode steps enqueued at once: one upload, the captured steps (each prepares the
-        next one's inputs on the device), one download of all their tokens."""
+        next one's inputs on the device); their tokens come back stretch by stretch and are handed to
+        the scheduler while the device runs the stretches behind."""
         ecfg = self.engine_config
         if ecfg.decode_burst < 2 or not ecfg.use_graph or not self._graphs:
             return None
@@ -180,20 +199,26 @@ class LLMEngine:
         graphed = self._graphs.get(_bucket(max(r, 1)))
         if graphed is None or graphed.graph is None:
             return None
-        k = self.scheduler.plan_burst(ecfg.decode_burst)
+        k = self.scheduler.plan_burst(min(graphed.max_steps, max_steps or graphed.max_steps))
         if k < 2:
             return None
         self.scheduler.fill(graphed.arena)
-        graphed.run_burst(k)
-        graphed.history_host[:k].copy_(graphed.history[:k], non_blocking=True)
-        torch.cuda.current_stream().synchronize()
-        tokens = np.ascontiguousarray(graphed.history_host.numpy()[:k, :r])
+        outs: List[RequestOutput] = []
+        stretches = graphed.run_burst(k)
+        for first, end, event in stretches:
+            event.synchronize()
+            tokens = np.ascontiguousarray(graphed.history_host.numpy()[first:end, :r])
+            outs += [RequestOutput(self._ids[sid], [token], finished, reason) for sid, token, finished, reason
+                     in self.scheduler.commit_burst(tokens, end - first, last=end == k)]
         self.num_graph_steps += k
-        return [RequestOutput(self._ids[sid], [token], finished, reason)
-                for sid, token, finished, reason in self.scheduler.commit_burst(tokens, k)]
+        return outs
 
-    def step(self) -> List[RequestOutput]:
-        burst = self._try_burst()
+    def step(self, max_decode_steps: Optional[int] = None) -> List[RequestOutput]:
+        """One step of the engine: admits, runs one batch (or, when every running request is decoding
+        and nobody waits, up to decode_burst x decode_chain decode steps back to back;
+        max_decode_steps lowers that bound), hands the sampled tokens to the scheduler.  Returns one
+        RequestOutput per token sampled."""
+        burst = self._try_burst(max_decode_steps) if max_decode_steps is None or max_decode_steps > 1 else None
         if burst is not None:
             return burst
         n, r, m = self.scheduler.schedule()
@@ -206,7 +231,8 @@ class LLMEngine:
             graphed = self._graphs.get(cap)
             if graphed is None:
                 graphed = self._graphs[cap] = _GraphedDecode(self.runner, self.sampler, cap,
-                                                             self.engine_config.decode_burst)
+                                                             self.engine_config.decode_burst,
+                                                             self.engine_config.decode_chain)
             arena = graphed.arena
         else:
             arena = self.runner.arena(n, r, m)

@@ -138,12 +138,13 @@ class Scheduler:
             raise SchedulerError(library.host_error())
         return k
 
-    def commit_burst(self, tokens: np.ndarray, k: int) -> List[Tuple[int, int, bool, Optional[str]]]:
-        """tokens[j, i]: what entry i sampled in step j of the burst."""
+    def commit_burst(self, tokens: np.ndarray, k: int, last: bool = True) -> List[Tuple[int, int, bool, Optional[str]]]:
+        """tokens[j, i]: what entry i sampled in step j of the burst.  A burst may be handed in in
+        several stretches of steps, in order; `last` says that this one ends it."""
         tokens = np.ascontiguousarray(tokens, dtype=np.int32)
         cap = tokens.size
         out = [np.zeros(max(cap, 1), dtype=np.int32) for _ in range(4)]
-        n = self._lib.mgpt_sched_commit_burst(self._h, _p(tokens), int(k), *[_p(a) for a in out], cap)
+        n = self._lib.mgpt_sched_commit_burst(self._h, _p(tokens), int(k), 1 if last else 0, *[_p(a) for a in out], cap)
         if n < 0:
             raise SchedulerError(f"commit_burst failed ({n}) {library.host_error()}")
         ids, toks, fin, why = out

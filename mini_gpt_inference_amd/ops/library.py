@@ -100,7 +100,7 @@ def host() -> ctypes.CDLL:
             "mgpt_sched_has_work": [P], "mgpt_sched_cancel": [P, I], "mgpt_sched_schedule": [P, P],
             "mgpt_sched_entries": [P, P, P, P, P, I],
             "mgpt_sched_fill": [P, P, I, I, I, I, I] + [P] * 14,
-            "mgpt_sched_plan_burst": [P, I], "mgpt_sched_commit_burst": [P, P, I, P, P, P, P, I],
+            "mgpt_sched_plan_burst": [P, I], "mgpt_sched_commit_burst": [P, P, I, I, P, P, P, P, I],
             "mgpt_sched_commit": [P, P, I, P, P, P, P, I],
             "mgpt_sched_queue": [P, I, P, I], "mgpt_sched_request_info": [P, I, P],
             "mgpt_sched_copy_output": [P, I, P, I],

@@ -252,6 +252,30 @@ def test_burst_is_planned_only_when_nothing_else_is_pending_and_ends_on_the_end_
     assert not s.has_work() and cm.num_free_pages() == 20 and cm.check() == 0
 
 
+def test_a_burst_handed_in_in_stretches_ends_like_one_handed_in_whole():
+    """The device is still at work on a burst's later steps when the first ones' tokens come back:
+    the scheduler takes them stretch by stretch, a request that met its end token in an earlier
+    stretch is passed over in the later ones, and entries last until the final stretch."""
+    results = []
+    for cuts in ([4], [1, 3], [2, 1, 1]):
+        cm, s = make(20, 4, max_batch=4, max_positions=64)
+        a = s.add_request([1, 2, 3], 10, eot=7)
+        b = s.add_request([1, 2, 3, 4, 5], 5)
+        step(s)
+        assert s.plan_burst(8) == 4
+        tokens = np.array([[5, 5], [7, 5], [6, 5], [6, 5]], dtype=np.int32)
+        outs, first = [], 0
+        for n in cuts:
+            assert len(s.entries()) == 2
+            outs += s.commit_burst(tokens[first:first + n], n, last=first + n == 4)
+            first += n
+        assert len(s.entries()) == 0
+        results.append((outs, s.output(a), s.output(b), cm.num_free_pages(), cm.check()))
+        assert s.info(a).status == FINISHED and s.info(b).status == FINISHED and not s.has_work()
+    assert results[0] == results[1] == results[2]
+    assert results[0][1] == [100, 5, 7] and results[0][3] == 20 and results[0][4] == 0
+
+
 def test_burst_needs_pages_for_every_step_or_does_not_start():
     cm, s = make(4, 4, max_batch=2, max_positions=64)
     a = s.add_request([1, 2, 3], 12)
