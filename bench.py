@@ -58,11 +58,16 @@ def decode_run(args, batch, steps, warmup, dtype):
     while sched.num_decode_tokens == 0:      # prompts, untimed
         engine.step()
 
-    def run_decode_steps(n):
+    samples = []     # (decode steps in the call, seconds) of every engine.step() call of the timed region
+
+    def run_decode_steps(n, record=False):
         """engine.step() until exactly n more decode steps have run (a call may run a burst of them)."""
         first, tokens = sched.num_steps, sched.num_decode_tokens
         while sched.num_steps - first < n:
+            before, t_call = sched.num_steps, time.perf_counter()
             engine.step(max_decode_steps=n - (sched.num_steps - first))
+            if record:
+                samples.append((sched.num_steps - before, time.perf_counter() - t_call))
         assert sched.num_steps - first == n, "the decode bursts do not divide the number of steps"
         assert sched.num_decode_tokens - tokens == n * batch, "a request dropped out of the decode steps"
 
@@ -71,9 +76,10 @@ def decode_run(args, batch, steps, warmup, dtype):
     torch.cuda.synchronize()
     start_ctx = args.prompt + 1 + (sched.num_steps - done)
     t0 = time.perf_counter()
-    run_decode_steps(steps)
+    run_decode_steps(steps, record=True)
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
+    engine.step_samples = samples
     mean_ctx = start_ctx + (steps - 1) / 2.0 + 1     # keys read per request and step, own token included
     return elapsed, mean_ctx, engine, cfg
 
@@ -201,6 +207,9 @@ def main() -> int:
                          "requests, a page pool too small for them: evictions)")
     ap.add_argument("--workload-layers", type=int, default=0, help="fewer layers for --workload (0 = the shape's)")
     ap.add_argument("--workload-requests", type=int, default=0, help="fewer requests for --workload")
+    ap.add_argument("--report", default=None,
+                    help="also write a JSON file with the raw timing samples, their median and quartiles, the "
+                         "commit and the software and device that ran them")
     ap.add_argument("--prefill-only", action="store_true",
                     help="run only the 2,048-token prefill and print its record (for profiling)")
     args = ap.parse_args()
@@ -216,6 +225,7 @@ def main() -> int:
         return 0
 
     elapsed, mean_ctx, engine, cfg = decode_run(args, args.batch, args.steps, args.warmup, args.dtype)
+    samples = engine.step_samples
     itemsize = 2 if args.dtype == "bfloat16" else 4
     step_s = elapsed / args.steps
     value = args.batch * args.steps / elapsed
@@ -250,7 +260,34 @@ def main() -> int:
             del eng
         record["points"] = points
     print(json.dumps(record))
+    if args.report:
+        write_report(args.report, record, samples)
     return 0
+
+
+def write_report(path, record, samples):
+    """The record, the raw samples behind it (one per engine.step() call of the timed region: decode
+    steps in the call, seconds; a call ends when its tokens are on the host), their median and
+    quartiles per step, and what ran them (the reference's timing rules, docs/PLAN.md:720-732)."""
+    import statistics
+    import subprocess
+
+    import torch
+
+    per_step = sorted(sec / n for n, sec in samples if n)
+    quart = statistics.quantiles(per_step, n=4) if len(per_step) >= 2 else [per_step[0]] * 3
+    try:
+        sha = subprocess.run(["git", "rev-parse", "HEAD"], capture_output=True, text=True, timeout=10).stdout.strip()
+    except Exception:
+        sha = ""
+    report = {"record": record,
+              "ms_per_step": {"median": quart[1] * 1e3, "q1": quart[0] * 1e3, "q3": quart[2] * 1e3,
+                              "calls": len(per_step)},
+              "samples": [[n, sec] for n, sec in samples],
+              "environment": {"git": sha, "torch": torch.__version__, "hip": torch.version.hip,
+                              "device": torch.cuda.get_device_name(0)}}
+    with open(path, "w", encoding="utf-8") as fh:
+        json.dump(report, fh, indent=1)
 
 
 if __name__ == "__main__":

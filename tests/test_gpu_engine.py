@@ -47,7 +47,7 @@ def _assert_greedy_within_tolerance(folder, prompt, tokens, dtype):
 
 @pytest.mark.parametrize("use_graph", [True, False])
 def test_greedy_generation_32bit_equals_plain_tokens(model_folders, use_graph):
-    # BASELINE configuration 1: three requests of 5/17/30 tokens, 12 greedy tokens, pages of 4
+    # The family's first tiny workload: three requests of 5/17/30 tokens, 12 greedy tokens, pages of 4
     prompts = _prompts("A", [5, 17, 30])
     want = _plain_greedy(model_folders["A"], prompts, 12)
     engine = LLMEngine.from_folder(model_folders["A"], EngineConfig(block_size=4, num_blocks=64, max_batch_size=4,
@@ -91,7 +91,7 @@ def test_chunked_mixed_and_whole_prompt_policies_give_the_same_tokens(model_fold
 
 
 def test_seeded_temperature_sampling_is_reproducible_and_independent_of_batching(model_folders):
-    # BASELINE configuration 2: five requests of 1/9/33/64/100 tokens, 16 tokens at temperature 0.8 from a
+    # The family's second tiny workload: five requests of 1/9/33/64/100 tokens, 16 tokens at temperature 0.8 from a
     # fixed sampler seed, prompt portions of 16, pages of 8
     prompts = _prompts("B", [1, 9, 33, 64, 100], seed=3)
     params = [SamplingParams(max_tokens=16, temperature=0.8, seed=100 + i) for i in range(5)]
