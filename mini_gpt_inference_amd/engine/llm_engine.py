@@ -22,7 +22,7 @@ from ..sampling.sampler import Sampler
 from ..weights.loader import load_model
 from ..weights.random_init import write_random_model
 from .request import Request, RequestOutput
-from .scheduler import Scheduler
+from .scheduler import FINISHED, Scheduler
 from .step import ModelRunner, StepArena, StepShape, _bucket
 
 _TORCH_DTYPES = {"bfloat16": torch.bfloat16, "float32": torch.float32}
@@ -143,6 +143,7 @@ class LLMEngine:
         self.sampler = Sampler(model.spec.vocab_size, engine_config.real_vocab_size, engine_config.seed)
         self._ids: Dict[int, str] = {}        # scheduler id -> caller's request id
         self._rids: Dict[str, int] = {}
+        self._generated = 0                   # requests that generate() has named so far
         self._graphs: Dict[int, _GraphedDecode] = {}
         self._tmpdir: Optional[str] = None
         self.num_graph_steps = 0
@@ -268,8 +269,8 @@ class LLMEngine:
                   else [sampling_params] * len(prompts))
         if len(params) != len(prompts):
             raise ValueError("one SamplingParams per prompt, or one for all")
-        base = len(self._rids)
-        names = [f"generate-{base + i}" for i in range(len(prompts))]
+        names = [f"generate-{self._generated + i}" for i in range(len(prompts))]
+        self._generated += len(prompts)
         got: Dict[str, List[int]] = {name: [] for name in names}
         for name, prompt, sp in zip(names, prompts, params):
             self.add_request(Request(name, list(prompt), sp, eot_token_id))
@@ -280,7 +281,18 @@ class LLMEngine:
                     got[out.request_id].extend(out.new_token_ids)
             if not outs and not self.scheduler.running:
                 raise RuntimeError("the scheduler cannot make progress: the waiting request does not fit")
+        self.forget_finished()
         return [got[name] for name in names]
+
+    def forget_finished(self) -> int:
+        """Drops what the engine still holds of finished requests (their ids and token lists), so that
+        an engine that serves for a long time does not grow; their ids may be used again.  Returns
+        how many were dropped.  generate() calls it; a loop around step() calls it when it likes."""
+        done = [sid for sid in self._ids if self.scheduler.info(sid).status == FINISHED]
+        for sid in done:
+            del self._rids[self._ids.pop(sid)]
+        self.scheduler.forget_finished()
+        return len(done)
 
     # ------------------------------------------------------------------ counters
     def fragmentation_stats(self, group: int = 0) -> Dict[str, int]:

@@ -188,6 +188,27 @@ def test_step_outputs_finish_reasons_eot_and_cancel(model_folders):
         engine.add_request(Request("bad", [1, 999], SamplingParams(max_tokens=2)))
 
 
+def test_finished_requests_are_forgotten_and_their_ids_can_be_used_again(model_folders):
+    engine = LLMEngine.from_folder(model_folders["A"], EngineConfig(block_size=4, num_blocks=64, max_batch_size=4,
+                                                                    dtype="float32"))
+    prompts = _prompts("A", [5, 9], seed=12)
+    first = engine.generate(prompts, SamplingParams(max_tokens=5, temperature=0.0))
+    assert not engine._ids and not engine._rids          # generate() leaves nothing behind
+    assert engine.generate(prompts, SamplingParams(max_tokens=5, temperature=0.0)) == first
+    engine.add_request(Request("mine", prompts[0], SamplingParams(max_tokens=3, temperature=0.0)))
+    with pytest.raises(ValueError):
+        engine.add_request(Request("mine", prompts[1], SamplingParams(max_tokens=3, temperature=0.0)))
+    while engine.has_unfinished_requests():
+        engine.step()
+    assert engine.forget_finished() == 1 and engine.forget_finished() == 0
+    engine.add_request(Request("mine", prompts[1], SamplingParams(max_tokens=3, temperature=0.0)))
+    got = []
+    while engine.has_unfinished_requests():
+        got += [t for out in engine.step() for t in out.new_token_ids]
+    assert got == first[1][:3]
+    assert engine.cache.num_free_pages() == 64 and engine.cache.check() == 0
+
+
 def test_real_vocabulary_bound_is_never_crossed(model_folders):
     engine = LLMEngine.from_folder(model_folders["A"], EngineConfig(block_size=4, num_blocks=32, max_batch_size=4,
                                                                     dtype="float32", real_vocab_size=40))
