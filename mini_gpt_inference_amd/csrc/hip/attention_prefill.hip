@@ -67,7 +67,11 @@ __global__ __launch_bounds__(256 * G) void prefill_attention_kernel(
     int single_below) {
   constexpr int THREADS = 256 * G;
   constexpr int SB = PF_KT * G;    // keys staged per step
-  constexpr int KLD = D + 8;       // key rows in LDS
+  // Key and value rows in LDS: as long as the head size where that is a power of two, the 16-byte
+  // chunks of a row XORed with the row's low bits (then neither the operand reads, 16 rows x 4 chunks
+  // an instruction, nor the transposing reads meet in a bank); padded by 16 bytes otherwise.
+  constexpr bool SWZ = (D & (D - 1)) == 0;
+  constexpr int KLD = SWZ ? D : D + 8;
   constexpr int KK = D / 32;       // MFMA k steps over the head size
   constexpr int DT = D / 16;       // 16-channel tiles of the output
   constexpr int KS_SIZE = SB * KLD;   // keys, and as much for values
@@ -111,14 +115,15 @@ __global__ __launch_bounds__(256 * G) void prefill_attention_kernel(
 #pragma unroll
   for (int dt = 0; dt < DT; ++dt) o[dt] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
 
-  // Staging: 2 threads per key row, each 16 bytes (8 channels) of the key row and of the value
-  // row at a time.
-  constexpr int TPR = THREADS / SB;
-  constexpr int CH = D / 8, NC = (CH + TPR - 1) / TPR;      // chunks per row, per thread
-  const int srow = tid / TPR, sc = tid % TPR;
-  bf16x8_t kst[NC], vst[NC];
-  bool k_ok;   // whether the fetched row is a visible key's: decided at fetch, applied at deposit,
-               // so that nothing touches a loaded value while the current stretch is multiplied
+  // Staging: the stretch's rows are dealt out 16 bytes (8 channels) at a time, a row's chunks to
+  // neighbouring threads, so that one load instruction of a wave covers whole rows (64 lanes: 8 rows
+  // of 128 bytes at head size 64) and the 64 chunks it later puts into LDS lie in as many places.
+  constexpr int CH = D / 8;                      // chunks per row
+  constexpr int NP = SB * CH / THREADS;          // chunks per thread (= D / 16)
+  static_assert(SB * CH % THREADS == 0, "the stretch's chunks must divide among the threads");
+  bf16x8_t kst[NP], vst[NP];
+  bool k_ok[NP];   // whether the fetched row is a visible key's: decided at fetch, applied at deposit,
+                   // so that nothing touches a loaded value while the current stretch is multiplied
 
   // the row index of key j, or -1; the block table entry is the only thing read from memory
   auto lookup = [&](int j) -> int {
@@ -126,26 +131,33 @@ __global__ __launch_bounds__(256 * G) void prefill_attention_kernel(
     const int pg = j / page_size;
     return (bt[pg] * n_kv_head + hk) * page_size + (j - pg * page_size);
   };
+  // where chunk c of LDS row `row` lies
+  auto chunk_at = [](int row, int c) -> int {
+    if (!SWZ) return c;
+    return D == 32 ? c ^ ((row >> 1) & 3) : c ^ (row & 7);
+  };
   auto fetch = [&](int step) {
-    const int row = row_tab[(step & 3) * SB + srow];
-    k_ok = row >= 0;
-    const long base = (long)(k_ok ? row : 0) * D;
 #pragma unroll
-    for (int u = 0; u < NC; ++u) {
-      const int c = sc + u * TPR;
-      kst[u] = *reinterpret_cast<const bf16x8_t*>(kpool + base + (c < CH ? c * 8 : 0));
-      vst[u] = *reinterpret_cast<const bf16x8_t*>(vpool + base + (c < CH ? c * 8 : 0));
+    for (int u = 0; u < NP; ++u) {
+      const int idx = u * THREADS + tid;
+      const int r = idx / CH, c = idx - r * CH;
+      const int row = row_tab[(step & 3) * SB + r];
+      k_ok[u] = row >= 0;
+      const long base = (long)(k_ok[u] ? row : 0) * D + c * 8;
+      kst[u] = *reinterpret_cast<const bf16x8_t*>(kpool + base);
+      vst[u] = *reinterpret_cast<const bf16x8_t*>(vpool + base);
     }
   };
   auto deposit = [&](int buf) {
     bf16_t* ks = pf_lds + buf * KS_SIZE;
     bf16_t* vs = pf_lds + (2 + buf) * KS_SIZE;
 #pragma unroll
-    for (int u = 0; u < NC; ++u) {
-      const int c = sc + u * TPR;
-      if (c >= CH) continue;
-      *reinterpret_cast<bf16x8_t*>(&ks[srow * KLD + c * 8]) = k_ok ? kst[u] : zero8;
-      *reinterpret_cast<bf16x8_t*>(&vs[srow * KLD + c * 8]) = k_ok ? vst[u] : zero8;
+    for (int u = 0; u < NP; ++u) {
+      const int idx = u * THREADS + tid;
+      const int r = idx / CH, c = idx - r * CH;
+      const int at = r * KLD + chunk_at(r, c) * 8;
+      *reinterpret_cast<bf16x8_t*>(&ks[at]) = k_ok[u] ? kst[u] : zero8;
+      *reinterpret_cast<bf16x8_t*>(&vs[at]) = k_ok[u] ? vst[u] : zero8;
     }
   };
 
@@ -185,7 +197,7 @@ __global__ __launch_bounds__(256 * G) void prefill_attention_kernel(
         for (int kk = 0; kk < KK; ++kk)
 #pragma unroll
           for (int kt = 0; kt < NKT; ++kt)
-            kf[kk][kt] = *reinterpret_cast<const bf16x8_t*>(&ks[(kt * 16 + qi) * KLD + kk * 32 + g * 8]);
+            kf[kk][kt] = *reinterpret_cast<const bf16x8_t*>(&ks[(kt * 16 + qi) * KLD + chunk_at(qi, kk * 4 + g) * 8]);
 #pragma unroll
         for (int kt = 0; kt < NKT; ++kt) s[kt] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
@@ -199,13 +211,16 @@ __global__ __launch_bounds__(256 * G) void prefill_attention_kernel(
       // key bb*32 + 16 + g*4 + (e - 4) otherwise; this lane points at row g*4 + qi/4 of those, chunk qi%4.
       bf16x4_t vlo[DT][NKT / 2], vhi[DT][NKT / 2];
       typedef bf16x4_t __attribute__((address_space(3))) * lds_b64_t;
-      const bf16_t* vlane = vs + (g * 4 + (qi >> 2)) * KLD + (qi & 3) * 4;
+      // row g*4 + qi/4 of each 16; its 8 bytes are half (qi & 1) of the 16-byte chunk dt*2 + (qi & 3)/2
+      const int vrow = g * 4 + (qi >> 2);
+      const bf16_t* vlane = vs + vrow * KLD + (qi & 1) * 4;
 #pragma unroll
       for (int bb = 0; bb < NKT / 2; ++bb)
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt) {
-          vlo[dt][bb] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_b64_t)(vlane + (bb * 32) * KLD + dt * 16));
-          vhi[dt][bb] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_b64_t)(vlane + (bb * 32 + 16) * KLD + dt * 16));
+          const int off = chunk_at(vrow, dt * 2 + ((qi & 3) >> 1)) * 8;   // rows 16 and 32 apart swizzle alike
+          vlo[dt][bb] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_b64_t)(vlane + (bb * 32) * KLD + off));
+          vhi[dt][bb] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_b64_t)(vlane + (bb * 32 + 16) * KLD + off));
         }
       __builtin_amdgcn_sched_barrier(0);   // or the compiler moves each read down to its use
 
@@ -328,7 +343,8 @@ extern "C" int mgpt_prefill_attention_bf16(
 #define PF_LAUNCH(DD, GG)                                                                                       \
   {                                                                                                             \
     constexpr int sb = PF_KT * GG;                                                                              \
-    constexpr int lds_bytes = 4 * sb * (DD + 8) * (int)sizeof(bf16_t) + 4 * sb * 4;                              \
+    constexpr int kld = (DD & (DD - 1)) == 0 ? DD : DD + 8;                                                     \
+    constexpr int lds_bytes = 4 * sb * kld * (int)sizeof(bf16_t) + 4 * sb * 4;                                  \
     static bool allowed = false; /* more LDS than a kernel gets without asking */                               \
     if (!allowed) {                                                                                             \
       const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(prefill_attention_kernel<DD, GG>), \
