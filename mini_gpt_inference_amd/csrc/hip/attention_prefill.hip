@@ -316,10 +316,15 @@ __global__ __launch_bounds__(256 * G) void prefill_attention_kernel(
   if (q_ok) {
     const float inv = 1.0f / l;
     bf16_t* orow = out + (long)(q_start + my_q) * ldo + (long)h * D;
+    // a lane's four neighbouring channels of a tile are one 8-byte store (the launcher has checked
+    // that rows start 8 bytes aligned)
 #pragma unroll
-    for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-      for (int i = 0; i < 4; ++i) orow[dt * 16 + g * 4 + i] = float_to_bf16(o[dt][i] * inv);
+    for (int dt = 0; dt < DT; ++dt) {
+      uint2 pk;
+      pk.x = pack_bf16x2(o[dt][0] * inv, o[dt][1] * inv);
+      pk.y = pack_bf16x2(o[dt][2] * inv, o[dt][3] * inv);
+      *reinterpret_cast<uint2*>(orow + dt * 16 + g * 4) = pk;
+    }
   }
 }
 
@@ -336,7 +341,8 @@ extern "C" int mgpt_prefill_attention_bf16(
   if (n_req == 0 || max_q_len == 0) return MGPT_OK;
   if (!q || !out || !kpool || !vpool || !block_tables || !cu_q || !seq_lens) return MGPT_ERR_NULL;
   if (n_req < 0 || max_q_len < 0 || n_head <= 0 || n_kv_head <= 0 || (n_head % n_kv_head) != 0 ||
-      page_size <= 0 || max_blocks <= 0 || window < 0 || (ldq % 8) != 0 || !(scale > 0.f))
+      page_size <= 0 || max_blocks <= 0 || window < 0 || (ldq % 8) != 0 || (ldo % 4) != 0 ||
+      (((size_t)out) & 7) != 0 || !(scale > 0.f))
     return MGPT_ERR_BAD_SHAPE;
   if (n_req > 65535 || n_head > 65535) return MGPT_ERR_TOO_LARGE;
   dim3 grid((max_q_len + PF_QT - 1) / PF_QT, n_req, n_head);
