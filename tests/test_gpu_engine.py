@@ -73,6 +73,29 @@ def test_greedy_generation_bfloat16_chooses_the_plain_argmax_up_to_rounding(mode
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("n_req", [20, 40])
+def test_many_requests_decode_from_padded_graphs(model_folders, dtype, n_req):
+    """20 and 40 requests: decode steps replayed from the graphs of 32 and 64 rows (padded), in chained
+    bursts; requests end at different lengths, so later steps fall into smaller graphs."""
+    rng = np.random.default_rng(31)
+    prompts = _prompts("B", [int(n) for n in rng.integers(1, 40, n_req)], seed=32)
+    news = [int(n) for n in rng.integers(3, 20, n_req)]
+    engine = LLMEngine.from_folder(model_folders["B"], EngineConfig(block_size=8, num_blocks=n_req * 8,
+                                                                    max_batch_size=n_req, dtype=dtype))
+    got = engine.generate(prompts, [SamplingParams(max_tokens=n, temperature=0.0) for n in news])
+    assert engine.stats()["graph_steps"] > 0
+    assert engine.cache.num_free_pages() == n_req * 8 and engine.cache.check() == 0
+    exact = 0
+    for prompt, tokens, n in zip(prompts, got, news):
+        assert len(tokens) == n
+        exact += _assert_greedy_within_tolerance(model_folders["B"], prompt, tokens, dtype)
+    if dtype == "float32":
+        assert exact == sum(news)
+    else:
+        assert exact >= 0.9 * sum(news)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_chunked_mixed_and_whole_prompt_policies_give_the_same_tokens(model_folders, dtype):
     prompts = _prompts("B", [1, 9, 33, 64, 100], seed=2)
     sp = SamplingParams(max_tokens=16, temperature=0.0)
