@@ -143,6 +143,29 @@ def test_trace_run_reports_a_pool_that_is_too_small(model_folders, tmp_path):
     assert proc.returncode == 1 and "used up" in proc.stderr and "done 0" not in proc.stdout
 
 
+def test_trace_run_says_what_is_wrong_with_a_line_or_a_model(model_folders, tmp_path):
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    base = [os.path.join(root, "bin", "trace_run"), "--dtype", "float32", "--out", str(tmp_path / "o"),
+            "--max-tokens", "128"]
+
+    def run(model, text):
+        return subprocess.run(base + ["--model", model], input=text, text=True, capture_output=True, timeout=300)
+
+    ok = json.dumps({"step": 0, "entries": [{"id": "a", "tokens": [1, 2], "want": [1]}], "end": []}) + "\n"
+    cases = {
+        "a token id the vocabulary lacks": json.dumps({"step": 1, "entries": [{"id": "a", "tokens": [100000], "want": []}]}),
+        "a position past the table": json.dumps({"step": 1, "entries": [{"id": "a", "tokens": [1] * 70, "want": []}]}),
+        "not JSON": "{step: 1",
+        "want outside the entry": json.dumps({"step": 1, "entries": [{"id": "a", "tokens": [1], "want": [3]}]}),
+    }
+    for what, line in cases.items():
+        proc = run(model_folders["A"], ok + line + "\n")
+        assert proc.returncode == 1 and "done 0" in proc.stdout and "done 1" not in proc.stdout, what
+        assert "trace_run:" in proc.stderr and "Traceback" not in proc.stderr, (what, proc.stderr)
+    proc = run(str(tmp_path / "no_such_model"), ok)
+    assert proc.returncode == 1 and "cannot load" in proc.stderr and "Traceback" not in proc.stderr
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_want_may_be_empty_or_partial_and_steps_without_logits_write_no_file(model_folders, dtype):
     cfg = helpers.CONFIGS["A"]
