@@ -94,7 +94,7 @@ def decode_bytes(cfg, batch, mean_ctx, itemsize):
     return weights + kv
 
 
-def prefill_run(args, dtype, reps=5):
+def prefill_run(args, dtype, reps=9):
     import numpy as np
     import torch
 
