@@ -49,7 +49,7 @@ def decode_run(args, batch, steps, warmup, dtype):
 
     engine, cfg = build_engine(args, batch, dtype)
     rng = np.random.default_rng(0)
-    budget = steps + warmup + 2 * args.burst * args.chain + 2
+    budget = steps + warmup + 3 * args.burst * args.chain + 2
     assert args.prompt + budget <= cfg.block_size, "prompt + decode steps exceed the model's positions"
     for i in range(batch):
         engine.add_request(Request(f"b{i}", rng.integers(0, cfg.vocab_size, args.prompt).tolist(),
@@ -68,6 +68,7 @@ def decode_run(args, batch, steps, warmup, dtype):
             engine.step(max_decode_steps=n - (sched.num_steps - first))
             if record:
                 samples.append((sched.num_steps - before, time.perf_counter() - t_call))
+        engine.step(max_decode_steps=0)      # what the last call enqueued ahead is taken in here
         assert sched.num_steps - first == n, "the decode bursts do not divide the number of steps"
         assert sched.num_decode_tokens - tokens == n * batch, "a request dropped out of the decode steps"
 

@@ -32,6 +32,8 @@ class EngineConfig:
     decode_chain: int = 4            # such graphs enqueued one behind the other before the host waits: it
                                      # launches the next and takes in the tokens of the last while the
                                      # device is at work
+    decode_ahead: bool = True        # before the host waits for a chain's last tokens it plans and enqueues
+                                     # the next chain, whose tokens the next step() call returns
     seed: int = 0                    # engine-wide sampler seed
     real_vocab_size: Optional[int] = None  # ids at or above it are never sampled
                                            # (src/minigpt_infer/tokenizer.py:37-46)

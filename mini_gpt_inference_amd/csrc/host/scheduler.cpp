@@ -154,6 +154,7 @@ void Scheduler::schedule_prompts(int& budget, bool allow_admission) {
 }
 
 const std::vector<StepEntry>& Scheduler::schedule() {
+  if (pending_ > 0) throw std::runtime_error("schedule(): a planned burst has not been handed in yet");
   entries_.clear();
   preempted_this_step_ = false;
   int budget = cfg_.max_num_batched_tokens;
@@ -204,11 +205,18 @@ const std::vector<StepOutput>& Scheduler::commit(const int* tokens, int n_tokens
 
 int Scheduler::plan_burst(int max_k) {
   if (max_k < 2 || running_.empty() || !waiting_.empty()) return 0;
+  if (pending_ > 0) {
+    // planning ahead of a burst that is not handed in yet: only while its requests are still the
+    // running ones, in their order (nobody has met an end token in the stretches handed in so far)
+    if (entries_.size() != running_.size()) return 0;
+    for (size_t i = 0; i < running_.size(); ++i)
+      if (entries_[i].id != running_[i]) return 0;
+  }
   int k = max_k;
   for (int id : running_) {
     const Request& r = *get(id);
     if (r.num_tokens() - r.num_computed != 1) return 0;  // still in its prompt
-    k = std::min(k, r.max_tokens - (int)r.output.size());
+    k = std::min(k, r.max_tokens - (int)r.output.size() - pending_);
   }
   if (k < 2) return 0;
   // pages for k more tokens each, or no burst at all
@@ -216,18 +224,19 @@ int Scheduler::plan_burst(int max_k) {
     long need = 0;
     for (int id : running_) {
       const Request& r = *get(id);
-      need += std::max(0, cache_->pages_needed(g, r.num_computed + k) - cache_->table_len(r.slot, g));
+      need += std::max(0, cache_->pages_needed(g, r.num_computed + pending_ + k) - cache_->table_len(r.slot, g));
     }
     if (need > cache_->num_free_pages(g)) return 0;
   }
   entries_.clear();
   for (int id : running_) {
     Request& r = *get(id);
-    cache_->reserve(r.slot, r.num_computed + k);
-    entries_.push_back({id, r.num_computed, 1, true});
+    cache_->reserve(r.slot, r.num_computed + pending_ + k);
+    entries_.push_back({id, r.num_computed + pending_, 1, true});
   }
   num_decode_tokens += (long)k * (long)entries_.size();
   num_steps += k;
+  pending_ += k;
   return k;
 }
 
@@ -250,7 +259,8 @@ const std::vector<StepOutput>& Scheduler::commit_burst(const int* tokens, int k,
       outputs_.push_back({r.id, token, why != NOT_FINISHED, (int)why});
     }
   }
-  if (last) entries_.clear();
+  pending_ = std::max(0, pending_ - k);
+  if (last && pending_ == 0) entries_.clear();
   return outputs_;
 }
 

@@ -93,11 +93,15 @@ class Scheduler {
   // one short of the first request's length limit, so nobody can end inside a burst except by its
   // end token.  Returns k >= 2 with entries() set to step 0, or 0 when a burst is not possible
   // (then nothing has changed).  Step j of a burst feeds position ctx + j.
+  // A further burst may be planned before the last one's tokens are all handed in (the device then
+  // never waits for the host between them): it starts where that one will end, and is refused (0) once
+  // a request of that one has ended, since the device goes on computing for the same requests.
   int plan_burst(int max_k);
   // tokens[j * n_entries + i]: what entry i sampled in step j.  A request that meets its end token
   // in step j ends there; what the device computed for it afterwards is dropped.  A burst may be
   // handed in in several stretches of steps, in order (the device is then still at work on the later
   // ones: pages that a request's end frees are given to nobody before the next plan); `last` ends it.
+  // The entries stay until every planned step has been handed in.
   const std::vector<StepOutput>& commit_burst(const int* tokens, int k, bool last = true);
 
   const Request* request(int id) const;
@@ -129,6 +133,7 @@ class Scheduler {
   std::vector<StepEntry> entries_;
   std::vector<StepOutput> outputs_;
   bool preempted_this_step_ = false;
+  int pending_ = 0;  // steps of planned bursts whose tokens have not been handed in yet
 };
 
 }  // namespace mgpt

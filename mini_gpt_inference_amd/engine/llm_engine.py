@@ -40,9 +40,12 @@ class _GraphedDecode:
         self.max_steps = self.burst * max(chain, 1)      # most steps enqueued from one upload
         self.arena = StepArena(cap, cap, cap, runner.n_groups, runner.max_blocks, runner.device)
         self.workspace = Workspace(runner.device)
-        self.history = torch.zeros(self.max_steps, cap, dtype=torch.int32, device=runner.device)
-        self.history_host = torch.zeros(self.max_steps, cap, dtype=torch.int32,
+        # two halves: a chain that goes on from the last one writes the other half, while the host
+        # still reads that one's tokens
+        self.history = torch.zeros(2 * self.max_steps, cap, dtype=torch.int32, device=runner.device)
+        self.history_host = torch.zeros(2 * self.max_steps, cap, dtype=torch.int32,
                                         pin_memory=runner.device.type == "cuda")
+        self.history_base = 0
         self.graph: Optional[torch.cuda.CUDAGraph] = None
         self.burst_graph: Optional[torch.cuda.CUDAGraph] = None
         self.shape: Optional[StepShape] = None   # of the last single step; launch geometry for captures
@@ -78,6 +81,8 @@ class _GraphedDecode:
 
     def run(self, shape: StepShape) -> None:
         """One step from the uploaded arena."""
+        self.arena.h["history_pos"][:] = 0
+        self.history_base = 0
         self.arena.upload()
         if self.graph is None:
             # once eagerly, so that every workspace buffer exists before capture
@@ -91,17 +96,25 @@ class _GraphedDecode:
         self.shape = shape
         self.graph.replay()
 
-    def run_burst(self, k: int):
-        """k steps from the uploaded arena, each feeding the next on the device.  They are enqueued in
-        stretches (whole captured bursts, then single steps); behind each stretch its rows of the
-        history are copied to the host and an event is recorded.  Returns [(first step, end step,
-        event)]: once a stretch's event has passed, history_host[first:end] holds its tokens, while
-        the device is at work on the stretches behind it."""
+    def run_burst(self, k: int, ahead: bool = False):
+        """k steps, each feeding the next on the device.  They are enqueued in stretches (whole
+        captured bursts, then single steps); behind each stretch its rows of the history are copied
+        to the host and an event is recorded.  Returns [(first row, end row, event)]: once a
+        stretch's event has passed, history_host[first:end] holds its tokens, while the device is at
+        work on the stretches behind it.  ahead: the steps go on from where the steps enqueued before
+        them will end (their tokens, positions and cache slots are the device's own); only the block
+        tables are uploaded, and the tokens go to the history's other half."""
         if self.graph is None:
             raise RuntimeError("a burst needs the single step's graph, which the first decode step captures")
         if k > self.max_steps:
             raise ValueError(f"{k} steps asked for, the history holds {self.max_steps}")
-        self.arena.upload()
+        base = (self.max_steps - self.history_base) if ahead else 0
+        self.history_base = base
+        self.arena.h["history_pos"][:] = base
+        if ahead:
+            self.arena.upload_tables()
+        else:
+            self.arena.upload()
         stretches, done = [], 0
         while done < k:
             if k - done >= self.burst > 1:
@@ -114,10 +127,10 @@ class _GraphedDecode:
                 while end < k:      # the rest: single steps one behind the other, one copy and one event
                     self.graph.replay()
                     end += 1
-            self.history_host[done:end].copy_(self.history[done:end], non_blocking=True)
+            self.history_host[base + done:base + end].copy_(self.history[base + done:base + end], non_blocking=True)
             event = torch.cuda.Event()
             event.record()
-            stretches.append((done, end, event))
+            stretches.append((base + done, base + end, event))
             done = end
         return stretches
 
@@ -144,6 +157,7 @@ class LLMEngine:
         self._ids: Dict[int, str] = {}        # scheduler id -> caller's request id
         self._rids: Dict[str, int] = {}
         self._generated = 0                   # requests that generate() has named so far
+        self._inflight = None                 # a chain of decode steps enqueued ahead, not yet taken in
         self._graphs: Dict[int, _GraphedDecode] = {}
         self._tmpdir: Optional[str] = None
         self.num_graph_steps = 0
@@ -189,10 +203,10 @@ class LLMEngine:
         return False if sid is None else self.scheduler.cancel(sid)
 
     # ------------------------------------------------------------------ stepping
-    def _try_burst(self, max_steps: Optional[int] = None) -> Optional[List[RequestOutput]]:
-        """Several decode steps enqueued at once: one upload, the captured steps (each prepares the
-        next one's inputs on the device); their tokens come back stretch by stretch and are handed to
-        the scheduler while the device runs the stretches behind."""
+    def _launch_chain(self, max_steps: Optional[int], ahead: bool):
+        """Plans up to decode_burst x decode_chain decode steps (at most max_steps) and enqueues them.
+        ahead: behind a chain whose last tokens the host has not seen yet.  Returns (graphs, requests,
+        steps, stretches), or None when no burst can be planned now."""
         ecfg = self.engine_config
         if ecfg.decode_burst < 2 or not ecfg.use_graph or not self._graphs:
             return None
@@ -200,28 +214,51 @@ class LLMEngine:
         graphed = self._graphs.get(_bucket(max(r, 1)))
         if graphed is None or graphed.graph is None:
             return None
-        k = self.scheduler.plan_burst(min(graphed.max_steps, max_steps or graphed.max_steps))
+        k = self.scheduler.plan_burst(graphed.max_steps if max_steps is None else min(graphed.max_steps, max_steps))
         if k < 2:
             return None
         self.scheduler.fill(graphed.arena)
+        self.num_graph_steps += k
+        return graphed, r, k, graphed.run_burst(k, ahead=ahead)
+
+    def _try_burst(self, max_steps: Optional[int] = None) -> Optional[List[RequestOutput]]:
+        """Several decode steps enqueued at once: one upload, the captured steps (each prepares the
+        next one's inputs on the device); their tokens come back stretch by stretch and are handed to
+        the scheduler while the device runs the stretches behind.  Before the host waits for the last
+        stretch it plans and enqueues the next chain (decode_ahead), which the next call then takes
+        in: as long as nothing else comes up, the device never waits for the host.  max_steps: the
+        most steps this call may plan; 0 only takes in what is enqueued."""
+        chain, self._inflight = self._inflight, None
+        if chain is None:
+            if max_steps is not None and max_steps < 2:
+                return None
+            chain = self._launch_chain(max_steps, ahead=False)
+            if chain is None:
+                return None
+            if max_steps is not None:
+                max_steps -= chain[2]
+        graphed, r, k, stretches = chain
         outs: List[RequestOutput] = []
-        stretches = graphed.run_burst(k)
-        for first, end, event in stretches:
+        for i, (first, end, event) in enumerate(stretches):
+            last = i == len(stretches) - 1
+            if last and self.engine_config.decode_ahead and (max_steps is None or max_steps >= 2):
+                self._inflight = self._launch_chain(max_steps, ahead=True)
             event.synchronize()
             tokens = np.ascontiguousarray(graphed.history_host.numpy()[first:end, :r])
             outs += [RequestOutput(self._ids[sid], [token], finished, reason) for sid, token, finished, reason
-                     in self.scheduler.commit_burst(tokens, end - first, last=end == k)]
-        self.num_graph_steps += k
+                     in self.scheduler.commit_burst(tokens, end - first, last=last)]
         return outs
 
     def step(self, max_decode_steps: Optional[int] = None) -> List[RequestOutput]:
         """One step of the engine: admits, runs one batch (or, when every running request is decoding
-        and nobody waits, up to decode_burst x decode_chain decode steps back to back;
-        max_decode_steps lowers that bound), hands the sampled tokens to the scheduler.  Returns one
-        RequestOutput per token sampled."""
-        burst = self._try_burst(max_decode_steps) if max_decode_steps is None or max_decode_steps > 1 else None
-        if burst is not None:
-            return burst
+        and nobody waits, up to decode_burst x decode_chain decode steps back to back), hands the
+        sampled tokens to the scheduler.  Returns one RequestOutput per token sampled.  With
+        decode_ahead a call may also enqueue the decode steps whose tokens the next call returns.
+        max_decode_steps bounds the decode steps that this call newly plans, those enqueued ahead
+        included; 0 only takes in what an earlier call enqueued."""
+        burst = self._try_burst(max_decode_steps)
+        if burst is not None or max_decode_steps == 0:
+            return burst or []
         n, r, m = self.scheduler.schedule()
         if r == 0:
             return []

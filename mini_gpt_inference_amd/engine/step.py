@@ -58,9 +58,12 @@ class StepArena:
             ("cu_q", r_cap + 1, np.int32), ("seq_lens", r_cap, np.int32), ("state_slots", r_cap, np.int32),
             ("logit_rows", m_cap, np.int32), ("slot_mapping", n_groups * n_cap, np.int32),
             ("block_tables", n_groups * r_cap * max_blocks, np.int32),
+            # where the device's history of sampled tokens goes on: every upload sets the device's count
+            # (zero unless the caller says otherwise); behind the cache slots and the block tables, so
+            # that the three can be uploaded alone (upload_tables)
+            ("history_pos", m_cap, np.int32),
             ("temperature", m_cap, np.float32), ("top_k", m_cap, np.int32), ("top_p", m_cap, np.float32),
             ("out_index", m_cap, np.int32),
-            ("history_pos", m_cap, np.int32),   # stays zero on the host: every upload restarts the device's count
         ]
         total = sum(_round_up(n, 4) for _, n, _ in fields)
         self.host_t = torch.zeros(total, dtype=torch.int32, pin_memory=device.type == "cuda")
@@ -73,7 +76,11 @@ class StepArena:
             self.h[name] = host_np[off:off + n].view(typ)
             dv = self.dev_t[off:off + n]
             self.d[name] = dv.view(torch.float32) if typ is np.float32 else dv
+            if name == "slot_mapping":
+                self._tables_begin = off
             off += _round_up(n, 4)
+            if name == "history_pos":
+                self._tables_end = off
         # the addresses of the arrays that the cache manager fills at every step
         self.h_addr: Dict[str, int] = {name: int(self.h[name].ctypes.data) for name in
                                        ("positions", "q_req", "cu_q", "seq_lens", "slot_mapping", "block_tables")}
@@ -85,6 +92,18 @@ class StepArena:
 
     def upload(self) -> None:
         self.dev_t.copy_(self.host_t, non_blocking=True)
+        if self.dev_t.is_cuda:
+            if self._uploaded is None:
+                self._uploaded = torch.cuda.Event()
+            self._uploaded.record()
+
+    def upload_tables(self) -> None:
+        """Uploads the cache slots of the step's tokens, the block tables and the history count only.
+        For steps that go on from what the device itself made of the last ones (tokens, positions,
+        lengths): the new pages, the slot of the first new token (the device looked it up before its
+        page was in the table) and where the history goes on are all the host has to add."""
+        a, b = self._tables_begin, self._tables_end
+        self.dev_t[a:b].copy_(self.host_t[a:b], non_blocking=True)
         if self.dev_t.is_cuda:
             if self._uploaded is None:
                 self._uploaded = torch.cuda.Event()

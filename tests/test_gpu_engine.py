@@ -260,17 +260,18 @@ def test_from_random_and_the_command_line(tmp_path, model_folders):
 def test_decode_bursts_change_nothing_but_the_pace(model_folders, dtype):
     """Steps enqueued back to back with tokens fed on the device give the tokens that one step at a
     time gives: greedy and seeded, with an end token met inside a burst; also with several bursts
-    enqueued before the host waits, whose tokens are taken in while the device runs the next."""
+    enqueued before the host waits, whose tokens are taken in while the device runs the next, and
+    with the next chain enqueued before the last tokens of this one are in."""
     prompts = _prompts("B", [3, 20, 41], seed=6)
     plain_first = _plain_greedy(model_folders["B"], prompts[:1], 12)[0]
     eot = plain_first[6]
     params = [SamplingParams(max_tokens=24, temperature=0.0), SamplingParams(max_tokens=17, temperature=0.9, seed=5),
               SamplingParams(max_tokens=24, temperature=0.7, top_k=20, seed=6)]
     outs, steps = [], []
-    for burst, chain in ((1, 1), (8, 1), (4, 3), (2, 4)):
+    for burst, chain, ahead in ((1, 1, False), (8, 1, False), (4, 3, False), (2, 4, True), (2, 1, True), (8, 2, True)):
         engine = LLMEngine.from_folder(model_folders["B"], EngineConfig(block_size=8, num_blocks=64, max_batch_size=4,
                                                                         dtype=dtype, decode_burst=burst,
-                                                                        decode_chain=chain, seed=3))
+                                                                        decode_chain=chain, decode_ahead=ahead, seed=3))
         for i, (p, sp) in enumerate(zip(prompts, params)):
             engine.add_request(Request(f"r{i}", p, sp, eot_token_id=eot if i == 0 else None))
         got = {f"r{i}": [] for i in range(3)}
@@ -282,7 +283,7 @@ def test_decode_bursts_change_nothing_but_the_pace(model_folders, dtype):
         outs.append(got)
         steps.append(calls)
         assert engine.cache.num_free_pages() == 64 and engine.cache.check() == 0
-    assert outs[0] == outs[1] == outs[2] == outs[3]
+    assert all(o == outs[0] for o in outs[1:])
     assert max(steps[1:]) < steps[0]                # the bursts were taken
     if dtype == "float32":
         assert outs[0]["r0"] == plain_first[:plain_first.index(eot) + 1]

@@ -276,6 +276,41 @@ def test_a_burst_handed_in_in_stretches_ends_like_one_handed_in_whole():
     assert results[0][1] == [100, 5, 7] and results[0][3] == 20 and results[0][4] == 0
 
 
+def test_a_burst_can_be_planned_ahead_of_one_whose_tokens_are_not_all_in():
+    """The device runs the next burst right behind the last one: the scheduler plans it from where
+    that one will end, reserves its pages, and refuses once a request of the last one has ended."""
+    cm, s = make(40, 4, max_batch=4, max_positions=64)
+    a = s.add_request([1, 2, 3], 20, eot=7)
+    b = s.add_request([1, 2, 3, 4, 5], 14)
+    step(s)
+    assert s.plan_burst(4) == 4                       # steps 0..3: a at 3.., b at 5..
+    toks = np.full((4, 2), 5, dtype=np.int32)
+    s.commit_burst(toks[:2], 2, last=False)           # two steps are in, two are not
+    assert s.plan_burst(4) == 4                       # ahead: starts where the first burst ends
+    ents = s.entries()
+    assert [(e.request, e.ctx) for e in ents] == [(a, 3 + 4), (b, 5 + 4)]
+    for e in ents:                                    # pages up to the end of the second burst
+        assert len(cm.table(s.info(e.request).slot)) * 4 >= e.ctx + 4
+    with pytest.raises(Exception):                    # no other scheduling while steps are out
+        s.schedule()
+    s.commit_burst(toks[2:], 2, last=True)            # the first burst's last stretch: entries stay
+    assert len(s.entries()) == 2
+    assert s.plan_burst(8) == 5                       # b has 14 - 5 - 4 = 5 left once the second burst is in
+    outs = s.commit_burst(toks, 4, last=True)
+    assert len(outs) == 8 and len(s.entries()) == 2   # the third burst is still out
+    # a meets its end token in the third burst's first step: no burst goes on behind that
+    toks5 = np.full((5, 2), 5, dtype=np.int32)
+    toks5[0, 0] = 7
+    s.commit_burst(toks5[:1], 1, last=False)
+    assert s.info(a).status == FINISHED
+    assert s.plan_burst(8) == 0
+    outs = s.commit_burst(toks5[1:], 4, last=True)
+    assert [o[0] for o in outs] == [b] * 4 and outs[-1][2:] == (True, "length") and len(s.entries()) == 0
+    assert s.output(a) == [100] + [5] * 8 + [7]
+    assert s.output(b) == [100] + [5] * 13
+    assert not s.has_work() and cm.num_free_pages() == 40 and cm.check() == 0
+
+
 def test_burst_needs_pages_for_every_step_or_does_not_start():
     cm, s = make(4, 4, max_batch=2, max_positions=64)
     a = s.add_request([1, 2, 3], 12)
