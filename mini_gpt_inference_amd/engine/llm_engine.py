@@ -247,7 +247,9 @@ class LLMEngine:
             tokens = np.ascontiguousarray(graphed.history_host.numpy()[first:end, :r])
             outs += [RequestOutput(self._ids[sid], [token], finished, reason) for sid, token, finished, reason
                      in self.scheduler.commit_burst(tokens, end - first, last=last)]
-        return outs
+        # a chain enqueued ahead for requests that have all ended since brings nothing: the caller goes on
+        # with an ordinary step
+        return outs if outs or self._inflight is not None else None
 
     def step(self, max_decode_steps: Optional[int] = None) -> List[RequestOutput]:
         """One step of the engine: admits, runs one batch (or, when every running request is decoding

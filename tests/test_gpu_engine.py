@@ -232,6 +232,34 @@ def test_finished_requests_are_forgotten_and_their_ids_can_be_used_again(model_f
     assert engine.cache.num_free_pages() == 64 and engine.cache.check() == 0
 
 
+def test_requests_that_end_while_the_next_chain_is_already_enqueued(model_folders):
+    """An end token met in a chain's last steps: the chain enqueued behind it computes for requests
+    that are over; its tokens are dropped, and the engine goes on with whoever comes next."""
+    prompts = _prompts("B", [7, 12], seed=40)
+    plain = _plain_greedy(model_folders["B"], prompts, 30)
+    engine = LLMEngine.from_folder(model_folders["B"], EngineConfig(block_size=8, num_blocks=64, max_batch_size=4,
+                                                                    dtype="float32", decode_burst=2, decode_chain=2))
+    # request 0 ends by its end token some chains in (further steps are planned ahead by then),
+    # request 1 is cancelled by the caller at that moment
+    first = [j for j in range(4, 30) if plain[0][j] not in plain[0][:j]]
+    assert first, "the plain tokens never bring a new token: choose another seed"
+    eot = plain[0][first[0]]
+    engine.add_request(Request("a", prompts[0], SamplingParams(max_tokens=30, temperature=0.0), eot_token_id=eot))
+    engine.add_request(Request("b", prompts[1], SamplingParams(max_tokens=30, temperature=0.0)))
+    got = {"a": [], "b": []}
+    while "a" in engine._rids and engine.scheduler.info(engine._rids["a"]).status != 2:
+        for out in engine.step():
+            got[out.request_id] += out.new_token_ids
+    assert got["a"] == plain[0][:first[0] + 1]
+    engine.cancel_request("b")
+    assert not engine.has_unfinished_requests()
+    assert got["b"] == plain[1][:len(got["b"])]
+    # the engine is used again while a chain for the two is still enqueued
+    again = engine.generate(prompts, SamplingParams(max_tokens=9, temperature=0.0))
+    assert again == [p[:9] for p in plain]
+    assert engine.cache.num_free_pages() == 64 and engine.cache.check() == 0 and engine._inflight is None
+
+
 def test_real_vocabulary_bound_is_never_crossed(model_folders):
     engine = LLMEngine.from_folder(model_folders["A"], EngineConfig(block_size=4, num_blocks=32, max_batch_size=4,
                                                                     dtype="float32", real_vocab_size=40))
