@@ -163,6 +163,9 @@ def serve_run(args, name):
                         max_num_batched_tokens=4096, prefill_chunk=w["prefill_chunk"], dtype=args.dtype,
                         use_graph=not args.no_graph, decode_burst=args.burst, decode_chain=args.chain)
     engine = LLMEngine.from_random(cfg, seed=0, engine_config=ecfg)
+    if not args.no_capture:
+        engine.capture_decode_graphs()      # before the clock starts, as a server does before it takes requests
+    before = engine.stats()
     for i, (p, o) in enumerate(requests):
         engine.add_request(Request(f"r{i}", p, SamplingParams(max_tokens=o, temperature=0.0)))
     torch.cuda.synchronize()
@@ -172,7 +175,8 @@ def serve_run(args, name):
         produced += len(engine.step())
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
-    stats = engine.stats()
+    stats = {key: value - before[key] if key.startswith(("num_", "graph_", "eager_", "replayed_")) else value
+             for key, value in engine.stats().items()}
     assert produced == sum(o for _, o in requests), "a request ended early or late"
     assert stats["free_blocks"] == pages, "pages were lost"
     return {"workload": name, "value": round(produced / elapsed, 1), "unit": "generated tokens/s",
@@ -206,6 +210,8 @@ def main() -> int:
                     help="instead of the decode measurement: a whole continuous-batching run with the shape "
                          "of GPT-2 small (64 mixed requests, prompt portions of 512) or of GPT-2 XL (256 "
                          "requests, a page pool too small for them: evictions)")
+    ap.add_argument("--no-capture", action="store_true",
+                    help="--workload: leave the decode graphs to be captured inside the timed run")
     ap.add_argument("--workload-layers", type=int, default=0, help="fewer layers for --workload (0 = the shape's)")
     ap.add_argument("--workload-requests", type=int, default=0, help="fewer requests for --workload")
     ap.add_argument("--report", default=None,

@@ -323,6 +323,50 @@ class LLMEngine:
         self.forget_finished()
         return [got[name] for name in names]
 
+    def capture_decode_graphs(self, batch_sizes: Optional[Sequence[int]] = None) -> List[int]:
+        """Captures the graphs of decode steps ahead of time, as a server does before it takes
+        requests (the reference's CUDAGraphRunner.capture does it for one batch size,
+        src/minigpt_infer/graphs.py:96-110): for every capacity that decode steps are padded to (the
+        powers of two up to max_batch_size, or those that hold the given batch sizes) it runs that many
+        made-up one-token requests for a few steps, which captures the single step and the burst.
+        A capacity whose requests the page pool cannot hold is left out.  Returns the capacities
+        captured.  The engine must be idle; its counters count these steps too, and requests that
+        bring no seed of their own draw from other streams than without this call."""
+        ecfg = self.engine_config
+        if self.has_unfinished_requests() or self._inflight is not None:
+            raise RuntimeError("capture_decode_graphs needs an idle engine")
+        if not ecfg.use_graph or not self.model.graph_safe:
+            return []
+        if batch_sizes is None:
+            caps, c = [], 1
+            while c < ecfg.max_batch_size:
+                caps.append(c)
+                c *= 2
+            caps.append(c)
+        else:
+            caps = sorted({_bucket(max(int(b), 1)) for b in batch_sizes})
+        steps = max(ecfg.decode_burst, 1) * max(ecfg.decode_chain, 1) + 3
+        if self.runner.max_positions is not None:
+            steps = min(steps, self.runner.max_positions - 1)
+        done: List[int] = []
+        for cap in caps:
+            n = min(cap, ecfg.max_batch_size)
+            if steps < 2 or _bucket(n) != cap:
+                continue
+            if any(n * self.cache.pages_needed(1 + steps, g) > self.cache.num_free_pages(g)
+                   for g in range(len(self.cache.groups))):
+                continue
+            for i in range(n):
+                self.add_request(Request(f"capture-{cap}-{i}-{self._generated}", [0],
+                                         SamplingParams(max_tokens=steps, temperature=0.0)))
+            self._generated += 1
+            while self.has_unfinished_requests():
+                self.step()
+            self.forget_finished()
+            if cap in self._graphs and self._graphs[cap].graph is not None:
+                done.append(cap)
+        return done
+
     def forget_finished(self) -> int:
         """Drops what the engine still holds of finished requests (their ids and token lists), so that
         an engine that serves for a long time does not grow; their ids may be used again.  Returns

@@ -260,6 +260,29 @@ def test_requests_that_end_while_the_next_chain_is_already_enqueued(model_folder
     assert engine.cache.num_free_pages() == 64 and engine.cache.check() == 0 and engine._inflight is None
 
 
+def test_decode_graphs_can_be_captured_before_the_first_request(model_folders):
+    prompts = _prompts("A", [5, 17, 30])
+    want = _plain_greedy(model_folders["A"], prompts, 12)
+    engine = LLMEngine.from_folder(model_folders["A"], EngineConfig(block_size=4, num_blocks=96, max_batch_size=4,
+                                                                    dtype="float32"))
+    assert engine.capture_decode_graphs() == [1, 2, 4]
+    assert engine.cache.num_free_pages() == 96 and engine.cache.check() == 0 and not engine._rids
+    graphs = {cap: (g.graph, g.burst_graph) for cap, g in engine._graphs.items()}
+    assert all(g is not None and b is not None for g, b in graphs.values())
+    eager_before = engine.stats()["eager_steps"]
+    assert engine.generate(prompts, SamplingParams(max_tokens=12, temperature=0.0)) == want
+    # nothing was captured again, and only the prompts' step ran outside a decode graph
+    assert {cap: (g.graph, g.burst_graph) for cap, g in engine._graphs.items()} == graphs
+    assert engine.stats()["eager_steps"] - eager_before == 1
+    # too few pages for four made-up requests: that capacity is left out
+    small = LLMEngine.from_folder(model_folders["A"], EngineConfig(block_size=4, num_blocks=20, max_batch_size=4,
+                                                                   dtype="float32"))
+    assert small.capture_decode_graphs() == [1, 2]
+    with pytest.raises(RuntimeError):
+        small.add_request(Request("x", [1, 2], SamplingParams(max_tokens=4)))
+        small.capture_decode_graphs()
+
+
 def test_real_vocabulary_bound_is_never_crossed(model_folders):
     engine = LLMEngine.from_folder(model_folders["A"], EngineConfig(block_size=4, num_blocks=32, max_batch_size=4,
                                                                     dtype="float32", real_vocab_size=40))
