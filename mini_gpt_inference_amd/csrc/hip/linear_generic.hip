@@ -82,16 +82,77 @@ __global__ __launch_bounds__(256) void linear_generic_kernel(
   }
 }
 
+// The same product for few rows (a decode step on the 32-bit path): with 64 x 64 tiles a product of
+// one row by 512 columns is eight workgroups that each walk the whole inner size.  Here a workgroup
+// owns 16 rows x 16 columns, one output element a thread, so there are as many workgroups as the
+// matrix has groups of 16 columns.  Every element is the same chain as above (acc = fma(a[k], w[k],
+// acc) for k = 0..K-1 from zero, then the bias): the two kernels agree bit for bit, and a token's
+// logits do not depend on which of them ran.
+#define ROWS_TILE 16
+#define ROWS_BK 64
+
+template <typename AT, typename WT, typename OT, int EPI>
+__global__ __launch_bounds__(256) void linear_generic_rows_kernel(
+    const AT* __restrict__ A, long lda, const WT* __restrict__ W, const float* __restrict__ bias,
+    OT* __restrict__ out, long ldo, int n_rows, int n_out, int k_dim) {
+  __shared__ float As[ROWS_TILE][ROWS_BK + 1];
+  __shared__ float Ws[ROWS_TILE][ROWS_BK + 1];
+  const int tid = threadIdx.x;
+  const int r = tid >> 4, c = tid & 15;        // the element this thread owns; also the row it stages
+  const int sk = (tid & 15) * 4;               // ... and which four k of a stage
+  const int row0 = blockIdx.y * ROWS_TILE, col0 = blockIdx.x * ROWS_TILE;
+  const bool a_ok = row0 + r < n_rows, w_ok = col0 + r < n_out;
+  const AT* ap = A + (long)(row0 + r) * lda + sk;
+  const WT* wp = W + (long)(col0 + r) * k_dim + sk;
+  float acc = 0.f;
+  for (int k0 = 0; k0 < k_dim; k0 += ROWS_BK) {
+    const int kmax = k_dim - k0 < ROWS_BK ? k_dim - k0 : ROWS_BK;   // a multiple of 16, so of 4
+    const bool k_ok = sk < kmax;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      As[r][sk + i] = (a_ok && k_ok) ? to_float<AT>(ap[k0 + i]) : 0.f;
+      Ws[r][sk + i] = (w_ok && k_ok) ? to_float<WT>(wp[k0 + i]) : 0.f;
+    }
+    __syncthreads();
+    if (kmax == ROWS_BK) {
+#pragma unroll
+      for (int kk = 0; kk < ROWS_BK; ++kk) acc = fmaf(As[r][kk], Ws[c][kk], acc);
+    } else {
+      for (int kk = 0; kk < kmax; ++kk) acc = fmaf(As[r][kk], Ws[c][kk], acc);
+    }
+    __syncthreads();
+  }
+  const int row = row0 + r, col = col0 + c;
+  if (row >= n_rows || col >= n_out) return;
+  float v = acc;
+  if (bias) v += bias[col];
+  if (EPI == EPI_GELU) v = gelu_tanh(v);
+  OT* dst = out + (long)row * ldo + col;
+  if (EPI == EPI_RESIDUAL) {
+    *dst = from_float<OT>(to_float<OT>(*dst) + v);
+  } else {
+    *dst = from_float<OT>(v);
+  }
+}
+
+#define ROWS_KERNEL_MAX_ROWS 32   // more rows than this: the 64 x 64 tiles
+
 template <typename AT, typename WT, typename OT>
 static int launch_epi(const void* A, long lda, const void* W, const float* bias, void* out, long ldo,
                       int n_rows, int n_out, int k_dim, int epi, hipStream_t stream) {
+  const bool few = n_rows <= ROWS_KERNEL_MAX_ROWS;
   dim3 grid((n_out + TILE - 1) / TILE, (n_rows + TILE - 1) / TILE), block(256);
-#define LAUNCH(E)                                                                               \
-  hipLaunchKernelGGL((linear_generic_kernel<AT, WT, OT, E>), grid, block, 0, stream, (const AT*)A, \
-                     lda, (const WT*)W, bias, (OT*)out, ldo, n_rows, n_out, k_dim)
-  if (epi == EPI_NONE) LAUNCH(EPI_NONE);
-  else if (epi == EPI_GELU) LAUNCH(EPI_GELU);
-  else if (epi == EPI_RESIDUAL) LAUNCH(EPI_RESIDUAL);
+  dim3 grid_rows((n_out + ROWS_TILE - 1) / ROWS_TILE, (n_rows + ROWS_TILE - 1) / ROWS_TILE);
+#define LAUNCH(E)                                                                                      \
+  if (few)                                                                                             \
+    hipLaunchKernelGGL((linear_generic_rows_kernel<AT, WT, OT, E>), grid_rows, block, 0, stream,       \
+                       (const AT*)A, lda, (const WT*)W, bias, (OT*)out, ldo, n_rows, n_out, k_dim);    \
+  else                                                                                                 \
+    hipLaunchKernelGGL((linear_generic_kernel<AT, WT, OT, E>), grid, block, 0, stream, (const AT*)A,   \
+                       lda, (const WT*)W, bias, (OT*)out, ldo, n_rows, n_out, k_dim)
+  if (epi == EPI_NONE) { LAUNCH(EPI_NONE); }
+  else if (epi == EPI_GELU) { LAUNCH(EPI_GELU); }
+  else if (epi == EPI_RESIDUAL) { LAUNCH(EPI_RESIDUAL); }
   else return MGPT_ERR_BAD_SHAPE;
 #undef LAUNCH
   return mgpt_last_error();

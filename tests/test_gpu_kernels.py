@@ -84,6 +84,30 @@ def test_linear_generic(a_dt, w_dt, o_dt, epi):
     helpers.assert_close(out, _linear_want(a, w, bias, epi, prev), tol, "linear_generic")
 
 
+@pytest.mark.parametrize("n_few", [1, 7, 16, 17, 32])
+@pytest.mark.parametrize("a_dt,w_dt,o_dt,epi", [("float32", "float32", "float32", kernels.EPI_NONE),
+                                                ("float32", "float32", "float32", kernels.EPI_RESIDUAL),
+                                                ("float32", "float32", "float32", kernels.EPI_GELU),
+                                                ("bfloat16", "float32", "bfloat16", kernels.EPI_GELU),
+                                                ("bfloat16", "bfloat16", "float32", kernels.EPI_NONE)])
+def test_linear_generic_few_rows_and_many_agree_bit_for_bit(a_dt, w_dt, o_dt, epi, n_few):
+    """Up to 32 rows go to a kernel with a workgroup per 16 x 16 outputs, more to 64 x 64 tiles: every
+    element is the same chain of fused multiply-adds along k in both, so a row's result is the same
+    bits whichever kernel its step's size chooses (a decode step against a prompt's step)."""
+    g = torch.Generator().manual_seed(23)
+    n, k, o = 50, 208, 137      # an inner size that is no multiple of the few-rows kernel's stage of 64
+    a, w, bias = rnd(g, n, k, dtype=a_dt), rnd(g, o, k, dtype=w_dt), rnd(g, o)
+    prev = rnd(g, n, o, dtype=o_dt)
+    many = prev.clone().to(DEV)
+    kernels.linear_generic(a.to(DEV), w.to(DEV), bias.to(DEV), many, n, epi)
+    few = prev.clone().to(DEV)
+    kernels.linear_generic(a.to(DEV), w.to(DEV), bias.to(DEV), few, n_few, epi)
+    assert torch.equal(few[:n_few], many[:n_few])
+    assert torch.equal(few[n_few:], prev[n_few:].to(DEV)), "rows beyond n_rows were written"
+    helpers.assert_close(few[:n_few], _linear_want(a, w, bias, epi, prev)[:n_few],
+                         "float32" if "bfloat16" not in (a_dt, w_dt, o_dt) else "bfloat16", "few rows")
+
+
 def test_linear_generic_refuses_bad_inner_size():
     a, w = torch.zeros(4, 40, device=DEV), torch.zeros(8, 40, device=DEV)
     with pytest.raises(kernels.KernelError, match="multiple of 16"):
