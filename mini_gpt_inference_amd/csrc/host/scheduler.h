@@ -90,7 +90,7 @@ class Scheduler {
   // A burst: up to max_k decode steps of the running requests planned at once, so that the device
   // can run them back to back while it feeds each step's tokens to the next by itself.  Only when
   // every running request is decoding, nobody waits, and pages for all k tokens are free; k stops
-  // one short of the first request's length limit, so nobody can end inside a burst except by its
+  // at the first request's length limit, so nobody can end before a burst's last step except by its
   // end token.  Returns k >= 2 with entries() set to step 0, or 0 when a burst is not possible
   // (then nothing has changed).  Step j of a burst feeds position ctx + j.
   // A further burst may be planned before the last one's tokens are all handed in (the device then
