@@ -162,7 +162,11 @@ int mgpt_sched_fill(void* sv, void* cm, int step_offset, int n_stride, int r_str
   for (int i = 0; i < R; ++i) {
     const mgpt::Request* r = s->request(e[i].id);
     state_slots[i] = r->slot;
-    for (int j = 0; j < e[i].q_len; ++j) token_ids[t++] = step_offset ? 0 : r->token_at(e[i].ctx + j);
+    // a burst planned ahead of one that is not handed in yet starts at a token only the device has
+    for (int j = 0; j < e[i].q_len; ++j) {
+      const int at = e[i].ctx + j;
+      token_ids[t++] = (step_offset || at >= r->num_tokens()) ? 0 : r->token_at(at);
+    }
     if (e[i].sample) {
       if (m >= m_stride) return -4;
       logit_rows[m] = t - 1;

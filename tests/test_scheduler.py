@@ -311,6 +311,29 @@ def test_a_burst_can_be_planned_ahead_of_one_whose_tokens_are_not_all_in():
     assert not s.has_work() and cm.num_free_pages() == 40 and cm.check() == 0
 
 
+def test_filling_a_burst_planned_ahead_reads_no_token_the_host_does_not_have():
+    """The first token of a burst planned ahead exists on the device only: the filled step names
+    position, cache slot and block table for it and leaves its token id at zero."""
+    import torch
+    from mini_gpt_inference_amd.engine.step import StepArena
+    cm, s = make(40, 4, max_batch=4, max_positions=64)
+    a = s.add_request([1, 2, 3], 20)
+    step(s)
+    assert s.plan_burst(4) == 4
+    arena = StepArena(4, 4, 4, 1, 16, torch.device("cpu"))
+    s.fill(arena)
+    assert arena.h["token_ids"][0] == 100 and arena.h["positions"][0] == 3
+    assert s.plan_burst(4) == 4                     # ahead of the four steps that are still out
+    arena.h["token_ids"][:] = -7
+    s.fill(arena)
+    slot = s.info(a).slot
+    assert arena.h["token_ids"][0] == 0 and arena.h["positions"][0] == 7 and arena.h["seq_lens"][0] == 8
+    assert arena.h["slot_mapping"][0] == cm.table(slot)[7 // 4] * 4 + 7 % 4
+    assert list(arena.h["block_tables"][:3]) == cm.table(slot)[:3]
+    s.commit_burst(np.full((8, 1), 5, dtype=np.int32), 8)
+    assert s.output(a) == [100] + [5] * 8
+
+
 def test_burst_needs_pages_for_every_step_or_does_not_start():
     cm, s = make(4, 4, max_batch=2, max_positions=64)
     a = s.add_request([1, 2, 3], 12)
