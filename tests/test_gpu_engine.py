@@ -340,6 +340,53 @@ def test_decode_bursts_change_nothing_but_the_pace(model_folders, dtype):
         assert outs[0]["r0"] == plain_first[:plain_first.index(eot) + 1]
 
 
+@pytest.mark.parametrize("name,seed", [("A", 0), ("A", 1), ("A", 2), ("A", 3), ("B", 4), ("B", 5), ("B", 6), ("B", 7),
+                                       ("C", 8), ("D", 9)])
+def test_random_engine_settings_give_the_tokens_of_one_step_at_a_time_32bit(model_folders, name, seed):
+    """Sampled and greedy requests with end tokens arrive over time; an engine with drawn settings
+    (page pool, batch size, token budget, portions, bursts, chains, steps enqueued ahead) gives every
+    request the tokens that an engine without bursts and with room for everything gives it."""
+    cfg = helpers.CONFIGS[name]
+    rng = np.random.default_rng(5000 + seed)
+    reqs = []
+    for i in range(int(rng.integers(6, 20))):
+        n = int(rng.integers(1, cfg.block_size // 2))
+        m = int(rng.integers(2, min(40, cfg.block_size - n)))
+        t = float(rng.choice([0.0, 0.7, 1.3]))
+        sp = SamplingParams(max_tokens=m, temperature=t, top_k=int(rng.integers(0, 30)) or None,
+                            top_p=float(rng.choice([1.0, 0.9, 0.5])) if t > 0 else None, seed=int(rng.integers(0, 1000)))
+        eot = int(rng.integers(0, cfg.vocab_size)) if rng.random() < 0.7 else None
+        reqs.append((helpers.random_ids(rng, cfg.vocab_size, n), sp, eot))
+    arrivals = sorted((int(rng.integers(0, 30)), i) for i in range(len(reqs)))
+    page = 4
+    pool = max(-(-(len(p) + sp.max_tokens) // page) for p, sp, _ in reqs) + int(rng.integers(2, 60))
+
+    def run(ecfg):
+        engine = LLMEngine.from_folder(model_folders[name], ecfg)
+        got = {i: [] for i in range(len(reqs))}
+        todo, step = list(arrivals), 0
+        while todo or engine.has_unfinished_requests():
+            while todo and todo[0][0] <= step:
+                _, i = todo.pop(0)
+                engine.add_request(Request(f"r{i}", reqs[i][0], reqs[i][1], eot_token_id=reqs[i][2]))
+            for out in engine.step():
+                got[int(out.request_id[1:])].extend(out.new_token_ids)
+            step += 1
+            if step % 7 == 0:
+                engine.forget_finished()
+            assert step < 5000, "the engine makes no progress"
+        engine.step(max_decode_steps=0)      # steps enqueued ahead for requests that ended since
+        assert engine.cache.check() == 0 and engine.cache.num_free_pages() == ecfg.num_blocks
+        return got
+
+    base = run(EngineConfig(block_size=page, num_blocks=pool + 50, max_batch_size=4, dtype="float32", decode_burst=1, seed=9))
+    drawn = EngineConfig(block_size=page, num_blocks=pool, max_batch_size=int(rng.integers(1, 24)),
+                         max_num_batched_tokens=int(rng.integers(8, 64)), prefill_chunk=int(rng.integers(0, 12)),
+                         dtype="float32", decode_burst=int(rng.integers(2, 9)), decode_chain=int(rng.integers(1, 5)),
+                         decode_ahead=True, seed=9)
+    assert run(drawn) == base, drawn
+
+
 @pytest.mark.parametrize("name,seed", [("A", 0), ("B", 1), ("C", 2)])
 def test_arrivals_evictions_bursts_and_cancels_together_32bit(model_folders, name, seed):
     """Requests arrive while others decode, the page pool is too small for all of them, prompts are
