@@ -41,10 +41,12 @@ __global__ __launch_bounds__(256) void linear_decode_kernel(SkinnyArgs a) {
   const int wo = min(o0 + lrow, a.n_out - 1);  // a column past the end reads the last row; never stored
   const int oc = o0 + g * 4;  // this lane's four output columns, of rows lrow + 16 t
   // rows of this workgroup: with gridDim.y > 1 the rows are dealt out in groups of NT * 16
-  const int r0 = (int)blockIdx.y * (NT * 16) + lrow;
+  // (one tile a workgroup: the group may be smaller than the tile, a.rows_per_group of its 16 rows)
+  const int rpg = NT == 1 ? a.rows_per_group : 16;
+  const int r0 = (int)blockIdx.y * (NT == 1 ? rpg : NT * 16) + lrow;
   bool row_ok[NT];
 #pragma unroll
-  for (int t = 0; t < NT; ++t) row_ok[t] = r0 + t * 16 < a.n_rows;
+  for (int t = 0; t < NT; ++t) row_ok[t] = lrow < rpg && r0 + t * 16 < a.n_rows;
 
   // ---- every load this lane will need, issued before anything waits.  Loads are unconditional
   // within a row (a k step past this wave's range reads the range's first step again and is not

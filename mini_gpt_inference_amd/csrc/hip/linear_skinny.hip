@@ -302,7 +302,8 @@ static int launch_nt(const SkinnyArgs& a, int epi, int out_dtype, dim3 grid, siz
 // act holds bfloat16 activations.  Refuses (MGPT_ERR_BAD_SHAPE) more than 64 rows and k_dim that
 // is no multiple of 16; the caller then takes the general kernels.  mode: 0 = the launcher chooses;
 // 1 keeps to this file's kernel also where linear_decode.hip would take the shape; SK_ROWS_SHARE_W
-// and SK_ROWS_GROUPS say how linear_decode.hip treats more than 16 rows (see there).  w_packed: optional, the
+// and SK_ROWS_GROUPS say how linear_decode.hip treats more than 16 rows (see there); 16, 8 or 4 in
+// the bits above the lowest eight fix the rows it gives a workgroup of one tile.  w_packed: optional, the
 // same matrix in mgpt_pack_weight's layout (only linear_decode.hip reads it).  partials: optional scratch of
 // mgpt_linear_skinny_partials(...) floats; with it a long inner size with many rows is split over
 // workgroups (two launches).
@@ -349,7 +350,8 @@ extern "C" int mgpt_linear_skinny(const void* act, long lda, const float* x, con
   a.n_kv_head = n_kv_head; a.page_size = page_size;
   // room for the parts of a split over workgroups, if the caller brought enough of it
   a.k_parts = 1;
-  a.rows_mode = (mode == SK_ROWS_SHARE_W || mode == SK_ROWS_GROUPS) ? mode : 0;
+  a.rows_mode = ((mode & 0xFF) == SK_ROWS_SHARE_W || (mode & 0xFF) == SK_ROWS_GROUPS) ? (mode & 0xFF) : 0;
+  a.rows_per_group = mode >> 8;
   a.partials = (partials && partials_floats >= mgpt_linear_decode_partials(n_rows, n_out, k_dim, ln, epilogue,
                                                                            a.rows_mode))
                    ? partials : nullptr;

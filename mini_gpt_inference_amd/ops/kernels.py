@@ -284,7 +284,7 @@ def linear_skinny(a: Optional[torch.Tensor], w: torch.Tensor, bias: Optional[tor
                   ln_colsum: Optional[torch.Tensor] = None, ln_eps: float = 0.0,
                   ln_rows: Optional[torch.Tensor] = None, scatter=None, general_only: bool = False,
                   partials: Optional[torch.Tensor] = None, w_packed: Optional[torch.Tensor] = None,
-                  rows_mode: int = 0) -> bool:
+                  rows_mode: int = 0, rows_per_group: int = 0) -> bool:
     """bfloat16 MFMA product for at most 64 rows.  With ln_x (the float32 residual stream; ln_rows an
     optional gather) the rows are read through a LayerNorm that fold_layer_norm folded into w, bias
     and ln_colsum.  scatter = (k_pool, v_pool, slot_mapping, q_width, kv_width) also stores the new
@@ -293,7 +293,8 @@ def linear_skinny(a: Optional[torch.Tensor], w: torch.Tensor, bias: Optional[tor
     float32 scratch of linear_skinny_partials(...) elements, with which a long inner size under many
     rows is split over workgroups.  w_packed: pack_weight(w), which the decode kernel reads faster
     than w itself.  rows_mode: how the decode kernel treats 17 to 64 rows (0: it chooses, ROWS_SHARE_W:
-    one workgroup per column tile takes all rows, ROWS_GROUPS: one per column tile and 16 rows).  Returns False, having launched nothing, when the kernel does not take the shape."""
+    one workgroup per column tile takes all rows, ROWS_GROUPS: one per column tile and 16 rows); rows_per_group:
+    16, 8 or 4 rows to a workgroup of one tile (0: the kernel's launcher chooses).  Returns False, having launched nothing, when the kernel does not take the shape."""
     if n_rows > _SKINNY_MAX_ROWS or w.dtype != torch.bfloat16:
         return False
     n_out, k_dim = w.shape
@@ -348,7 +349,7 @@ def linear_skinny(a: Optional[torch.Tensor], w: torch.Tensor, bias: Optional[tor
         _ptr(a if ln_x is None else None), lda, _ptr(ln_x), _ptr(ln_rows), _ptr(ln_colsum),
         float(ln_eps), _ptr(w), _ptr(w_packed), _ptr(bias), _ptr(out), _dtype_code(out), out.stride(0), n_rows,
         n_out, k_dim, epilogue, _ptr(kp), _ptr(vp), _ptr(sm), q_width, kv_width, head_dim, n_kv_head, page_size,
-        1 if general_only else rows_mode, _ptr(partials), 0 if partials is None else partials.numel(), _stream())
+        1 if general_only else rows_mode | (rows_per_group << 8), _ptr(partials), 0 if partials is None else partials.numel(), _stream())
     if rc == -2:
         return False
     _check(rc, "linear_skinny")
