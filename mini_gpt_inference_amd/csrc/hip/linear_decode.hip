@@ -55,18 +55,23 @@ int mgpt_launch_linear_decode(const SkinnyArgs& a, int epilogue, int out_dtype, 
   const int per = (a.k_dim / 32 + 3) / 4;  // k steps of the first waves
   // Rows of a group: 16 fill the MFMA's tile, but while the workgroups are few, fewer rows to a
   // workgroup (the tile's other rows stay zero and are never loaded) make a workgroup's share of the
-  // activations smaller and the workgroups more: 8 or 4 rows as long as there are no more than 256
-  // workgroups, and only for a matrix small enough that reading it once more per group costs
-  // nothing ([512 x 2048] at 16 rows: 3.6 us with groups of 4 against 4.4; [1600 x 6400] at 8 rows:
-  // 11.5 against 8.7).  The sums are the same whatever the groups.  (rows_per_group forced: by the
+  // activations smaller and the workgroups more: the fewest rows of 1, 2, 4, 8 with which there are
+  // no more than 256 workgroups, and only for a matrix small enough that reading it once more per
+  // group costs nothing ([512 x 2048] at 16 rows: 3.4 us with groups of 2, 3.6 with groups of 4,
+  // 4.4 with one of 16, and 4.2 with groups of 1, which are 512 workgroups; [1600 x 6400] at 8 rows:
+  // 11.5 with groups of 4 against 8.7).  The sums are the same whatever the groups.  (rows_per_group forced: by the
   // caller's wish.)
   SkinnyArgs b = a;
-  if (b.rows_per_group != 4 && b.rows_per_group != 8 && b.rows_per_group != 16) {
+  if (b.rows_per_group != 1 && b.rows_per_group != 2 && b.rows_per_group != 4 && b.rows_per_group != 8 &&
+      b.rows_per_group != 16) {
     b.rows_per_group = 16;
     const long tiles = (a.n_out + 15) / 16;
     if ((long)a.n_out * a.k_dim * (long)sizeof(bf16_t) <= SK_ROW_GROUPS_MAX_BYTES) {
-      if (a.n_rows > 4 && tiles * ((a.n_rows + 3) / 4) <= 256) b.rows_per_group = 4;
-      else if (a.n_rows > 8 && tiles * ((a.n_rows + 7) / 8) <= 256) b.rows_per_group = 8;
+      for (int rpg = 1; rpg < 16; rpg *= 2)
+        if (a.n_rows > rpg && tiles * ((a.n_rows + rpg - 1) / rpg) <= 256) {
+          b.rows_per_group = rpg;
+          break;
+        }
     }
   }
   dim3 grid((a.n_out + 15) / 16, (a.n_rows + b.rows_per_group - 1) / b.rows_per_group);

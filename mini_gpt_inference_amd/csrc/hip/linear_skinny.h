@@ -37,7 +37,7 @@ struct SkinnyArgs {
   // more than 16 rows in linear_decode.hip: 0 = the launcher chooses, SK_ROWS_SHARE_W = one workgroup
   // per column tile takes all rows, SK_ROWS_GROUPS = one workgroup per column tile and 16 rows
   int rows_mode;
-  int rows_per_group;  // linear_decode.hip, one tile a workgroup: rows of a group, 16, 8 or 4 (set by its launcher)
+  int rows_per_group;  // linear_decode.hip, one tile a workgroup: rows of a group, 16, 8, 4, 2 or 1 (set by its launcher)
   // key/value scatter (SK_EPI_QKV)
   bf16_t* kpool;
   bf16_t* vpool;

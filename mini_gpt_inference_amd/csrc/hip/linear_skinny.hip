@@ -302,7 +302,7 @@ static int launch_nt(const SkinnyArgs& a, int epi, int out_dtype, dim3 grid, siz
 // act holds bfloat16 activations.  Refuses (MGPT_ERR_BAD_SHAPE) more than 64 rows and k_dim that
 // is no multiple of 16; the caller then takes the general kernels.  mode: 0 = the launcher chooses;
 // 1 keeps to this file's kernel also where linear_decode.hip would take the shape; SK_ROWS_SHARE_W
-// and SK_ROWS_GROUPS say how linear_decode.hip treats more than 16 rows (see there); 16, 8 or 4 in
+// and SK_ROWS_GROUPS say how linear_decode.hip treats more than 16 rows (see there); 16, 8, 4, 2 or 1 in
 // the bits above the lowest eight fix the rows it gives a workgroup of one tile.  w_packed: optional, the
 // same matrix in mgpt_pack_weight's layout (only linear_decode.hip reads it).  partials: optional scratch of
 // mgpt_linear_skinny_partials(...) floats; with it a long inner size with many rows is split over

@@ -294,7 +294,7 @@ def linear_skinny(a: Optional[torch.Tensor], w: torch.Tensor, bias: Optional[tor
     rows is split over workgroups.  w_packed: pack_weight(w), which the decode kernel reads faster
     than w itself.  rows_mode: how the decode kernel treats 17 to 64 rows (0: it chooses, ROWS_SHARE_W:
     one workgroup per column tile takes all rows, ROWS_GROUPS: one per column tile and 16 rows); rows_per_group:
-    16, 8 or 4 rows to a workgroup of one tile (0: the kernel's launcher chooses).  Returns False, having launched nothing, when the kernel does not take the shape."""
+    16, 8, 4, 2 or 1 rows to a workgroup of one tile (0: the kernel's launcher chooses).  Returns False, having launched nothing, when the kernel does not take the shape."""
     if n_rows > _SKINNY_MAX_ROWS or w.dtype != torch.bfloat16:
         return False
     n_out, k_dim = w.shape

@@ -143,15 +143,15 @@ def test_linear_skinny(n, k, o, epi, o_dt, general):
                                          rows_mode=mode)
             helpers.assert_close(out_m[:n], _linear_want(a, w, bias, epi, prev)[:n], "bfloat16", f"rows mode {mode}")
             assert torch.equal(out_m[n:], prev[n:].to(DEV)), "rows beyond n_rows were written"
-        # 16, 8 or 4 rows to a workgroup: the same sums whatever the groups
+        # 16, 8, 4 or 1 rows to a workgroup: the same sums whatever the groups
         outs = []
-        for rpg in (16, 8, 4):
+        for rpg in (16, 8, 1):
             out_g = prev.clone().to(DEV)
             assert kernels.linear_skinny(a.to(DEV), w.to(DEV), bias.to(DEV), out_g, n, epi, w_packed=packed,
                                          rows_mode=kernels.ROWS_GROUPS, rows_per_group=rpg)
             outs.append(out_g)
         assert torch.equal(outs[0], outs[1]) and torch.equal(outs[0], outs[2]), "the groups' size changes the result"
-        helpers.assert_close(outs[2][:n], _linear_want(a, w, bias, epi, prev)[:n], "bfloat16", "groups of 4 rows")
+        helpers.assert_close(outs[2][:n], _linear_want(a, w, bias, epi, prev)[:n], "bfloat16", "groups of 1 row")
         assert torch.equal(outs[2][n:], prev[n:].to(DEV)), "rows beyond n_rows were written"
     helpers.assert_close(out[:n], _linear_want(a, w, bias, epi, prev)[:n], "bfloat16", f"skinny {n}x{k}x{o}")
     assert torch.equal(out[n:], prev[n:].to(DEV)), "rows beyond n_rows were written"
@@ -288,7 +288,7 @@ def test_linear_skinny_through_a_folded_layer_norm(n, k, o, ln_bias, gather, gen
                                  f"LN + skinny, rows mode {mode}")
             assert torch.isnan(out_m[n:]).all(), "rows beyond n_rows were written"
         outs = []
-        for rpg in (16, 8, 4):
+        for rpg in (16, 4, 2):
             out_g = torch.full((n + 1, o), float("nan"), dtype=torch.float32, device=DEV)
             assert kernels.linear_skinny(None, wf, bias_f, out_g, n, kernels.EPI_NONE, ln_x=x.to(DEV),
                                          ln_colsum=colsum, ln_eps=1e-5, ln_rows=i32(rows) if gather else None,
@@ -302,7 +302,8 @@ def test_linear_skinny_through_a_folded_layer_norm(n, k, o, ln_bias, gather, gen
                                                      (False, 40, kernels.ROWS_SHARE_W, 0),
                                                      (False, 40, kernels.ROWS_GROUPS, 0), (False, 64, kernels.ROWS_GROUPS, 0),
                                                      (False, 6, kernels.ROWS_GROUPS, 4), (False, 13, kernels.ROWS_GROUPS, 8),
-                                                     (False, 40, kernels.ROWS_GROUPS, 4), (False, 16, 0, 0)])
+                                                     (False, 40, kernels.ROWS_GROUPS, 4), (False, 16, 0, 0), (False, 7, kernels.ROWS_GROUPS, 1),
+                                                     (False, 9, kernels.ROWS_GROUPS, 2)])
 def test_linear_skinny_stores_keys_and_values(general, n, rows_mode, rpg):
     g = torch.Generator().manual_seed(5)
     k, h, hk, d, page, pages = 64, 4, 2, 16, 4, 23
