@@ -48,6 +48,11 @@ def decode_run(args, batch, steps, warmup, dtype):
     from mini_gpt_inference_amd import Request, SamplingParams
 
     engine, cfg = build_engine(args, batch, dtype)
+    if not args.no_graph:
+        # every graph that the timed steps replay (the single step's and the burst's) is recorded
+        # here, before any request: the reference captures before it times as well
+        # (src/minigpt_infer/graphs.py:96-110)
+        assert engine.capture_decode_graphs([batch]), "the decode graphs could not be captured ahead"
     rng = np.random.default_rng(0)
     budget = steps + warmup + 3 * args.burst * args.chain + 2
     assert args.prompt + budget <= cfg.block_size, "prompt + decode steps exceed the model's positions"
@@ -76,13 +81,31 @@ def decode_run(args, batch, steps, warmup, dtype):
     run_decode_steps(warmup)
     torch.cuda.synchronize()
     start_ctx = args.prompt + 1 + (sched.num_steps - done)
+    before = engine.stats()
+    engine.stretch_times = stretches = []
     t0 = time.perf_counter()
     run_decode_steps(steps, record=True)
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
+    engine.stretch_times = None
+    after = engine.stats()
+    assert after["graph_captures"] == before["graph_captures"], "a HIP graph was recorded inside the timed steps"
+    if not args.no_graph:
+        assert after["graph_steps"] - before["graph_steps"] == steps, "a timed step did not come from a graph"
     engine.step_samples = samples
+    # the device's pace: from the arrival of one stretch's tokens (a captured burst, or the single
+    # steps that end a chain) to the arrival of the next one's
+    engine.stretch_samples = [(n, t1 - t_prev) for (_, t_prev), (n, t1) in zip(stretches, stretches[1:])]
     mean_ctx = start_ctx + (steps - 1) / 2.0 + 1     # keys read per request and step, own token included
     return elapsed, mean_ctx, engine, cfg
+
+
+def kernels_per_step(engine, batch):
+    """Kernels that one captured decode step of this batch launches (0 without graphs)."""
+    from mini_gpt_inference_amd.engine.step import _bucket
+
+    graphed = engine._graphs.get(_bucket(max(batch, 1)))
+    return graphed.kernels_per_step if graphed is not None else 0
 
 
 def decode_bytes(cfg, batch, mean_ctx, itemsize):
@@ -232,7 +255,7 @@ def main() -> int:
         return 0
 
     elapsed, mean_ctx, engine, cfg = decode_run(args, args.batch, args.steps, args.warmup, args.dtype)
-    samples = engine.step_samples
+    samples = engine.stretch_samples or engine.step_samples
     itemsize = 2 if args.dtype == "bfloat16" else 4
     step_s = elapsed / args.steps
     value = args.batch * args.steps / elapsed
@@ -253,6 +276,7 @@ def main() -> int:
             "hip_graph": bool(stats["graph_steps"]), "decode_burst": args.burst, "decode_chain": args.chain,
             "parallelism": "single-gpu",
         },
+        "kernels_per_step": kernels_per_step(engine, args.batch),
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 5)},
     }
@@ -273,9 +297,11 @@ def main() -> int:
 
 
 def write_report(path, record, samples):
-    """The record, the raw samples behind it (one per engine.step() call of the timed region: decode
-    steps in the call, seconds; a call ends when its tokens are on the host), their median and
-    quartiles per step, and what ran them (the reference's timing rules, docs/PLAN.md:720-732)."""
+    """The record, the raw samples behind it (one per stretch of decode steps enqueued at once, a
+    captured burst mostly: decode steps, seconds from the arrival of the stretch before it on the
+    host to its own), their median and quartiles per step, and what ran them (the reference's timing
+    rules: warm-up, synchronisation around the timed region, median and quartiles over at least 30
+    repeats, docs/PLAN.md:720-732, bench/common.py:118-157)."""
     import statistics
     import subprocess
 
@@ -283,10 +309,15 @@ def write_report(path, record, samples):
 
     per_step = sorted(sec / n for n, sec in samples if n)
     quart = statistics.quantiles(per_step, n=4) if len(per_step) >= 2 else [per_step[0]] * 3
-    try:
-        sha = subprocess.run(["git", "rev-parse", "HEAD"], capture_output=True, text=True, timeout=10).stdout.strip()
-    except Exception:
-        sha = ""
+    import os
+
+    sha = os.environ.get("MGPT_GIT_SHA", "")      # where the tree is a copy without its history
+    if not sha:
+        try:
+            sha = subprocess.run(["git", "rev-parse", "HEAD"], capture_output=True, text=True, timeout=10,
+                                 cwd=os.path.dirname(os.path.abspath(__file__))).stdout.strip()
+        except Exception:
+            sha = ""
     report = {"record": record,
               "ms_per_step": {"median": quart[1] * 1e3, "q1": quart[0] * 1e3, "q3": quart[2] * 1e3,
                               "calls": len(per_step)},

@@ -3,12 +3,15 @@ runtime (g++), each into one shared library next to the sources.
 
 The libraries are loaded with ctypes; nothing here needs torch's extension
 builder, a writable HOME or a network.  ``build_*`` always compiles;
-``ensure_*`` compiles only when the library is missing.
+``ensure_*`` compiles when the library is missing or was built from other
+sources than those that lie beside it now (a digest of the sources is kept next
+to each library).
 """
 
 from __future__ import annotations
 
 import glob
+import hashlib
 import os
 import shutil
 import subprocess
@@ -31,6 +34,9 @@ HIP_FLAGS = [
     # accumulation registers and copies each one out again for the arithmetic that follows
     "-mllvm", "-amdgpu-mfma-vgpr-form=1",
 ]
+
+
+HOST_FLAGS = ["-O2", "-std=c++17", "-fPIC", "-shared", "-Wall", "-D_GLIBCXX_ASSERTIONS"]
 
 
 class BuildError(RuntimeError):
@@ -81,6 +87,42 @@ def _writable_target(path: str) -> str:
     return os.path.join(alt, os.path.basename(path))
 
 
+def kernel_sources() -> list[str]:
+    return sorted(glob.glob(os.path.join(HIP_DIR, "*.hip")) + glob.glob(os.path.join(HIP_DIR, "*.h")))
+
+
+def host_sources() -> list[str]:
+    return sorted(glob.glob(os.path.join(HOST_DIR, "*.cpp")) + glob.glob(os.path.join(HOST_DIR, "*.h")))
+
+
+def sources_digest(files: list[str], flags: list[str]) -> str:
+    """A digest of the sources' names and contents and of the compiler's flags."""
+    h = hashlib.sha256(" ".join(flags).encode())
+    for path in files:
+        h.update(os.path.basename(path).encode() + b"\0")
+        with open(path, "rb") as fh:
+            h.update(fh.read())
+    return h.hexdigest()
+
+
+def _stamp(lib: str) -> str:
+    return lib + ".digest"
+
+
+def _write_stamp(lib: str, digest: str) -> None:
+    with open(_stamp(lib), "w", encoding="ascii") as fh:
+        fh.write(digest)
+
+
+def is_current(lib: str, digest: str) -> bool:
+    """Whether the library exists and was built from sources with this digest."""
+    try:
+        with open(_stamp(lib), encoding="ascii") as fh:
+            return os.path.isfile(lib) and fh.read().strip() == digest
+    except OSError:
+        return False
+
+
 def kernel_lib_path() -> str:
     return KERNEL_LIB if os.path.isfile(KERNEL_LIB) else _writable_target(KERNEL_LIB)
 
@@ -119,8 +161,10 @@ def build_kernels() -> str:
         if errors:
             raise errors[0]
         tmp = target + f".tmp{os.getpid()}"
+        digest = sources_digest(kernel_sources(), HIP_FLAGS)
         _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", *objects, "-o", tmp], "kernel library")
         os.replace(tmp, target)
+        _write_stamp(target, digest)
     finally:
         shutil.rmtree(objdir, ignore_errors=True)
     _say(f"built {target}")
@@ -138,24 +182,30 @@ def build_host() -> str:
     # _GLIBCXX_ASSERTIONS: an index past the end of a vector stops the process with a message instead
     # of reading whatever lies there (the scheduler's and the cache manager's work is small: the
     # checks cost nothing that a step would notice)
-    _run([cxx, "-O2", "-std=c++17", "-fPIC", "-shared", "-Wall", "-D_GLIBCXX_ASSERTIONS", "-I", HOST_DIR, *sources,
-          "-o", tmp],
-         "host runtime")
+    digest = sources_digest(host_sources(), HOST_FLAGS)
+    _run([cxx, *HOST_FLAGS, "-I", HOST_DIR, *sources, "-o", tmp], "host runtime")
     os.replace(tmp, target)
+    _write_stamp(target, digest)
     _say(f"built {target}")
     return target
 
 
 def ensure_kernels() -> str:
+    """The kernel library's path; compiles it first if there is none or if a source has changed
+    since it was built."""
     path = kernel_lib_path()
-    if not os.path.isfile(path):
+    if not is_current(path, sources_digest(kernel_sources(), HIP_FLAGS)):
+        if os.path.isfile(path):
+            _say("the kernel sources have changed since the library was built")
         path = build_kernels()
     return path
 
 
 def ensure_host() -> str:
     path = host_lib_path()
-    if not os.path.isfile(path):
+    if not is_current(path, sources_digest(host_sources(), HOST_FLAGS)):
+        if os.path.isfile(path):
+            _say("the host sources have changed since the library was built")
         path = build_host()
     return path
 

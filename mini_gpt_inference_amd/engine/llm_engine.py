@@ -8,6 +8,7 @@ from __future__ import annotations
 
 import shutil
 import tempfile
+import time
 from typing import Dict, List, Optional, Sequence, Union
 
 import numpy as np
@@ -49,6 +50,7 @@ class _GraphedDecode:
         self.graph: Optional[torch.cuda.CUDAGraph] = None
         self.burst_graph: Optional[torch.cuda.CUDAGraph] = None
         self.shape: Optional[StepShape] = None   # of the last single step; launch geometry for captures
+        self.kernels_per_step = 0                # kernels that the captured step launches
 
     def _launch(self, shape: StepShape) -> None:
         ctx = self.runner.context(self.arena, shape, padded=True, workspace=self.workspace)
@@ -59,14 +61,17 @@ class _GraphedDecode:
             self.sampler.sample(logits, self.arena, self.cap, advance=(self.runner.page_sizes, self.history))
 
     def _capture(self, shape: StepShape, times: int) -> torch.cuda.CUDAGraph:
+        self.runner.num_graph_captures += 1
         graph = torch.cuda.CUDAGraph()
         side = torch.cuda.Stream()
         side.wait_stream(torch.cuda.current_stream())
+        launched = kernels.launches
         with torch.cuda.stream(side):
             graph.capture_begin()
             try:
                 for _ in range(times):
                     self._launch(shape)
+                self.kernels_per_step = (kernels.launches - launched) // times
             except BaseException:
                 # never leave the stream capturing: the graph object's destructor synchronizes the
                 # device, which a stream that is still capturing turns into an abort of the process
@@ -159,9 +164,13 @@ class LLMEngine:
         self._generated = 0                   # requests that generate() has named so far
         self._inflight = None                 # a chain of decode steps enqueued ahead, not yet taken in
         self._graphs: Dict[int, _GraphedDecode] = {}
+        self._unseeded = 0                    # requests so far that brought no seed of their own
         self._tmpdir: Optional[str] = None
         self.num_graph_steps = 0
         self.num_eager_steps = 0
+        # a list here collects (decode steps, time.perf_counter()) whenever the tokens of a stretch of
+        # enqueued decode steps have arrived on the host: the device's pace, for measurements
+        self.stretch_times: Optional[List] = None
 
     # ------------------------------------------------------------------ constructors
     @classmethod
@@ -190,8 +199,14 @@ class LLMEngine:
         vocab = self.model.spec.vocab_size
         if any((t < 0 or t >= vocab) for t in request.prompt_token_ids):
             raise ValueError(f"prompt token id outside 0..{vocab - 1}")
+        seed = sp.seed
+        if seed is None:
+            # a stream of its own per request in the order of arrival; the made-up requests of
+            # capture_decode_graphs bring a seed, so that calling it changes nobody's tokens
+            seed = self._unseeded
+            self._unseeded += 1
         sid = self.scheduler.add_request(request.prompt_token_ids, sp.max_tokens, request.eot_token_id,
-                                         sp.temperature, sp.top_k, sp.top_p, sp.seed)
+                                         sp.temperature, sp.top_k, sp.top_p, seed)
         self._ids[sid] = request.request_id
         self._rids[request.request_id] = sid
 
@@ -244,6 +259,8 @@ class LLMEngine:
             if last and self.engine_config.decode_ahead and (max_steps is None or max_steps >= 2):
                 self._inflight = self._launch_chain(max_steps, ahead=True)
             event.synchronize()
+            if self.stretch_times is not None:
+                self.stretch_times.append((end - first, time.perf_counter()))
             tokens = np.ascontiguousarray(graphed.history_host.numpy()[first:end, :r])
             outs += [RequestOutput(self._ids[sid], [token], finished, reason) for sid, token, finished, reason
                      in self.scheduler.commit_burst(tokens, end - first, last=last)]
@@ -330,8 +347,8 @@ class LLMEngine:
         powers of two up to max_batch_size, or those that hold the given batch sizes) it runs that many
         made-up one-token requests for a few steps, which captures the single step and the burst.
         A capacity whose requests the page pool cannot hold is left out.  Returns the capacities
-        captured.  The engine must be idle; its counters count these steps too, and requests that
-        bring no seed of their own draw from other streams than without this call."""
+        captured.  The engine must be idle; its counters count these steps too.  The tokens of later
+        requests do not depend on whether this was called."""
         ecfg = self.engine_config
         if self.has_unfinished_requests() or self._inflight is not None:
             raise RuntimeError("capture_decode_graphs needs an idle engine")
@@ -358,7 +375,7 @@ class LLMEngine:
                 continue
             for i in range(n):
                 self.add_request(Request(f"capture-{cap}-{i}-{self._generated}", [0],
-                                         SamplingParams(max_tokens=steps, temperature=0.0)))
+                                         SamplingParams(max_tokens=steps, temperature=0.0, seed=0)))
             self._generated += 1
             while self.has_unfinished_requests():
                 self.step()
@@ -400,4 +417,5 @@ class LLMEngine:
             "allocated_blocks": self.cache.groups[0].num_pages - self.cache.num_free_pages(0),
             "graph_steps": self.num_graph_steps, "eager_steps": self.num_eager_steps,
             "replayed_eager_steps": self.runner.num_replayed_steps,
+            "graph_captures": self.runner.num_graph_captures,
         }

@@ -162,6 +162,7 @@ class ModelRunner:
         self._step_graphs: Dict[Tuple, _StepGraph] = {}     # by exact shape; emptied when it has MAX_STEP_GRAPHS
         self._bucket_graphs: Dict[Tuple, _StepGraph] = {}   # by capacities: as many as there are buckets
         self.num_replayed_steps = 0
+        self.num_graph_captures = 0       # HIP graphs recorded so far, decode steps' and other steps'
         self._arenas: Dict[Tuple[int, int, int], StepArena] = {}
         self.n_groups = len(cache.groups)
         self.page_sizes = torch.tensor([g.page_size for g in cache.groups], dtype=torch.int32, device=device)
@@ -317,6 +318,7 @@ class ModelRunner:
             with kernels.pinned_stream():
                 return self.model.forward(ctx)
         entry.graph = None
+        self.num_graph_captures += 1
         if lead_cap is not None:
             forward()
         graph = torch.cuda.CUDAGraph()

@@ -67,8 +67,13 @@ def pinned_stream():
         _pinned_stream = previous
 
 
-def _check(rc: int, what: str) -> None:
+launches = 0     # kernels launched so far (a product split over workgroups counts its second kernel too)
+
+
+def _check(rc: int, what: str, n_kernels: int = 1) -> None:
+    global launches
     if rc == 0:
+        launches += n_kernels
         return
     if rc < 0:
         raise KernelError(f"{what}: refused, {_ERRORS.get(rc, rc)}")
@@ -352,7 +357,7 @@ def linear_skinny(a: Optional[torch.Tensor], w: torch.Tensor, bias: Optional[tor
         1 if general_only else rows_mode | (rows_per_group << 8), _ptr(partials), 0 if partials is None else partials.numel(), _stream())
     if rc == -2:
         return False
-    _check(rc, "linear_skinny")
+    _check(rc, "linear_skinny", 2 if partials is not None else 1)
     return True
 
 
@@ -520,7 +525,7 @@ def linear_mfma(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], 
                                                           0 if k_parts is None else int(k_parts), *args)
     if rc == -2:
         return False
-    _check(rc, "linear_mfma")
+    _check(rc, "linear_mfma", 2 if partials is not None else 1)
     return True
 
 

@@ -13,6 +13,18 @@ def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs an MI355X; run with -m gpu")
 
 
+def pytest_report_header(config):
+    """Which native libraries the tests will load, and whether they were built from the sources beside them."""
+    from mini_gpt_inference_amd.csrc import build
+
+    lines = []
+    for path, files, flags in ((build.kernel_lib_path(), build.kernel_sources(), build.HIP_FLAGS),
+                               (build.host_lib_path(), build.host_sources(), build.HOST_FLAGS)):
+        state = "current" if build.is_current(path, build.sources_digest(files, flags)) else "missing or stale: rebuilt at first use"
+        lines.append(f"native library {path}: {state}")
+    return lines
+
+
 def pytest_collection_modifyitems(config, items):
     import torch
 

@@ -34,9 +34,12 @@ def test_no_silent_fallback_when_the_kernel_library_cannot_be_loaded(tmp_path):
 
 
 def test_bench_prints_one_record_with_the_agreed_fields():
-    """A short run of bench.py: one JSON line, the fields the measurement is read from, a flat `config`."""
+    """A short run of bench.py with a step count that whole bursts do not divide and a warm-up shorter
+    than a burst: one JSON line, the fields the measurement is read from, a flat `config`.  bench.py
+    itself asserts that no HIP graph was recorded inside the timed steps and that every timed step
+    came from a graph."""
     import json
-    proc = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--steps", "16", "--warmup", "8",
+    proc = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--steps", "20", "--warmup", "5",
                            "--layers", "2", "--no-extras"], capture_output=True, text=True, timeout=300)
     assert proc.returncode == 0, proc.stderr[-2000:]
     lines = [line for line in proc.stdout.splitlines() if line.startswith("{")]
@@ -45,7 +48,8 @@ def test_bench_prints_one_record_with_the_agreed_fields():
     for key in ("metric", "value", "unit", "n_gpus", "steps", "warmup", "ms_per_step", "higher_is_better", "scaling",
                 "vs_baseline", "dtype", "data", "config", "roofline"):
         assert key in rec, key
-    assert rec["n_gpus"] == 1 and rec["steps"] == 16 and rec["warmup"] == 8 and rec["value"] > 0
+    assert rec["n_gpus"] == 1 and rec["steps"] == 20 and rec["warmup"] == 5 and rec["value"] > 0
+    assert rec["config"]["hip_graph"] is True and 0 < rec["kernels_per_step"] < 40
     assert rec["config"]["n_layer"] == 2 and rec["config"]["n_layer_full"] == 8      # fewer layers are named
     assert len(rec["config"]) <= 20 and not any(isinstance(v, (dict, list)) for v in rec["config"].values())
     assert abs(rec["roofline"]["frac"] - rec["roofline"]["achieved"] / rec["roofline"]["peak"]) < 1e-4
