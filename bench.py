@@ -60,7 +60,8 @@ def decode_run(args, batch, steps, warmup, dtype):
         engine.add_request(Request(f"b{i}", rng.integers(0, cfg.vocab_size, args.prompt).tolist(),
                                    SamplingParams(max_tokens=budget, temperature=0.0)))
     sched = engine.scheduler
-    while sched.num_decode_tokens == 0:      # prompts, untimed
+    decoded_before = sched.num_decode_tokens
+    while sched.num_decode_tokens == decoded_before:      # prompts, untimed
         engine.step()
 
     samples = []     # (decode steps in the call, seconds) of every engine.step() call of the timed region
