@@ -52,3 +52,23 @@ int mgpt_launch_linear_decode(const SkinnyArgs& a, int epilogue, int out_dtype, 
 long mgpt_linear_decode_partials(int n_rows, int n_out, int k_dim, bool ln, int epilogue, int rows_mode);
 // whether 17 to 64 rows of this shape go to one workgroup per column tile and 16 rows
 bool mgpt_linear_decode_row_groups(int n_rows, int n_out, int k_dim, int rows_mode);
+
+// mgpt_linear_skinny for callers that cannot allocate device memory and bring no scratch of their
+// own (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  It has
+// no counterpart in the reference.  Where mgpt_linear_skinny would split a long inner size over
+// workgroups (17 to 64 rows, see mgpt_linear_skinny_partials) the partial sums go to an array that
+// the library itself holds in device memory, MGPT_STATIC_SCRATCH_FLOATS floats (1 MiB) on every GPU
+// the library runs on, until the process ends; a shape that needs more is refused with
+// MGPT_ERR_SCRATCH and nothing is launched.  The call allocates and frees nothing.  Every call on
+// a GPU uses that GPU's one array, so calls that overlap on one GPU (on different streams, or from
+// different threads) race; calls on one stream follow each other and are safe.  Nothing in the
+// array has to start at zero: the first kernel writes every partial sum that the second reads.
+#define MGPT_STATIC_SCRATCH_FLOATS (4L * 64 * 1024)
+#define MGPT_ERR_SCRATCH (-5)
+extern "C" int mgpt_linear_skinny_static_scratch(
+    const void* act, long lda, const float* x, const int* rows, const float* colsum, float eps, const void* w,
+    const void* w_packed, const float* bias, void* out, int out_dtype, long ldo, int n_rows, int n_out, int k_dim,
+    int epilogue, void* kpool, void* vpool, const int* slot_mapping, int q_width, int kv_width, int head_dim,
+    int n_kv_head, int page_size, int mode, hipStream_t stream);
+// the array's size in floats
+extern "C" long mgpt_linear_skinny_static_scratch_floats();

@@ -23,6 +23,8 @@
 // their cache pages by slot_mapping (src/minigpt_infer/cache/paged.py:125-137).
 #include "linear_skinny.h"
 
+#include <mutex>
+
 __device__ __forceinline__ bf16x8_t load8(const bf16_t* p) {
   return *reinterpret_cast<const bf16x8_t*>(p);
 }
@@ -389,4 +391,52 @@ extern "C" long mgpt_linear_skinny_partials(int n_rows, int n_out, int k_dim, in
 // folded LayerNorm costs a workgroup no more than at 16 rows)
 extern "C" int mgpt_linear_skinny_row_groups(int n_rows, int n_out, int k_dim) {
   return mgpt_linear_decode_row_groups(n_rows, n_out, k_dim, 0) ? 1 : 0;
+}
+
+// ---- the variant that allocates nothing (declared in linear_skinny.h)
+static __device__ __align__(256) float scratch[MGPT_STATIC_SCRATCH_FLOATS];
+
+#define MGPT_MAX_DEVICES 64
+static float* scratch_of_device[MGPT_MAX_DEVICES];  // the array's address on each GPU, asked for once
+static std::mutex scratch_mutex;
+
+// The device address of `scratch` on the current GPU.  In host code the array's name is only a
+// handle for the runtime, not an address a kernel could use: the address comes from
+// hipGetSymbolAddress, and every GPU has its own.
+static int static_scratch(float** ptr) {
+  int dev = -1;
+  hipError_t err = hipGetDevice(&dev);
+  if (err != hipSuccess) return (int)err;
+  if (dev < 0 || dev >= MGPT_MAX_DEVICES) return MGPT_ERR_TOO_LARGE;
+  std::lock_guard<std::mutex> lock(scratch_mutex);
+  if (!scratch_of_device[dev]) {
+    void* p = nullptr;
+    err = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (err != hipSuccess) return (int)err;
+    if (!p) return MGPT_ERR_NULL;
+    scratch_of_device[dev] = (float*)p;
+  }
+  *ptr = scratch_of_device[dev];
+  return MGPT_OK;
+}
+
+extern "C" long mgpt_linear_skinny_static_scratch_floats() { return MGPT_STATIC_SCRATCH_FLOATS; }
+
+extern "C" int mgpt_linear_skinny_static_scratch(
+    const void* act, long lda, const float* x, const int* rows, const float* colsum, float eps, const void* w,
+    const void* w_packed, const float* bias, void* out, int out_dtype, long ldo, int n_rows, int n_out, int k_dim,
+    int epilogue, void* kpool, void* vpool, const int* slot_mapping, int q_width, int kv_width, int head_dim,
+    int n_kv_head, int page_size, int mode, hipStream_t stream) {
+  if (n_rows < 0 || n_rows > 64 || n_out < 0 || k_dim <= 0) return MGPT_ERR_BAD_SHAPE;
+  const int rows_mode = ((mode & 0xFF) == SK_ROWS_SHARE_W || (mode & 0xFF) == SK_ROWS_GROUPS) ? (mode & 0xFF) : 0;
+  const long need = mode == 1 ? 0 : mgpt_linear_decode_partials(n_rows, n_out, k_dim, x != nullptr, epilogue, rows_mode);
+  if (need > MGPT_STATIC_SCRATCH_FLOATS) return MGPT_ERR_SCRATCH;
+  float* partials = nullptr;
+  if (need > 0) {
+    const int rc = static_scratch(&partials);
+    if (rc != MGPT_OK) return rc;
+  }
+  return mgpt_linear_skinny(act, lda, x, rows, colsum, eps, w, w_packed, bias, out, out_dtype, ldo, n_rows, n_out,
+                            k_dim, epilogue, kpool, vpool, slot_mapping, q_width, kv_width, head_dim, n_kv_head,
+                            page_size, mode, partials, need, stream);
 }

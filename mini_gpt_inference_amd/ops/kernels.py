@@ -24,6 +24,7 @@ _ERRORS = {
     -2: "unsupported shape",
     -3: "size beyond what the launch grid can hold",
     -4: "null pointer",
+    -5: "the shape needs more scratch than the library's own array holds",
 }
 
 
