@@ -1,0 +1,1057 @@
+// The fused kernels of a decode step with few rows (bfloat16): two kernels a layer.
+//
+//  * fused_attention_decode_kernel, one workgroup per (token, head): adds up the residual row that
+//    the kernels before it left as a sum (fused_decode.h), LayerNorm, this head's query, key and
+//    value (src/minigpt_infer/model.py:43,49-53), the key and value into their page
+//    (src/minigpt_infer/cache/paged.py:125-137), attention over the request's pages and the new
+//    key (model.py:61-87; the Triton decode kernel src/minigpt_infer/attention/triton_paged.py:44-123),
+//    and this head's share of the output projection (model.py:89-90), left as one of n_head partial
+//    sums of the residual.
+//  * fused_mlp_decode_kernel, one workgroup per 64 hidden units (and group of rows): adds up the
+//    residual rows, LayerNorm, its slice of the first product with bias and GELU-tanh, and that
+//    slice's share of the second product (model.py:96-101), left as one of hidden/64 partial sums.
+//  * residual_layernorm_kernel and residual_settle_kernel: the LayerNorm of rows that are still such
+//    a sum (the final norm, model.py:186), and the sum itself for whoever needs plain rows.
+//
+// A decode step at a few rows is a chain of dependent kernels that each wait for one memory round
+// trip; every load whose address does not depend on the step's data (weights, block table) is
+// issued first, the sums of the residual and the LayerNorm happen while they are on their way.
+// Sums are added in a fixed order, so results do not depend on timing.
+#include "fused_decode.h"
+
+typedef __attribute__((ext_vector_type(2))) __bf16 fd_bf16x2_t;
+
+// A barrier between the waves of a workgroup that waits for this wave's LDS traffic only.
+// __syncthreads() also waits for every global load in flight, and here the loads of the weights
+// (and of keys and values) are meant to stay in flight across the barriers of the work that does
+// not need them yet.  Only LDS is exchanged across these barriers, never global memory.
+__device__ __forceinline__ void fd_barrier() {
+  asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
+
+#ifdef FD_TRACE
+// time stamps (100 MHz) of the first workgroup's first thread, for measurements of where a kernel's time goes
+__device__ unsigned long long fd_trace_buf[64];
+#define FD_STAMP(k)                                                                  \
+  do {                                                                               \
+    if (blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x == 0) fd_trace_buf[k] = wall_clock64(); \
+  } while (0)
+// a stamp once the value v has arrived in its register
+#define FD_STAMP_AFTER(k, v)              \
+  do {                                    \
+    asm volatile("" ::"v"(v) : "memory"); \
+    FD_STAMP(k);                          \
+  } while (0)
+extern "C" int mgpt_fd_trace(unsigned long long* host) {
+  return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(fd_trace_buf), sizeof(fd_trace_buf));
+}
+#else
+#define FD_STAMP(k)
+#define FD_STAMP_AFTER(k, v)
+#endif
+
+template <int CTRL>
+__device__ __forceinline__ float fd_dpp(float v) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, false));
+}
+
+// sum over the LPK neighbouring lanes of an aligned group; every lane of the group gets it
+template <int LPK>
+__device__ __forceinline__ float fd_group_sum(float v) {
+  v += fd_dpp<MGPT_DPP_XOR1>(v);
+  if (LPK >= 4) v += fd_dpp<MGPT_DPP_XOR2>(v);
+  if (LPK >= 8) v += fd_dpp<MGPT_DPP_HALF_MIRROR>(v);
+  if (LPK >= 16) v += fd_dpp<MGPT_DPP_MIRROR>(v);
+  return v;
+}
+
+__device__ __forceinline__ float fd_dot2(unsigned int a, unsigned int b, float c) {
+  return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(fd_bf16x2_t, a), __builtin_bit_cast(fd_bf16x2_t, b),
+                                         c, false);
+}
+
+__device__ __forceinline__ float4 fd_add4(float4 a, float4 b) {
+  return make_float4(a.x + b.x, a.y + b.y, a.z + b.z, a.w + b.w);
+}
+
+__device__ __forceinline__ float4 fd_keep4(bool keep, float4 v) {
+  return make_float4(keep ? v.x : 0.f, keep ? v.y : 0.f, keep ? v.z : 0.f, keep ? v.w : 0.f);
+}
+
+__device__ __forceinline__ float4 fd_bf16x4(uint2 t) {
+  return make_float4(__uint_as_float(t.x << 16), __uint_as_float(t.x & 0xffff0000u), __uint_as_float(t.y << 16),
+                     __uint_as_float(t.y & 0xffff0000u));
+}
+
+__device__ __forceinline__ float fd_sum4(float4 v) { return (v.x + v.y) + (v.z + v.w); }
+
+// the block (row tile, k step) of a packed matrix (fold_norm.hip: pack_weight_kernel), this lane's 8 values
+__device__ __forceinline__ bf16x8_t fd_packed(const bf16_t* w, long tile, int k_steps, int s, int lane) {
+  return *reinterpret_cast<const bf16x8_t*>(w + ((tile * k_steps + s) * 64 + lane) * 8);
+}
+
+// ---- A residual row added up by a whole workgroup.  The row has V = width / 4 vectors of four; the
+// workgroup's threads form G = FUSED_THREADS / V groups of V, and group q loads the parts q, q + G,
+// q + 2 G, q + 3 G (group 0 also the base): FUSED_GROUP_PARTS * G parts at most.  The loads are
+// issued by fd_row_issue and used by fd_row_sum, so that the caller can issue other loads between
+// the two; there is no branch between a load and the next (a load past the parts reads part 0
+// again and is dropped), because the compiler waits for every load in flight where control flow
+// joins.
+struct FdRowLoads {
+  float4 base;
+  float4 part[FUSED_GROUP_PARTS];
+};
+
+// TABLES: the row is the token's and the position's table rows (no base, no parts)
+template <bool TABLES>
+__device__ __forceinline__ void fd_row_issue(const FusedResidual& r, long row, int id, int pos, int V, int G,
+                                             FdRowLoads& L) {
+  const int tid = threadIdx.x;
+  const int gq = tid / V, vq = tid - gq * V;
+  const int gc = gq < G ? gq : 0;
+  if (TABLES) {
+    const bool has_pos = r.pos_table != nullptr;
+    const uint2 t = reinterpret_cast<const uint2*>(r.tok_table)[(long)id * V + vq];
+    const uint2 q = reinterpret_cast<const uint2*>(has_pos ? r.pos_table : r.tok_table)[(long)(has_pos ? pos : id) * V + vq];
+    L.base = fd_add4(fd_bf16x4(t), fd_keep4(has_pos, fd_bf16x4(q)));
+  } else {
+    L.base = reinterpret_cast<const float4*>(r.base)[row * V + vq];
+    const float* parts = r.n_parts > 0 ? r.partials : r.base;  // no parts: every load below reads the base again
+#pragma unroll
+    for (int u = 0; u < FUSED_GROUP_PARTS; ++u) {
+      const int p = gc + u * G;
+      L.part[u] = reinterpret_cast<const float4*>(parts + (p < r.n_parts ? p * r.part_stride : 0))[row * V + vq];
+    }
+  }
+}
+
+// Returns, in the threads tid < V, the row's vector tid; xs: LDS for G * V vectors.  One barrier inside.
+template <bool TABLES>
+__device__ __forceinline__ float4 fd_row_sum(const FusedResidual& r, int V, int G, const FdRowLoads& L, float* xs) {
+  const int tid = threadIdx.x;
+  const int gq = tid / V, vq = tid - gq * V;
+  float4 s = fd_keep4(gq == 0, L.base);
+  if (!TABLES) {
+#pragma unroll
+    for (int u = 0; u < FUSED_GROUP_PARTS; ++u) s = fd_add4(s, fd_keep4(gq + u * G < r.n_parts, L.part[u]));
+  }
+  if (gq < G) reinterpret_cast<float4*>(xs)[gq * V + vq] = s;
+  fd_barrier();
+  float4 xv = make_float4(0.f, 0.f, 0.f, 0.f);
+  if (tid < V) {
+    // groups beyond the parts hold zeros: only the groups that had something are read
+    const int used = TABLES ? 1 : min(G, max(r.n_parts, 1));
+    xv = reinterpret_cast<const float4*>(xs)[tid];
+#pragma unroll 8
+    for (int q = 1; q < used; ++q) xv = fd_add4(xv, reinterpret_cast<const float4*>(xs)[q * V + tid]);
+  }
+  return xv;
+}
+
+// LayerNorm of the row that the threads tid < V hold (xv), through two barriers: returns the normed
+// values of this thread's vector (gain and beta applied) in the threads tid < V.
+__device__ __forceinline__ float4 fd_row_norm(float4 xv, int V, int C, float eps, float4 gain4, float4 beta4,
+                                              float* mean_s, float* var_s) {
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int waves_used = (V + 63) >> 6;  // the waves that hold the row
+  const float ws = wave_sum(fd_sum4(xv));
+  if (lane == 0) mean_s[wave] = ws;
+  fd_barrier();
+  float mean = 0.f;
+  for (int w = 0; w < waves_used; ++w) mean += mean_s[w];
+  mean /= (float)C;
+  float4 d = make_float4(0.f, 0.f, 0.f, 0.f);
+  if (tid < V) d = make_float4(xv.x - mean, xv.y - mean, xv.z - mean, xv.w - mean);
+  const float wq = wave_sum((d.x * d.x + d.y * d.y) + (d.z * d.z + d.w * d.w));
+  if (lane == 0) var_s[wave] = wq;
+  fd_barrier();
+  float var = 0.f;
+  for (int w = 0; w < waves_used; ++w) var += var_s[w];
+  const float rstd = 1.0f / sqrtf(var / (float)C + eps);
+  return make_float4(d.x * rstd * gain4.x + beta4.x, d.y * rstd * gain4.y + beta4.y, d.z * rstd * gain4.z + beta4.z,
+                     d.w * rstd * gain4.w + beta4.w);
+}
+
+struct FusedAttnArgs {
+  FusedResidual res;
+  const float* gain;
+  const float* beta;  // or null
+  float eps;
+  const bf16_t* wqkv;  // packed [3 * n_head * D rows, width]
+  const float* bqkv;   // or null
+  const bf16_t* wproj;  // packed [width rows, n_head * D]
+  const float* bproj;   // or null
+  float* out_partials;  // [n_head][part_rows][width]
+  long out_part_stride;
+  bf16_t* kpool;
+  bf16_t* vpool;
+  const int* slot_mapping;
+  const int* block_tables;
+  int max_blocks;
+  const int* positions;
+  const int* q_req;
+  int width, n_head, page_shift, num_pages;
+  unsigned int page_bytes;
+  float scale_log2e;
+};
+
+// Sixteen waves a workgroup: a compute unit takes in about 200 KB a microsecond when sixteen waves
+// each have up to sixteen loads of 16 bytes a lane in flight, and half of that with eight waves
+// that have twice as many each.  A wave therefore holds few loads at a time, and a lane at most
+// 128 registers.
+template <int D, bool TABLES>
+__global__ __launch_bounds__(FUSED_THREADS) void fused_attention_decode_kernel(FusedAttnArgs a) {
+  constexpr int T = 3 * D / 16;                  // row tiles of this head's q, k and v
+  constexpr int TG = T < 12 ? T : 12;            // of them in flight together
+  constexpr int NG = T / TG;
+  constexpr int SMAX = 12 / TG;                  // k steps whose loads are in flight together
+  constexpr int LPK = D / 8, KPI = 64 / LPK;     // lanes per key, keys per load instruction
+  constexpr int NI = LPK / 2 < 2 ? 2 : LPK / 2;  // load instructions of a wave's keys in one pass
+  constexpr int CHUNK = NI * KPI;                // keys of a wave in one pass
+  constexpr int ROWS = FUSED_WAVES * KPI;        // partial results of attention: one per (key subgroup, wave)
+  constexpr int SUBSETS = FUSED_THREADS / D;     // groups of 8 partial rows, one thread per channel each
+  constexpr int NK2 = D <= 32 ? 1 : D / 32;      // k steps of the projection that hold this head's columns
+  constexpr int TP2 = 4 / NK2 > 0 ? 4 / NK2 : 1; // its row tiles per wave whose loads are in flight together
+  static_assert(ROWS == SUBSETS * 8, "the merge deals eight partial rows to a thread");
+  // one pool for what is never alive together: the row's partial sums, then the waves' sums of
+  // q, k, v, then attention's partial results
+  constexpr int POOL_FLOATS = ROWS * D > 4096 ? ROWS * D : 4096;
+  static_assert(FUSED_WAVES * T * 16 <= POOL_FLOATS, "the pool holds the waves' sums of q, k, v");
+  __shared__ __align__(16) float pool[POOL_FLOATS];
+  __shared__ __align__(16) bf16_t act_s[FUSED_MAX_WIDTH];
+  __shared__ float mean_s[FUSED_WAVES], var_s[FUSED_WAVES];
+  __shared__ __align__(16) bf16_t q_s[D];
+  __shared__ __align__(16) bf16_t k_s[D];
+  __shared__ __align__(16) bf16_t v_s[D];
+  __shared__ __align__(16) bf16_t y_s[D];
+  __shared__ float m_s[FUSED_WAVES];
+  __shared__ float l_s[ROWS];
+  __shared__ float part_s[SUBSETS * D];
+  __shared__ float lpart_s[SUBSETS];
+  float* const xs = pool;
+  float* const red_s = pool;
+  float* const acc_s = pool;
+
+  const int h = blockIdx.x, n = blockIdx.y;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int lrow = lane & 15, g = lane >> 4;
+  const int sub = lane / LPK, dg = lane % LPK;
+  const int C = a.width, KS = C >> 5, V = C >> 2;
+
+  FD_STAMP(0);
+  // ---- The prologue.  A compute unit issues a wave's 16-byte loads at about a kilobyte every
+  // ten clocks, and a barrier lets a wave pass only when every other wave has issued what stands
+  // before it: the weights' loads (most of the traffic) are therefore dealt out in four pieces
+  // between the barriers of the residual row's sum and LayerNorm, which need the row's loads only
+  // and happen while the pieces are on their way.  A wave's loads come back in order: the step's
+  // numbers and the row first, keys and values last.
+  const int qr = a.q_req[n];
+  const int qpos = a.positions[n];
+  const int slot = a.slot_mapping[n];
+  const int* bt = a.block_tables + (long)n * a.max_blocks;  // a decode-only step: token n is request n
+  int page0[NI];
+#pragma unroll
+  for (int i = 0; i < NI; ++i) {
+    const int e = (wave * CHUNK + i * KPI + sub) >> a.page_shift;
+    page0[i] = bt[e < a.max_blocks ? e : a.max_blocks - 1];
+  }
+  // the row: V vectors of four; the threads form G groups of V, group q adds up the parts q, q + G, ...
+  // (group 0 the base as well)
+  const int G = FUSED_THREADS / V;
+  const int gq = tid / V, vq = tid - gq * V;
+  float4 piece = make_float4(0.f, 0.f, 0.f, 0.f);
+  float4 part[FUSED_GROUP_PARTS];
+  if (TABLES) {
+    if (gq == 0) {
+      const uint2 t = reinterpret_cast<const uint2*>(a.res.tok_table)[(long)a.res.ids[n] * V + vq];
+      piece = fd_bf16x4(t);
+      if (a.res.pos_table)
+        piece = fd_add4(piece, fd_bf16x4(reinterpret_cast<const uint2*>(a.res.pos_table)[(long)a.res.positions[n] * V + vq]));
+    }
+  } else {
+    if (gq == 0) piece = reinterpret_cast<const float4*>(a.res.base)[(long)n * V + vq];
+#pragma unroll
+    for (int u = 0; u < FUSED_GROUP_PARTS; ++u) {
+      part[u] = make_float4(0.f, 0.f, 0.f, 0.f);
+      const int p = gq + u * G;
+      if (gq < G && p < a.res.n_parts)
+        part[u] = reinterpret_cast<const float4*>(a.res.partials + p * a.res.part_stride)[(long)n * V + vq];
+    }
+  }
+  const int vc = tid < V ? tid : 0;
+  float4 gain4 = make_float4(0.f, 0.f, 0.f, 0.f), beta4 = make_float4(0.f, 0.f, 0.f, 0.f);
+  if (tid < V) {
+    gain4 = reinterpret_cast<const float4*>(a.gain)[vc];
+    if (a.beta) beta4 = reinterpret_cast<const float4*>(a.beta)[vc];
+  }
+  const int per = (KS + FUSED_WAVES - 1) / FUSED_WAVES;  // k steps of a wave
+  const int ks0 = wave * per;
+  const int nks = max(0, min(per, KS - ks0));
+  const int tiles_per_part = a.n_head * (D / 16);
+  constexpr int NW = TG * SMAX;  // loads of the weights' first pass, dealt out in four pieces
+  static_assert(NW % 4 == 0, "four pieces");
+  bf16x8_t wv[TG][SMAX];
+#define FA_LOAD_W(piece_no)                                                                                 \
+  _Pragma("unroll") for (int q_ = 0; q_ < NW / 4; ++q_) {                                                  \
+    const int idx_ = (piece_no) * (NW / 4) + q_, tt_ = idx_ / SMAX, i_ = idx_ % SMAX;                       \
+    const long tile_ = (long)(tt_ / (D / 16)) * tiles_per_part + h * (D / 16) + (tt_ % (D / 16));           \
+    wv[tt_][i_] = fd_packed(a.wqkv, tile_, KS, i_ < nks ? ks0 + i_ : 0, lane);                              \
+  }
+  FA_LOAD_W(0)
+  if (qr < 0) return;  // a token of the padding (the whole workgroup)
+  FD_STAMP_AFTER(16, piece.x);
+
+  // ---- the residual row's sum and LayerNorm
+  if (!TABLES) {
+#pragma unroll
+    for (int u = 0; u < FUSED_GROUP_PARTS; ++u) piece = fd_add4(piece, part[u]);
+  }
+  if (gq < G) reinterpret_cast<float4*>(xs)[gq * V + vq] = piece;
+  fd_barrier();
+  FD_STAMP(17);
+  FA_LOAD_W(1)
+  float4 xv = make_float4(0.f, 0.f, 0.f, 0.f);
+  if (tid < V) {
+    // groups beyond the parts hold zeros: only the groups that had something are read
+    const int used = TABLES ? 1 : min(G, max(a.res.n_parts, 1));
+    xv = reinterpret_cast<const float4*>(xs)[tid];
+#pragma unroll 8
+    for (int q = 1; q < used; ++q) xv = fd_add4(xv, reinterpret_cast<const float4*>(xs)[q * V + tid]);
+    if (h == 0 && a.res.settled) reinterpret_cast<float4*>(a.res.settled + (long)n * C)[tid] = xv;
+  }
+  const int waves_used = (V + 63) >> 6;  // the waves that hold the row
+  {
+    const float ws = wave_sum(fd_sum4(xv));
+    if (lane == 0) mean_s[wave] = ws;
+  }
+  fd_barrier();
+  FD_STAMP(18);
+  FA_LOAD_W(2)
+  float mean = 0.f;
+  for (int w = 0; w < waves_used; ++w) mean += mean_s[w];
+  mean /= (float)C;
+  float4 dv = make_float4(0.f, 0.f, 0.f, 0.f);
+  if (tid < V) dv = make_float4(xv.x - mean, xv.y - mean, xv.z - mean, xv.w - mean);
+  {
+    const float wq = wave_sum((dv.x * dv.x + dv.y * dv.y) + (dv.z * dv.z + dv.w * dv.w));
+    if (lane == 0) var_s[wave] = wq;
+  }
+  fd_barrier();
+  FD_STAMP(19);
+  FA_LOAD_W(3)
+#undef FA_LOAD_W
+  // keys and values of the first pass: their addresses need the block table and the position only
+  const int kv_end = qpos;  // the keys before the token's own
+  const int page_mask = (1 << a.page_shift) - 1;
+  const unsigned int lane_off = ((unsigned int)(h << a.page_shift) * D + dg * 8) * 2u;
+  uint4 kraw[NI], vraw[NI];
+  const int c00 = wave * CHUNK;
+  if (c00 < kv_end) {  // the same in all lanes of a wave
+#pragma unroll
+    for (int i = 0; i < NI; ++i) {
+      const int j = c00 + i * KPI + sub;
+      const bool follow = j < kv_end && (unsigned int)page0[i] < (unsigned int)a.num_pages;
+      const unsigned int row_off = ((unsigned int)page0[i] * a.page_bytes) + (unsigned int)(j & page_mask) * (D * 2u);
+      const unsigned int off = follow ? row_off + lane_off : 0u;
+      kraw[i] = *reinterpret_cast<const uint4*>(reinterpret_cast<const char*>(a.kpool) + off);
+      vraw[i] = *reinterpret_cast<const uint4*>(reinterpret_cast<const char*>(a.vpool) + off);
+    }
+  }
+  {
+    float var = 0.f;
+    for (int w = 0; w < waves_used; ++w) var += var_s[w];
+    const float rstd = 1.0f / sqrtf(var / (float)C + a.eps);
+    if (tid < V) {
+      uint2 pk;
+      pk.x = pack_bf16x2(dv.x * rstd * gain4.x + beta4.x, dv.y * rstd * gain4.y + beta4.y);
+      pk.y = pack_bf16x2(dv.z * rstd * gain4.z + beta4.z, dv.w * rstd * gain4.w + beta4.w);
+      reinterpret_cast<uint2*>(act_s)[tid] = pk;
+    }
+  }
+  fd_barrier();  // also: everybody has read the row's partial sums, whose place the waves' sums take now
+  FD_STAMP(1);
+
+  // ---- q, k, v of this head: every wave a stretch of k over all the row tiles; the waves' sums
+  // meet in LDS (every column of the MFMA's output holds the one token: the lanes of column 0 speak)
+  for (int s0 = 0, first = 1;; first = 0) {
+#pragma unroll
+    for (int grp = 0; grp < NG; ++grp) {
+      if (grp > 0 || !first) {
+#pragma unroll
+        for (int tt = 0; tt < TG; ++tt) {
+          const int t2 = grp * TG + tt;
+          const long tile = (long)(t2 / (D / 16)) * tiles_per_part + h * (D / 16) + (t2 % (D / 16));
+#pragma unroll
+          for (int i = 0; i < SMAX; ++i) wv[tt][i] = fd_packed(a.wqkv, tile, KS, s0 + i < nks ? ks0 + s0 + i : 0, lane);
+        }
+      }
+      bf16x8_t b[SMAX];
+#pragma unroll
+      for (int i = 0; i < SMAX; ++i)
+        b[i] = *reinterpret_cast<const bf16x8_t*>(act_s + (s0 + i < nks ? ks0 + s0 + i : 0) * 32 + g * 8);
+#pragma unroll
+      for (int tt = 0; tt < TG; ++tt) {
+        f32x4_t acc = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int i = 0; i < SMAX; ++i)
+          if (s0 + i < nks) acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wv[tt][i], b[i], acc, 0, 0, 0);
+        if (lrow == 0) {
+          float4* r = reinterpret_cast<float4*>(red_s + (wave * T + grp * TG + tt) * 16 + g * 4);
+          float4 v = make_float4(acc[0], acc[1], acc[2], acc[3]);
+          if (s0 > 0) v = fd_add4(v, *r);
+          *r = v;
+        }
+      }
+    }
+    s0 += SMAX;
+    if (s0 >= per) break;
+  }
+  // the output projection's matrix for this head: asked for now, used after attention
+  const int ks_b = (h * D) >> 5;
+  const int KS2 = (a.n_head * D) >> 5;
+  const int n_tiles2 = C >> 4;
+  bf16x8_t w2[TP2][NK2];
+#pragma unroll
+  for (int j = 0; j < TP2; ++j) {
+    const int tile = wave + FUSED_WAVES * j;
+#pragma unroll
+    for (int i = 0; i < NK2; ++i) w2[j][i] = fd_packed(a.wproj, tile < n_tiles2 ? tile : 0, KS2, ks_b + i, lane);
+  }
+  fd_barrier();
+  FD_STAMP(2);
+  if (tid < 3 * D) {
+    float v = 0.f;
+#pragma unroll
+    for (int w = 0; w < FUSED_WAVES; ++w) v += red_s[w * T * 16 + tid];
+    const int part = tid / D, d = tid - part * D;
+    if (a.bqkv) v += a.bqkv[part * a.n_head * D + h * D + d];
+    const bf16_t b = float_to_bf16(v);
+    if (part == 0) {
+      q_s[d] = b;
+    } else {
+      (part == 1 ? k_s : v_s)[d] = b;
+      if (slot >= 0) {
+        const long page = slot >> a.page_shift;
+        const int off = slot & page_mask;
+        const long dst = ((((page * a.n_head + h) << a.page_shift) + off) * (long)D) + d;
+        (part == 1 ? a.kpool : a.vpool)[dst] = b;
+      }
+    }
+  }
+  fd_barrier();  // also: the waves' sums are read, their place takes attention's partial results
+  FD_STAMP(3);
+
+  // ---- attention over the keys before the token's own (from the pages) and its own (from LDS)
+  const uint4 qraw = *reinterpret_cast<const uint4*>(q_s + dg * 8);
+  float m = -INFINITY, l = 0.f;
+  float acc[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) acc[e] = 0.f;
+  for (int c_base = 0; c_base < kv_end; c_base += CHUNK * FUSED_WAVES) {
+    const int c0 = c_base + wave * CHUNK;
+    if (c_base > 0 && c0 < kv_end) {
+      int page[NI];
+#pragma unroll
+      for (int i = 0; i < NI; ++i) {
+        const int e = (c0 + i * KPI + sub) >> a.page_shift;
+        page[i] = bt[e < a.max_blocks ? e : a.max_blocks - 1];
+      }
+#pragma unroll
+      for (int i = 0; i < NI; ++i) {
+        const int j = c0 + i * KPI + sub;
+        const bool follow = j < kv_end && (unsigned int)page[i] < (unsigned int)a.num_pages;
+        const unsigned int row_off = ((unsigned int)page[i] * a.page_bytes) + (unsigned int)(j & page_mask) * (D * 2u);
+        const unsigned int off = follow ? row_off + lane_off : 0u;
+        kraw[i] = *reinterpret_cast<const uint4*>(reinterpret_cast<const char*>(a.kpool) + off);
+        vraw[i] = *reinterpret_cast<const uint4*>(reinterpret_cast<const char*>(a.vpool) + off);
+      }
+    }
+    if (__builtin_amdgcn_readfirstlane(c0 >= kv_end)) continue;
+    bool valid[NI];
+#pragma unroll
+    for (int i = 0; i < NI; ++i) {
+      valid[i] = c0 + i * KPI + sub < kv_end;
+      if (!valid[i]) vraw[i] = make_uint4(0, 0, 0, 0);  // its weight is 0, but 0 * NaN is not
+    }
+    float s[NI];
+    float cmax = -INFINITY;
+#pragma unroll
+    for (int i = 0; i < NI; ++i) {
+      float dot = fd_dot2(qraw.x, kraw[i].x, 0.f);
+      dot = fd_dot2(qraw.y, kraw[i].y, dot);
+      dot = fd_dot2(qraw.z, kraw[i].z, dot);
+      dot = fd_dot2(qraw.w, kraw[i].w, dot);
+      dot = fd_group_sum<LPK>(dot) * a.scale_log2e;
+      s[i] = valid[i] ? dot : -INFINITY;
+      cmax = fmaxf(cmax, s[i]);
+    }
+    const float m_new = fmaxf(m, wave_max(cmax));
+    if (m_new != -INFINITY) {  // the same in all lanes; false only while the wave has seen no key
+      const float alpha = __builtin_amdgcn_exp2f(m - m_new);  // m = -inf: 0
+      l *= alpha;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) acc[e] *= alpha;
+      m = m_new;
+#pragma unroll
+      for (int i = 0; i < NI; i += 2) {
+        const float pa = __builtin_amdgcn_exp2f(s[i] - m_new), pb = __builtin_amdgcn_exp2f(s[i + 1] - m_new);
+        l += pa + pb;
+        const unsigned int pp = pack_bf16x2(pa, pb);
+        const unsigned int va[4] = {vraw[i].x, vraw[i].y, vraw[i].z, vraw[i].w};
+        const unsigned int vb[4] = {vraw[i + 1].x, vraw[i + 1].y, vraw[i + 1].z, vraw[i + 1].w};
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+          // (va.low half, vb.low half) and (va.high half, vb.high half): channel 2w and 2w+1 of both keys
+          const unsigned int lo = __builtin_amdgcn_perm(vb[w], va[w], 0x05040100u);
+          const unsigned int hi = __builtin_amdgcn_perm(vb[w], va[w], 0x07060302u);
+          acc[2 * w] = fd_dot2(pp, lo, acc[2 * w]);
+          acc[2 * w + 1] = fd_dot2(pp, hi, acc[2 * w + 1]);
+        }
+      }
+    }
+  }
+  if (wave == 0) {
+    // the token's own key and value: the first wave takes them in, its first key group holds the weight
+    const uint4 kk = *reinterpret_cast<const uint4*>(k_s + dg * 8);
+    const uint4 vv = *reinterpret_cast<const uint4*>(v_s + dg * 8);
+    float dot = fd_dot2(qraw.x, kk.x, 0.f);
+    dot = fd_dot2(qraw.y, kk.y, dot);
+    dot = fd_dot2(qraw.z, kk.z, dot);
+    dot = fd_dot2(qraw.w, kk.w, dot);
+    dot = fd_group_sum<LPK>(dot) * a.scale_log2e;
+    const float m_new = fmaxf(m, dot);
+    const float alpha = __builtin_amdgcn_exp2f(m - m_new);
+    l *= alpha;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc[e] *= alpha;
+    m = m_new;
+    const float p = __builtin_amdgcn_exp2f(dot - m_new);
+    if (sub == 0) {
+      l += p;
+      const unsigned int pp = pack_bf16x2(p, 0.f);
+      const unsigned int vw[4] = {vv.x, vv.y, vv.z, vv.w};
+#pragma unroll
+      for (int w = 0; w < 4; ++w) {
+        acc[2 * w] = fd_dot2(pp, vw[w] & 0xffffu, acc[2 * w]);
+        acc[2 * w + 1] = fd_dot2(pp, vw[w] >> 16, acc[2 * w + 1]);
+      }
+    }
+  }
+  FD_STAMP(4);
+
+  // ---- merge of the waves' partial results (rows [sub][wave] of D channels; a key's weight sits on
+  // LPK lanes, so lane dg == 0 speaks for the group's sum)
+  if (lane == 0) m_s[wave] = m;
+  if (dg == 0) l_s[sub * FUSED_WAVES + wave] = l;
+  {
+    float4* dst = reinterpret_cast<float4*>(acc_s + (sub * FUSED_WAVES + wave) * D + dg * 8);
+    dst[0] = make_float4(acc[0], acc[1], acc[2], acc[3]);
+    dst[1] = make_float4(acc[4], acc[5], acc[6], acc[7]);
+  }
+  fd_barrier();
+  {
+    float mx = m_s[0];
+#pragma unroll
+    for (int w = 1; w < FUSED_WAVES; ++w) mx = fmaxf(mx, m_s[w]);
+    const int c = tid % D, sset = tid / D;  // this thread: channel c of the partial rows 8 sset ..
+    float av = 0.f, lt = 0.f;
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+      const int r = sset * 8 + k;
+      const float f = __builtin_amdgcn_exp2f(m_s[r & (FUSED_WAVES - 1)] - mx);  // a wave without keys: 0, and its sums are 0
+      av = fmaf(acc_s[r * D + c], f, av);
+      lt = fmaf(l_s[r], f, lt);
+    }
+    part_s[sset * D + c] = av;
+    if (c == 0) lpart_s[sset] = lt;
+  }
+  fd_barrier();
+  if (tid < D) {
+    float av = 0.f, lt = 0.f;
+#pragma unroll
+    for (int s2 = 0; s2 < SUBSETS; ++s2) {
+      av += part_s[s2 * D + tid];
+      lt += lpart_s[s2];
+    }
+    y_s[tid] = float_to_bf16(av / lt);
+  }
+  fd_barrier();
+  FD_STAMP(5);
+
+  // ---- this head's share of the output projection: row tiles dealt out to the waves
+  {
+    const bf16x8_t zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+    bf16x8_t yb[NK2];
+#pragma unroll
+    for (int i = 0; i < NK2; ++i) {
+      const int idx0 = (ks_b + i) * 32 + g * 8 - h * D;  // where this lane's 8 values of k lie in the head
+      yb[i] = (idx0 >= 0 && idx0 < D) ? *reinterpret_cast<const bf16x8_t*>(y_s + idx0) : zero8;
+    }
+    float* orow = a.out_partials + h * a.out_part_stride + (long)n * C;
+    for (int pass = 0;; ++pass) {
+#pragma unroll
+      for (int j = 0; j < TP2; ++j) {
+        const int tile = wave + FUSED_WAVES * (pass * TP2 + j);
+        if (tile < n_tiles2) {
+          f32x4_t o = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+          for (int i = 0; i < NK2; ++i) o = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w2[j][i], yb[i], o, 0, 0, 0);
+          if (lrow == 0) {
+            const int oc = tile * 16 + g * 4;
+            float4 v = make_float4(o[0], o[1], o[2], o[3]);
+            if (h == 0 && a.bproj) v = fd_add4(v, *reinterpret_cast<const float4*>(a.bproj + oc));
+            *reinterpret_cast<float4*>(orow + oc) = v;
+          }
+        }
+      }
+      if (FUSED_WAVES * (pass + 1) * TP2 >= n_tiles2) break;
+#pragma unroll
+      for (int j = 0; j < TP2; ++j) {
+        const int tile = wave + FUSED_WAVES * ((pass + 1) * TP2 + j);
+#pragma unroll
+        for (int i = 0; i < NK2; ++i) w2[j][i] = fd_packed(a.wproj, tile < n_tiles2 ? tile : 0, KS2, ks_b + i, lane);
+      }
+    }
+  }
+  FD_STAMP(6);
+}
+
+struct FusedMlpArgs {
+  FusedResidual res;
+  const float* gain;
+  const float* beta;  // or null
+  float eps;
+  const bf16_t* wfc;    // packed [hidden rows, width]
+  const float* bfc;     // or null
+  const bf16_t* wproj;  // packed [width rows, hidden]
+  const float* bproj;   // or null
+  float* out_partials;  // [hidden / FUSED_MLP_SLICE][part_rows][width]
+  long out_part_stride;
+  int n_rows, width, hidden, rows_per_wg;
+};
+
+#define FM_TS (FUSED_MLP_SLICE / 16)   // row tiles of a workgroup's slice of the first product
+#define FM_KQ (FUSED_WAVES / FM_TS)    // waves that share a row tile, each a stretch of k
+#define FM_SMAX 4                      // k steps of it whose loads are in flight together
+#define FM_NK2 (FUSED_MLP_SLICE / 32)  // k steps of the second product that the slice covers
+#define FM_TP2 2                       // row tiles of the second product per wave in flight together
+#define FM_GS (FUSED_MLP_SLICE + 8)    // row stride of the slice's activations in LDS
+#define FM_RED_BYTES (FM_KQ * FM_TS * 64 * 4 * 4)
+#define FM_WAVE_PARTS 8                // parts of a residual row that one wave adds up
+
+// VU: vectors of four that a lane holds of a row (width <= 256 VU).  The workgroup has rows_per_wg
+// rows (a power of two up to 16); a row belongs to 16 / rows_per_wg waves, of which each adds up
+// every (16 / rows_per_wg)-th part of it (FM_WAVE_PARTS at most), and the first the base as well.
+template <int VU>
+__global__ __launch_bounds__(FUSED_THREADS) void fused_mlp_decode_kernel(FusedMlpArgs a) {
+  // the waves' sums of their rows [16][width] (later: of the first product), then the normed rows
+  // [rows_per_wg][width + 8]
+  extern __shared__ __align__(16) char smem[];
+  __shared__ __align__(16) bf16_t g_s[16 * FM_GS];
+  const int j = blockIdx.x, r0 = blockIdx.y * a.rows_per_wg;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int lrow = lane & 15, g = lane >> 4;
+  const int C = a.width, KS = C >> 5, V = C >> 2;
+  const int RW = a.rows_per_wg;
+  const int lda = C + 8;
+  float* xs = reinterpret_cast<float*>(smem);
+  float* red = reinterpret_cast<float*>(smem);
+  const int xs_bytes = FUSED_WAVES * C * 4 > FM_RED_BYTES ? FUSED_WAVES * C * 4 : FM_RED_BYTES;
+  bf16_t* act_s = reinterpret_cast<bf16_t*>(smem + xs_bytes);
+
+  FD_STAMP(8);
+  // ---- loads in the order in which their data is needed: this wave's share of a residual row,
+  // then the weights of both products (the second product's behind the barrier that the rows'
+  // sums need: a wave passes a barrier only when all others have issued what stands before it)
+  const int wpr = FUSED_WAVES / RW;           // waves of a row
+  const int lr = wave / wpr, sw = wave - lr * wpr;
+  const int row = r0 + lr;
+  const bool has_row = row < a.n_rows;        // the same in all lanes, like everything that decides a load here
+  float4 xs4[VU], gv[VU], bv[VU];
+#pragma unroll
+  for (int u = 0; u < VU; ++u) xs4[u] = gv[u] = bv[u] = make_float4(0.f, 0.f, 0.f, 0.f);
+  if (has_row) {
+    float4 xp[VU][FM_WAVE_PARTS];
+#pragma unroll
+    for (int u = 0; u < VU; ++u) {
+      const int c4 = lane + 64 * u;
+      const int cc = c4 < V ? c4 : 0;
+      if (sw == 0) {
+        xs4[u] = reinterpret_cast<const float4*>(a.res.base)[(long)row * V + cc];
+        gv[u] = reinterpret_cast<const float4*>(a.gain)[cc];
+        if (a.beta) bv[u] = reinterpret_cast<const float4*>(a.beta)[cc];
+      }
+#pragma unroll
+      for (int k = 0; k < FM_WAVE_PARTS; ++k) {
+        xp[u][k] = make_float4(0.f, 0.f, 0.f, 0.f);
+        const int p = sw + k * wpr;
+        if (p < a.res.n_parts)
+          xp[u][k] = reinterpret_cast<const float4*>(a.res.partials + p * a.res.part_stride)[(long)row * V + cc];
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < VU; ++u)
+#pragma unroll
+      for (int k = 0; k < FM_WAVE_PARTS; ++k) xs4[u] = fd_add4(xs4[u], xp[u][k]);
+  }
+  const int tt = wave & (FM_TS - 1), kq = wave / FM_TS;  // this wave's row tile and stretch of k
+  const int per = (KS + FM_KQ - 1) / FM_KQ;
+  const int ks0 = kq * per;
+  const int nks = max(0, min(per, KS - ks0));
+  bf16x8_t wv[FM_SMAX];
+#pragma unroll
+  for (int i = 0; i < FM_SMAX; ++i) wv[i] = fd_packed(a.wfc, (long)j * FM_TS + tt, KS, i < nks ? ks0 + i : 0, lane);
+
+  // ---- the waves' shares of the rows meet in LDS; a row's first wave adds them, LayerNorm, bfloat16
+#pragma unroll
+  for (int u = 0; u < VU; ++u) {
+    const int c4 = lane + 64 * u;
+    if (c4 < V) reinterpret_cast<float4*>(xs + wave * C)[c4] = xs4[u];
+  }
+  fd_barrier();
+  const int KS2 = a.hidden >> 5;
+  const int n_tiles2 = C >> 4;
+  bf16x8_t w2[FM_TP2][FM_NK2];
+#pragma unroll
+  for (int q = 0; q < FM_TP2; ++q) {
+    const int tile = wave + FUSED_WAVES * q;
+#pragma unroll
+    for (int i = 0; i < FM_NK2; ++i) w2[q][i] = fd_packed(a.wproj, tile < n_tiles2 ? tile : 0, KS2, j * FM_NK2 + i, lane);
+  }
+  if (sw == 0 && has_row) {
+    const int used = min(wpr, max(a.res.n_parts, 1));  // waves beyond the parts hold zeros
+    float4 xv[VU];
+    float s1 = 0.f;
+#pragma unroll
+    for (int u = 0; u < VU; ++u) {
+      const int c4 = lane + 64 * u;
+      xv[u] = make_float4(0.f, 0.f, 0.f, 0.f);
+      if (c4 < V) {
+        xv[u] = xs4[u];
+        for (int q = 1; q < used; ++q) xv[u] = fd_add4(xv[u], reinterpret_cast<const float4*>(xs + (wave + q) * C)[c4]);
+        if (j == 0 && a.res.settled) reinterpret_cast<float4*>(a.res.settled + (long)row * C)[c4] = xv[u];
+        s1 += fd_sum4(xv[u]);
+      }
+    }
+    const float mean = wave_sum(s1) / (float)C;
+    float sq = 0.f;
+#pragma unroll
+    for (int u = 0; u < VU; ++u) {
+      const bool in = lane + 64 * u < V;
+      xv[u] = in ? make_float4(xv[u].x - mean, xv[u].y - mean, xv[u].z - mean, xv[u].w - mean)
+                 : make_float4(0.f, 0.f, 0.f, 0.f);
+      sq += (xv[u].x * xv[u].x + xv[u].y * xv[u].y) + (xv[u].z * xv[u].z + xv[u].w * xv[u].w);
+    }
+    const float rstd = 1.0f / sqrtf(wave_sum(sq) / (float)C + a.eps);
+#pragma unroll
+    for (int u = 0; u < VU; ++u) {
+      const int c4 = lane + 64 * u;
+      if (c4 < V) {
+        uint2 pk;
+        pk.x = pack_bf16x2(xv[u].x * rstd * gv[u].x + bv[u].x, xv[u].y * rstd * gv[u].y + bv[u].y);
+        pk.y = pack_bf16x2(xv[u].z * rstd * gv[u].z + bv[u].z, xv[u].w * rstd * gv[u].w + bv[u].w);
+        *reinterpret_cast<uint2*>(act_s + lr * lda + c4 * 4) = pk;
+      }
+    }
+  }
+  fd_barrier();
+  FD_STAMP(9);
+
+  // ---- first product: a wave one row tile of the slice over its stretch of k
+  // (a column of the MFMA beyond the workgroup's rows repeats its first row and is never stored)
+  const int arow = (lrow < RW && r0 + lrow < a.n_rows) ? lrow : 0;
+  f32x4_t acc = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+  for (int s0 = 0;;) {
+#pragma unroll
+    for (int i = 0; i < FM_SMAX; ++i)
+      if (s0 + i < nks) {
+        const bf16x8_t b = *reinterpret_cast<const bf16x8_t*>(act_s + arow * lda + (ks0 + s0 + i) * 32 + g * 8);
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wv[i], b, acc, 0, 0, 0);
+      }
+    s0 += FM_SMAX;
+    if (s0 >= per) break;
+#pragma unroll
+    for (int i = 0; i < FM_SMAX; ++i)
+      wv[i] = fd_packed(a.wfc, (long)j * FM_TS + tt, KS, s0 + i < nks ? ks0 + s0 + i : 0, lane);
+  }
+  // (the rows' sums were read before the last barrier: their place takes the waves' sums of the product)
+  *reinterpret_cast<float4*>(red + ((kq * FM_TS + tt) * 64 + lane) * 4) = make_float4(acc[0], acc[1], acc[2], acc[3]);
+  fd_barrier();
+  FD_STAMP(10);
+  {
+    // a thread one hidden unit of one row: the waves' sums in the order of k, bias, GELU
+    const int t2 = tid >> 8, ln = (tid >> 2) & 63, i4 = tid & 3;
+    float v = 0.f;
+#pragma unroll
+    for (int q = 0; q < FM_KQ; ++q) v += red[((q * FM_TS + t2) * 64 + ln) * 4 + i4];
+    const int o = t2 * 16 + (ln >> 4) * 4 + i4;  // hidden unit within the slice
+    if (a.bfc) v += a.bfc[j * FUSED_MLP_SLICE + o];
+    g_s[(ln & 15) * FM_GS + o] = float_to_bf16(gelu_tanh_fast(v));
+  }
+  fd_barrier();
+  FD_STAMP(11);
+
+  // ---- the slice's share of the second product: row tiles dealt out to the waves
+  bf16x8_t yb[FM_NK2];
+#pragma unroll
+  for (int i = 0; i < FM_NK2; ++i) yb[i] = *reinterpret_cast<const bf16x8_t*>(g_s + lrow * FM_GS + i * 32 + g * 8);
+  const bool store = lrow < RW && r0 + lrow < a.n_rows;
+  float* orow = a.out_partials + j * a.out_part_stride + (long)(r0 + lrow) * C;
+  for (int pass = 0;; ++pass) {
+#pragma unroll
+    for (int q = 0; q < FM_TP2; ++q) {
+      const int tile = wave + FUSED_WAVES * (pass * FM_TP2 + q);
+      if (tile < n_tiles2) {
+        f32x4_t o = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int i = 0; i < FM_NK2; ++i) o = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w2[q][i], yb[i], o, 0, 0, 0);
+        if (store) {
+          const int oc = tile * 16 + g * 4;
+          float4 v = make_float4(o[0], o[1], o[2], o[3]);
+          if (j == 0 && a.bproj) v = fd_add4(v, *reinterpret_cast<const float4*>(a.bproj + oc));
+          *reinterpret_cast<float4*>(orow + oc) = v;
+        }
+      }
+    }
+    if (FUSED_WAVES * (pass + 1) * FM_TP2 >= n_tiles2) break;
+#pragma unroll
+    for (int q = 0; q < FM_TP2; ++q) {
+      const int tile = wave + FUSED_WAVES * ((pass + 1) * FM_TP2 + q);
+#pragma unroll
+      for (int i = 0; i < FM_NK2; ++i) w2[q][i] = fd_packed(a.wproj, tile < n_tiles2 ? tile : 0, KS2, j * FM_NK2 + i, lane);
+    }
+  }
+  FD_STAMP(12);
+}
+
+// out[i] = LayerNorm(row rows[i] (or i) of a residual that is still a sum); a workgroup a row
+template <typename OT>
+__global__ __launch_bounds__(FUSED_THREADS) void residual_layernorm_kernel(FusedResidual res, const float* __restrict__ gain,
+                                                                           const float* __restrict__ beta, float eps,
+                                                                           const int* __restrict__ rows,
+                                                                           OT* __restrict__ out, int width) {
+  __shared__ __align__(16) float xs[4 * FUSED_THREADS];
+  __shared__ float mean_s[FUSED_WAVES], var_s[FUSED_WAVES];
+  const int i = blockIdx.x, tid = threadIdx.x;
+  const int V = width >> 2, G = FUSED_THREADS / V;
+  const long row = rows ? rows[i] : i;
+  FdRowLoads L;
+  fd_row_issue<false>(res, row, 0, 0, V, G, L);
+  const int vc = tid < V ? tid : 0;
+  const float4 gain4 = reinterpret_cast<const float4*>(gain)[vc];
+  const float4 beta4 = fd_keep4(beta != nullptr, reinterpret_cast<const float4*>(beta ? beta : gain)[vc]);
+  const float4 xv = fd_row_sum<false>(res, V, G, L, xs);
+  const float4 y = fd_row_norm(xv, V, width, eps, gain4, beta4, mean_s, var_s);
+  if (tid < V) {
+    OT* orow = out + (long)i * width;
+    if (sizeof(OT) == 4) {
+      reinterpret_cast<float4*>(orow)[tid] = y;
+    } else {
+      uint2 pk;
+      pk.x = pack_bf16x2(y.x, y.y);
+      pk.y = pack_bf16x2(y.z, y.w);
+      reinterpret_cast<uint2*>(orow)[tid] = pk;
+    }
+  }
+}
+
+// settled[row] = the row's sum; a thread four values (settled may be the base itself).  Not on
+// the path of a decode step: for parts that need plain rows.
+__global__ __launch_bounds__(256) void residual_settle_kernel(FusedResidual res, int n_rows, int width) {
+  const int V = width >> 2;
+  const long idx = (long)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= (long)n_rows * V) return;
+  const long row = idx / V;
+  const int c4 = (int)(idx - row * V);
+  float4 s = reinterpret_cast<const float4*>(res.base)[row * V + c4];
+  for (int p = 0; p < res.n_parts; ++p) s = fd_add4(s, reinterpret_cast<const float4*>(res.partials + p * res.part_stride)[row * V + c4]);
+  reinterpret_cast<float4*>(res.settled)[row * V + c4] = s;
+}
+
+// What every launcher checks of a residual that is still a sum.  tables_ok: the kernel can look the
+// rows up in the token and position tables itself.
+static int check_residual(const FusedResidual& r, int width, bool tables_ok) {
+  if (width <= 0 || (width % 32) != 0 || width > FUSED_MAX_WIDTH) return MGPT_ERR_BAD_SHAPE;
+  if (!r.base) {
+    if (!tables_ok || r.n_parts != 0) return MGPT_ERR_BAD_SHAPE;
+    if (!r.tok_table || !r.ids || (r.pos_table && !r.positions)) return MGPT_ERR_NULL;
+  }
+  if (r.n_parts < 0 || (r.n_parts > 0 && !r.partials)) return MGPT_ERR_NULL;
+  if (r.n_parts > 0 && r.part_stride < width) return MGPT_ERR_BAD_SHAPE;
+  const size_t align = (size_t)r.base | (size_t)r.partials | (size_t)r.settled | (size_t)(r.part_stride * 4);
+  if ((align & 15) != 0 || (((size_t)r.tok_table | (size_t)r.pos_table) & 7) != 0) return MGPT_ERR_BAD_SHAPE;
+  return MGPT_OK;
+}
+
+// parts that a workgroup of FUSED_THREADS threads adds up of one row (fd_row_issue)
+static int group_parts_limit(int width) { return FUSED_GROUP_PARTS * (FUSED_THREADS / (width / 4)); }
+
+static FusedResidual make_residual(const float* base, const float* partials, int n_parts, long part_stride,
+                                   const void* tok_table, const void* pos_table, const int* ids,
+                                   const int* positions, float* settled) {
+  FusedResidual r;
+  r.base = base; r.partials = n_parts > 0 ? partials : nullptr; r.n_parts = n_parts; r.part_stride = part_stride;
+  r.tok_table = (const bf16_t*)tok_table; r.pos_table = (const bf16_t*)pos_table; r.ids = ids;
+  r.positions = positions; r.settled = settled;
+  return r;
+}
+
+// Most parts of a pending residual of this width that the fused kernels take (0: the width is not taken).
+extern "C" int mgpt_fused_parts_limit(int width) {
+  if (width <= 0 || (width % 32) != 0 || width > FUSED_MAX_WIDTH) return 0;
+  const int a = group_parts_limit(width), b = FM_WAVE_PARTS * FUSED_WAVES;
+  return a < b ? a : b;
+}
+
+// The attention half of a layer for the single tokens of a decode-only step (token n is request n or,
+// with q_req[n] < 0, padding).  Refuses (MGPT_ERR_BAD_SHAPE) head sizes other than 16, 32, 64, 128,
+// widths beyond FUSED_MAX_WIDTH or no multiple of 32, n_head * head_dim no multiple of 32, pages that
+// are no power of two, pools of 4 GiB or more, more parts than mgpt_fused_parts_limit.
+// out_partials gets n_head parts.
+extern "C" int mgpt_fused_attention_decode(
+    const float* base, const float* partials, int n_parts, long part_stride, const void* tok_table,
+    const void* pos_table, const int* ids, const int* token_positions, float* settled, const float* gain,
+    const float* beta, float eps, const void* wqkv_packed, const float* bqkv, const void* wproj_packed,
+    const float* bproj, float* out_partials, long out_part_stride, void* kpool, void* vpool,
+    const int* slot_mapping, const int* block_tables, int max_blocks, const int* positions, const int* q_req,
+    int n_rows, int width, int n_head, int head_dim, int page_size, int num_pages, float scale,
+    hipStream_t stream) {
+  if (n_rows == 0) return MGPT_OK;
+  if (!gain || !wqkv_packed || !wproj_packed || !out_partials || !kpool || !vpool || !slot_mapping ||
+      !block_tables || !positions || !q_req)
+    return MGPT_ERR_NULL;
+  FusedAttnArgs a;
+  a.res = make_residual(base, partials, n_parts, part_stride, tok_table, pos_table, ids, token_positions, settled);
+  int rc = check_residual(a.res, width, true);
+  if (rc != MGPT_OK) return rc;
+  if (n_rows < 0 || n_head <= 0 || max_blocks <= 0 || num_pages <= 0 || ((n_head * head_dim) % 32) != 0 ||
+      n_parts > group_parts_limit(width) || out_part_stride < (long)n_rows * width || ((out_part_stride * 4) & 15) != 0 ||
+      (((size_t)out_partials | (size_t)gain | (size_t)beta | (size_t)bproj) & 15) != 0)
+    return MGPT_ERR_BAD_SHAPE;
+  if (n_rows > 65535) return MGPT_ERR_TOO_LARGE;
+  int page_shift = -1;
+  for (int s = 0; s < 30; ++s)
+    if ((1 << s) == page_size) page_shift = s;
+  if (page_shift < 0) return MGPT_ERR_BAD_SHAPE;
+  const long pool_bytes = (long)num_pages * n_head * page_size * head_dim * 2;
+  if (pool_bytes >= (1L << 32)) return MGPT_ERR_BAD_SHAPE;
+  a.gain = gain; a.beta = beta; a.eps = eps;
+  a.wqkv = (const bf16_t*)wqkv_packed; a.bqkv = bqkv; a.wproj = (const bf16_t*)wproj_packed; a.bproj = bproj;
+  a.out_partials = out_partials; a.out_part_stride = out_part_stride;
+  a.kpool = (bf16_t*)kpool; a.vpool = (bf16_t*)vpool; a.slot_mapping = slot_mapping;
+  a.block_tables = block_tables; a.max_blocks = max_blocks; a.positions = positions; a.q_req = q_req;
+  a.width = width; a.n_head = n_head; a.page_shift = page_shift; a.num_pages = num_pages;
+  a.page_bytes = (unsigned int)(n_head * page_size * head_dim * 2);
+  a.scale_log2e = scale * 1.4426950408889634f;
+  // the head is the fast index: the workgroups of a head (one per token) then land on the same
+  // XCD when the number of heads is a multiple of 8, and share its copy of the head's weights
+  dim3 grid(n_head, n_rows), block(FUSED_THREADS);
+#define FA_LAUNCH(DD)                                                                                     \
+  do {                                                                                                    \
+    if (base) hipLaunchKernelGGL((fused_attention_decode_kernel<DD, false>), grid, block, 0, stream, a);  \
+    else hipLaunchKernelGGL((fused_attention_decode_kernel<DD, true>), grid, block, 0, stream, a);        \
+  } while (0)
+  switch (head_dim) {
+    case 16: FA_LAUNCH(16); break;
+    case 32: FA_LAUNCH(32); break;
+    case 64: FA_LAUNCH(64); break;
+    case 128: FA_LAUNCH(128); break;
+    default: return MGPT_ERR_BAD_SHAPE;
+  }
+#undef FA_LAUNCH
+  return mgpt_last_error();
+}
+
+// rows of a workgroup of the feed-forward kernel, a power of two: as few as keep the workgroups
+// within 256, and no more than leave every row the waves that its parts need
+static int mlp_rows_per_wg(int n_rows, int hidden, int n_parts) {
+  const int slices = hidden / FUSED_MLP_SLICE;
+  int most = FUSED_WAVES;  // a row needs a wave per FM_WAVE_PARTS parts
+  while (most > 1 && (FUSED_WAVES / most) * FM_WAVE_PARTS < n_parts) most >>= 1;
+  int rw = 1;
+  while (rw < most && (long)slices * ((n_rows + rw - 1) / rw) > 256) rw <<= 1;
+  return rw;
+}
+
+// The feed-forward half of a layer.  hidden must be a multiple of FUSED_MLP_SLICE; the residual must
+// have a base (no table rows); out_partials gets hidden / FUSED_MLP_SLICE parts.
+extern "C" int mgpt_fused_mlp_decode(const float* base, const float* partials, int n_parts, long part_stride,
+                                     const void* tok_table, const void* pos_table, const int* ids,
+                                     const int* token_positions, float* settled, const float* gain,
+                                     const float* beta, float eps, const void* wfc_packed, const float* bfc,
+                                     const void* wproj_packed, const float* bproj, float* out_partials,
+                                     long out_part_stride, int n_rows, int width, int hidden, hipStream_t stream) {
+  if (n_rows == 0) return MGPT_OK;
+  if (!gain || !wfc_packed || !wproj_packed || !out_partials) return MGPT_ERR_NULL;
+  FusedMlpArgs a;
+  a.res = make_residual(base, partials, n_parts, part_stride, tok_table, pos_table, ids, token_positions, settled);
+  int rc = check_residual(a.res, width, false);
+  if (rc != MGPT_OK) return rc;
+  if (n_rows < 0 || hidden <= 0 || (hidden % FUSED_MLP_SLICE) != 0 || n_parts > FM_WAVE_PARTS * FUSED_WAVES ||
+      out_part_stride < (long)n_rows * width || ((out_part_stride * 4) & 15) != 0 ||
+      (((size_t)out_partials | (size_t)gain | (size_t)beta | (size_t)bproj) & 15) != 0)
+    return MGPT_ERR_BAD_SHAPE;
+  a.gain = gain; a.beta = beta; a.eps = eps;
+  a.wfc = (const bf16_t*)wfc_packed; a.bfc = bfc; a.wproj = (const bf16_t*)wproj_packed; a.bproj = bproj;
+  a.out_partials = out_partials; a.out_part_stride = out_part_stride;
+  a.n_rows = n_rows; a.width = width; a.hidden = hidden;
+  a.rows_per_wg = mlp_rows_per_wg(n_rows, hidden, n_parts);
+  const int groups = (n_rows + a.rows_per_wg - 1) / a.rows_per_wg;
+  if (groups > 65535) return MGPT_ERR_TOO_LARGE;
+  dim3 grid(hidden / FUSED_MLP_SLICE, groups), block(FUSED_THREADS);
+  size_t smem = (size_t)FUSED_WAVES * width * 4;
+  if (smem < FM_RED_BYTES) smem = FM_RED_BYTES;
+  smem += (size_t)a.rows_per_wg * (width + 8) * 2;
+  if (width <= 256) hipLaunchKernelGGL(fused_mlp_decode_kernel<1>, grid, block, smem, stream, a);
+  else hipLaunchKernelGGL(fused_mlp_decode_kernel<2>, grid, block, smem, stream, a);
+  return mgpt_last_error();
+}
+
+extern "C" int mgpt_fused_mlp_parts(int hidden) {
+  return (hidden > 0 && (hidden % FUSED_MLP_SLICE) == 0) ? hidden / FUSED_MLP_SLICE : 0;
+}
+
+// out[i] = LayerNorm of row rows[i] (or i) of a residual that is still a sum (with a base); out float32 or bfloat16
+extern "C" int mgpt_residual_layernorm(const float* base, const float* partials, int n_parts, long part_stride,
+                                       const void* tok_table, const void* pos_table, const int* ids,
+                                       const int* token_positions, const float* gain, const float* beta,
+                                       float eps, const int* rows, void* out, int out_dtype, int n_rows, int width,
+                                       hipStream_t stream) {
+  if (n_rows == 0) return MGPT_OK;
+  if (!gain || !out) return MGPT_ERR_NULL;
+  const FusedResidual r = make_residual(base, partials, n_parts, part_stride, tok_table, pos_table, ids,
+                                        token_positions, nullptr);
+  int rc = check_residual(r, width, false);
+  if (rc != MGPT_OK) return rc;
+  if (n_rows < 0 || n_parts > group_parts_limit(width) || (((size_t)out | (size_t)gain | (size_t)beta) & 15) != 0)
+    return MGPT_ERR_BAD_SHAPE;
+  dim3 grid(n_rows), block(FUSED_THREADS);
+  if (out_dtype == MGPT_F32)
+    hipLaunchKernelGGL(residual_layernorm_kernel<float>, grid, block, 0, stream, r, gain, beta, eps, rows, (float*)out, width);
+  else if (out_dtype == MGPT_BF16)
+    hipLaunchKernelGGL(residual_layernorm_kernel<bf16_t>, grid, block, 0, stream, r, gain, beta, eps, rows, (bf16_t*)out, width);
+  else
+    return MGPT_ERR_BAD_DTYPE;
+  return mgpt_last_error();
+}
+
+// settled[row] = base[row] + the parts; settled may be base
+extern "C" int mgpt_residual_settle(const float* base, const float* partials, int n_parts, long part_stride,
+                                    const void* tok_table, const void* pos_table, const int* ids,
+                                    const int* token_positions, float* settled, int n_rows, int width,
+                                    hipStream_t stream) {
+  if (n_rows == 0) return MGPT_OK;
+  if (!settled) return MGPT_ERR_NULL;
+  const FusedResidual r = make_residual(base, partials, n_parts, part_stride, tok_table, pos_table, ids,
+                                        token_positions, settled);
+  int rc = check_residual(r, width, false);
+  if (rc != MGPT_OK) return rc;
+  if (n_rows < 0) return MGPT_ERR_BAD_SHAPE;
+  const long total = (long)n_rows * (width / 4);
+  hipLaunchKernelGGL(residual_settle_kernel, dim3((unsigned int)((total + 255) / 256)), dim3(256), 0, stream, r,
+                     n_rows, width);
+  return mgpt_last_error();
+}

@@ -564,3 +564,189 @@ def prefill_attention_bf16(q: torch.Tensor, out: torch.Tensor, k_pool: torch.Ten
         return False
     _check(rc, "prefill_attention_bf16")
     return True
+
+
+# ---------------------------------------------------------------- decode steps of few rows, fused
+FUSED_MAX_WIDTH = 512
+FUSED_MLP_SLICE = 64
+
+
+def fused_parts_limit(width: int) -> int:
+    """Most pending sums of a residual of this width that the fused kernels add up on their way in
+    (0: they do not take the width)."""
+    if width <= 0 or width % 32 or width > FUSED_MAX_WIDTH:
+        return 0
+    return int(library.kernels().mgpt_fused_parts_limit(width))
+
+
+def _residual_args(pending, width: int):
+    """The argument block of a residual that is still a sum (ops.residual.PendingSums)."""
+    base, partials, n_parts = pending.base, pending.partials, pending.n_parts
+    tok = pos = ids = positions = None
+    if base is None:
+        tok, pos, ids, positions = pending.tables
+        _need_cuda(tok, pos, ids, positions)
+        _need(tok.dtype == torch.bfloat16 and tok.is_contiguous() and tok.shape[1] == width,
+              "the token table must be dense bfloat16 [vocab, width]")
+        _need(pos is None or (pos.dtype == torch.bfloat16 and pos.is_contiguous() and pos.shape[1] == width),
+              "the position table must be dense bfloat16 [positions, width]")
+    else:
+        _need_cuda(base)
+        _need(base.dtype == torch.float32 and base.is_contiguous() and base.shape[1] == width,
+              "the residual rows must be dense float32 [rows, width]")
+    stride = 0
+    if n_parts:
+        _need_cuda(partials)
+        _need(partials.dtype == torch.float32 and partials.dim() == 3 and partials.is_contiguous()
+              and partials.shape[0] >= n_parts and partials.shape[2] == width,
+              "pending sums must be dense float32 [parts, rows, width]")
+        stride = partials.stride(0)
+    return (_ptr(base), _ptr(partials) if n_parts else None, n_parts, stride, _ptr(tok), _ptr(pos), _ptr(ids),
+            _ptr(positions))
+
+
+def _residual_rows(pending) -> int:
+    """Rows that every array of a pending residual holds."""
+    rows = 1 << 30
+    if pending.base is not None:
+        rows = min(rows, pending.base.shape[0])
+    else:
+        rows = min(rows, pending.tables[2].numel())
+    if pending.n_parts:
+        rows = min(rows, pending.partials.shape[1])
+    return rows
+
+
+def fused_attention_decode(pending, settled: torch.Tensor, gain: torch.Tensor, beta: Optional[torch.Tensor],
+                           eps: float, wqkv_packed: torch.Tensor, bqkv: Optional[torch.Tensor],
+                           wproj_packed: torch.Tensor, bproj: Optional[torch.Tensor], out_partials: torch.Tensor,
+                           k_pool: torch.Tensor, v_pool: torch.Tensor, slot_mapping: torch.Tensor,
+                           block_tables: torch.Tensor, positions: torch.Tensor, q_req: torch.Tensor, n_rows: int,
+                           n_head: int, scale: float) -> bool:
+    """LayerNorm, one head's q/k/v, cache write, attention and that head's share of the output
+    projection, for the single tokens of a decode-only step: out_partials[h, n] is head h's share
+    of what token n adds to the residual.  The residual comes as a sum (pending), whose value is
+    stored to `settled` on the way.  False, having launched nothing, if the kernel does not take
+    the shape."""
+    width = gain.numel()
+    _need_cuda(settled, gain, beta, wqkv_packed, bqkv, wproj_packed, bproj, out_partials, k_pool, v_pool,
+               slot_mapping, block_tables, positions, q_req)
+    _need(k_pool.shape == v_pool.shape and k_pool.dim() == 4 and k_pool.is_contiguous() and v_pool.is_contiguous()
+          and k_pool.dtype == torch.bfloat16 and v_pool.dtype == torch.bfloat16,
+          "key and value pools must be dense bfloat16 [pages, kv_heads, page_size, head_dim]")
+    num_pages, n_kv_head, page_size, head_dim = k_pool.shape
+    q_width = n_head * head_dim
+    if (n_kv_head != n_head or head_dim not in (16, 32, 64, 128) or width % 32 or width > FUSED_MAX_WIDTH
+            or q_width % 32 or page_size & (page_size - 1) or pending.n_parts > fused_parts_limit(width)):
+        return False
+    args = _residual_args(pending, width)
+    _need(_residual_rows(pending) >= n_rows, "the pending residual holds fewer rows than the step")
+    _need(settled.dtype == torch.float32 and settled.is_contiguous() and settled.shape[1] == width
+          and settled.shape[0] >= n_rows and (pending.base is None or settled.data_ptr() != pending.base.data_ptr()),
+          "the settled rows need a dense float32 array of their own")
+    for name, t, numel in (("gain", gain, width), ("beta", beta, width), ("qkv bias", bqkv, 3 * q_width),
+                           ("projection bias", bproj, width)):
+        _need(t is None or (t.dtype == torch.float32 and t.numel() == numel), f"{name} must be float32 [{numel}]")
+    _need(wqkv_packed.dtype == torch.bfloat16 and wqkv_packed.numel() == 3 * q_width * width,
+          "wqkv_packed must be pack_weight of the [3 * heads * head_dim, width] matrix")
+    _need(wproj_packed.dtype == torch.bfloat16 and wproj_packed.numel() == width * q_width,
+          "wproj_packed must be pack_weight of the [width, heads * head_dim] matrix")
+    _need(out_partials.dtype == torch.float32 and out_partials.dim() == 3 and out_partials.is_contiguous()
+          and out_partials.shape[0] >= n_head and out_partials.shape[1] >= n_rows and out_partials.shape[2] == width,
+          "out_partials must be dense float32 [>=heads, >=rows, width]")
+    _need(block_tables.dtype == torch.int32 and block_tables.dim() == 2 and block_tables.is_contiguous()
+          and block_tables.shape[0] >= n_rows, "block_tables must be dense int32 [>=rows, blocks]")
+    _need_i32("slot_mapping", slot_mapping, n_rows)
+    _need_i32("positions", positions, n_rows)
+    _need_i32("q_req", q_req, n_rows)
+    rc = library.kernels().mgpt_fused_attention_decode(
+        *args, _ptr(settled), _ptr(gain), _ptr(beta), float(eps), _ptr(wqkv_packed), _ptr(bqkv), _ptr(wproj_packed),
+        _ptr(bproj), _ptr(out_partials), out_partials.stride(0), _ptr(k_pool), _ptr(v_pool), _ptr(slot_mapping),
+        _ptr(block_tables), block_tables.shape[1], _ptr(positions), _ptr(q_req), n_rows, width, n_head, head_dim,
+        page_size, num_pages, float(scale), _stream())
+    if rc == -2:
+        return False
+    _check(rc, "fused_attention_decode")
+    return True
+
+
+def fused_mlp_parts(hidden: int) -> int:
+    """Parts that fused_mlp_decode leaves of its output (0: it does not take this hidden size)."""
+    return hidden // FUSED_MLP_SLICE if hidden > 0 and hidden % FUSED_MLP_SLICE == 0 else 0
+
+
+def fused_mlp_decode(pending, settled: torch.Tensor, gain: torch.Tensor, beta: Optional[torch.Tensor], eps: float,
+                     wfc_packed: torch.Tensor, bfc: Optional[torch.Tensor], wproj_packed: torch.Tensor,
+                     bproj: Optional[torch.Tensor], out_partials: torch.Tensor, n_rows: int, hidden: int) -> bool:
+    """LayerNorm, 64 hidden units of the first product with bias and GELU-tanh, and their share of
+    the second product, per workgroup: out_partials[j, n] is what hidden units 64 j .. add to row n
+    of the residual.  False, having launched nothing, if the kernel does not take the shape."""
+    width = gain.numel()
+    parts = fused_mlp_parts(hidden)
+    if not parts or width % 32 or width > FUSED_MAX_WIDTH or pending.base is None \
+            or pending.n_parts > fused_parts_limit(width):
+        return False
+    _need_cuda(settled, gain, beta, wfc_packed, bfc, wproj_packed, bproj, out_partials)
+    args = _residual_args(pending, width)
+    _need(_residual_rows(pending) >= n_rows, "the pending residual holds fewer rows than the step")
+    _need(settled.dtype == torch.float32 and settled.is_contiguous() and settled.shape[1] == width
+          and settled.shape[0] >= n_rows and (pending.base is None or settled.data_ptr() != pending.base.data_ptr()),
+          "the settled rows need a dense float32 array of their own")
+    for name, t, numel in (("gain", gain, width), ("beta", beta, width), ("first bias", bfc, hidden),
+                           ("second bias", bproj, width)):
+        _need(t is None or (t.dtype == torch.float32 and t.numel() == numel), f"{name} must be float32 [{numel}]")
+    _need(wfc_packed.dtype == torch.bfloat16 and wfc_packed.numel() == hidden * width
+          and wproj_packed.dtype == torch.bfloat16 and wproj_packed.numel() == hidden * width,
+          "the matrices must be pack_weight of [hidden, width] and [width, hidden]")
+    _need(out_partials.dtype == torch.float32 and out_partials.dim() == 3 and out_partials.is_contiguous()
+          and out_partials.shape[0] >= parts and out_partials.shape[1] >= n_rows and out_partials.shape[2] == width,
+          "out_partials must be dense float32 [>=hidden/64, >=rows, width]")
+    rc = library.kernels().mgpt_fused_mlp_decode(
+        *args, _ptr(settled), _ptr(gain), _ptr(beta), float(eps), _ptr(wfc_packed), _ptr(bfc), _ptr(wproj_packed),
+        _ptr(bproj), _ptr(out_partials), out_partials.stride(0), n_rows, width, hidden, _stream())
+    if rc == -2:
+        return False
+    _check(rc, "fused_mlp_decode")
+    return True
+
+
+def residual_layer_norm(pending, gain: torch.Tensor, beta: Optional[torch.Tensor], eps: float,
+                        rows: Optional[torch.Tensor], out: torch.Tensor, n_rows: int) -> bool:
+    """out[i] = LayerNorm of row rows[i] (or i) of a residual that is still a sum.  False if the
+    width is not taken."""
+    width = gain.numel()
+    if width % 32 or width > FUSED_MAX_WIDTH or pending.base is None or pending.n_parts > fused_parts_limit(width):
+        return False
+    _need_cuda(gain, beta, rows, out)
+    args = _residual_args(pending, width)
+    _need(gain.dtype == torch.float32 and (beta is None or (beta.dtype == torch.float32 and beta.numel() == width)),
+          "gain and beta must be float32 [width]")
+    _need(out.is_contiguous() and out.shape[1] == width and out.shape[0] >= n_rows, "LayerNorm output too small")
+    if rows is None:
+        _need(_residual_rows(pending) >= n_rows, "the pending residual holds fewer rows than asked for")
+    else:
+        _need_i32("rows", rows, n_rows)
+    rc = library.kernels().mgpt_residual_layernorm(*args, _ptr(gain), _ptr(beta), float(eps), _ptr(rows), _ptr(out),
+                                                   _dtype_code(out), n_rows, width, _stream())
+    if rc == -2:
+        return False
+    _check(rc, "residual_layer_norm")
+    return True
+
+
+def residual_settle(pending, settled: torch.Tensor, n_rows: int) -> bool:
+    """settled[:n_rows] = the rows of a residual that is still a sum (settled may be its base).
+    False if the width is not taken."""
+    width = settled.shape[1]
+    if width % 32 or width > FUSED_MAX_WIDTH or pending.base is None:
+        return False
+    _need_cuda(settled)
+    args = _residual_args(pending, width)
+    _need(settled.dtype == torch.float32 and settled.is_contiguous() and settled.shape[0] >= n_rows,
+          "the settled rows must be dense float32")
+    _need(_residual_rows(pending) >= n_rows, "the pending residual holds fewer rows than asked for")
+    rc = library.kernels().mgpt_residual_settle(*args, _ptr(settled), n_rows, width, _stream())
+    if rc == -2:
+        return False
+    _check(rc, "residual_settle")
+    return True

@@ -7,7 +7,7 @@ from typing import Optional, Union
 
 import torch
 
-from . import kernels
+from . import kernels, residual
 
 
 class LazyNorm:
@@ -22,7 +22,18 @@ class LazyNorm:
     def tensor(self, ctx) -> torch.Tensor:
         if self._tensor is None:
             h = ctx.workspace.get(self.buffer, self.n_rows, self.x.shape[1], ctx.dtype)
-            self.norm.forward(ctx, self.x, h, self.n_rows, rows=self.rows)
+            pending = getattr(ctx, "pending", None)
+            if pending is not None:
+                # the residual is still a sum: a LayerNorm adds it up on its way in, anything else
+                # needs plain rows first
+                norm = self.norm
+                if not (getattr(norm, "fusable_layer_norm", False)
+                        and kernels.residual_layer_norm(pending, norm.weight, norm.bias, norm.eps, self.rows, h,
+                                                        self.n_rows)):
+                    residual.settle(ctx, self.x, ctx.n_rows)
+                    pending = None
+            if pending is None:
+                self.norm.forward(ctx, self.x, h, self.n_rows, rows=self.rows)
             self._tensor = h
         return self._tensor
 
@@ -99,6 +110,8 @@ def linear(ctx, a: Union[torch.Tensor, LazyNorm], w: torch.Tensor, bias: Optiona
     pages by the same kernel; the return value says whether that was done."""
     if n_rows == 0:
         return scatter is not None
+    if isinstance(a, LazyNorm) and getattr(ctx, "pending", None) is not None:
+        a = a.tensor(ctx)      # the kernels below read plain residual rows
     fast = w.dtype == torch.bfloat16 and not ctx.exact and ctx.dtype == torch.bfloat16
     wide_out = w.shape[0] >= WIDE_OUT and n_rows * w.shape[1] > WIDE_OUT_DECODE_WORK
     if fast and n_rows <= 64 and not wide_out:

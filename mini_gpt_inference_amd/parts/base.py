@@ -57,6 +57,9 @@ class Part:
     # graph and replayed.  A part that looks at ctx.host_ctx_lens or ctx.host_state_slots, or that
     # allocates, is not.
     graph_safe = False
+    # True if the part reads the residual stream through ops.residual (it takes sums that are still
+    # pending, or settles them itself); every other part is handed a plain residual stream
+    takes_pending_residual = False
 
     def weight_requests(self) -> Dict[str, WeightRequest]:
         """Parameter name -> shape and role of every tensor this part needs."""
@@ -187,3 +190,5 @@ class StepContext:
     padded: bool = False         # rows and requests are padded to a bucket's sizes (n_rows, cu_q.numel() - 1):
                                  # the host values above then describe the bucket, not the step
     lead_cap: int = 0            # padded steps: the decoding requests' tokens lie among the first lead_cap
+    # sums that are still to be added to the residual stream (ops.residual.PendingSums); None: it is plain
+    pending: Optional[Any] = None

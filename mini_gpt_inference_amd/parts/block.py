@@ -4,6 +4,7 @@ from __future__ import annotations
 
 import torch
 
+from ..ops import residual
 from ..ops.linear import LazyNorm
 from .base import CacheBinding, Part, StepContext, register_arrangement
 from .feedforward import FeedForward
@@ -24,13 +25,19 @@ class PreNorm(Arrangement):
     """x = x + mixer(norm1(x)); x = x + ff(norm2(x)) (reference: src/minigpt_infer/model.py:112-115)."""
 
     graph_safe = True
+    takes_pending_residual = True
 
     def __init__(self, width: int) -> None:
         self.width = int(width)
 
     def run(self, ctx, x, norm1, mixer, norm2, feed_forward, binding, position) -> None:
         # the norms are handed on uncomputed: a linear layer that can normalise in its prologue
-        # does, everything else calls .tensor(ctx) and gets the normed rows
+        # does, everything else calls .tensor(ctx) and gets the normed rows.  A part that does not
+        # know of a residual whose sums are still pending gets a plain one.
         n = ctx.n_rows
+        if not mixer.takes_pending_residual:
+            residual.settle(ctx, x, n)
         mixer.forward_add(ctx, LazyNorm(norm1, x, n), x, binding, position)
+        if not feed_forward.takes_pending_residual:
+            residual.settle(ctx, x, n)
         feed_forward.forward_add(ctx, LazyNorm(norm2, x, n), x)

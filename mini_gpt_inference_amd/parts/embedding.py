@@ -6,7 +6,7 @@ from typing import Dict, Optional
 
 import torch
 
-from ..ops import kernels
+from ..ops import kernels, residual
 from ..ops.linear import linear
 from .base import MATRIX, Part, StepContext, TABLE, WeightRequest, register_embedding, register_head
 from .positions import PositionEncoding
@@ -29,7 +29,14 @@ class TokenEmbedding(Part):
         return {"weight": WeightRequest((self.vocab_size, self.width), TABLE)}
 
     def forward(self, ctx: StepContext, position: PositionEncoding, x: torch.Tensor) -> None:
-        kernels.embed(ctx.token_ids, ctx.positions, self.weight, position.embedding_table(), x, ctx.n_rows)
+        table = position.embedding_table()
+        if (residual.usable(ctx, self.width, 1) and self.weight.dtype == torch.bfloat16
+                and (table is None or table.dtype == torch.bfloat16)):
+            # a decode-only step of few rows: the rows are looked up by the kernel that reads the
+            # residual first (or by ops.residual.settle, for a part that needs plain rows)
+            ctx.pending = residual.PendingSums(None, None, 0, (self.weight, table, ctx.token_ids, ctx.positions))
+            return
+        kernels.embed(ctx.token_ids, ctx.positions, self.weight, table, x, ctx.n_rows)
 
 
 @register_head("linear_head")

@@ -6,8 +6,8 @@ from typing import Dict
 
 import torch
 
-from ..ops import kernels
-from ..ops.linear import linear
+from ..ops import kernels, residual
+from ..ops.linear import LazyNorm, linear, packed_weight
 from .base import MATRIX, Part, StepContext, VECTOR, WeightRequest, register_feed_forward
 
 _ACTIVATIONS = {"gelu_tanh": kernels.EPI_GELU}
@@ -28,6 +28,7 @@ class DenseMLP(FeedForward):
     a parameter)."""
 
     graph_safe = True
+    takes_pending_residual = True
 
     def __init__(self, width: int, hidden: int, bias: bool, activation: str = "gelu_tanh") -> None:
         if activation not in _ACTIVATIONS:
@@ -44,7 +45,36 @@ class DenseMLP(FeedForward):
             req["proj_bias"] = WeightRequest((self.width,), VECTOR)
         return req
 
+    def _forward_add_fused(self, ctx: StepContext, h, x: torch.Tensor) -> bool:
+        """A decode-only step of few rows: one kernel from the residual (a sum, as the kernels
+        before left it) through LayerNorm, both products and the activation to this part's addition
+        to the residual, left as one partial sum per 64 hidden units.  False, with nothing launched,
+        where that kernel does not apply."""
+        parts_n = kernels.fused_mlp_parts(self.hidden)
+        if not (isinstance(h, LazyNorm) and h._tensor is None and h.rows is None and h.x is x
+                and getattr(h.norm, "fusable_layer_norm", False) and parts_n and residual.usable(ctx, self.width, parts_n)
+                and self.activation == "gelu_tanh" and self.fc_weight.dtype == torch.bfloat16
+                and self.proj_weight.dtype == torch.bfloat16):
+            return False
+        wfc, wproj = packed_weight(self.fc_weight), packed_weight(self.proj_weight)
+        if wfc is None or wproj is None:
+            return False
+        n = ctx.n_rows
+        if ctx.pending is not None and ctx.pending.base is None:
+            residual.settle(ctx, x, n)      # table rows: this kernel reads residual rows only
+        pending, settled = residual.take(ctx, x)
+        parts = ctx.workspace.get("feed_forward_parts", parts_n * n, self.width, torch.float32) \
+            [:parts_n * n].view(parts_n, n, self.width)
+        if not kernels.fused_mlp_decode(pending, settled, h.norm.weight, h.norm.bias, h.norm.eps, wfc, self.fc_bias,
+                                        wproj, self.proj_bias, parts, n, self.hidden):
+            return False
+        ctx.pending = residual.PendingSums(settled, parts, parts_n)
+        return True
+
     def forward_add(self, ctx: StepContext, h: torch.Tensor, x: torch.Tensor) -> None:
+        if self._forward_add_fused(ctx, h, x):
+            return
+        residual.settle(ctx, x, ctx.n_rows)
         n = ctx.n_rows
         u = ctx.workspace.get("ff_hidden", n, self.hidden, ctx.dtype)
         linear(ctx, h, self.fc_weight, self.fc_bias, u, n, _ACTIVATIONS[self.activation])

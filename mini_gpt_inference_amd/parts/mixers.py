@@ -7,8 +7,8 @@ from typing import Dict, Optional, Union
 import torch
 
 from ..ops import attention as attention_ops
-from ..ops import kernels
-from ..ops.linear import linear
+from ..ops import kernels, residual
+from ..ops.linear import LazyNorm, linear, packed_weight
 from .base import (CacheBinding, KVNeed, MATRIX, Part, StateNeed, StepContext, VECTOR, WeightRequest,
                    register_mixer)
 from .positions import PositionEncoding
@@ -41,6 +41,7 @@ class PagedCausalAttention(Mixer):
     head-major; out = y Wproj^T (+ b) (model.py:89-90), added into the residual (model.py:113)."""
 
     graph_safe = True
+    takes_pending_residual = True
 
     def __init__(self, width: int, n_head: int, head_dim: int, bias: bool, n_kv_head: Optional[int] = None,
                  scale: Optional[float] = None, window: int = 0) -> None:
@@ -69,8 +70,39 @@ class PagedCausalAttention(Mixer):
     def cache_need(self) -> KVNeed:
         return KVNeed(self.n_kv_head, self.head_dim, self.window)
 
+    def _forward_add_fused(self, ctx: StepContext, h, x: torch.Tensor, binding: CacheBinding,
+                           position: PositionEncoding) -> bool:
+        """A decode-only step of few rows: one kernel from the residual (as the kernels before left
+        it: a sum) through LayerNorm, projections, cache write and attention to this mixer's
+        addition to the residual, left as one partial sum per head.  False, with nothing launched,
+        where that kernel does not apply."""
+        if not (isinstance(h, LazyNorm) and h._tensor is None and h.rows is None and h.x is x
+                and getattr(h.norm, "fusable_layer_norm", False) and residual.usable(ctx, self.width, self.n_head)
+                and binding.writes and not position.rotates and self.window == 0
+                and self.n_kv_head == self.n_head and self.qkv_weight.dtype == torch.bfloat16
+                and self.proj_weight.dtype == torch.bfloat16):
+            return False
+        wqkv, wproj = packed_weight(self.qkv_weight), packed_weight(self.proj_weight)
+        if wqkv is None or wproj is None:
+            return False
+        n = ctx.n_rows
+        group = ctx.groups[binding.group]
+        pending, settled = residual.take(ctx, x)
+        parts = ctx.workspace.get("attention_parts", self.n_head * n, self.width, torch.float32) \
+            [:self.n_head * n].view(self.n_head, n, self.width)
+        if not kernels.fused_attention_decode(
+                pending, settled, h.norm.weight, h.norm.bias, h.norm.eps, wqkv, self.qkv_bias, wproj, self.proj_bias,
+                parts, group.k_pools[binding.index], group.v_pools[binding.index], group.slot_mapping,
+                group.block_tables, ctx.positions, ctx.q_req, n, self.n_head, self.scale):
+            return False
+        ctx.pending = residual.PendingSums(settled, parts, self.n_head)
+        return True
+
     def forward_add(self, ctx: StepContext, h: torch.Tensor, x: torch.Tensor, binding: CacheBinding,
                     position: PositionEncoding) -> None:
+        if self._forward_add_fused(ctx, h, x, binding, position):
+            return
+        residual.settle(ctx, x, ctx.n_rows)
         n = ctx.n_rows
         total = self.q_width + 2 * self.kv_width
         qkv = ctx.workspace.get("qkv", n, total, ctx.dtype)

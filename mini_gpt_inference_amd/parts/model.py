@@ -13,6 +13,7 @@ from typing import Dict, List, Optional, Tuple
 
 import torch
 
+from ..ops import residual
 from ..ops.linear import LazyNorm
 from . import block as _block  # noqa: F401  (registers the parts)
 from . import embedding as _embedding  # noqa: F401
@@ -171,9 +172,12 @@ class DecoderModel:
         n = ctx.n_rows
         ws = ctx.workspace
         x = ws.get("residual", n, self.spec.width, torch.float32)
+        ctx.pending = None
         self.embedding.forward(ctx, self.position, x)
         for run, binding in zip(self.spec.order, self.cache_layout.bindings):
             layer = self.layers[run.layer]
+            if not layer.arrangement.takes_pending_residual:
+                residual.settle(ctx, x, n)
             layer.arrangement.run(ctx, x, layer.norm1, layer.mixer, layer.norm2, layer.feed_forward, binding,
                                   self.position)
         m = ctx.m_rows
@@ -184,4 +188,5 @@ class DecoderModel:
         if m:
             self.head.forward(ctx, LazyNorm(self.final_norm, x, m, rows=ctx.logit_rows, buffer="final_normed"),
                               logits, m)
+        ctx.pending = None
         return logits[:m]
