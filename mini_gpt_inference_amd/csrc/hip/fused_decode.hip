@@ -65,6 +65,21 @@ __device__ __forceinline__ float fd_group_sum(float v) {
   return v;
 }
 
+// sum over the lanes that hold the same channels of different keys (lane = key group * LPK + channel
+// group): rotations within the rows of 16 lanes, then the four rows; no trip through LDS
+template <int LPK>
+__device__ __forceinline__ float fd_sum_over_keys(float v) {
+  if (LPK <= 8) v += fd_dpp<0x128>(v);  // row_ror:8
+  if (LPK <= 4) v += fd_dpp<0x124>(v);  // row_ror:4
+  if (LPK <= 2) v += fd_dpp<0x122>(v);  // row_ror:2
+  const unsigned int u = __float_as_uint(v);
+  const auto a = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+  const float x = __uint_as_float(a[0]) + __uint_as_float(a[1]);
+  const unsigned int ux = __float_as_uint(x);
+  const auto b = __builtin_amdgcn_permlane32_swap(ux, ux, false, false);
+  return __uint_as_float(b[0]) + __uint_as_float(b[1]);
+}
+
 __device__ __forceinline__ float fd_dot2(unsigned int a, unsigned int b, float c) {
   return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(fd_bf16x2_t, a), __builtin_bit_cast(fd_bf16x2_t, b),
                                          c, false);
@@ -209,15 +224,13 @@ __global__ __launch_bounds__(FUSED_THREADS) void fused_attention_decode_kernel(F
   constexpr int LPK = D / 8, KPI = 64 / LPK;     // lanes per key, keys per load instruction
   constexpr int NI = LPK / 2 < 2 ? 2 : LPK / 2;  // load instructions of a wave's keys in one pass
   constexpr int CHUNK = NI * KPI;                // keys of a wave in one pass
-  constexpr int ROWS = FUSED_WAVES * KPI;        // partial results of attention: one per (key subgroup, wave)
-  constexpr int SUBSETS = FUSED_THREADS / D;     // groups of 8 partial rows, one thread per channel each
   constexpr int NK2 = D <= 32 ? 1 : D / 32;      // k steps of the projection that hold this head's columns
   constexpr int TP2 = 4 / NK2 > 0 ? 4 / NK2 : 1; // its row tiles per wave whose loads are in flight together
-  static_assert(ROWS == SUBSETS * 8, "the merge deals eight partial rows to a thread");
   // one pool for what is never alive together: the row's partial sums, then the waves' sums of
   // q, k, v, then attention's partial results
-  constexpr int POOL_FLOATS = ROWS * D > 4096 ? ROWS * D : 4096;
+  constexpr int POOL_FLOATS = FUSED_WAVES * T * 16 > 4096 ? FUSED_WAVES * T * 16 : 4096;
   static_assert(FUSED_WAVES * T * 16 <= POOL_FLOATS, "the pool holds the waves' sums of q, k, v");
+  static_assert(FUSED_WAVES * D <= POOL_FLOATS, "the pool holds the waves' sums of attention");
   __shared__ __align__(16) float pool[POOL_FLOATS];
   __shared__ __align__(16) bf16_t act_s[FUSED_MAX_WIDTH];
   __shared__ float mean_s[FUSED_WAVES], var_s[FUSED_WAVES];
@@ -226,9 +239,7 @@ __global__ __launch_bounds__(FUSED_THREADS) void fused_attention_decode_kernel(F
   __shared__ __align__(16) bf16_t v_s[D];
   __shared__ __align__(16) bf16_t y_s[D];
   __shared__ float m_s[FUSED_WAVES];
-  __shared__ float l_s[ROWS];
-  __shared__ float part_s[SUBSETS * D];
-  __shared__ float lpart_s[SUBSETS];
+  __shared__ float l_s[FUSED_WAVES];
   float* const xs = pool;
   float* const red_s = pool;
   float* const acc_s = pool;
@@ -285,6 +296,18 @@ __global__ __launch_bounds__(FUSED_THREADS) void fused_attention_decode_kernel(F
   if (tid < V) {
     gain4 = reinterpret_cast<const float4*>(a.gain)[vc];
     if (a.beta) beta4 = reinterpret_cast<const float4*>(a.beta)[vc];
+  }
+  // what the epilogues add: this thread's bias of q, k or v, and (first head) the projection's
+  float qkv_bias = 0.f;
+  if (tid < 3 * D && a.bqkv) qkv_bias = a.bqkv[(tid / D) * a.n_head * D + h * D + tid % D];
+  const int n_tiles2 = C >> 4;
+  float4 proj_bias[TP2];
+#pragma unroll
+  for (int j = 0; j < TP2; ++j) {
+    proj_bias[j] = make_float4(0.f, 0.f, 0.f, 0.f);
+    const int tile = wave + FUSED_WAVES * j;
+    if (h == 0 && a.bproj && lrow == 0 && tile < n_tiles2)
+      proj_bias[j] = *reinterpret_cast<const float4*>(a.bproj + tile * 16 + g * 4);
   }
   const int per = (KS + FUSED_WAVES - 1) / FUSED_WAVES;  // k steps of a wave
   const int ks0 = wave * per;
@@ -411,7 +434,6 @@ __global__ __launch_bounds__(FUSED_THREADS) void fused_attention_decode_kernel(F
   // the output projection's matrix for this head: asked for now, used after attention
   const int ks_b = (h * D) >> 5;
   const int KS2 = (a.n_head * D) >> 5;
-  const int n_tiles2 = C >> 4;
   bf16x8_t w2[TP2][NK2];
 #pragma unroll
   for (int j = 0; j < TP2; ++j) {
@@ -426,8 +448,7 @@ __global__ __launch_bounds__(FUSED_THREADS) void fused_attention_decode_kernel(F
 #pragma unroll
     for (int w = 0; w < FUSED_WAVES; ++w) v += red_s[w * T * 16 + tid];
     const int part = tid / D, d = tid - part * D;
-    if (a.bqkv) v += a.bqkv[part * a.n_head * D + h * D + d];
-    const bf16_t b = float_to_bf16(v);
+    const bf16_t b = float_to_bf16(v + qkv_bias);
     if (part == 0) {
       q_s[d] = b;
     } else {
@@ -541,39 +562,31 @@ __global__ __launch_bounds__(FUSED_THREADS) void fused_attention_decode_kernel(F
   }
   FD_STAMP(4);
 
-  // ---- merge of the waves' partial results (rows [sub][wave] of D channels; a key's weight sits on
-  // LPK lanes, so lane dg == 0 speaks for the group's sum)
-  if (lane == 0) m_s[wave] = m;
-  if (dg == 0) l_s[sub * FUSED_WAVES + wave] = l;
-  {
-    float4* dst = reinterpret_cast<float4*>(acc_s + (sub * FUSED_WAVES + wave) * D + dg * 8);
+  // ---- merge: first across the key groups of a wave (lanes that differ above the LPK lanes of a
+  // key: the maximum is the wave's already, so the sums simply add), then across the waves in LDS
+  l = fd_sum_over_keys<LPK>(l);
+#pragma unroll
+  for (int e = 0; e < 8; ++e) acc[e] = fd_sum_over_keys<LPK>(acc[e]);
+  if (lane == 0) {
+    m_s[wave] = m;
+    l_s[wave] = l;
+  }
+  if (lane < LPK) {
+    float4* dst = reinterpret_cast<float4*>(acc_s + wave * D + dg * 8);
     dst[0] = make_float4(acc[0], acc[1], acc[2], acc[3]);
     dst[1] = make_float4(acc[4], acc[5], acc[6], acc[7]);
   }
   fd_barrier();
-  {
+  if (tid < D) {
     float mx = m_s[0];
 #pragma unroll
     for (int w = 1; w < FUSED_WAVES; ++w) mx = fmaxf(mx, m_s[w]);
-    const int c = tid % D, sset = tid / D;  // this thread: channel c of the partial rows 8 sset ..
     float av = 0.f, lt = 0.f;
 #pragma unroll
-    for (int k = 0; k < 8; ++k) {
-      const int r = sset * 8 + k;
-      const float f = __builtin_amdgcn_exp2f(m_s[r & (FUSED_WAVES - 1)] - mx);  // a wave without keys: 0, and its sums are 0
-      av = fmaf(acc_s[r * D + c], f, av);
-      lt = fmaf(l_s[r], f, lt);
-    }
-    part_s[sset * D + c] = av;
-    if (c == 0) lpart_s[sset] = lt;
-  }
-  fd_barrier();
-  if (tid < D) {
-    float av = 0.f, lt = 0.f;
-#pragma unroll
-    for (int s2 = 0; s2 < SUBSETS; ++s2) {
-      av += part_s[s2 * D + tid];
-      lt += lpart_s[s2];
+    for (int w = 0; w < FUSED_WAVES; ++w) {
+      const float f = __builtin_amdgcn_exp2f(m_s[w] - mx);  // a wave without keys: exp2(-inf) = 0, and its sums are 0
+      av = fmaf(acc_s[w * D + tid], f, av);
+      lt = fmaf(l_s[w], f, lt);
     }
     y_s[tid] = float_to_bf16(av / lt);
   }
@@ -601,7 +614,8 @@ __global__ __launch_bounds__(FUSED_THREADS) void fused_attention_decode_kernel(F
           if (lrow == 0) {
             const int oc = tile * 16 + g * 4;
             float4 v = make_float4(o[0], o[1], o[2], o[3]);
-            if (h == 0 && a.bproj) v = fd_add4(v, *reinterpret_cast<const float4*>(a.bproj + oc));
+            if (pass == 0) v = fd_add4(v, proj_bias[j]);
+            else if (h == 0 && a.bproj) v = fd_add4(v, *reinterpret_cast<const float4*>(a.bproj + oc));
             *reinterpret_cast<float4*>(orow + oc) = v;
           }
         }
@@ -697,6 +711,16 @@ __global__ __launch_bounds__(FUSED_THREADS) void fused_mlp_decode_kernel(FusedMl
 #pragma unroll
       for (int k = 0; k < FM_WAVE_PARTS; ++k) xs4[u] = fd_add4(xs4[u], xp[u][k]);
   }
+  // what the epilogues add: this thread's bias of the first product, and (first slice) the second's
+  float fc_bias = 0.f;
+  if (a.bfc) fc_bias = a.bfc[j * FUSED_MLP_SLICE + (tid >> 8) * 16 + (((tid >> 2) & 63) >> 4) * 4 + (tid & 3)];
+  float4 proj_bias[FM_TP2];
+#pragma unroll
+  for (int q = 0; q < FM_TP2; ++q) {
+    proj_bias[q] = make_float4(0.f, 0.f, 0.f, 0.f);
+    const int tile = wave + FUSED_WAVES * q;
+    if (j == 0 && a.bproj && tile < (C >> 4)) proj_bias[q] = *reinterpret_cast<const float4*>(a.bproj + tile * 16 + g * 4);
+  }
   const int tt = wave & (FM_TS - 1), kq = wave / FM_TS;  // this wave's row tile and stretch of k
   const int per = (KS + FM_KQ - 1) / FM_KQ;
   const int ks0 = kq * per;
@@ -788,8 +812,7 @@ __global__ __launch_bounds__(FUSED_THREADS) void fused_mlp_decode_kernel(FusedMl
 #pragma unroll
     for (int q = 0; q < FM_KQ; ++q) v += red[((q * FM_TS + t2) * 64 + ln) * 4 + i4];
     const int o = t2 * 16 + (ln >> 4) * 4 + i4;  // hidden unit within the slice
-    if (a.bfc) v += a.bfc[j * FUSED_MLP_SLICE + o];
-    g_s[(ln & 15) * FM_GS + o] = float_to_bf16(gelu_tanh_fast(v));
+    g_s[(ln & 15) * FM_GS + o] = float_to_bf16(gelu_tanh_fast(v + fc_bias));
   }
   fd_barrier();
   FD_STAMP(11);
@@ -811,7 +834,8 @@ __global__ __launch_bounds__(FUSED_THREADS) void fused_mlp_decode_kernel(FusedMl
         if (store) {
           const int oc = tile * 16 + g * 4;
           float4 v = make_float4(o[0], o[1], o[2], o[3]);
-          if (j == 0 && a.bproj) v = fd_add4(v, *reinterpret_cast<const float4*>(a.bproj + oc));
+          if (pass == 0) v = fd_add4(v, proj_bias[q]);
+          else if (j == 0 && a.bproj) v = fd_add4(v, *reinterpret_cast<const float4*>(a.bproj + oc));
           *reinterpret_cast<float4*>(orow + oc) = v;
         }
       }
