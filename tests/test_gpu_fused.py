@@ -1,0 +1,235 @@
+"""The fused kernels of a decode step with few rows, each alone against the plain functions, at sizes
+other than the engine's: a residual that arrives as a base plus pending partial sums (or as table
+rows), widths, head sizes and counts that are no powers of two, contexts around the edges of a
+wave's share of keys and of a pass, a far key that decides the softmax, NaN in everything a kernel
+must not read, padded tokens."""
+
+import math
+
+import pytest
+import torch
+
+import helpers
+import plain_gpt as P
+from mini_gpt_inference_amd.ops import kernels
+from mini_gpt_inference_amd.ops.residual import PendingSums
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+
+
+def rnd(gen, *shape, scale=1.0):
+    return torch.randn(*shape, generator=gen, dtype=torch.float32) * scale
+
+
+def bf(t):
+    return t.to(torch.bfloat16)
+
+
+def i32(values):
+    return torch.tensor(list(values), dtype=torch.int32, device=DEV)
+
+
+def _pending(gen, rows, width, n_parts, extra_rows=2):
+    """A residual as the kernels before would have left it: base + parts, with rows of padding behind
+    that hold NaN.  Returns (PendingSums on the device, the rows' true values in float64)."""
+    base = rnd(gen, rows + extra_rows, width, scale=2.0) + 0.5
+    base[rows:] = float("nan")
+    parts = rnd(gen, max(n_parts, 1), rows + extra_rows, width, scale=0.7)
+    parts[:, rows:] = float("nan")
+    true = base[:rows].double() + (parts[:n_parts, :rows].double().sum(0) if n_parts else 0)
+    return PendingSums(base.to(DEV), parts.to(DEV) if n_parts else None, n_parts), true
+
+
+ATTN_CASES = [
+    # width, heads, head size, page, contexts (keys before the token's own), parts of the residual, biases
+    dict(c=512, h=8, d=64, page=16, ctx=[256, 0, 1, 31, 32, 33, 511, 512, 513, 700], parts=8, bias=True),
+    dict(c=512, h=8, d=64, page=16, ctx=[5, 130], parts=32, bias=True),
+    dict(c=96, h=3, d=32, page=8, ctx=[0, 17, 100, 515], parts=3, bias=False),
+    dict(c=64, h=4, d=16, page=4, ctx=[60, 3, 1029], parts=4, bias=True),
+    dict(c=256, h=2, d=128, page=32, ctx=[40, 600], parts=0, bias=True),
+    dict(c=320, h=5, d=64, page=16, ctx=[77, 0, 300], parts=12, bias=False),
+    dict(c=128, h=6, d=32, page=2, ctx=[9, 64], parts=1, bias=True),     # heads * head size wider than the model
+]
+
+
+@pytest.mark.parametrize("tables", [False, True])
+@pytest.mark.parametrize("case", range(len(ATTN_CASES)))
+def test_fused_attention_decode(case, tables):
+    spec = ATTN_CASES[case]
+    c, h, d, page, ctxs = spec["c"], spec["h"], spec["d"], spec["page"], spec["ctx"]
+    g = torch.Generator().manual_seed(100 + case)
+    n = len(ctxs)
+    rows = n + 1                                  # one padded token behind the real ones
+    qw = h * d
+    gain, beta = 1 + 0.1 * rnd(g, c), rnd(g, c, scale=0.1)
+    wqkv, wproj = bf(rnd(g, 3 * qw, c, scale=c ** -0.5)), bf(rnd(g, c, qw, scale=qw ** -0.5))
+    bqkv, bproj = (rnd(g, 3 * qw, scale=0.2), rnd(g, c, scale=0.2)) if spec["bias"] else (None, None)
+    eps, scale = 1e-5, (0.21 if case % 2 else 1.0 / math.sqrt(d))
+    if tables:
+        vocab, n_pos = 61, max(ctxs) + 1
+        tok, pos = bf(rnd(g, vocab, c)), bf(rnd(g, n_pos, c, scale=0.5))
+        ids = torch.randint(0, vocab, (rows,), generator=g)
+        pending = PendingSums(None, None, 0, (tok.to(DEV), pos.to(DEV), i32(ids), i32(ctxs + [0])))
+        true = tok.double()[ids[:n]] + pos.double()[ctxs]
+    else:
+        pending, true = _pending(g, n, c, spec["parts"], extra_rows=1)
+    # the cache: every request's earlier keys and values in pages handed out in a shuffled order
+    max_blocks = max(-(-(x + 1) // page) for x in ctxs) + 1
+    n_pages = sum(-(-(x + 1) // page) for x in ctxs) + 3
+    order = torch.randperm(n_pages, generator=g).tolist()
+    kp = torch.full((n_pages, h, page, d), float("nan"), dtype=torch.bfloat16)
+    vp = kp.clone()
+    bt = torch.full((rows, max_blocks), 10 ** 6, dtype=torch.int32)      # unused entries point far outside the pool
+    past_k, past_v, slots = [], [], []
+    for r, ctx in enumerate(ctxs):
+        k_r, v_r = bf(rnd(g, ctx, h, d)), bf(rnd(g, ctx, h, d))
+        past_k.append(k_r)
+        past_v.append(v_r)
+        for b in range(-(-(ctx + 1) // page)):
+            bt[r, b] = order.pop()
+        for t in range(ctx):
+            kp[bt[r, t // page], :, t % page] = k_r[t]
+            vp[bt[r, t // page], :, t % page] = v_r[t]
+        slots.append(int(bt[r, ctx // page]) * page + ctx % page)
+    # what the kernel must compute, in float64 from the rounded inputs
+    hn = P.plain_layer_norm(true, gain.double(), beta.double(), eps)
+    qkv = P.plain_linear(bf(hn).double(), wqkv.double(), None if bqkv is None else bqkv.double())
+    # a far key decides the first long request's softmax: a key at position 3 that points along the query
+    far = next((r for r, ctx in enumerate(ctxs) if ctx > 200), None)
+    if far is not None:
+        qf = bf(qkv[far, :d]).double()
+        key = bf((6.0 / scale / qf.norm() ** 2 * qf).float())
+        past_k[far][3, 0] = key
+        kp[bt[far, 3 // page], 0, 3 % page] = key
+    want = torch.empty(n, c, dtype=torch.float64)
+    for r, ctx in enumerate(ctxs):
+        q, k, v = P.plain_split_heads(bf(qkv[r:r + 1]).double(), h)
+        keys = torch.cat([past_k[r].double().transpose(0, 1), k], dim=1)        # [H, ctx + 1, D]
+        vals = torch.cat([past_v[r].double().transpose(0, 1), v], dim=1)
+        y = P.plain_causal_attention(q, keys, vals, scale=scale, causal=False)   # one query sees all ctx + 1 keys
+        want[r] = P.plain_linear(bf(y).double(), wproj.double(), None if bproj is None else bproj.double())
+    dev = lambda t: None if t is None else t.to(DEV)
+    settled = torch.full((rows, c), float("nan"), device=DEV)
+    out = torch.full((h, rows, c), float("nan"), device=DEV)
+    kp_d, vp_d = kp.to(DEV), vp.to(DEV)
+    took = kernels.fused_attention_decode(
+        pending, settled, dev(gain), dev(beta), eps, kernels.pack_weight(wqkv.to(DEV)), dev(bqkv),
+        kernels.pack_weight(wproj.to(DEV)), dev(bproj), out, kp_d, vp_d, i32(slots + [-1]), bt.to(DEV),
+        i32(ctxs + [0]), i32(list(range(n)) + [-1]), rows, h, scale)
+    assert took
+    torch.cuda.synchronize()
+    helpers.assert_close(settled[:n], true, "float32", "the settled rows")
+    helpers.assert_close(out[:, :n].sum(0), want, "bfloat16", f"fused attention case {case}")
+    assert torch.isnan(out[:, n]).all() and torch.isnan(settled[n]).all(), "the padded token's rows were written"
+    for r, ctx in enumerate(ctxs):                 # the token's key and value are in its page, nothing else changed
+        page_i, off = slots[r] // page, slots[r] % page
+        _, k, v = P.plain_split_heads(qkv[r:r + 1], h)
+        helpers.assert_close(kp_d[page_i, :, off], k[:, 0], "bfloat16", "the stored key")
+        helpers.assert_close(vp_d[page_i, :, off], v[:, 0], "bfloat16", "the stored value")
+        kp[page_i, :, off] = kp_d[page_i, :, off].cpu()
+        vp[page_i, :, off] = vp_d[page_i, :, off].cpu()
+    same = lambda a, b: torch.equal(a.view(torch.int16), b.view(torch.int16))
+    assert same(kp_d.cpu(), kp) and same(vp_d.cpu(), vp), "the cache changed beyond the new slots"
+
+
+MLP_CASES = [
+    # width, hidden, rows, parts of the residual, biases
+    dict(c=512, f=2048, rows=1, parts=8, bias=True),
+    dict(c=512, f=2048, rows=8, parts=8, bias=True),
+    dict(c=512, f=2048, rows=16, parts=8, bias=False),
+    dict(c=512, f=2048, rows=23, parts=12, bias=True),      # more parts than a wave adds: fewer rows a workgroup
+    dict(c=96, f=384, rows=5, parts=3, bias=False),
+    dict(c=64, f=256, rows=3, parts=0, bias=True),
+    dict(c=320, f=1280, rows=9, parts=5, bias=True),
+    dict(c=256, f=64, rows=2, parts=40, bias=True),
+    dict(c=128, f=8192, rows=40, parts=2, bias=True),       # more workgroups than compute units
+]
+
+
+@pytest.mark.parametrize("case", range(len(MLP_CASES)))
+def test_fused_mlp_decode(case):
+    spec = MLP_CASES[case]
+    c, f, rows = spec["c"], spec["f"], spec["rows"]
+    g = torch.Generator().manual_seed(200 + case)
+    pending, true = _pending(g, rows, c, spec["parts"])
+    gain, beta = 1 + 0.1 * rnd(g, c), rnd(g, c, scale=0.1)
+    wfc, wproj = bf(rnd(g, f, c, scale=c ** -0.5)), bf(rnd(g, c, f, scale=f ** -0.5))
+    bfc, bproj = (rnd(g, f, scale=0.3), rnd(g, c, scale=0.3)) if spec["bias"] else (None, None)
+    eps = 1e-6 if case % 2 else 1e-5
+    hn = bf(P.plain_layer_norm(true, gain.double(), beta.double(), eps)).double()
+    u = P.plain_gelu_tanh(P.plain_linear(hn, wfc.double(), None if bfc is None else bfc.double()))
+    want = P.plain_linear(bf(u).double(), wproj.double(), None if bproj is None else bproj.double())
+    dev = lambda t: None if t is None else t.to(DEV)
+    n_parts = kernels.fused_mlp_parts(f)
+    assert n_parts == f // 64
+    settled = torch.full((rows + 2, c), float("nan"), device=DEV)
+    out = torch.full((n_parts, rows + 2, c), float("nan"), device=DEV)
+    took = kernels.fused_mlp_decode(pending, settled, dev(gain), dev(beta), eps, kernels.pack_weight(wfc.to(DEV)),
+                                    dev(bfc), kernels.pack_weight(wproj.to(DEV)), dev(bproj), out, rows, f)
+    assert took
+    torch.cuda.synchronize()
+    helpers.assert_close(settled[:rows], true, "float32", "the settled rows")
+    helpers.assert_close(out[:, :rows].sum(0), want, "bfloat16", f"fused feed-forward case {case}")
+    assert torch.isnan(out[:, rows:]).all() and torch.isnan(settled[rows:]).all(), "rows beyond the step were written"
+
+
+@pytest.mark.parametrize("out_dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("c,parts,bias", [(512, 32, True), (96, 3, False), (64, 0, True), (320, 12, True), (32, 100, True)])
+def test_residual_layer_norm_and_settle(c, parts, bias, out_dtype):
+    g = torch.Generator().manual_seed(300 + c)
+    rows = 7
+    pending, true = _pending(g, rows, c, parts)
+    gain, beta = 1 + 0.1 * rnd(g, c), rnd(g, c, scale=0.1) if bias else None
+    want = P.plain_layer_norm(true, gain.double(), None if beta is None else beta.double(), 1e-5)
+    dev = lambda t: None if t is None else t.to(DEV)
+    tdt = torch.float32 if out_dtype == "float32" else torch.bfloat16
+    out = torch.full((rows, c), float("nan"), dtype=tdt, device=DEV)
+    assert kernels.residual_layer_norm(pending, dev(gain), dev(beta), 1e-5, None, out, rows)
+    helpers.assert_close(out, want, out_dtype, "LayerNorm of a pending residual")
+    pick = [6, 0, 3, 3]
+    out2 = torch.full((4, c), float("nan"), dtype=tdt, device=DEV)
+    assert kernels.residual_layer_norm(pending, dev(gain), dev(beta), 1e-5, i32(pick), out2, 4)
+    helpers.assert_close(out2, want[pick], out_dtype, "LayerNorm of chosen rows of a pending residual")
+    # the sum itself: into another array, and into the base
+    settled = torch.full((rows + 2, c), float("nan"), device=DEV)
+    assert kernels.residual_settle(pending, settled, rows)
+    helpers.assert_close(settled[:rows], true, "float32", "settle")
+    assert torch.isnan(settled[rows:]).all()
+    assert kernels.residual_settle(pending, pending.base, rows)
+    helpers.assert_close(pending.base[:rows], true, "float32", "settle in place")
+
+
+def test_fused_kernels_refuse_what_they_cannot_do():
+    """Widths beyond 512 or no multiple of 32, more pending sums than a reader adds up on its way in,
+    key/value groups, head sizes outside 16/32/64/128, a hidden size that is no multiple of 64: False,
+    and nothing is written."""
+    assert kernels.fused_parts_limit(512) == 32 and kernels.fused_parts_limit(544) == 0
+    assert kernels.fused_parts_limit(48) == 0 and kernels.fused_parts_limit(64) >= 128
+    g = torch.Generator().manual_seed(5)
+    for c, f, parts in [(544, 2176, 2), (48, 192, 2), (512, 2048, 33), (512, 2000, 2)]:
+        base = rnd(g, 2, c).to(DEV)
+        pending = PendingSums(base, rnd(g, parts, 2, c).to(DEV), parts)
+        out = torch.full((max(f // 64, 1), 2, c), 7.0, device=DEV)
+        settled = torch.full((2, c), 7.0, device=DEV)
+        w = torch.zeros(f * c, dtype=torch.bfloat16, device=DEV)
+        assert not kernels.fused_mlp_decode(pending, settled, torch.ones(c, device=DEV), None, 1e-5, w, None, w, None,
+                                            out, 2, f)
+        torch.cuda.synchronize()
+        assert bool((out == 7.0).all()) and bool((settled == 7.0).all())
+        if c % 32 or c > 512 or parts > 32:
+            assert not kernels.residual_layer_norm(pending, torch.ones(c, device=DEV), None, 1e-5, None,
+                                                   torch.zeros(2, c, device=DEV), 2)
+    # attention: two key/value heads under four query heads, and a head size of 48
+    for hk, d in [(2, 64), (4, 48)]:
+        c, h = 256, 4
+        pending = PendingSums(rnd(g, 1, c).to(DEV), None, 0)
+        pools = torch.zeros(4, hk, 16, d, dtype=torch.bfloat16, device=DEV)
+        w1 = torch.zeros(3 * h * d * c, dtype=torch.bfloat16, device=DEV)
+        w2 = torch.zeros(c * h * d, dtype=torch.bfloat16, device=DEV)
+        out = torch.full((h, 1, c), 7.0, device=DEV)
+        assert not kernels.fused_attention_decode(pending, torch.zeros(1, c, device=DEV), torch.ones(c, device=DEV), None,
+                                                  1e-5, w1, None, w2, None, out, pools, pools.clone(), i32([0]),
+                                                  torch.zeros(1, 4, dtype=torch.int32, device=DEV), i32([0]), i32([0]),
+                                                  1, h, 0.125)
+        assert bool((out == 7.0).all())
