@@ -95,6 +95,38 @@ def test_many_requests_decode_from_padded_graphs(model_folders, dtype, n_req):
         assert exact >= 0.9 * sum(news)
 
 
+@pytest.mark.parametrize("shape,n_req", [("50M", 8), ("small", 20), ("xl", 64)])
+def test_real_widths_decode_through_graphs_and_bursts(tmp_path, shape, n_req):
+    """The benchmarked shapes through the engine itself (padded graphs, bursts of steps fed on the
+    device): every greedy choice is the plain implementation's argmax up to the logits' tolerance."""
+    from mini_gpt_inference_amd import GPTConfig
+    from mini_gpt_inference_amd.weights.random_init import write_random_model
+    family = {"50M": dict(n_layer=2, n_embd=512, n_head=8, vocab_size=50304),
+              "small": dict(n_layer=1, n_embd=768, n_head=12, vocab_size=50257),
+              "xl": dict(n_layer=1, n_embd=1600, n_head=25, vocab_size=50257)}[shape]
+    cfg = GPTConfig("gpt2-mini", block_size=64, bias=True, layer_norm_eps=1e-5, **family)
+    folder = write_random_model(str(tmp_path / shape), cfg, 11, std_scale=3.0)
+    rng = np.random.default_rng(n_req)
+    prompts = [helpers.random_ids(rng, cfg.vocab_size, int(n)) for n in rng.integers(1, 9, n_req)]
+    n_new = 20
+    engine = LLMEngine.from_folder(folder, EngineConfig(block_size=16, num_blocks=n_req * 2, max_batch_size=n_req,
+                                                        dtype="bfloat16"))
+    got = engine.generate(prompts, SamplingParams(max_tokens=n_new, temperature=0.0))
+    assert engine.stats()["graph_steps"] >= n_new - 4
+    pcfg, w = P.read_model_folder(folder)
+    exact = total = 0
+    for prompt, tokens in list(zip(prompts, got))[::max(1, n_req // 8)]:      # a sample of the requests: the plain model is slow
+        assert len(tokens) == n_new
+        ids = list(prompt)
+        for tok in tokens:
+            logits = P.plain_forward(w, pcfg, ids)[-1].numpy()
+            assert logits[tok] >= logits.max() - 2 * helpers.TOL["bfloat16"] * max(1.0, np.abs(logits).max())
+            exact += tok == int(np.argmax(logits))
+            total += 1
+            ids.append(tok)
+    assert exact >= 0.9 * total
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_chunked_mixed_and_whole_prompt_policies_give_the_same_tokens(model_folders, dtype):
     prompts = _prompts("B", [1, 9, 33, 64, 100], seed=2)

@@ -311,6 +311,64 @@ def test_real_family_sizes(tmp_path, shape, dtype):
     helpers.assert_close(torch.cat(got), want[[0, 33, 69, 70, 86, 87, 88, 89]], dtype, f"{shape} {dtype}")
 
 
+_family_cache = {}
+
+
+def _family_model(tmp_path_factory, shape):
+    """(folder, config, plain config, plain weights) of a family shape, written once per session."""
+    if shape not in _family_cache:
+        from mini_gpt_inference_amd import GPTConfig
+        from mini_gpt_inference_amd.weights.random_init import write_random_model
+        cfg = GPTConfig("gpt2-mini", layer_norm_eps=1e-5, **FAMILY[shape])
+        folder = write_random_model(str(tmp_path_factory.mktemp("family") / shape), cfg, 7, std_scale=2.0)
+        pcfg, w = P.read_model_folder(folder)
+        _family_cache[shape] = (folder, cfg, pcfg, w)
+    return _family_cache[shape]
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("shape", ["small", "xl", "50M"])
+def test_real_family_sizes_mixed_with_page_reuse(tmp_path_factory, shape, dtype):
+    """The real widths under the mixed schedule: up to four live requests, portions of some beside
+    single tokens of others, a NaN-poisoned pool so small that pages are used again."""
+    folder, cfg, pcfg, w = _family_model(tmp_path_factory, shape)
+    rng = np.random.default_rng(21)
+    reqs = {f"r{i}": helpers.random_ids(rng, cfg.vocab_size, n) for i, n in enumerate([50, 37, 64, 20, 45, 33])}
+    plan = helpers.plan_mixed(reqs, np.random.default_rng(8), tail=12)
+    replayer = TraceReplayer(folder, dtype, plan.tight_tokens(16), poison=True)
+    assert sum(-(-len(t) // 16) for t in reqs.values()) > replayer.num_pages, "no page would be used twice"
+    got = plan.assemble(helpers.run_plan_in_process(replayer, plan), {r: len(t) for r, t in reqs.items()},
+                        cfg.vocab_size)
+    for rid, ids in reqs.items():
+        helpers.assert_close(got[rid], P.plain_forward(w, pcfg, ids).numpy(), dtype, f"{shape} {dtype} mixed {rid}")
+    assert replayer.cache.check() == 0 and replayer.cache.num_free_pages() == replayer.num_pages
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("n_req", [8, 17, 40, 64])
+@pytest.mark.parametrize("shape", ["small", "xl", "50M"])
+def test_real_family_sizes_many_requests_decoding(tmp_path_factory, shape, dtype, n_req):
+    """Decode steps of 8, 17, 40 and 64 requests at the real widths, as logits: the decode products
+    change kernels with the rows and the matrix's size (rows dealt out in groups, the inner size
+    split over workgroups, the head's hand-over to the tiled kernel, the fused kernels of few rows).
+    The same step comes several times, so the later ones are graph replays."""
+    folder, cfg, pcfg, w = _family_model(tmp_path_factory, shape)
+    rng = np.random.default_rng(100 + n_req)
+    steps = 4
+    seqs = [helpers.random_ids(rng, cfg.vocab_size, int(rng.integers(1, 6)) + steps) for _ in range(n_req)]
+    want = [P.plain_forward(w, pcfg, s).numpy() for s in seqs]
+    rep = TraceReplayer(folder, dtype, n_req * 16, max_live=n_req, poison=True)
+    heads = [len(s) - steps for s in seqs]
+    rep.run_step({"step": 0, "entries": [{"id": f"r{i}", "tokens": s[:h], "want": []}
+                                         for i, (s, h) in enumerate(zip(seqs, heads))], "end": []})
+    for j in range(steps):
+        got = rep.run_step({"step": 1 + j, "entries": [{"id": f"r{i}", "tokens": [s[h + j]], "want": [0]}
+                                                       for i, (s, h) in enumerate(zip(seqs, heads))], "end": []})
+        ref = np.stack([wv[h + j] for wv, h in zip(want, heads)])
+        helpers.assert_close(got, ref, dtype, f"{shape} {dtype}: decode step {j} of {n_req} requests")
+    assert rep.runner.num_replayed_steps >= 1
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_step_shapes_that_repeat_are_replayed_from_a_graph_with_the_same_logits(model_folders, dtype):
     """Single tokens and portions of four, over and over: from the fourth step of a shape on the
