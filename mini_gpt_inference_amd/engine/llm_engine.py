@@ -410,7 +410,12 @@ class LLMEngine:
 
     def stats(self) -> Dict[str, int]:
         s = self.scheduler
+        weight_bytes, derived_bytes = self.model.weight_bytes()
         return {
+            # device memory of the weights as loaded, and of the copies made of them at first use
+            # (packed for the decode kernels, folded with a LayerNorm)
+            "weight_bytes": weight_bytes, "derived_weight_bytes": derived_bytes,
+            "cache_bytes": self.store.bytes(),
             "num_preemptions": s.num_preemptions, "num_steps": s.num_steps,
             "num_prompt_tokens": s.num_prompt_tokens, "num_decode_tokens": s.num_decode_tokens,
             "free_blocks": self.cache.num_free_pages(0),

@@ -54,6 +54,29 @@ def _derived(w: torch.Tensor) -> dict:
     return tables.setdefault((w.data_ptr(), tuple(w.shape), tuple(w.stride())), {})
 
 
+def derived_bytes(w: torch.Tensor) -> int:
+    """Bytes of device memory that the derived copies of w hold (folded with a LayerNorm, packed
+    for the decode kernels), counting every copy of every view of w's storage once."""
+    owner = w._base if w._base is not None else w
+    seen, total = set(), 0
+
+    def walk(obj) -> None:
+        nonlocal total
+        if isinstance(obj, torch.Tensor):
+            if obj.data_ptr() not in seen:
+                seen.add(obj.data_ptr())
+                total += obj.numel() * obj.element_size()
+        elif isinstance(obj, (tuple, list)):
+            for item in obj:
+                walk(item)
+        elif isinstance(obj, dict):
+            for item in obj.values():
+                walk(item)
+
+    walk(getattr(owner, _DERIVED, None))
+    return total
+
+
 def folded_layer_norm(norm, w: torch.Tensor, bias: Optional[torch.Tensor]):
     """(folded matrix, column sums, folded bias): the matrix with the LayerNorm's gain and bias
     folded in, made once per (norm, matrix, bias)."""

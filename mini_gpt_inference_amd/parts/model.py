@@ -124,8 +124,25 @@ class DecoderModel:
         return wanted
 
     def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
+        self._bound = {name: tensors[name] for name in self.weight_requests()}
         for part, spec in self._named_parts():
             part.bind({local: tensors[spec.weights[local]] for local in part.weight_requests()})
+
+    def weight_bytes(self) -> Tuple[int, int]:
+        """(bytes of the tensors as loaded, bytes of the copies derived from them since: matrices
+        folded with a LayerNorm or packed for the decode kernels, made at first use).  A tensor that
+        two parts share (a tied head) counts once."""
+        from ..ops.linear import derived_bytes
+
+        loaded = derived = 0
+        seen = set()
+        for tensor in getattr(self, "_bound", {}).values():
+            if tensor.data_ptr() in seen:
+                continue
+            seen.add(tensor.data_ptr())
+            loaded += tensor.numel() * tensor.element_size()
+            derived += derived_bytes(tensor)
+        return loaded, derived
 
     # ------------------------------------------------------------------ cache
     def _plan_cache(self) -> CacheLayout:

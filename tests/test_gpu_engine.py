@@ -315,6 +315,25 @@ def test_decode_graphs_can_be_captured_before_the_first_request(model_folders):
         small.capture_decode_graphs()
 
 
+def test_stats_count_the_weights_and_the_copies_made_of_them(model_folders):
+    """stats() reports the bytes of the tensors as loaded (the tied head once) and of the copies the
+    kernels made of the matrices at first use, which are none before the first step."""
+    cfg = helpers.CONFIGS["A"]
+    engine = LLMEngine.from_folder(model_folders["A"], EngineConfig(block_size=4, num_blocks=32, max_batch_size=2,
+                                                                    dtype="bfloat16"))
+    c, f, v, p, L = cfg.n_embd, 4 * cfg.n_embd, cfg.vocab_size, cfg.block_size, cfg.n_layer
+    matrices = (v * c + p * c + L * (3 * c * c + c * c + 2 * f * c)) * 2
+    vectors = ((2 * L + 1) * 2 * c + L * (3 * c + c + f + c)) * 4
+    before = engine.stats()
+    assert before["weight_bytes"] == matrices + vectors and before["derived_weight_bytes"] == 0
+    assert before["cache_bytes"] == L * 2 * 32 * cfg.n_head * 4 * cfg.head_dim * 2
+    engine.generate([[1, 2, 3]], SamplingParams(max_tokens=4, temperature=0.0))
+    after = engine.stats()
+    assert after["weight_bytes"] == before["weight_bytes"]
+    # every matrix of the layers has at least its packed copy by now
+    assert after["derived_weight_bytes"] >= L * (3 * c * c + c * c + 2 * f * c) * 2
+
+
 def test_real_vocabulary_bound_is_never_crossed(model_folders):
     engine = LLMEngine.from_folder(model_folders["A"], EngineConfig(block_size=4, num_blocks=32, max_batch_size=4,
                                                                     dtype="float32", real_vocab_size=40))

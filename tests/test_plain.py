@@ -135,6 +135,45 @@ def test_block_reduces_to_library_pre_norm_layer():
     assert torch.allclose(got, want, atol=1e-10)
 
 
+def test_whole_model_is_a_library_encoder_stack_between_embeddings_and_a_tied_head():
+    """The whole composition beside the block: torch.nn.TransformerEncoder (pre-norm layers in order,
+    then its final norm) fed with the summed embeddings and followed by the tied head is the plain
+    forward.  A dropped or misplaced final norm, blocks out of order, a head that is not the token
+    table, positions that start at 1: each fails it.  The layers differ from each other (every
+    tensor is drawn afresh), so their order shows."""
+    cfg = {"n_layer": 3, "n_embd": 48, "n_head": 3, "vocab_size": 29, "block_size": 20, "layer_norm_eps": 1e-3}
+    w = _weights(cfg, seed=11)
+    def encoder_layer():
+        return torch.nn.TransformerEncoderLayer(48, 3, dim_feedforward=192, dropout=0.0, batch_first=True,
+                                                norm_first=True, layer_norm_eps=1e-3,
+                                                activation=lambda u: F.gelu(u, approximate="tanh"))
+    stack = torch.nn.TransformerEncoder(encoder_layer(), num_layers=3, norm=torch.nn.LayerNorm(48, eps=1e-3),
+                                        enable_nested_tensor=False).double().eval()
+    with torch.no_grad():
+        for i, layer in enumerate(stack.layers):
+            p = f"blocks.{i}."
+            layer.self_attn.in_proj_weight.copy_(w[p + "attn.qkv.weight"])
+            layer.self_attn.in_proj_bias.copy_(w[p + "attn.qkv.bias"])
+            layer.self_attn.out_proj.weight.copy_(w[p + "attn.proj.weight"])
+            layer.self_attn.out_proj.bias.copy_(w[p + "attn.proj.bias"])
+            layer.linear1.weight.copy_(w[p + "mlp.fc.weight"]); layer.linear1.bias.copy_(w[p + "mlp.fc.bias"])
+            layer.linear2.weight.copy_(w[p + "mlp.proj.weight"]); layer.linear2.bias.copy_(w[p + "mlp.proj.bias"])
+            layer.norm1.weight.copy_(w[p + "ln1.weight"]); layer.norm1.bias.copy_(w[p + "ln1.bias"])
+            layer.norm2.weight.copy_(w[p + "ln2.weight"]); layer.norm2.bias.copy_(w[p + "ln2.bias"])
+        stack.norm.weight.copy_(w["ln_f.weight"]); stack.norm.bias.copy_(w["ln_f.bias"])
+    ids = torch.tensor([3, 28, 0, 7, 7, 19, 4, 11, 2])
+    x = F.embedding(ids, w["tok_emb.weight"]) + F.embedding(torch.arange(9), w["pos_emb.weight"])
+    mask = torch.triu(torch.full((9, 9), float("-inf"), dtype=P.DT), diagonal=1)
+    with torch.no_grad():
+        want = F.linear(stack(x[None], mask=mask)[0], w["tok_emb.weight"])
+    got = P.plain_forward(w, cfg, ids.tolist())
+    assert torch.allclose(got, want, atol=1e-9), (got - want).abs().max()
+    # the check can fail: the same stack without its final norm, or with two layers swapped, is far off
+    stack.norm = None
+    with torch.no_grad():
+        assert not torch.allclose(F.linear(stack(x[None], mask=mask)[0], w["tok_emb.weight"]), got, atol=1e-3)
+
+
 def test_forward_head_is_tied_and_prefix_property_holds():
     cfg = {"n_layer": 2, "n_embd": 32, "n_head": 2, "vocab_size": 23, "block_size": 16, "layer_norm_eps": 1e-5}
     w = _weights(cfg, seed=3)
