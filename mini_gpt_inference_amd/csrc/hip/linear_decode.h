@@ -111,7 +111,12 @@ __global__ __launch_bounds__(256) void linear_decode_kernel(SkinnyArgs a) {
   for (int t = 0; t < NT; ++t) {
     acc[t] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
     x0[t] = sd[t] = sq[t] = 0.f;
-    if (LN && row_ok[t]) x0[t] = a.x[(long)src[t] * K];
+    // the shift of a row: the median of three of its values, so that one channel that stands far
+    // out (residual streams have such) does not become the shift
+    if (LN && row_ok[t]) {
+      const float* xr = a.x + (long)src[t] * K;
+      x0[t] = __builtin_amdgcn_fmed3f(xr[0], xr[K >> 1], xr[K - 1]);
+    }
   }
   // W as it is (a wave's load is sixteen rows' 64 bytes), or packed so that it is 1 KB in one piece
   const bf16_t* wp = a.w_packed ? a.w_packed + (((long)(o0 >> 4) * (K >> 5) + (kb >> 5)) * 64 + lane) * 8
@@ -142,8 +147,11 @@ __global__ __launch_bounds__(256) void linear_decode_kernel(SkinnyArgs a) {
       for (int t = 0; t < NT; ++t) {
 #pragma unroll
         for (int i = 0; i < SMAX; ++i) {
-          const float f[8] = {lo[t][i].x, lo[t][i].y, lo[t][i].z, lo[t][i].w,
-                              hi[t][i].x, hi[t][i].y, hi[t][i].z, hi[t][i].w};
+          // what is rounded to bfloat16 is the distance from the row's first value: a row far from
+          // zero loses nothing to its offset (the epilogue corrects with the mean of the distances);
+          // a row that is not loaded has x0 = 0 and zeros
+          const float f[8] = {lo[t][i].x - x0[t], lo[t][i].y - x0[t], lo[t][i].z - x0[t], lo[t][i].w - x0[t],
+                              hi[t][i].x - x0[t], hi[t][i].y - x0[t], hi[t][i].z - x0[t], hi[t][i].w - x0[t]};
           typedef __attribute__((__vector_size__(4 * sizeof(unsigned int)))) unsigned int u32x4_t;
           const u32x4_t pk = {pack_bf16x2(f[0], f[1]), pack_bf16x2(f[2], f[3]), pack_bf16x2(f[4], f[5]),
                               pack_bf16x2(f[6], f[7])};
@@ -151,9 +159,8 @@ __global__ __launch_bounds__(256) void linear_decode_kernel(SkinnyArgs a) {
           if (s0 + i < steps) {
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
-              const float d = f[e] - x0[t];
-              sd[t] += d;
-              sq[t] = fmaf(d, d, sq[t]);
+              sd[t] += f[e];
+              sq[t] = fmaf(f[e], f[e], sq[t]);
             }
           }
         }
@@ -234,17 +241,16 @@ __global__ __launch_bounds__(256) void linear_decode_kernel(SkinnyArgs a) {
     if (!row_ok[t]) continue;
     OT* orow = out + (long)(r0 + t * 16) * a.ldo;
     float v[4];
-    float mean = 0.f, rstd = 1.f;
+    float md = 0.f, rstd = 1.f;
     if (LN) {
       const float inv_k = 1.0f / (float)K;
-      const float md = sd[t] * inv_k;  // mean of x - x0
-      mean = x0[t] + md;
+      md = sd[t] * inv_k;  // mean of x - x0, and the products were of x - x0 as well
       rstd = 1.0f / sqrtf(fmaxf(sq[t] * inv_k - md * md, 0.f) + a.eps);
     }
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       v[i] = acc[t][i];
-      if (LN) v[i] = rstd * (v[i] - mean * cs4[i]);
+      if (LN) v[i] = rstd * (v[i] - md * cs4[i]);
       v[i] += bias4[i];
       if (EPI == SK_EPI_GELU) v[i] = gelu_tanh_fast(v[i]);
       if (EPI == SK_EPI_RESIDUAL) v[i] += old4[t][i];

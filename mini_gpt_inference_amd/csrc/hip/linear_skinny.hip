@@ -66,7 +66,9 @@ __global__ __launch_bounds__(WAVES * 64) void linear_skinny_kernel(SkinnyArgs a)
       const int n = t * 16 + lrow;
       const int src = n < a.n_rows ? (a.rows ? a.rows[n] : n) : 0;
       xrow[t] = a.x + (long)src * K;
-      x0[t] = xrow[t][0];
+      // the shift of a row: the median of three of its values, so that one channel that stands
+      // far out (residual streams have such) does not become the shift
+      x0[t] = __builtin_amdgcn_fmed3f(xrow[t][0], xrow[t][K >> 1], xrow[t][K - 1]);
     }
   }
   auto load_w = [&](bf16x8_t (&dst)[SK_BATCH], int o0, int sb) {
@@ -104,7 +106,9 @@ __global__ __launch_bounds__(WAVES * 64) void linear_skinny_kernel(SkinnyArgs a)
           bf16x8_t v;
 #pragma unroll
           for (int e = 0; e < 8; ++e) {
-            v[e] = (short)float_to_bf16(f[e]);
+            // what is rounded to bfloat16 is the distance from the row's first value: a row far from
+            // zero loses nothing to its offset (the epilogue corrects with the mean of the distances)
+            v[e] = (short)float_to_bf16(f[e] - x0[t]);
             if (ok && stats) {
               const float d = f[e] - x0[t];
               sd[t] += d;
@@ -225,16 +229,15 @@ __global__ __launch_bounds__(WAVES * 64) void linear_skinny_kernel(SkinnyArgs a)
       const int n = t * 16 + lrow;
       if (n >= a.n_rows) continue;
       float v[4];
-      float mean = 0.f, rstd = 1.f;
+      float md = 0.f, rstd = 1.f;
       if (LN) {
-        const float md = sd[t] / (float)K;   // mean of x - x0
-        mean = x0[t] + md;
+        md = sd[t] / (float)K;   // mean of x - x0, and the products were of x - x0 as well
         rstd = 1.0f / sqrtf(fmaxf(sq[t] / (float)K - md * md, 0.f) + a.eps);
       }
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         v[i] = acc[t][i];
-        if (LN && oc + i < a.n_out) v[i] = rstd * (v[i] - mean * a.colsum[oc + i]);
+        if (LN && oc + i < a.n_out) v[i] = rstd * (v[i] - md * a.colsum[oc + i]);
         if (a.bias && oc + i < a.n_out) v[i] += a.bias[oc + i];
         if (EPI == SK_EPI_GELU) v[i] = gelu_tanh_fast(v[i]);
       }

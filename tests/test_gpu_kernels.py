@@ -298,6 +298,27 @@ def test_linear_skinny_through_a_folded_layer_norm(n, k, o, ln_bias, gather, gen
         assert torch.isnan(outs[2][n:]).all(), "rows beyond n_rows were written"
 
 
+@pytest.mark.parametrize("general", [False, True])
+@pytest.mark.parametrize("outlier", [None, 0, 7])
+def test_folded_layer_norm_of_rows_far_from_zero(general, outlier):
+    """Rows whose values lie 50 standard deviations from zero (and one channel further out still, also
+    the first one): what the product rounds to bfloat16 must be the distance from a value of the
+    row, not the value, or the rounding error of the offset drowns the row."""
+    g = torch.Generator().manual_seed(40)
+    n, k, o = 6, 256, 96
+    x = rnd(g, n, k, scale=1.0) + torch.tensor([100.0, -100.0, 50.0, 0.0, 300.0, -75.0])[:, None]
+    if outlier is not None:
+        x[:, outlier] += 400.0
+    lw, lb = 1 + 0.1 * rnd(g, k), rnd(g, k)
+    w, bias = rnd(g, o, k, dtype="bfloat16", scale=k ** -0.5), rnd(g, o)
+    wf, colsum, bias_f = kernels.fold_layer_norm(w.to(DEV), lw.to(DEV), lb.to(DEV), bias.to(DEV))
+    out = torch.empty(n, o, dtype=torch.float32, device=DEV)
+    assert kernels.linear_skinny(None, wf, bias_f, out, n, kernels.EPI_NONE, ln_x=x.to(DEV), ln_colsum=colsum,
+                                 ln_eps=1e-5, general_only=general)
+    h = P.plain_layer_norm(x.double(), lw.double(), lb.double(), 1e-5)
+    helpers.assert_close(out, P.plain_linear(h, w.double(), bias.double()), "bfloat16", "LN of rows far from zero")
+
+
 @pytest.mark.parametrize("general,n,rows_mode,rpg", [(False, 6, 0, 0), (True, 6, 0, 0), (True, 40, 0, 0),
                                                      (False, 40, kernels.ROWS_SHARE_W, 0),
                                                      (False, 40, kernels.ROWS_GROUPS, 0), (False, 64, kernels.ROWS_GROUPS, 0),
