@@ -23,6 +23,35 @@ class CacheError(RuntimeError):
     pass
 
 
+NOMINAL_SPAN = 4096   # tokens a request is taken to hold where the model puts no bound on positions
+
+
+def plan_group_pages(groups, page_size: int, num_blocks: int, kv_cache_bytes, itemsize: int,
+                     max_positions=None) -> List[int]:
+    """Pages of every cache group.  groups: the layout's CacheGroupSpec list (n_kv_head, head_dim,
+    window, n_pools).  Without kv_cache_bytes every group gets num_blocks pages (the one-group
+    shorthand, the reference's num_blocks).  With it the bytes are split so that every group holds
+    the same number of full-length requests: a group's page costs n_pools * 2 * n_kv_head * page_size
+    * head_dim * itemsize bytes, and a full-length request holds its whole span in a group that
+    keeps all keys but only a window (and the page being written) in one that keeps a window."""
+    if kv_cache_bytes is None:
+        return [int(num_blocks)] * len(groups)
+    span_all = int(max_positions) if max_positions else NOMINAL_SPAN
+    page_bytes, pages_per_request = [], []
+    for g in groups:
+        page_bytes.append(g.n_pools * 2 * g.n_kv_head * page_size * g.head_dim * itemsize)
+        span = min(g.window + page_size, span_all) if g.window else span_all
+        pages_per_request.append(-(-span // page_size))
+    per_request = sum(b * n for b, n in zip(page_bytes, pages_per_request))
+    if per_request <= 0:
+        return [1] * len(groups)
+    requests = kv_cache_bytes / per_request
+    if requests < 1.0:
+        raise CacheError(f"kv_cache_bytes = {kv_cache_bytes} does not hold one request of full length "
+                         f"({per_request} bytes over {len(groups)} cache groups)")
+    return [max(n, int(requests * n)) for n in pages_per_request]
+
+
 def _ip(a):
     """The address of an int32 array for the library; an address (int) passes through, which lets a
     caller that fills the same arrays at every step look them up once."""

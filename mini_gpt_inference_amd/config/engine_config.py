@@ -17,7 +17,10 @@ from typing import Optional
 @dataclass
 class EngineConfig:
     block_size: int = 16             # tokens per KV page (the reference's "KV block")
-    num_blocks: int = 2048           # pages in the fixed pool, per cache group
+    num_blocks: int = 2048           # pages in the fixed pool, per cache group (the reference's num_blocks)
+    kv_cache_bytes: Optional[int] = None   # instead of num_blocks: device memory for all cache groups together,
+                                           # split so that every group holds the same number of full-length
+                                           # requests (groups differ in bytes per token and in their window)
     max_batch_size: int = 256        # most requests running at once (= state slots)
     max_num_batched_tokens: int = 4096   # token budget of one step
     prefill_chunk: int = 0           # largest prompt portion per request and step; 0 = no limit
@@ -41,6 +44,8 @@ class EngineConfig:
     def __post_init__(self) -> None:
         if self.block_size <= 0 or self.num_blocks <= 0 or self.max_batch_size <= 0:
             raise ValueError("block_size, num_blocks and max_batch_size must be positive")
+        if self.kv_cache_bytes is not None and self.kv_cache_bytes <= 0:
+            raise ValueError("kv_cache_bytes must be positive")
         if self.max_num_batched_tokens <= 0:
             raise ValueError("max_num_batched_tokens must be positive")
         if self.decode_burst < 1 or self.decode_chain < 1:

@@ -15,7 +15,7 @@ import numpy as np
 import torch
 
 from ..cache.kv_store import KVStore
-from ..cache.manager import CacheManager, GroupGeometry
+from ..cache.manager import CacheManager, GroupGeometry, plan_group_pages
 from ..config.engine_config import EngineConfig, SamplingParams
 from ..ops import kernels
 from ..parts.base import Workspace
@@ -146,8 +146,10 @@ class LLMEngine:
         self.device = torch.device(device)
         self.dtype = _TORCH_DTYPES[engine_config.dtype]
         layout = model.cache_layout
-        geometry = [GroupGeometry(engine_config.block_size, engine_config.num_blocks, g.window)
-                    for g in layout.groups]
+        pages = plan_group_pages(layout.groups, engine_config.block_size, engine_config.num_blocks,
+                                 engine_config.kv_cache_bytes, 2 if self.dtype == torch.bfloat16 else 4,
+                                 model.spec.max_positions)
+        geometry = [GroupGeometry(engine_config.block_size, n, g.window) for g, n in zip(layout.groups, pages)]
         self.cache = CacheManager(geometry, engine_config.max_batch_size)
         self.store = KVStore(layout, geometry, engine_config.max_batch_size, self.dtype, self.device)
         max_positions = model.spec.max_positions

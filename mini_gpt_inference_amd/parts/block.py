@@ -2,6 +2,8 @@
 
 from __future__ import annotations
 
+from typing import Mapping, Optional, Tuple
+
 import torch
 
 from ..ops import residual
@@ -13,10 +15,15 @@ from .positions import PositionEncoding
 
 
 class Arrangement(Part):
-    category = "arrangement"
+    """How a layer's parts sit around the residual stream.  `roles` names the parts it arranges (the
+    model refuses a layer whose parts are others); run() gets them by role, and for every mixer role
+    the binding of this run's cache."""
 
-    def run(self, ctx: StepContext, x: torch.Tensor, norm1: Part, mixer: Mixer, norm2: Part,
-            feed_forward: FeedForward, binding: CacheBinding, position: PositionEncoding) -> None:
+    category = "arrangement"
+    roles: Optional[Tuple[str, ...]] = None     # None: whatever the layer brings
+
+    def run(self, ctx: StepContext, x: torch.Tensor, parts: Mapping[str, Part],
+            bindings: Mapping[str, CacheBinding], position: PositionEncoding) -> None:
         raise NotImplementedError
 
 
@@ -26,11 +33,14 @@ class PreNorm(Arrangement):
 
     graph_safe = True
     takes_pending_residual = True
+    roles = ("norm1", "mixer", "norm2", "feed_forward")
 
     def __init__(self, width: int) -> None:
         self.width = int(width)
 
-    def run(self, ctx, x, norm1, mixer, norm2, feed_forward, binding, position) -> None:
+    def run(self, ctx, x, parts, bindings, position) -> None:
+        norm1, mixer, norm2, feed_forward = (parts[r] for r in self.roles)
+        binding = bindings["mixer"]
         # the norms are handed on uncomputed: a linear layer that can normalise in its prologue
         # does, everything else calls .tensor(ctx) and gets the normed rows.  A part that does not
         # know of a residual whose sums are still pending gets a plain one.

@@ -9,7 +9,7 @@ the same step writes (then it only reads).  A layer may appear in several runs.
 from __future__ import annotations
 
 from dataclasses import dataclass, field
-from typing import Dict, List, Optional, Tuple
+from typing import Dict, List, Mapping, Optional, Tuple
 
 import torch
 
@@ -25,13 +25,41 @@ from .base import (ARRANGEMENTS, CacheBinding, EMBEDDINGS, FEED_FORWARDS, HEADS,
                    POSITIONS, Part, PartSpec, StateNeed, StepContext, WeightRequest)
 
 
-@dataclass(frozen=True)
+# categories of a layer's parts, and the registry of each
+_LAYER_REGISTRIES = {"norm": NORMS, "mixer": MIXERS, "feed_forward": FEED_FORWARDS}
+
+
 class LayerSpec:
-    arrangement: PartSpec
-    norm1: PartSpec
-    mixer: PartSpec
-    norm2: PartSpec
-    feed_forward: PartSpec
+    """A layer: an arrangement and the parts it arranges, each under a role name.
+
+    parts: role -> (category, PartSpec) with category "norm", "mixer" or "feed_forward"; which
+    roles there are is the arrangement's business (a pre-norm block has norm1, mixer, norm2,
+    feed_forward; a block with one norm or two mixers has other roles).  The four roles of the
+    pre-norm block can be given by keyword, or in that order."""
+
+    def __init__(self, arrangement: PartSpec, norm1: Optional[PartSpec] = None, mixer: Optional[PartSpec] = None,
+                 norm2: Optional[PartSpec] = None, feed_forward: Optional[PartSpec] = None, *,
+                 parts: Optional[Mapping[str, Tuple[str, PartSpec]]] = None) -> None:
+        named: Dict[str, Tuple[str, PartSpec]] = {}
+        for role, (category, spec) in (parts or {}).items():
+            if category not in _LAYER_REGISTRIES:
+                raise ValueError(f"part {role!r}: category {category!r} is none of {sorted(_LAYER_REGISTRIES)}")
+            named[role] = (category, spec)
+        for role, category, spec in (("norm1", "norm", norm1), ("mixer", "mixer", mixer), ("norm2", "norm", norm2),
+                                     ("feed_forward", "feed_forward", feed_forward)):
+            if spec is not None:
+                named[role] = (category, spec)
+        self.arrangement = arrangement
+        self.parts = named
+
+    def __getattr__(self, role: str) -> PartSpec:
+        parts = self.__dict__.get("parts", {})
+        if role in parts:
+            return parts[role][1]
+        raise AttributeError(role)
+
+    def roles(self, category: str) -> List[str]:
+        return [role for role, (cat, _) in self.parts.items() if cat == category]
 
 
 @dataclass(frozen=True)
@@ -67,17 +95,27 @@ class CacheGroupSpec:
 @dataclass
 class CacheLayout:
     groups: List[CacheGroupSpec]
-    state_numels: List[int]            # one entry per run that keeps per-request state
-    bindings: List[CacheBinding]       # one per run
+    state_numels: List[int]                        # one entry per (run, mixer) that keeps per-request state
+    run_bindings: List[Dict[str, CacheBinding]]    # per run: mixer role -> where it keeps what it remembers
+
+    @property
+    def bindings(self) -> List[CacheBinding]:
+        """One binding per run, for models whose layers have exactly one mixer each."""
+        return [next(iter(b.values())) if len(b) == 1 else None for b in self.run_bindings]
 
 
-@dataclass
 class _Layer:
-    arrangement: Part
-    norm1: Part
-    mixer: Part
-    norm2: Part
-    feed_forward: Part
+    """The built parts of a layer, by role (also as attributes)."""
+
+    def __init__(self, arrangement: Part, parts: Dict[str, Part]) -> None:
+        self.arrangement = arrangement
+        self.parts = parts
+
+    def __getattr__(self, role: str) -> Part:
+        parts = self.__dict__.get("parts", {})
+        if role in parts:
+            return parts[role]
+        raise AttributeError(role)
 
 
 class DecoderModel:
@@ -85,11 +123,15 @@ class DecoderModel:
         self.spec = spec
         self.embedding = EMBEDDINGS.build(spec.embedding)
         self.position = POSITIONS.build(spec.position)
-        self.layers: List[_Layer] = [
-            _Layer(ARRANGEMENTS.build(ls.arrangement), NORMS.build(ls.norm1), MIXERS.build(ls.mixer),
-                   NORMS.build(ls.norm2), FEED_FORWARDS.build(ls.feed_forward))
-            for ls in spec.layers
-        ]
+        self.layers: List[_Layer] = []
+        for i, ls in enumerate(spec.layers):
+            arrangement = ARRANGEMENTS.build(ls.arrangement)
+            wanted = getattr(arrangement, "roles", None)
+            if wanted is not None and set(wanted) != set(ls.parts):
+                raise ValueError(f"layer {i}: arrangement {ls.arrangement.kind!r} arranges the parts "
+                                 f"{sorted(wanted)}, the layer has {sorted(ls.parts)}")
+            self.layers.append(_Layer(arrangement, {role: _LAYER_REGISTRIES[category].build(part_spec)
+                                                    for role, (category, part_spec) in ls.parts.items()}))
         self.final_norm = NORMS.build(spec.final_norm)
         self.head = HEADS.build(spec.head)
         for i, run in enumerate(spec.order):
@@ -103,8 +145,7 @@ class DecoderModel:
     def _named_parts(self) -> List[Tuple[Part, PartSpec]]:
         pairs = [(self.embedding, self.spec.embedding), (self.position, self.spec.position)]
         for layer, ls in zip(self.layers, self.spec.layers):
-            pairs += [(layer.norm1, ls.norm1), (layer.mixer, ls.mixer), (layer.norm2, ls.norm2),
-                      (layer.feed_forward, ls.feed_forward)]
+            pairs += [(layer.parts[role], part_spec) for role, (_, part_spec) in ls.parts.items()]
         pairs += [(self.final_norm, self.spec.final_norm), (self.head, self.spec.head)]
         return pairs
 
@@ -149,36 +190,42 @@ class DecoderModel:
         groups: List[CacheGroupSpec] = []
         keys: List[Tuple[int, int, int]] = []
         state_numels: List[int] = []
-        bindings: List[CacheBinding] = []
+        run_bindings: List[Dict[str, CacheBinding]] = []
         for i, run in enumerate(self.spec.order):
-            need = self.layers[run.layer].mixer.cache_need()
-            if run.reads_cache_of is not None:
-                src = bindings[run.reads_cache_of]
-                src_need = self.layers[self.spec.order[run.reads_cache_of].layer].mixer.cache_need()
-                if need != src_need or src.kind != "kv":
-                    raise ValueError(f"run {i} cannot read the cache of run {run.reads_cache_of}: different needs")
-                bindings.append(CacheBinding("kv", src.group, src.index, writes=False))
-            elif isinstance(need, KVNeed):
-                key = (need.n_kv_head, need.head_dim, need.window)
-                if key not in keys:
-                    keys.append(key)
-                    groups.append(CacheGroupSpec(need.n_kv_head, need.head_dim, need.window, 0))
-                g = keys.index(key)
-                bindings.append(CacheBinding("kv", g, groups[g].n_pools, writes=True))
-                groups[g] = CacheGroupSpec(*key, groups[g].n_pools + 1)
-            elif isinstance(need, StateNeed):
-                bindings.append(CacheBinding("state", -1, len(state_numels), writes=True))
-                state_numels.append(int(need.numel))
-            else:
-                bindings.append(CacheBinding("none"))
-        return CacheLayout(groups, state_numels, bindings)
+            layer, layer_spec = self.layers[run.layer], self.spec.layers[run.layer]
+            bindings: Dict[str, CacheBinding] = {}
+            for role in layer_spec.roles("mixer"):
+                need = layer.parts[role].cache_need()
+                if run.reads_cache_of is not None:
+                    src_run = self.spec.order[run.reads_cache_of]
+                    src = run_bindings[run.reads_cache_of].get(role)
+                    src_need = (self.layers[src_run.layer].parts[role].cache_need()
+                                if role in self.layers[src_run.layer].parts else None)
+                    if src is None or need != src_need or src.kind != "kv":
+                        raise ValueError(f"run {i} cannot read the cache of run {run.reads_cache_of}: different needs")
+                    bindings[role] = CacheBinding("kv", src.group, src.index, writes=False)
+                elif isinstance(need, KVNeed):
+                    key = (need.n_kv_head, need.head_dim, need.window)
+                    if key not in keys:
+                        keys.append(key)
+                        groups.append(CacheGroupSpec(need.n_kv_head, need.head_dim, need.window, 0))
+                    g = keys.index(key)
+                    bindings[role] = CacheBinding("kv", g, groups[g].n_pools, writes=True)
+                    groups[g] = CacheGroupSpec(*key, groups[g].n_pools + 1)
+                elif isinstance(need, StateNeed):
+                    bindings[role] = CacheBinding("state", -1, len(state_numels), writes=True)
+                    state_numels.append(int(need.numel))
+                else:
+                    bindings[role] = CacheBinding("none")
+            run_bindings.append(bindings)
+        return CacheLayout(groups, state_numels, run_bindings)
 
     @property
     def graph_safe(self) -> bool:
         """Whether every part of the model allows a step to be captured in a HIP graph (Part.graph_safe)."""
         parts = [self.embedding, self.position, self.final_norm, self.head]
         for layer in self.layers:
-            parts += [layer.arrangement, layer.norm1, layer.mixer, layer.norm2, layer.feed_forward]
+            parts += [layer.arrangement, *layer.parts.values()]
         return all(getattr(p, "graph_safe", False) for p in parts if p is not None)
 
     # ------------------------------------------------------------------ forward
@@ -191,12 +238,11 @@ class DecoderModel:
         x = ws.get("residual", n, self.spec.width, torch.float32)
         ctx.pending = None
         self.embedding.forward(ctx, self.position, x)
-        for run, binding in zip(self.spec.order, self.cache_layout.bindings):
+        for run, bindings in zip(self.spec.order, self.cache_layout.run_bindings):
             layer = self.layers[run.layer]
             if not layer.arrangement.takes_pending_residual:
                 residual.settle(ctx, x, n)
-            layer.arrangement.run(ctx, x, layer.norm1, layer.mixer, layer.norm2, layer.feed_forward, binding,
-                                  self.position)
+            layer.arrangement.run(ctx, x, layer.parts, bindings, self.position)
         m = ctx.m_rows
         # rows start 16 bytes apart at least: the sampling kernel then reads them four floats at a time
         # whatever the vocabulary's size (50257 is odd)

@@ -147,3 +147,24 @@ def test_random_orders_of_requests_lose_no_page():
         cm.free_slot(s)
     assert cm.num_free_pages(0) == 64 and cm.num_free_pages(1) == 64 and cm.num_free_slots == 6
     assert cm.check() == 0
+
+
+def test_cache_groups_are_sized_by_bytes_so_that_each_holds_the_same_requests():
+    """kv_cache_bytes is split over the groups by what a full-length request costs in each: a group
+    with a window needs few pages per request, one with more heads costs more per page."""
+    from types import SimpleNamespace as G
+    from mini_gpt_inference_amd.cache.manager import CacheError, plan_group_pages
+    full = G(n_kv_head=8, head_dim=64, window=0, n_pools=6)
+    windowed = G(n_kv_head=2, head_dim=64, window=128, n_pools=2)
+    assert plan_group_pages([full, windowed], 16, 777, None, 2, 1024) == [777, 777]       # the shorthand
+    page_full, page_win = 6 * 2 * 8 * 16 * 64 * 2, 2 * 2 * 2 * 16 * 64 * 2
+    per_request = 64 * page_full + 9 * page_win         # 1024 / 16 pages, and (128 + 16) / 16
+    pages = plan_group_pages([full, windowed], 16, 777, 10 * per_request + 5, 2, 1024)
+    assert pages == [640, 90]
+    assert pages[0] * page_full + pages[1] * page_win <= 10 * per_request + 5
+    one = plan_group_pages([full], 16, 1, 3 * 64 * page_full, 2, 1024)
+    assert one == [192]
+    assert plan_group_pages([full], 16, 1, 2 * 256 * (page_full * 2), 4, None) == [512]    # no bound on positions: 4096 tokens
+    import pytest
+    with pytest.raises(CacheError, match="does not hold one request"):
+        plan_group_pages([full, windowed], 16, 1, per_request - 1, 2, 1024)

@@ -189,6 +189,7 @@ def test_cache_layout_groups_runs_by_what_their_mixers_keep():
     layout = DecoderModel(_spec(ORDER)).cache_layout
     assert [(g.n_kv_head, g.window, g.n_pools) for g in layout.groups] == [(HK, WINDOW, 2), (H, 0, 1)]
     assert layout.state_numels == [C]
+    assert all(sorted(b) == ["mixer"] for b in layout.run_bindings)       # one mixer a layer: one binding a run
     kinds = [(b.kind, b.group, b.index, b.writes) for b in layout.bindings]
     assert kinds == [("kv", 0, 0, True), ("state", -1, 0, True), ("kv", 1, 0, True), ("kv", 0, 1, True),
                      ("kv", 1, 0, False)]
@@ -589,3 +590,100 @@ def test_toy_rotation_decodes_from_graphs(dtype):
             margin = 2 * helpers.TOL[dtype] * max(1.0, np.abs(logits).max())
             assert logits[tok] >= logits.max() - margin
             ids.append(tok)
+
+
+# ----------------------------------------------------------------------------- a toy arrangement
+from mini_gpt_inference_amd.parts.base import register_arrangement      # noqa: E402
+from mini_gpt_inference_amd.parts.block import Arrangement              # noqa: E402
+
+
+@register_arrangement("toy_parallel")
+class ToyParallel(Arrangement):
+    """x = x + attention(h) + state_mixer(h) + ff(h) with h = norm(x): one norm, and two mixers beside
+    the feed-forward, all reading the same normed rows.  Defined here and registered without a change
+    to the framework: a layer is a map of roles to parts, and this arrangement names other roles than
+    the pre-norm block does."""
+
+    roles = ("norm", "attention", "memory", "feed_forward")
+
+    def __init__(self, width: int) -> None:
+        self.width = int(width)
+
+    def run(self, ctx, x, parts, bindings, position) -> None:
+        h = as_tensor(ctx, LazyNorm(parts["norm"], x, ctx.n_rows)).clone()      # every branch reads the rows as they were
+        parts["attention"].forward_add(ctx, h, x, bindings["attention"], position)
+        parts["memory"].forward_add(ctx, h, x, bindings["memory"], position)
+        parts["feed_forward"].forward_add(ctx, h, x)
+
+
+def _parallel_spec():
+    a0, a1 = (_attn_layer(i, C, H, H, D, 0, 1 / math.sqrt(D), HID, EPS) for i in (0, 1))
+    parallel = LayerSpec(PartSpec("toy_parallel", {"width": C}),
+                         parts={"norm": ("norm", a1.norm1), "attention": ("mixer", a1.mixer),
+                                "memory": ("mixer", PartSpec("toy_decay", {"width": C, "decay": 0.25},
+                                                             {"mix_weight": "L1.mix.w"})),
+                                "feed_forward": ("feed_forward", a1.feed_forward)})
+    return ModelSpec(width=C, vocab_size=V,
+                     embedding=PartSpec("token_embedding", {"vocab_size": V, "width": C}, {"weight": "emb.w"}),
+                     position=PartSpec("learned_absolute", {"max_positions": 50, "width": C}, {"weight": "pos.w"}),
+                     layers=(a0, parallel), order=(LayerRun(0), LayerRun(1), LayerRun(0), LayerRun(1)),
+                     final_norm=_norm("nf.", C, EPS),
+                     head=PartSpec("linear_head", {"vocab_size": V, "width": C, "tied": True}, {"weight": "emb.w"}),
+                     max_positions=50)
+
+
+def _plain_parallel_model(w, ids):
+    x = P.plain_embed(torch.tensor(ids), w["emb.w"].double(), w["pos.w"].double())
+    for layer in (0, 1, 0, 1):
+        p = f"L{layer}."
+        h = _pl_norm(x, w, p + "n1.", EPS)
+        a, _ = _pl_attn(h, w, p, H, H, 1 / math.sqrt(D), 0)
+        if layer == 0:
+            x = x + a
+            x = x + _pl_mlp(_pl_norm(x, w, p + "n2.", EPS), w, p)
+        else:
+            x = x + a + plain_toy(h, w[p + "mix.w"].double(), 0.25) + _pl_mlp(h, w, p)
+    return _pl_norm(x, w, "nf.", EPS) @ w["emb.w"].double().t()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_toy_arrangement_with_one_norm_and_two_mixers(dtype):
+    """A parallel block registered by the test: its layer has the roles norm / attention / memory /
+    feed_forward, the model gives each of its two mixers a cache of its own in every run (pages for
+    one, a state slot for the other), and steps cut anywhere give the plain model's logits."""
+    model = DecoderModel(_parallel_spec())
+    layout = model.cache_layout
+    assert [sorted(b) for b in layout.run_bindings] == [["mixer"], ["attention", "memory"]] * 2
+    assert [g.n_pools for g in layout.groups] == [4] and layout.state_numels == [C, C]
+    assert [layout.run_bindings[i]["memory"].index for i in (1, 3)] == [0, 1]
+    assert not model.graph_safe                              # the toy parts make no such promise
+    with pytest.raises(ValueError, match="arranges the parts"):
+        DecoderModel(ModelSpec(**{**_parallel_spec().__dict__, "layers": (
+            LayerSpec(PartSpec("toy_parallel", {"width": C}), norm1=_norm("L0.n1.", C, EPS)),)}))
+    weights = _random_weights(model, 21)
+    _bind(model, weights, dtype)
+    rng = np.random.default_rng(4)
+    reqs = [rng.integers(0, V, n).tolist() for n in (19, 33)]
+    want = [_plain_parallel_model(weights, ids).numpy() for ids in reqs]
+    runner, cache = _runner(model, dtype)
+    slots = [cache.acquire_slot() for _ in reqs]
+    done = [0, 0]
+    got = [[], []]
+    sizes = [[6, 1, 1, 4, 1, 2, 9], [11, 1, 7, 1, 1, 20]]
+    step = 0
+    while any(d < len(r) for d, r in zip(done, reqs)):
+        batch = [(i, min(sizes[i][step % len(sizes[i])], len(reqs[i]) - done[i])) for i in range(2)
+                 if done[i] < len(reqs[i])]
+        step += 1
+        for i, q in batch:
+            assert cache.reserve(slots[i], done[i] + q)
+        toks = sum((reqs[i][done[i]:done[i] + q] for i, q in batch), [])
+        out = runner.step([slots[i] for i, _ in batch], [done[i] for i, _ in batch], [q for _, q in batch], toks,
+                          list(range(len(toks))))
+        o = 0
+        for i, q in batch:
+            got[i].append(out[o:o + q].cpu())
+            o += q
+            done[i] += q
+    for i in range(2):
+        helpers.assert_close(torch.cat(got[i]), want[i], dtype, f"parallel block, request {i}")
