@@ -212,6 +212,71 @@ def serve_run(args, name):
             "prompt_tokens_computed": stats["num_prompt_tokens"], "dtype": args.dtype, "weights": "random"}
 
 
+def host_cost_run(args):
+    """What the host pays to launch one mixed step of the GPT-2-small shape (eight single tokens
+    beside a prompt portion of 300, no HIP graph): through the model's Python, and from the plan
+    recorded at the shape's first coming (one call into the kernel library).  Host time is the time
+    until the launching call returns; the device is idle before each."""
+    import numpy as np
+    import torch
+
+    from mini_gpt_inference_amd import EngineConfig, GPTConfig
+    from mini_gpt_inference_amd.engine.llm_engine import LLMEngine
+    from mini_gpt_inference_amd.ops import kernels
+
+    w = WORKLOADS["small-mixed"]
+    layers = args.workload_layers or w["layers"]
+    cfg = GPTConfig("gpt2-mini", n_layer=layers, n_embd=w["width"], n_head=w["heads"], vocab_size=w["vocab"],
+                    block_size=w["positions"], bias=True, layer_norm_eps=1e-5)
+    engine = LLMEngine.from_random(cfg, seed=0, engine_config=EngineConfig(
+        block_size=args.kv_block, num_blocks=1024, max_batch_size=16, dtype=args.dtype, use_graph=False))
+    runner, cache = engine.runner, engine.cache
+    rng = np.random.default_rng(3)
+    q_lens = [1] * 8 + [300]
+    ctx_lens = [int(c) for c in rng.integers(20, 200, 8)] + [212]
+    slots = [cache.acquire_slot() for _ in q_lens]
+    for s, c, q in zip(slots, ctx_lens, q_lens):
+        assert cache.reserve(s, c + q)
+    tokens = rng.integers(0, cfg.vocab_size, sum(q_lens)).astype(np.int32)
+    rows = list(range(8)) + [sum(q_lens) - 1]
+
+    def one(plans):
+        runner.plan_steps = plans
+        torch.cuda.synchronize()
+        before, t0 = kernels.launches, time.perf_counter()
+        runner.step(slots, ctx_lens, q_lens, tokens, rows)
+        host = time.perf_counter() - t0
+        torch.cuda.synchronize()
+        return host, kernels.launches - before, time.perf_counter() - t0
+
+    one(True)                                   # first coming: buffers made, matrices packed, the plan recorded
+    one(True)
+    python_runs = [one(False) for _ in range(args.host_cost_reps)]
+    planned_before = runner.num_planned_steps
+    plan_runs = [one(True) for _ in range(args.host_cost_reps)]
+    assert runner.num_planned_steps - planned_before == args.host_cost_reps, "the steps did not come from the plan"
+    med = lambda runs, i: sorted(r[i] for r in runs)[len(runs) // 2]
+    n_kernels = plan_runs[0][1]      # launcher calls (one whose product is split along k is two kernels)
+    # the launches alone, without describing the step and uploading its arrays
+    plan = runner._entry((tuple(q_lens), len(rows))).plan
+    alone = []
+    for _ in range(args.host_cost_reps):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        plan.run()
+        alone.append(time.perf_counter() - t0)
+    torch.cuda.synchronize()
+    alone_us = sorted(alone)[len(alone) // 2] * 1e6
+    return {"workload": "host cost of an eager mixed step", "n_layer": cfg.n_layer, "n_embd": cfg.n_embd,
+            "tokens": int(sum(q_lens)), "requests": len(q_lens), "kernels": n_kernels, "dtype": args.dtype,
+            "python_host_us": round(med(python_runs, 0) * 1e6, 1),
+            "python_host_us_per_kernel": round(med(python_runs, 0) * 1e6 / n_kernels, 2),
+            "plan_host_us": round(med(plan_runs, 0) * 1e6, 1),
+            "plan_host_us_per_kernel": round(med(plan_runs, 0) * 1e6 / n_kernels, 2),
+            "plan_launches_alone_us": round(alone_us, 1), "plan_launches_alone_us_per_kernel": round(alone_us / n_kernels, 2),
+            "python_step_us": round(med(python_runs, 2) * 1e6, 1), "plan_step_us": round(med(plan_runs, 2) * 1e6, 1)}
+
+
 def main() -> int:
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
     ap.add_argument("--gpus", type=int, default=1)
@@ -238,6 +303,10 @@ def main() -> int:
                     help="--workload: leave the decode graphs to be captured inside the timed run")
     ap.add_argument("--workload-layers", type=int, default=0, help="fewer layers for --workload (0 = the shape's)")
     ap.add_argument("--workload-requests", type=int, default=0, help="fewer requests for --workload")
+    ap.add_argument("--host-step-cost", action="store_true",
+                    help="instead of the decode measurement: the host's time to launch an eager mixed step of the "
+                         "GPT-2-small shape, through the model's Python and from its recorded plan")
+    ap.add_argument("--host-cost-reps", type=int, default=15)
     ap.add_argument("--report", default=None,
                     help="also write a JSON file with the raw timing samples, their median and quartiles, the "
                          "commit and the software and device that ran them")
@@ -250,6 +319,9 @@ def main() -> int:
 
     if args.prefill_only:
         print(json.dumps({"prefill": prefill_run(args, args.dtype, reps=10)}))
+        return 0
+    if args.host_step_cost:
+        print(json.dumps(host_cost_run(args)))
         return 0
     if args.workload:
         print(json.dumps(serve_run(args, args.workload)))

@@ -14,6 +14,7 @@
 // partial results (max, sum, weighted values) are merged through LDS in wave order.
 // Slots outside the visible range are never loaded.
 #include "common.h"
+#include "launchers.h"
 
 #define AD_WAVES 4
 #define AD_MAX_DPL 4  // head_dim <= 256

@@ -22,6 +22,7 @@
 //  * the waves' partial results (maximum, sum, weighted values per key subgroup) are merged
 //    through LDS once, in a fixed order.
 #include "common.h"
+#include "launchers.h"
 
 #define AW_WAVES 8
 

@@ -17,6 +17,7 @@
 // tokens were cut into steps or what else is in the batch.  Slots outside
 // [begin, end) are never loaded.
 #include "common.h"
+#include "launchers.h"
 
 template <typename T>
 __global__ void kv_write_kernel(const T* __restrict__ qkv, long ld, int k_off, int v_off,

@@ -23,6 +23,7 @@
 // log2 e), the maximum over the four lanes that share a query goes through two lane swaps
 // instead of LDS, and the row sum stays split over those lanes until the end.
 #include "common.h"
+#include "launchers.h"
 
 typedef __attribute__((__vector_size__(8 * sizeof(short)))) short bf16x8_t;
 typedef __attribute__((__vector_size__(4 * sizeof(short)))) short bf16x4_t;

@@ -5,6 +5,7 @@
 // LayerNorm: y = (x - mean) / sqrt(var_biased + eps) * w (+ b) over the last dim
 //            (reference: nn.LayerNorm at src/minigpt_infer/model.py:107,109,127)
 #include "common.h"
+#include "launchers.h"
 
 template <typename WT>
 __global__ void embed_kernel(const int* __restrict__ ids, const int* __restrict__ pos,

@@ -8,6 +8,7 @@
 // LayerNorm as in src/minigpt_infer/model.py:107,109,127; the linear layers that read it:
 // model.py:43,96,128.
 #include "common.h"
+#include "launchers.h"
 
 __global__ void fold_layernorm_kernel(const bf16_t* __restrict__ w, const float* __restrict__ gain,
                                       const float* __restrict__ beta, const float* __restrict__ bias,

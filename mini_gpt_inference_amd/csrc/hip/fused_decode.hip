@@ -18,6 +18,7 @@
 // issued first, the sums of the residual and the LayerNorm happen while they are on their way.
 // Sums are added in a fixed order, so results do not depend on timing.
 #include "fused_decode.h"
+#include "launchers.h"
 
 typedef __attribute__((ext_vector_type(2))) __bf16 fd_bf16x2_t;
 

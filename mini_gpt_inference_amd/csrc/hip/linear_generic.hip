@@ -8,6 +8,7 @@
 // the launch.  The bfloat16 serving path uses it only for shapes the MFMA
 // kernels refuse.
 #include "common.h"
+#include "launchers.h"
 
 #define EPI_NONE 0
 #define EPI_GELU 1

@@ -27,6 +27,7 @@
 // of its own) form a block of a few row tiles by a few column tiles, whose operands that L2 holds.
 #include "common.h"
 #include <type_traits>
+#include "launchers.h"
 
 typedef __attribute__((__vector_size__(8 * sizeof(short)))) short bf16x8_t;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4_t;

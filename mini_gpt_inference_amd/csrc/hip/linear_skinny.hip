@@ -24,6 +24,7 @@
 #include "linear_skinny.h"
 
 #include <mutex>
+#include "launchers.h"
 
 __device__ __forceinline__ bf16x8_t load8(const bf16_t* p) {
   return *reinterpret_cast<const bf16x8_t*>(p);

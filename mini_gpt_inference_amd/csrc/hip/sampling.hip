@@ -13,6 +13,7 @@
 // pure function of (engine seed, request seed, index of the output token), so a
 // request's tokens do not depend on batching or preemption.
 #include "common.h"
+#include "launchers.h"
 
 #define SAMPLE_THREADS 1024
 #define SAMPLE_WAVES (SAMPLE_THREADS / MGPT_WAVE)

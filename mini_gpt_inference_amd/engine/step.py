@@ -18,7 +18,8 @@ import torch
 
 from ..cache.kv_store import KVStore
 from ..cache.manager import CacheManager
-from ..ops import kernels
+from ..ops import kernels, library
+from ..ops.plan import LaunchPlan
 from ..parts.base import GroupView, StepContext, Workspace, WorkspaceFrozen
 from ..parts.model import DecoderModel
 
@@ -130,22 +131,28 @@ class StepShape:
 
 @dataclass
 class _StepGraph:
-    """A step shape seen before: how often, and once captured the graph with what it is bound to."""
+    """A step shape seen before: how often; its launches as a plan (recorded when it first came) and,
+    once captured, the graph; each with the arena and the state of the workspace it is bound to."""
     seen: int = 0
     graph: Optional[torch.cuda.CUDAGraph] = None
     arena: Optional[StepArena] = None
     generation: int = -1
     logits: Optional[torch.Tensor] = None
+    plan: Optional[LaunchPlan] = None
+    plan_arena: Optional[StepArena] = None
+    plan_generation: int = -1
+    plan_logits: Optional[torch.Tensor] = None
 
 
 class ModelRunner:
     """Owns the device side of stepping: arenas, workspace, the cache's pools, the model.
 
-    Steps run eagerly, one launch per kernel from Python; for a model whose parts all allow it
-    (Part.graph_safe) a step shape that keeps coming is replayed from a HIP graph captured at its
-    third coming, since the host's launches, not the kernels, bound a step of a few hundred
-    tokens.  A shape is the tuple of the requests' token counts and the number of logit rows;
-    everything else a kernel reads comes from the arena's device arrays."""
+    A step's first coming runs the model's Python, one launch per kernel (about 10 us of host time
+    each), and for a model whose parts all allow it (Part.graph_safe) records the launches; the
+    second coming of the shape makes them from C++ (ops.plan.LaunchPlan), the third captures them in
+    a HIP graph that every later one replays, since the host's launches, not the kernels, bound a
+    step of a few hundred tokens.  A shape is the tuple of the requests' token counts and the number
+    of logit rows; everything else a kernel reads comes from the arena's device arrays."""
 
     MAX_STEP_GRAPHS = 64
     CAPTURE_AT = 3     # a shape is captured when it comes for the third time (capturing costs a step's launches again)
@@ -159,6 +166,8 @@ class ModelRunner:
         self.vocab_size = model.spec.vocab_size
         self.workspace = Workspace(device)
         self.graph_steps = graph_steps and device.type == "cuda" and model.graph_safe
+        self.plan_steps = device.type == "cuda" and model.plan_safe      # launches recorded and made again from C++
+        self.num_planned_steps = 0        # steps whose launches came from a recorded plan
         self._step_graphs: Dict[Tuple, _StepGraph] = {}     # by exact shape; emptied when it has MAX_STEP_GRAPHS
         self._bucket_graphs: Dict[Tuple, _StepGraph] = {}   # by capacities: as many as there are buckets
         self.num_replayed_steps = 0
@@ -270,10 +279,12 @@ class ModelRunner:
         single-token requests may take), padded to those, which serves every step of the bucket
         whatever its requests bring."""
         arena.upload()
-        if not self.graph_steps:
+        if not self.plan_steps and not self.graph_steps:
             with kernels.pinned_stream():
                 return self.model.forward(self.context(arena, shape, padded=False))
         exact = self._entry((tuple(shape.q_lens), shape.n_logits))
+        if not self.graph_steps:
+            return self._planned_or_recorded(exact, arena, shape)
         if self._live(exact, arena):
             exact.graph.replay()
             self.num_replayed_steps += 1
@@ -289,12 +300,31 @@ class ModelRunner:
             bucket.graph.replay()
             self.num_replayed_steps += 1
             return bucket.logits[:shape.n_logits]
-        with kernels.pinned_stream():
-            logits = self.model.forward(self.context(arena, shape, padded=False))
+        logits = self._planned_or_recorded(exact, arena, shape)
         if exact.seen >= self.CAPTURE_AT:
             self._capture(exact, arena, shape, None)
         elif bucket.seen >= self.CAPTURE_AT and not self._live(bucket, arena):
             self._capture(bucket, arena, shape, lead_cap)
+        return logits
+
+    def _plan_live(self, entry: _StepGraph, arena: StepArena) -> bool:
+        return (entry.plan is not None and entry.plan_arena is arena
+                and entry.plan_generation == self.workspace.generation)
+
+    def _planned_or_recorded(self, entry: _StepGraph, arena: StepArena, shape: StepShape) -> torch.Tensor:
+        """The step's own rows, eagerly: from the shape's recorded plan if it has a valid one, else
+        through the model's Python, which records the plan."""
+        with kernels.pinned_stream():
+            if not self.plan_steps:
+                return self.model.forward(self.context(arena, shape, padded=False))
+            if self._plan_live(entry, arena):
+                entry.plan.run()
+                self.num_planned_steps += 1
+                return entry.plan_logits
+            with library.record() as launches:
+                logits = self.model.forward(self.context(arena, shape, padded=False))
+        entry.plan, entry.plan_arena = LaunchPlan(launches), arena
+        entry.plan_generation, entry.plan_logits = self.workspace.generation, logits
         return logits
 
     def _entry(self, key: Tuple) -> _StepGraph:
@@ -314,8 +344,11 @@ class ModelRunner:
         bucket.  A bucket's graph runs over more rows than the eager step before it did, so it runs
         once eagerly first: every buffer it needs exists then."""
         def forward():
-            ctx = self.context(arena, shape, padded=lead_cap is not None, lead_cap=lead_cap)
             with kernels.pinned_stream():
+                if lead_cap is None and self._plan_live(entry, arena):
+                    entry.plan.run()       # the same launches, without the model's Python
+                    return entry.plan_logits
+                ctx = self.context(arena, shape, padded=lead_cap is not None, lead_cap=lead_cap)
                 return self.model.forward(ctx)
         entry.graph = None
         self.num_graph_captures += 1

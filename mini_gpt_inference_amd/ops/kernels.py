@@ -279,8 +279,9 @@ def fold_layer_norm(w: torch.Tensor, gain: torch.Tensor, beta: Optional[torch.Te
     w_out = torch.empty_like(w)
     colsum = torch.empty(n_out, dtype=torch.float32, device=w.device)
     bias_out = torch.empty(n_out, dtype=torch.float32, device=w.device)
-    rc = library.kernels().mgpt_fold_layernorm(_ptr(w), _ptr(gain), _ptr(beta), _ptr(bias), _ptr(w_out),
-                                               _ptr(colsum), _ptr(bias_out), n_out, k_dim, _stream())
+    with library.unrecorded():
+        rc = library.kernels().mgpt_fold_layernorm(_ptr(w), _ptr(gain), _ptr(beta), _ptr(bias), _ptr(w_out),
+                                                   _ptr(colsum), _ptr(bias_out), n_out, k_dim, _stream())
     _check(rc, "fold_layer_norm")
     return w_out, colsum, bias_out
 
@@ -372,7 +373,8 @@ def pack_weight(w: torch.Tensor) -> Optional[torch.Tensor]:
     if k_dim % 32 != 0 or w.data_ptr() % 16 != 0:
         return None
     packed = torch.empty(-(-n_out // 16) * 16 * k_dim, dtype=torch.bfloat16, device=w.device)
-    _check(library.kernels().mgpt_pack_weight(_ptr(w), _ptr(packed), n_out, k_dim, _stream()), "pack_weight")
+    with library.unrecorded():
+        _check(library.kernels().mgpt_pack_weight(_ptr(w), _ptr(packed), n_out, k_dim, _stream()), "pack_weight")
     return packed
 
 

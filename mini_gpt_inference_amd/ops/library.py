@@ -14,6 +14,7 @@ from ..csrc import build as _build
 
 _kernels = None
 _host = None
+_recording = None      # a list that collects (launcher name, arguments) of every launch, or None
 
 
 class NativeLibraryError(RuntimeError):
@@ -46,8 +47,74 @@ def kernels() -> ctypes.CDLL:
                      "mgpt_paged_attention_generic", "mgpt_sample", "mgpt_sample_advance"):
             getattr(lib, name).restype = I
         _declare_optional(lib)
-        _kernels = lib
+        lib.mgpt_plan_create.restype = c_void_p
+        lib.mgpt_plan_create.argtypes = []
+        lib.mgpt_plan_destroy.restype = None
+        lib.mgpt_plan_destroy.argtypes = [c_void_p]
+        lib.mgpt_plan_size.argtypes = [c_void_p]
+        lib.mgpt_plan_add.argtypes = [c_void_p, c_char_p, POINTER(c_ulonglong), c_int]
+        lib.mgpt_plan_run.argtypes = [c_void_p, c_void_p, POINTER(c_int)]
+        for name in ("mgpt_plan_size", "mgpt_plan_add", "mgpt_plan_run"):
+            getattr(lib, name).restype = c_int
+        _kernels = _Recording(lib)
     return _kernels
+
+
+class _Recording:
+    """The kernel library with its launchers wrapped: while a recording is on (record()), every
+    launch that was made (return code 0) is noted with its arguments, for ops.plan.LaunchPlan."""
+
+    def __init__(self, lib: ctypes.CDLL) -> None:
+        self._lib = lib
+
+    def __getattr__(self, name: str):
+        fn = getattr(self._lib, name)
+        argtypes = getattr(fn, "argtypes", None)
+        # launchers take the stream last; everything else (queries, the plan's own calls) passes through
+        if not name.startswith("mgpt_") or name.startswith("mgpt_plan_") or not argtypes or argtypes[-1] is not c_void_p \
+                or fn.restype is not c_int:
+            setattr(self, name, fn)
+            return fn
+
+        def launch(*args):
+            rc = fn(*args)
+            if _recording is not None and rc == 0:
+                _recording.append((name, argtypes, args))
+            return rc
+
+        setattr(self, name, launch)
+        return launch
+
+
+class unrecorded:
+    """Launches inside the block are not noted: work done once (a matrix packed or folded at its
+    first use) is no part of a step's plan."""
+
+    def __enter__(self):
+        global _recording
+        self._outer = _recording
+        _recording = None
+
+    def __exit__(self, *exc):
+        global _recording
+        _recording = self._outer
+        return False
+
+
+class record:
+    """with record() as launches: ... collects (launcher, argtypes, arguments) of every launch made
+    inside the block."""
+
+    def __enter__(self):
+        global _recording
+        self._outer = _recording
+        _recording = []
+        return _recording
+
+    def __exit__(self, *exc):
+        global _recording
+        _recording = self._outer
+        return False
 
 
 def _declare_optional(lib: ctypes.CDLL) -> None:

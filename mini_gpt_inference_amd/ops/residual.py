@@ -23,8 +23,9 @@ from . import kernels
 
 # most rows of a decode-only step that go through the fused kernels (one workgroup per token and
 # head re-reads the head's weights from the L2: beyond this the kernels that share a matrix
-# among the rows are faster)
-FUSED_MAX_ROWS = 16
+# among the rows are faster; the 50.9M model's step takes 184 us against 203 at 32 rows, 282
+# against 256 at 48)
+FUSED_MAX_ROWS = 32
 
 
 @dataclass

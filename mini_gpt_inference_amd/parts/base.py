@@ -57,6 +57,10 @@ class Part:
     # graph and replayed.  A part that looks at ctx.host_ctx_lens or ctx.host_state_slots, or that
     # allocates, is not.
     graph_safe = False
+    # True if, beyond graph_safe, forward() computes through the kernel library's launchers only
+    # (ops.kernels), with no operator of the tensor library: then a step's launches can be recorded
+    # once and made again from C++ (ops.plan.LaunchPlan), which sees no other work than theirs.
+    plan_safe = False
     # True if the part reads the residual stream through ops.residual (it takes sums that are still
     # pending, or settles them itself); every other part is handed a plain residual stream
     takes_pending_residual = False

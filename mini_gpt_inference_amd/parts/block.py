@@ -32,6 +32,8 @@ class PreNorm(Arrangement):
     """x = x + mixer(norm1(x)); x = x + ff(norm2(x)) (reference: src/minigpt_infer/model.py:112-115)."""
 
     graph_safe = True
+
+    plan_safe = True
     takes_pending_residual = True
     roles = ("norm1", "mixer", "norm2", "feed_forward")
 

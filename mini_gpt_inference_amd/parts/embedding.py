@@ -19,6 +19,8 @@ class TokenEmbedding(Part):
 
     graph_safe = True
 
+    plan_safe = True
+
     category = "embedding"
 
     def __init__(self, vocab_size: int, width: int) -> None:
@@ -46,6 +48,8 @@ class LinearHead(Part):
     (src/minigpt_infer/model.py:129-130)."""
 
     graph_safe = True
+
+    plan_safe = True
 
     category = "head"
 

@@ -28,6 +28,8 @@ class DenseMLP(FeedForward):
     a parameter)."""
 
     graph_safe = True
+
+    plan_safe = True
     takes_pending_residual = True
 
     def __init__(self, width: int, hidden: int, bias: bool, activation: str = "gelu_tanh") -> None:

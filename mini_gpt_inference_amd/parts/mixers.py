@@ -41,6 +41,8 @@ class PagedCausalAttention(Mixer):
     head-major; out = y Wproj^T (+ b) (model.py:89-90), added into the residual (model.py:113)."""
 
     graph_safe = True
+
+    plan_safe = True
     takes_pending_residual = True
 
     def __init__(self, width: int, n_head: int, head_dim: int, bias: bool, n_kv_head: Optional[int] = None,

@@ -228,6 +228,14 @@ class DecoderModel:
             parts += [layer.arrangement, *layer.parts.values()]
         return all(getattr(p, "graph_safe", False) for p in parts if p is not None)
 
+    @property
+    def plan_safe(self) -> bool:
+        """Whether every part of the model computes through the kernel library only (Part.plan_safe)."""
+        parts = [self.embedding, self.position, self.final_norm, self.head]
+        for layer in self.layers:
+            parts += [layer.arrangement, *layer.parts.values()]
+        return self.graph_safe and all(getattr(p, "plan_safe", False) for p in parts if p is not None)
+
     # ------------------------------------------------------------------ forward
     def forward(self, ctx: StepContext) -> torch.Tensor:
         """Runs the step's tokens through every run of the order and returns float32 logits

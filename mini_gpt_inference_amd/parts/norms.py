@@ -18,6 +18,8 @@ class LayerNorm(Part):
 
     graph_safe = True
 
+    plan_safe = True
+
     category = "norm"
     fusable_layer_norm = True   # a linear kernel may fold weight and bias into its matrix and apply mean, rstd itself
 

@@ -35,6 +35,8 @@ class LearnedAbsolutePositions(PositionEncoding):
 
     graph_safe = True
 
+    plan_safe = True
+
     def __init__(self, max_positions: int, width: int) -> None:
         self.max_positions, self.width = int(max_positions), int(width)
         self.weight: Optional[torch.Tensor] = None
@@ -51,6 +53,8 @@ class NoPositions(PositionEncoding):
     """No position signal at all."""
 
     graph_safe = True
+
+    plan_safe = True
 
     def __init__(self) -> None:
         pass

@@ -393,10 +393,10 @@ def test_step_shapes_that_repeat_are_replayed_from_a_graph_with_the_same_logits(
         step += 1
         helpers.assert_close(got, ref[s:s + n], dtype, f"step {step}: tokens {s}..{s + n}")
 
-    for _ in range(8):                      # shape (1,): eager, eager, capture, then replays
+    for _ in range(8):                      # shape (1,): recorded, from the plan, captured, then replays
         feed(1); fed += 1
     first = rep.runner.num_replayed_steps
-    assert first >= 4
+    assert first >= 4 and rep.runner.num_planned_steps >= 1
     for _ in range(6):                      # shape (4,) between them
         feed(4); fed += 4
         feed(1); fed += 1
@@ -408,6 +408,55 @@ def test_step_shapes_that_repeat_are_replayed_from_a_graph_with_the_same_logits(
         feed(4); fed += 4
     assert rep.runner.num_replayed_steps >= before + 8   # captured again and replayed again
     for i in range(60, 64):                 # and the other request goes on where it stood
+        feed(1, "y", other, want_other, i)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_shape_seen_before_is_launched_from_its_recorded_plan(model_folders, dtype):
+    """Without HIP graphs every repeat of a step shape makes its launches from the plan recorded at
+    the shape's first coming (one call into the kernel library instead of the model's Python); every
+    such step is checked against the plain implementation, other shapes come between them, and a
+    larger step that makes the workspace grow retires the plans, which are then recorded again."""
+    cfg = helpers.CONFIGS["A"]
+    rng = np.random.default_rng(8)
+    ids = helpers.random_ids(rng, cfg.vocab_size, 60)
+    other = helpers.random_ids(rng, cfg.vocab_size, 50)
+    pcfg, w = P.read_model_folder(model_folders["A"])
+    want, want_other = P.plain_forward(w, pcfg, ids).numpy(), P.plain_forward(w, pcfg, other).numpy()
+    rep = TraceReplayer(model_folders["A"], dtype, 128, page_size=4, poison=True)
+    rep.runner.graph_steps = False
+    assert rep.runner.plan_steps
+    fed = step = 0
+
+    def feed(n, rid="x", seq=ids, ref=want, start=None):
+        nonlocal step
+        s = fed if start is None else start
+        got = rep.run_step({"step": step, "entries": [{"id": rid, "tokens": seq[s:s + n], "want": list(range(n))}],
+                            "end": []}).cpu()
+        step += 1
+        helpers.assert_close(got, ref[s:s + n], dtype, f"step {step}: tokens {s}..{s + n}")
+
+    for _ in range(2):                           # both shapes twice: the workspace has all its buffers by then
+        feed(3); fed += 3
+        feed(1); fed += 1
+    settled = rep.runner.num_planned_steps
+    for _ in range(3):
+        feed(3); fed += 3
+        feed(1); fed += 1
+    assert rep.runner.num_planned_steps == settled + 6 and rep.runner.num_replayed_steps == 0
+    feed(40, "y", other, want_other, 0)          # the workspace grows: the plans hold stale addresses
+    before = rep.runner.num_planned_steps
+    feed(3); fed += 3
+    feed(1); fed += 1
+    assert rep.runner.num_planned_steps == before, "a plan recorded before the workspace grew was used"
+    feed(3); fed += 3
+    feed(1); fed += 1
+    before = rep.runner.num_planned_steps
+    for _ in range(3):
+        feed(3); fed += 3
+        feed(1); fed += 1
+    assert rep.runner.num_planned_steps == before + 6
+    for i in range(40, 44):                      # the other request goes on where it stood, from its own plans
         feed(1, "y", other, want_other, i)
 
 
