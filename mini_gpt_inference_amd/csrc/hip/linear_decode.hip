@@ -46,6 +46,13 @@ int mgpt_launch_linear_decode(const SkinnyArgs& a, int epilogue, int out_dtype, 
   // the scatter stores four neighbouring columns of a head at once
   if (epilogue == SK_EPI_QKV && ((a.n_out % 16) != 0 || (a.ldo % 4) != 0 || (((size_t)a.out) & 15) != 0))
     return MGPT_ERR_BAD_SHAPE;
+  if (a.n_rows <= 16 && a.partials != nullptr && a.rows_per_group == 0 && decode_vec_ok(a) &&
+      mgpt_linear_decode_partials(a.n_rows, a.n_out, a.k_dim, a.x != nullptr, epilogue, a.rows_mode) > 0) {
+    // few rows under a long inner size and few column tiles: the inner size split over workgroups
+    SkinnyArgs b = a;
+    b.rows_per_group = 16;
+    return mgpt_launch_linear_decode_rows(b, epilogue, out_dtype, stream);
+  }
   if (a.n_rows > 16 && !mgpt_linear_decode_row_groups(a.n_rows, a.n_out, a.k_dim, a.rows_mode))
   {
     SkinnyArgs b = a;

@@ -37,10 +37,17 @@ static int launch_tiles_unaligned_head(const SkinnyArgs& a, hipStream_t s) {
 // order and applies bias, GELU or the residual add.
 #define LDR_PARTS 4
 
+// Up to 16 rows are split as well when the inner size is long and the column tiles are few: a tile's
+// workgroup then streams 16 x k_dim of the matrix through one compute unit (205 KB for k = 6400),
+// and fewer workgroups than compute units do ([1600 x 6400] at one row: 11.5 us as 100 workgroups).
+// Below 3072 the second kernel costs more than the split saves (64 KB a workgroup at k = 2048).
+#define LDR_FEW_ROWS_MIN_K 3072
 long mgpt_linear_decode_partials(int n_rows, int n_out, int k_dim, bool ln, int epilogue, int rows_mode) {
-  if (ln || epilogue == SK_EPI_QKV || n_rows <= 16 || n_rows > 64) return 0;
+  if (ln || epilogue == SK_EPI_QKV || n_rows <= 0 || n_rows > 64) return 0;
+  if ((k_dim % (32 * LDR_PARTS)) != 0 || (n_out % 16) != 0 || n_out / 16 >= 128) return 0;
+  if (n_rows <= 16) return k_dim >= LDR_FEW_ROWS_MIN_K ? (long)LDR_PARTS * n_rows * n_out : 0;
   if (mgpt_linear_decode_row_groups(n_rows, n_out, k_dim, rows_mode)) return 0;
-  if (k_dim < 1024 || (k_dim % (32 * LDR_PARTS)) != 0 || (n_out % 16) != 0 || n_out / 16 >= 128) return 0;
+  if (k_dim < 1024) return 0;
   return (long)LDR_PARTS * n_rows * n_out;
 }
 
@@ -109,6 +116,7 @@ int mgpt_launch_linear_decode_rows(const SkinnyArgs& a, int epilogue, int out_dt
   if (a.partials != nullptr && decode_vec_ok(a) &&
       mgpt_linear_decode_partials(a.n_rows, a.n_out, a.k_dim, a.x != nullptr, epilogue, a.rows_mode) > 0) {
     switch (nt) {
+      case 1: return launch_split<1>(a, epilogue, out_dtype, stream);
       case 2: return launch_split<2>(a, epilogue, out_dtype, stream);
       case 3: return launch_split<3>(a, epilogue, out_dtype, stream);
       case 4: return launch_split<4>(a, epilogue, out_dtype, stream);

@@ -105,6 +105,10 @@ def packed_weight(w: torch.Tensor) -> Optional[torch.Tensor]:
 # with the fold and 0.375 ms without).
 FOLD_MAX_ROWS = 32
 FOLD_MAX_OUT = 4096
+# ... except at few rows, where the LayerNorm kernel's own launch costs more than the conversion
+# (the GPT-2-XL shape, outputs of 4800 and 6400: 957 us a step of 24 layers against 1062 at one
+# row, 1361 against 1399 at 16 rows, 1923 against 1741 at 32)
+FOLD_ANY_OUT_MAX_ROWS = 16
 # A very wide output (the head, 8192 columns and more) goes to the decode kernel while rows x inner
 # size stays within this, and to the tiled kernel beyond: that one streams the matrix at nearly the
 # same rate whatever the rows (50304 x 512: 10.2 us at 1 row, 11.4 at 32, 14.0 at 64), the decode
@@ -112,9 +116,6 @@ FOLD_MAX_OUT = 4096
 # row (9.4, 16.4, 28.5 us; at an inner size of 1600 it is behind from 4 rows on).
 WIDE_OUT = 8192
 WIDE_OUT_DECODE_WORK = 8192
-# A long inner size is split over workgroups (a second kernel then adds the parts) from more than
-# this many rows on.
-SPLIT_MIN_ROWS = 16
 
 
 def as_tensor(ctx, a: Union[torch.Tensor, LazyNorm]) -> torch.Tensor:
@@ -140,7 +141,7 @@ def linear(ctx, a: Union[torch.Tensor, LazyNorm], w: torch.Tensor, bias: Optiona
     if fast and n_rows <= 64 and not wide_out:
         epi = kernels.SK_EPI_QKV if scatter is not None else epilogue
         if (isinstance(a, LazyNorm) and getattr(a.norm, "fusable_layer_norm", False) and a._tensor is None
-                and w.shape[0] <= FOLD_MAX_OUT
+                and (w.shape[0] <= FOLD_MAX_OUT or n_rows <= FOLD_ANY_OUT_MAX_ROWS)
                 and (n_rows <= FOLD_MAX_ROWS or kernels.linear_skinny_row_groups(n_rows, w.shape[0], w.shape[1]))):
             wf, colsum, bias_f = folded_layer_norm(a.norm, w, bias)
             if kernels.linear_skinny(None, wf, bias_f, out, n_rows, epi, ln_x=a.x, ln_colsum=colsum,
@@ -148,8 +149,7 @@ def linear(ctx, a: Union[torch.Tensor, LazyNorm], w: torch.Tensor, bias: Optiona
                                      w_packed=packed_weight(wf)):
                 return scatter is not None
         partials = None
-        need = kernels.linear_skinny_partials(n_rows, w.shape[0], w.shape[1], False, epi) \
-            if n_rows > SPLIT_MIN_ROWS else 0
+        need = kernels.linear_skinny_partials(n_rows, w.shape[0], w.shape[1], False, epi)
         if need:
             partials = ctx.workspace.get("linear_partials", need, 1, torch.float32)
         if kernels.linear_skinny(as_tensor(ctx, a), w, bias, out, n_rows, epi, scatter=scatter, partials=partials,

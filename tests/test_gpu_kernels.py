@@ -369,7 +369,8 @@ def test_linear_skinny_with_the_inner_size_split_over_workgroups(n, k, o, epi, o
     groups = kernels.linear_skinny_row_groups(n, o, k)
     assert groups == (o * k * 2 <= 6 << 20 if k <= 2048 else n > 32 and o * k * 2 <= 8 << 20)
     assert kernels.linear_skinny_partials(n, o, k, False, epi) == (0 if groups else need)
-    assert kernels.linear_skinny_partials(16, o, k, False, epi) == 0          # few rows: one launch is as fast
+    # up to 16 rows: split only from an inner size of 3072 on
+    assert kernels.linear_skinny_partials(16, o, k, False, epi) == (4 * 16 * o if k >= 3072 else 0)
     assert kernels.linear_skinny_partials(n, o, 512, False, epi) == 0         # a short inner size
     assert kernels.linear_skinny_partials(n, o, k, True, epi) == 0            # not through a folded LayerNorm
     a, w, bias = rnd(g, n + 2, k, dtype="bfloat16"), rnd(g, o, k, dtype="bfloat16", scale=k ** -0.5), rnd(g, o)
@@ -389,6 +390,35 @@ def test_linear_skinny_with_the_inner_size_split_over_workgroups(n, k, o, epi, o
                                  rows_mode=kernels.ROWS_SHARE_W)
     assert torch.isnan(partials).all(), "too little scratch was written to"
     helpers.assert_close(out2[:n], _linear_want(a, w, bias, epi, prev)[:n], "bfloat16", "unsplit")
+
+
+@pytest.mark.parametrize("n,k,o", [(1, 3072, 768), (8, 6400, 1600), (16, 3072, 48), (3, 4096, 512)])
+@pytest.mark.parametrize("epi,o_dt", [(kernels.EPI_NONE, "bfloat16"), (kernels.EPI_GELU, "bfloat16"),
+                                      (kernels.EPI_RESIDUAL, "float32")])
+def test_linear_skinny_few_rows_with_a_long_inner_size_split_over_workgroups(n, k, o, epi, o_dt):
+    """Up to 16 rows under an inner size of 3072 and more and few column tiles: four workgroups per
+    tile take a quarter of the inner size each when the caller brings scratch, one takes it all
+    without; both against the plain product."""
+    g = torch.Generator().manual_seed(61)
+    need = kernels.linear_skinny_partials(n, o, k, False, epi)
+    assert need == 4 * n * o
+    assert kernels.linear_skinny_partials(n, o, 2048, False, epi) == 0       # not worth a second kernel
+    assert kernels.linear_skinny_partials(n, 2048, k, False, epi) == 0       # column tiles enough
+    a, w, bias = rnd(g, n + 1, k, dtype="bfloat16"), rnd(g, o, k, dtype="bfloat16", scale=k ** -0.5), rnd(g, o)
+    prev = rnd(g, n + 1, o, dtype=o_dt)
+    want = _linear_want(a, w, bias, epi, prev)
+    partials = torch.full((need,), float("nan"), device=DEV)
+    packed = kernels.pack_weight(w.to(DEV))
+    for wp in (None, packed):
+        out = prev.clone().to(DEV)
+        assert kernels.linear_skinny(a.to(DEV), w.to(DEV), bias.to(DEV), out, n, epi, partials=partials, w_packed=wp)
+        assert not torch.isnan(partials).any(), "the parts were not written: no split happened"
+        partials.fill_(float("nan"))
+        helpers.assert_close(out[:n], want[:n], "bfloat16", f"few rows split {n}x{k}x{o}")
+        assert torch.equal(out[n:], prev[n:].to(DEV)), "rows beyond n_rows were written"
+    whole = prev.clone().to(DEV)
+    assert kernels.linear_skinny(a.to(DEV), w.to(DEV), bias.to(DEV), whole, n, epi)
+    helpers.assert_close(whole[:n], want[:n], "bfloat16", "unsplit")
 
 
 @pytest.mark.parametrize("n,shape", [(70, None), (300, 3), (1100, 2), (300, 1), (520, 0)])
