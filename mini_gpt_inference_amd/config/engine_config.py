@@ -26,6 +26,9 @@ class EngineConfig:
     prefill_chunk: int = 0           # largest prompt portion per request and step; 0 = no limit
     mixed_batches: bool = True       # False: a step with admissions runs prompts only,
                                      # as the reference does (scheduler.py:52-56)
+    evict: str = "newest"            # when pages run out during decoding: "newest" evicts the newest running
+                                     # request, also when it is the one that asks; "newest_other" never the
+                                     # asker while another runs, as the reference does (scheduler.py:66-82)
     dtype: str = "bfloat16"          # "bfloat16" (serving) or "float32" (true 32-bit path)
     use_graph: bool = True           # replay decode-only steps, and other steps whose shape repeats, from
                                      # captured HIP graphs
@@ -52,6 +55,8 @@ class EngineConfig:
             raise ValueError("decode_burst and decode_chain must be at least 1")
         if self.prefill_chunk < 0:
             raise ValueError("prefill_chunk must be >= 0")
+        if self.evict not in ("newest", "newest_other"):
+            raise ValueError(f"evict must be 'newest' or 'newest_other', got {self.evict!r}")
         if self.dtype in ("bf16",):
             self.dtype = "bfloat16"
         if self.dtype in ("fp32",):

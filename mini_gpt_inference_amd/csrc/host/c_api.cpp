@@ -83,9 +83,10 @@ int mgpt_cache_build_step(void* cm, int n_req, const int* slots, const int* ctx_
 
 // ---------------------------------------------------------------- scheduler
 void* mgpt_sched_create(void* cm, int max_batch_size, int max_num_batched_tokens, int prefill_chunk,
-                        int mixed, int max_positions) {
+                        int mixed, int max_positions, int spare_asker) {
   GUARD_BEGIN
-  SchedulerConfig cfg{max_batch_size, max_num_batched_tokens, prefill_chunk, mixed != 0, max_positions};
+  SchedulerConfig cfg{max_batch_size, max_num_batched_tokens, prefill_chunk, mixed != 0, max_positions,
+                      spare_asker != 0};
   return new Scheduler(static_cast<CacheManager*>(cm), cfg);
   GUARD_END(nullptr)
 }

@@ -97,8 +97,11 @@ void Scheduler::ensure_capacity_for_decode() {
     while (!cache_->reserve(r.slot, r.num_computed + 1)) {
       // Evict the newest running request.  The reference never evicts the one that asks
       // (scheduler.py:78-82 picks the newest other one), which lets a newcomer push out an older
-      // request; here the asker itself goes when it is the newest.
-      Request& victim = *get(running_.back());
+      // request; by default the asker itself goes when it is the newest, and spare_asker brings the
+      // reference's rule back (the asker then goes only when it is the last one running).
+      int vid = running_.back();
+      if (cfg_.spare_asker && vid == id && running_.size() > 1) vid = running_[running_.size() - 2];
+      Request& victim = *get(vid);
       const bool self = victim.id == id;
       preempt(victim);
       if (self) break;

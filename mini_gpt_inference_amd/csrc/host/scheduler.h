@@ -33,6 +33,8 @@ struct SchedulerConfig {
   int prefill_chunk;           // largest prompt portion per request and step; 0 = no limit
   bool mixed;                  // prompt portions beside decode tokens in one step
   int max_positions;           // prompt + max_tokens may not exceed it (engine.py:83-88)
+  bool spare_asker = false;    // when pages run out: true = evict the newest running request other than
+                               // the one that asks (scheduler.py:66-82); false = the newest, the asker too
 };
 
 struct Request {

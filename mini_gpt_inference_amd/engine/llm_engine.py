@@ -159,7 +159,8 @@ class LLMEngine:
             self.cache, engine_config.max_batch_size,
             max(engine_config.max_num_batched_tokens, engine_config.max_batch_size),
             engine_config.prefill_chunk, engine_config.mixed_batches,
-            max_positions if max_positions is not None else 2 ** 30)
+            max_positions if max_positions is not None else 2 ** 30,
+            spare_asker=engine_config.evict == "newest_other")
         self.sampler = Sampler(model.spec.vocab_size, engine_config.real_vocab_size, engine_config.seed)
         self._ids: Dict[int, str] = {}        # scheduler id -> caller's request id
         self._rids: Dict[str, int] = {}

@@ -50,12 +50,12 @@ def _p(a: np.ndarray):
 
 class Scheduler:
     def __init__(self, cache: CacheManager, max_batch_size: int, max_num_batched_tokens: int,
-                 prefill_chunk: int, mixed: bool, max_positions: int) -> None:
+                 prefill_chunk: int, mixed: bool, max_positions: int, spare_asker: bool = False) -> None:
         self._lib = library.host()
         self.cache = cache
         self.max_batch_size = max_batch_size
         self._h = self._lib.mgpt_sched_create(cache.handle, max_batch_size, max_num_batched_tokens,
-                                              prefill_chunk, int(mixed), max_positions)
+                                              prefill_chunk, int(mixed), max_positions, int(spare_asker))
         if not self._h:
             raise SchedulerError(library.host_error())
         self._counts = np.zeros(3, dtype=np.int32)

@@ -183,7 +183,7 @@ def host() -> ctypes.CDLL:
             fn.argtypes = args
             fn.restype = I
         lib.mgpt_sched_create.restype = P
-        lib.mgpt_sched_create.argtypes = [P, I, I, I, I, I]
+        lib.mgpt_sched_create.argtypes = [P, I, I, I, I, I, I]
         lib.mgpt_sched_destroy.argtypes = [P]
         lib.mgpt_sched_destroy.restype = None
         lib.mgpt_sched_counter.argtypes = [P, I]

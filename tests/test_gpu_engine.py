@@ -172,15 +172,16 @@ def test_seeded_temperature_sampling_is_reproducible_and_independent_of_batching
             ids.append(tok)
 
 
+@pytest.mark.parametrize("evict", ["newest", "newest_other"])
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-def test_pages_run_out_preempted_request_is_recomputed_and_ends_with_the_same_tokens(model_folders, dtype):
+def test_pages_run_out_preempted_request_is_recomputed_and_ends_with_the_same_tokens(model_folders, dtype, evict):
     # reference tests/test_paged.py:107-143: pages of 2, four pages, two prompts of 2, 4 new tokens each
     prompts = [[1, 2], [4, 5]]
     sp = SamplingParams(max_tokens=4, temperature=0.0)
     roomy = LLMEngine.from_folder(model_folders["A"], EngineConfig(block_size=2, num_blocks=64, max_batch_size=2,
                                                                    dtype=dtype)).generate(prompts, sp)
     engine = LLMEngine.from_folder(model_folders["A"], EngineConfig(block_size=2, num_blocks=4, max_batch_size=2,
-                                                                    dtype=dtype))
+                                                                    dtype=dtype, evict=evict))
     tight = engine.generate(prompts, sp)
     assert engine.stats()["num_preemptions"] > 0
     assert engine.cache.num_free_pages() == 4 and engine.cache.check() == 0

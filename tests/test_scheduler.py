@@ -11,9 +11,9 @@ from mini_gpt_inference_amd.cache.manager import CacheManager, GroupGeometry
 from mini_gpt_inference_amd.engine.scheduler import FINISHED, RUNNING, WAITING, Scheduler, SchedulerError
 
 
-def make(num_pages, page_size, max_batch, budget=64, chunk=0, mixed=True, max_positions=1024):
+def make(num_pages, page_size, max_batch, budget=64, chunk=0, mixed=True, max_positions=1024, spare_asker=False):
     cm = CacheManager([GroupGeometry(page_size, num_pages, 0)], max_batch)
-    return cm, Scheduler(cm, max_batch, budget, chunk, mixed, max_positions)
+    return cm, Scheduler(cm, max_batch, budget, chunk, mixed, max_positions, spare_asker)
 
 
 def step(sched, token=lambda rid, idx: 100 + idx):
@@ -164,6 +164,30 @@ def test_evicted_request_goes_to_the_front_of_waiting():
     assert s.running == [old] and s.waiting == [new, later] and s.num_preemptions == 1
     assert len(cm.table(s.info(old).slot)) == 2   # the survivor got the freed page
     assert s.info(new).num_computed == 0 and s.info(new).output_len == 1 and s.info(new).status == WAITING
+
+
+def test_the_references_victim_rule_can_be_switched_back_on():
+    # The same three pages as above.  The older request takes the free page; then the newer one asks.
+    # The reference (scheduler.py:66-82) never evicts the one that asks while another runs, so the
+    # older request goes and the newer keeps decoding; both finish, and no page is lost.
+    cm, s = make(3, 4, max_batch=2, mixed=False, max_positions=64, spare_asker=True)
+    old = s.add_request(list(range(4)), 5)
+    new = s.add_request(list(range(4)), 5)
+    step(s)
+    assert s.running == [old, new] and cm.num_free_pages() == 1
+    ents, _ = step(s)
+    assert [e.request for e in ents] == [new]
+    assert s.running == [new] and s.waiting == [old] and s.num_preemptions == 1
+    assert len(cm.table(s.info(new).slot)) == 2
+    assert s.info(old).num_computed == 0 and s.info(old).status == WAITING
+    # the last one running still gives way to nobody but itself: it is never asked to
+    for _ in range(40):
+        if not s.has_work():
+            break
+        step(s)
+        assert cm.check() == 0
+    assert not s.has_work() and cm.num_free_pages() == 3
+    assert len(s.output(old)) == 5 and len(s.output(new)) == 5
 
 
 def test_requests_that_can_never_run_are_refused():
