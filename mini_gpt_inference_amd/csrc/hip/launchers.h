@@ -89,16 +89,22 @@ int mgpt_linear_skinny(const void* act, long lda, const float* x, const int* row
     n_rows, int n_out, int k_dim, int epilogue, void* kpool, void* vpool, const int* slot_mapping, int
     q_width, int kv_width, int head_dim, int n_kv_head, int page_size, int mode, float* partials, long
     partials_floats, hipStream_t stream);
+// linear_skinny.hip
+int mgpt_linear_head_best(const void* act, long lda, const float* x, const int* rows, const float* colsum,
+    float eps, const void* w, const void* w_packed, const float* bias, float* out, long ldo, int n_rows, int
+    n_out, int k_dim, float* best_val, int* best_idx, int best_limit, hipStream_t stream);
 // sampling.hip
 int mgpt_sample(const float* logits, long ld, int n_rows, int vocab, int real_vocab, const float* temperature,
     const int* top_k, const float* top_p, const uint64_t* request_seed, const int* out_index, uint64_t
-    engine_seed, int* out_tokens, hipStream_t stream);
+    engine_seed, int* out_tokens, const float* tile_best, const int* tile_best_idx, int n_tiles, hipStream_t
+    stream);
 // sampling.hip
 int mgpt_sample_advance(const float* logits, long ld, int n_rows, int vocab, int real_vocab, const float*
     temperature, const int* top_k, const float* top_p, const uint64_t* request_seed, int* out_index, uint64_t
     engine_seed, int* out_tokens, int* token_ids, int* positions, int* seq_lens, const int* q_req, int*
     slot_mapping, const int* block_tables, const int* page_sizes, int n_groups, int n_stride, int r_stride,
-    int max_blocks, int* history, int* history_pos, int history_rows, int history_stride, hipStream_t stream);
+    int max_blocks, int* history, int* history_pos, int history_rows, int history_stride, const float*
+    tile_best, const int* tile_best_idx, int n_tiles, hipStream_t stream);
 }
 
 // MGPT_FOR_EACH_LAUNCHER(X) expands X(name) for every launcher above
@@ -122,5 +128,6 @@ int mgpt_sample_advance(const float* logits, long ld, int n_rows, int vocab, int
   X(mgpt_linear_mfma_shape) \
   X(mgpt_linear_mfma_qkv) \
   X(mgpt_linear_skinny) \
+  X(mgpt_linear_head_best) \
   X(mgpt_sample) \
   X(mgpt_sample_advance)

@@ -257,6 +257,26 @@ __global__ __launch_bounds__(256) void linear_decode_kernel(SkinnyArgs a) {
     }
     if (VEC && sizeof(OT) == 4) {
       *reinterpret_cast<float4*>(orow + oc) = make_float4(v[0], v[1], v[2], v[3]);
+      if (NT == 1 && EPI == SK_EPI_NONE && a.best_val != nullptr) {
+        // the row's best of this tile: of this lane's four columns in rising order, then over the
+        // four lanes that hold the row (all of them are here: VEC means whole tiles)
+        float bv = -INFINITY;
+        int bi = 0x7fffffff;
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          if (oc + i < a.best_limit && v[i] > bv) { bv = v[i]; bi = oc + i; }
+#pragma unroll
+        for (int m = 16; m <= 32; m <<= 1) {
+          const float ov = __shfl_xor(bv, m, 64);
+          const int oi = __shfl_xor(bi, m, 64);
+          if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
+        }
+        if (g == 0) {
+          const long at = (long)(r0 + t * 16) * (a.n_out >> 4) + (o0 >> 4);
+          a.best_val[at] = bv;
+          a.best_idx[at] = bi;
+        }
+      }
     } else if (VEC) {
       uint2 pk;
       pk.x = pack_bf16x2(v[0], v[1]);

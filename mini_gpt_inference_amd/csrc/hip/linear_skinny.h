@@ -43,6 +43,12 @@ struct SkinnyArgs {
   bf16_t* vpool;
   const int* slot_mapping;
   int q_width, kv_width, head_dim, n_kv_head, page_size;
+  // linear_decode.hip, one tile a workgroup, float32 output without an epilogue: per row and column
+  // tile the largest value among the tile's columns below best_limit and its column (the lowest
+  // among equals), to best_val / best_idx [n_rows][n_out / 16]; null: off
+  float* best_val;
+  int* best_idx;
+  int best_limit;
 };
 
 // linear_decode.hip: at most 64 rows, k_dim a multiple of 32.  Returns

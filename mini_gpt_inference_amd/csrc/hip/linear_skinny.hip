@@ -313,13 +313,14 @@ static int launch_nt(const SkinnyArgs& a, int epi, int out_dtype, dim3 grid, siz
 // same matrix in mgpt_pack_weight's layout (only linear_decode.hip reads it).  partials: optional scratch of
 // mgpt_linear_skinny_partials(...) floats; with it a long inner size with many rows is split over
 // workgroups (two launches).
-extern "C" int mgpt_linear_skinny(const void* act, long lda, const float* x, const int* rows,
-                                  const float* colsum, float eps, const void* w, const void* w_packed,
-                                  const float* bias, void* out, int out_dtype, long ldo, int n_rows,
-                                  int n_out, int k_dim, int epilogue, void* kpool, void* vpool,
-                                  const int* slot_mapping, int q_width, int kv_width, int head_dim,
-                                  int n_kv_head, int page_size, int mode, float* partials,
-                                  long partials_floats, hipStream_t stream) {
+static int linear_skinny_launch(const void* act, long lda, const float* x, const int* rows,
+                                const float* colsum, float eps, const void* w, const void* w_packed,
+                                const float* bias, void* out, int out_dtype, long ldo, int n_rows,
+                                int n_out, int k_dim, int epilogue, void* kpool, void* vpool,
+                                const int* slot_mapping, int q_width, int kv_width, int head_dim,
+                                int n_kv_head, int page_size, int mode, float* partials,
+                                long partials_floats, float* best_val, int* best_idx, int best_limit,
+                                hipStream_t stream) {
   if (n_rows == 0 || n_out == 0) return MGPT_OK;
   if (!w || !out || (!act && !x)) return MGPT_ERR_NULL;
   if (n_rows < 0 || n_rows > 64 || n_out < 0 || k_dim <= 0 || (k_dim % 16) != 0 || ldo < n_out)
@@ -354,6 +355,7 @@ extern "C" int mgpt_linear_skinny(const void* act, long lda, const float* x, con
   a.k_dim = k_dim; a.ksplit = ks; a.kpool = (bf16_t*)kpool; a.vpool = (bf16_t*)vpool;
   a.slot_mapping = slot_mapping; a.q_width = q_width; a.kv_width = kv_width; a.head_dim = head_dim;
   a.n_kv_head = n_kv_head; a.page_size = page_size;
+  a.best_val = best_val; a.best_idx = best_idx; a.best_limit = best_limit;
   // room for the parts of a split over workgroups, if the caller brought enough of it
   a.k_parts = 1;
   a.rows_mode = ((mode & 0xFF) == SK_ROWS_SHARE_W || (mode & 0xFF) == SK_ROWS_GROUPS) ? (mode & 0xFF) : 0;
@@ -364,7 +366,7 @@ extern "C" int mgpt_linear_skinny(const void* act, long lda, const float* x, con
   if (mode != 1) {
     // the rows of a decode step: the kernel laid out for latency, where it takes the shape
     const int rc = mgpt_launch_linear_decode(a, epilogue, out_dtype, stream);
-    if (rc != MGPT_ERR_BAD_SHAPE) return rc;
+    if (rc != MGPT_ERR_BAD_SHAPE || best_val) return rc;
   }
   const int cw_per_wg = waves / ks;
   const int n_groups = (tiles + cw_per_wg - 1) / cw_per_wg;
@@ -384,6 +386,38 @@ extern "C" int mgpt_linear_skinny(const void* act, long lda, const float* x, con
     default: return SK_NT(4);
   }
 #undef SK_NT
+}
+
+extern "C" int mgpt_linear_skinny(const void* act, long lda, const float* x, const int* rows,
+                                  const float* colsum, float eps, const void* w, const void* w_packed,
+                                  const float* bias, void* out, int out_dtype, long ldo, int n_rows,
+                                  int n_out, int k_dim, int epilogue, void* kpool, void* vpool,
+                                  const int* slot_mapping, int q_width, int kv_width, int head_dim,
+                                  int n_kv_head, int page_size, int mode, float* partials,
+                                  long partials_floats, hipStream_t stream) {
+  return linear_skinny_launch(act, lda, x, rows, colsum, eps, w, w_packed, bias, out, out_dtype, ldo, n_rows, n_out,
+                              k_dim, epilogue, kpool, vpool, slot_mapping, q_width, kv_width, head_dim, n_kv_head,
+                              page_size, mode, partials, partials_floats, nullptr, nullptr, 0, stream);
+}
+
+// The output head of a decode step: float32 logits for at most 16 rows, and with them, per row and
+// tile of 16 columns, the largest logit among the columns below best_limit and its column
+// (best_val, best_idx: [n_rows][n_out / 16]), so that a greedy choice need not read the logits again
+// (mgpt_sample's best_* arguments).  Takes what linear_decode.hip takes with whole tiles and aligned
+// rows; MGPT_ERR_BAD_SHAPE otherwise, having launched nothing (mgpt_linear_skinny then does the product).
+// The tied head of src/minigpt_infer/model.py:128-130,187 before the argmax of sampling.py:97-103.
+extern "C" int mgpt_linear_head_best(const void* act, long lda, const float* x, const int* rows,
+                                     const float* colsum, float eps, const void* w, const void* w_packed,
+                                     const float* bias, float* out, long ldo, int n_rows, int n_out, int k_dim,
+                                     float* best_val, int* best_idx, int best_limit, hipStream_t stream) {
+  if (n_rows == 0 || n_out == 0) return MGPT_OK;
+  if (!best_val || !best_idx) return MGPT_ERR_NULL;
+  if (n_rows > 16 || (k_dim % 32) != 0 || (n_out % 16) != 0 || (ldo % 4) != 0 || best_limit <= 0 ||
+      ((((size_t)out) | ((size_t)bias) | ((size_t)colsum)) & 15) != 0)
+    return MGPT_ERR_BAD_SHAPE;
+  return linear_skinny_launch(act, lda, x, rows, colsum, eps, w, w_packed, bias, out, MGPT_F32, ldo, n_rows, n_out,
+                              k_dim, SK_EPI_NONE, nullptr, nullptr, nullptr, 0, 0, 0, 0, 0, 0, nullptr, 0, best_val,
+                              best_idx, best_limit, stream);
 }
 
 // floats of scratch with which mgpt_linear_skinny splits this shape's inner size over workgroups; 0: it would not

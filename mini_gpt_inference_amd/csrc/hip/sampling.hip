@@ -169,7 +169,8 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
     const float* __restrict__ logits, long ld, int vocab, int real_vocab,
     const float* __restrict__ temperature, const int* __restrict__ top_k,
     const float* __restrict__ top_p, const uint64_t* __restrict__ request_seed,
-    const int* out_index, uint64_t engine_seed, int* out_tokens, AdvanceArgs adv) {
+    const int* out_index, uint64_t engine_seed, int* out_tokens, AdvanceArgs adv,
+    const float* __restrict__ tile_best, const int* __restrict__ tile_best_idx, int n_tiles) {
   __shared__ float red_f[SAMPLE_WAVES];
   __shared__ int red_i[SAMPLE_WAVES];
   __shared__ float part[SAMPLE_THREADS];
@@ -186,7 +187,26 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
     // strictly larger value is all it has to look for; four logits are compared as their maximum.
     float best = -INFINITY;
     int best_i = 0x7fffffff;
-    if ((reinterpret_cast<uintptr_t>(lg) & 15) == 0) {
+    if (tile_best != nullptr) {
+      // the kernel that made the logits has left every tile's best (mgpt_linear_head_best, which
+      // already kept to the columns below real_vocab): a few kilobytes to read instead of the row
+      const float* tb = tile_best + (long)row * n_tiles;
+      const int* ti = tile_best_idx + (long)row * n_tiles;
+      constexpr int U = 4;
+      for (int base = tid; base < n_tiles; base += SAMPLE_THREADS * U) {
+        float v[U];
+        int ix[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+          const int i = base + u * SAMPLE_THREADS;
+          v[u] = tb[i < n_tiles ? i : base];
+          ix[u] = ti[i < n_tiles ? i : base];
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+          if (base + u * SAMPLE_THREADS < n_tiles && v[u] > best) { best = v[u]; best_i = ix[u]; }
+      }
+    } else if ((reinterpret_cast<uintptr_t>(lg) & 15) == 0) {
       const int n4 = nv >> 2;
       const float4* lg4 = reinterpret_cast<const float4*>(lg);
       constexpr int U = 16;  // loads in flight per thread: one pass covers 64 Ki logits
@@ -346,27 +366,32 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
 }
 
 // logits: [n_rows, vocab] floats with row stride ld.  top_k (0 = off), top_p (1 = off),
-// request_seed and out_index may be null.
+// request_seed and out_index may be null.  tile_best, tile_best_idx [n_rows][n_tiles] (optional): what
+// mgpt_linear_head_best left beside these logits with best_limit = real_vocab; greedy rows then read
+// those instead of the logits.
 static int launch_sample(const float* logits, long ld, int n_rows, int vocab, int real_vocab,
                          const float* temperature, const int* top_k, const float* top_p,
                          const uint64_t* request_seed, const int* out_index, uint64_t engine_seed,
-                         int* out_tokens, const AdvanceArgs& adv, hipStream_t stream) {
+                         int* out_tokens, const AdvanceArgs& adv, const float* tile_best,
+                         const int* tile_best_idx, int n_tiles, hipStream_t stream) {
   if (n_rows == 0) return MGPT_OK;
   if (!logits || !temperature || !out_tokens) return MGPT_ERR_NULL;
   if (n_rows < 0 || vocab <= 0 || real_vocab <= 0 || ld < vocab) return MGPT_ERR_BAD_SHAPE;
+  if (tile_best && (!tile_best_idx || n_tiles <= 0)) return MGPT_ERR_BAD_SHAPE;
   hipLaunchKernelGGL(sample_kernel, dim3(n_rows), dim3(SAMPLE_THREADS), 0, stream, logits, ld, vocab,
                      real_vocab, temperature, top_k, top_p, request_seed, out_index, engine_seed,
-                     out_tokens, adv);
+                     out_tokens, adv, tile_best, tile_best_idx, n_tiles);
   return mgpt_last_error();
 }
 
 extern "C" int mgpt_sample(const float* logits, long ld, int n_rows, int vocab, int real_vocab,
                            const float* temperature, const int* top_k, const float* top_p,
                            const uint64_t* request_seed, const int* out_index, uint64_t engine_seed,
-                           int* out_tokens, hipStream_t stream) {
+                           int* out_tokens, const float* tile_best, const int* tile_best_idx, int n_tiles,
+                           hipStream_t stream) {
   AdvanceArgs adv = {};
   return launch_sample(logits, ld, n_rows, vocab, real_vocab, temperature, top_k, top_p, request_seed,
-                       out_index, engine_seed, out_tokens, adv, stream);
+                       out_index, engine_seed, out_tokens, adv, tile_best, tile_best_idx, n_tiles, stream);
 }
 
 // mgpt_sample, then each row prepares the next decode step on the device (AdvanceArgs above).
@@ -378,7 +403,8 @@ extern "C" int mgpt_sample_advance(const float* logits, long ld, int n_rows, int
                                    const int* q_req, int* slot_mapping, const int* block_tables,
                                    const int* page_sizes, int n_groups, int n_stride, int r_stride,
                                    int max_blocks, int* history, int* history_pos, int history_rows,
-                                   int history_stride, hipStream_t stream) {
+                                   int history_stride, const float* tile_best, const int* tile_best_idx,
+                                   int n_tiles, hipStream_t stream) {
   if (!token_ids || !positions || !seq_lens || !out_index || !q_req || !slot_mapping || !block_tables ||
       !page_sizes || !history || !history_pos)
     return MGPT_ERR_NULL;
@@ -388,5 +414,5 @@ extern "C" int mgpt_sample_advance(const float* logits, long ld, int n_rows, int
   AdvanceArgs adv = {token_ids, positions, seq_lens, out_index, q_req, slot_mapping, block_tables, page_sizes,
                      n_groups, n_stride, r_stride, max_blocks, history, history_pos, history_rows, history_stride};
   return launch_sample(logits, ld, n_rows, vocab, real_vocab, temperature, top_k, top_p, request_seed,
-                       out_index, engine_seed, out_tokens, adv, stream);
+                       out_index, engine_seed, out_tokens, adv, tile_best, tile_best_idx, n_tiles, stream);
 }

@@ -18,6 +18,7 @@ from ..cache.kv_store import KVStore
 from ..cache.manager import CacheManager, GroupGeometry, plan_group_pages
 from ..config.engine_config import EngineConfig, SamplingParams
 from ..ops import kernels
+from ..ops.linear import TileBest
 from ..parts.base import Workspace
 from ..sampling.sampler import Sampler
 from ..weights.loader import load_model
@@ -51,14 +52,18 @@ class _GraphedDecode:
         self.burst_graph: Optional[torch.cuda.CUDAGraph] = None
         self.shape: Optional[StepShape] = None   # of the last single step; launch geometry for captures
         self.kernels_per_step = 0                # kernels that the captured step launches
+        self.tile_best_used = False              # greedy rows choose from what the head left per tile
 
     def _launch(self, shape: StepShape) -> None:
         ctx = self.runner.context(self.arena, shape, padded=True, workspace=self.workspace)
         # launch geometry must not depend on this step's lengths: size it for the longest sequence
         ctx.max_seq_len = self.runner.max_positions or ctx.max_seq_len
+        ctx.tile_best = TileBest(self.sampler.real_vocab)
         with kernels.pinned_stream():
             logits = self.runner.model.forward(ctx)
-            self.sampler.sample(logits, self.arena, self.cap, advance=(self.runner.page_sizes, self.history))
+            self.sampler.sample(logits, self.arena, self.cap, advance=(self.runner.page_sizes, self.history),
+                                tile_best=ctx.tile_best)
+        self.tile_best_used = ctx.tile_best.filled
 
     def _capture(self, shape: StepShape, times: int) -> torch.cuda.CUDAGraph:
         self.runner.num_graph_captures += 1

@@ -210,8 +210,12 @@ def paged_attention_generic(q: torch.Tensor, out: torch.Tensor, k_pool: torch.Te
 
 def sample(logits: torch.Tensor, n_rows: int, real_vocab: int, temperature: torch.Tensor,
            top_k: Optional[torch.Tensor], top_p: Optional[torch.Tensor], request_seed: Optional[torch.Tensor],
-           out_index: Optional[torch.Tensor], engine_seed: int, out_tokens: torch.Tensor, advance=None) -> None:
+           out_index: Optional[torch.Tensor], engine_seed: int, out_tokens: torch.Tensor, advance=None,
+           tile_best=None) -> None:
     """One token per row of float32 logits: argmax where temperature <= 0, else seeded sampling.
+
+    tile_best = (values, columns), float32 and int32 [>=n_rows, tiles]: what linear_head_best left
+    beside these logits with limit = real_vocab; greedy rows then read those instead of the logits.
 
     advance = (token_ids, positions, seq_lens, q_req, slot_mapping [groups, n_stride], block_tables
     [groups, r_stride, max_blocks], page_sizes [groups], history [rows, stride], history_pos): after
@@ -230,6 +234,15 @@ def sample(logits: torch.Tensor, n_rows: int, real_vocab: int, temperature: torc
     _need(out_index is None or (out_index.dtype == torch.int32 and out_index.numel() >= n_rows),
           "out_index must be int32 [rows]")
     _need_i32("out_tokens", out_tokens, n_rows)
+    tb = ti = None
+    n_tiles = 0
+    if tile_best is not None:
+        tb, ti = tile_best
+        _need_cuda(tb, ti)
+        _need(tb.dtype == torch.float32 and ti.dtype == torch.int32 and tb.dim() == 2 and tb.is_contiguous()
+              and ti.is_contiguous() and tb.shape == ti.shape and tb.shape[0] >= n_rows,
+              "tile_best must be dense float32 values and int32 columns [>=n_rows, tiles]")
+        n_tiles = tb.shape[1]
     if advance is not None:
         token_ids, positions, seq_lens, q_req, slot_mapping, block_tables, page_sizes, history, history_pos = advance
         _need_cuda(*advance)
@@ -252,13 +265,13 @@ def sample(logits: torch.Tensor, n_rows: int, real_vocab: int, temperature: torc
             _ptr(request_seed), _ptr(out_index), ctypes.c_ulonglong(engine_seed & (2**64 - 1)), _ptr(out_tokens),
             _ptr(token_ids), _ptr(positions), _ptr(seq_lens), _ptr(q_req), _ptr(slot_mapping), _ptr(block_tables),
             _ptr(page_sizes), n_groups, n_stride, r_stride, max_blocks, _ptr(history), _ptr(history_pos),
-            history.shape[0], history.stride(0), _stream())
+            history.shape[0], history.stride(0), _ptr(tb), _ptr(ti), n_tiles, _stream())
         _check(rc, "sample_advance")
         return
     rc = library.kernels().mgpt_sample(_ptr(logits), logits.stride(0), n_rows, vocab, real_vocab,
                                        _ptr(temperature), _ptr(top_k), _ptr(top_p), _ptr(request_seed),
                                        _ptr(out_index), ctypes.c_ulonglong(engine_seed & (2**64 - 1)),
-                                       _ptr(out_tokens), _stream())
+                                       _ptr(out_tokens), _ptr(tb), _ptr(ti), n_tiles, _stream())
     _check(rc, "sample")
 
 
@@ -379,6 +392,45 @@ def pack_weight(w: torch.Tensor) -> Optional[torch.Tensor]:
 
 
 ROWS_SHARE_W, ROWS_GROUPS = 2, 3
+
+
+def linear_head_best(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor, n_rows: int,
+                     best_val: torch.Tensor, best_idx: torch.Tensor, limit: int,
+                     w_packed: Optional[torch.Tensor] = None) -> bool:
+    """out[:n_rows] = a[:n_rows] @ w.T (+ bias) in float32 for at most 16 bfloat16 rows, and beside it,
+    per row and tile of 16 columns, the largest value among the columns below `limit` and its column
+    (the lowest among equals): best_val float32, best_idx int32, both [>=n_rows, out / 16].  What
+    sample() takes as tile_best.  False, having launched nothing, if the decode kernel does not take
+    the shape."""
+    n_out, k_dim = w.shape
+    if (n_rows > 16 or w.dtype != torch.bfloat16 or a.dtype != torch.bfloat16 or out.dtype != torch.float32
+            or k_dim % 32 or n_out % 16 or a.stride(0) % 8 or a.data_ptr() % 16 or out.stride(0) % 4
+            or out.data_ptr() % 16):
+        return False
+    _need_cuda(a, w, bias, out, best_val, best_idx, w_packed)
+    _need(w.is_contiguous(), "weight must be dense [out, in]")
+    _need(a.dim() == 2 and a.stride(1) == 1 and a.shape[1] == k_dim and a.shape[0] >= n_rows,
+          "activation must be [>=n_rows, inner] with unit inner stride")
+    _need(out.dim() == 2 and out.stride(1) == 1 and out.shape[1] >= n_out and out.shape[0] >= n_rows,
+          "output must be [>=n_rows, >=out] with unit inner stride")
+    _need(bias is None or (bias.dtype == torch.float32 and bias.numel() == n_out and bias.data_ptr() % 16 == 0),
+          "bias must be aligned float32 [out]")
+    tiles = n_out // 16
+    _need(best_val.dtype == torch.float32 and best_idx.dtype == torch.int32 and best_val.is_contiguous()
+          and best_idx.is_contiguous() and tuple(best_val.shape) == tuple(best_idx.shape)
+          and best_val.dim() == 2 and best_val.shape[0] >= n_rows and best_val.shape[1] == tiles,
+          "best_val and best_idx must be dense float32 / int32 [>=n_rows, out / 16]")
+    _need(0 < limit <= n_out, "limit must lie in 1..out")
+    if w_packed is not None:
+        _need(w_packed.dtype == torch.bfloat16 and w_packed.is_contiguous() and w_packed.numel() == n_out * k_dim
+              and w_packed.data_ptr() % 16 == 0, "w_packed must be pack_weight(w)")
+    rc = library.kernels().mgpt_linear_head_best(
+        _ptr(a), a.stride(0), None, None, None, 0.0, _ptr(w), _ptr(w_packed), _ptr(bias), _ptr(out), out.stride(0),
+        n_rows, n_out, k_dim, _ptr(best_val), _ptr(best_idx), int(limit), _stream())
+    if rc == -2:
+        return False
+    _check(rc, "linear_head_best")
+    return True
 
 
 def linear_skinny_row_groups(n_rows: int, n_out: int, k_dim: int) -> bool:

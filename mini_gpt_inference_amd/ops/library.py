@@ -40,9 +40,9 @@ def kernels() -> ctypes.CDLL:
         lib.mgpt_linear_generic.argtypes = [P, I, L, P, I, P, P, I, L, I, I, I, I, P]
         lib.mgpt_kv_write.argtypes = [P, I, L, I, I, P, P, P, I, I, I, I, P]
         lib.mgpt_paged_attention_generic.argtypes = [P, L, P, L, P, P, P, I, P, P, P, I, I, I, I, I, F, I, I, I, P]
-        lib.mgpt_sample.argtypes = [P, L, I, I, I, P, P, P, P, P, c_ulonglong, P, P]
+        lib.mgpt_sample.argtypes = [P, L, I, I, I, P, P, P, P, P, c_ulonglong, P, P, P, I, P]
         lib.mgpt_sample_advance.argtypes = [P, L, I, I, I, P, P, P, P, P, c_ulonglong, P,
-                                            P, P, P, P, P, P, P, I, I, I, I, P, P, I, I, P]
+                                            P, P, P, P, P, P, P, I, I, I, I, P, P, I, I, P, P, I, P]
         for name in ("mgpt_embed", "mgpt_layernorm", "mgpt_linear_generic", "mgpt_kv_write",
                      "mgpt_paged_attention_generic", "mgpt_sample", "mgpt_sample_advance"):
             getattr(lib, name).restype = I
@@ -122,6 +122,7 @@ def _declare_optional(lib: ctypes.CDLL) -> None:
     P, I, L, F = c_void_p, c_int, c_long, c_float
     table = {
         "mgpt_linear_skinny": [P, L, P, P, P, F, P, P, P, P, I, L, I, I, I, I, P, P, P, I, I, I, I, I, I, P, L, P],
+        "mgpt_linear_head_best": [P, L, P, P, P, F, P, P, P, P, L, I, I, I, P, P, I, P],
         "mgpt_pack_weight": [P, P, I, I, P],
         "mgpt_linear_skinny_partials": [I, I, I, I, I],
         "mgpt_linear_skinny_row_groups": [I, I, I],

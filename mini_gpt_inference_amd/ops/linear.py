@@ -122,8 +122,21 @@ def as_tensor(ctx, a: Union[torch.Tensor, LazyNorm]) -> torch.Tensor:
     return a.tensor(ctx) if isinstance(a, LazyNorm) else a
 
 
+class TileBest:
+    """Asks a product for the best column of every tile of 16 beside its float32 output: the largest
+    value among the columns below `limit` and its column.  The product that can, fills values and
+    columns ([rows, out / 16], from the workspace) and sets `filled`."""
+
+    def __init__(self, limit: int) -> None:
+        self.limit = int(limit)
+        self.values: Optional[torch.Tensor] = None
+        self.columns: Optional[torch.Tensor] = None
+        self.filled = False
+
+
 def linear(ctx, a: Union[torch.Tensor, LazyNorm], w: torch.Tensor, bias: Optional[torch.Tensor],
-           out: torch.Tensor, n_rows: int, epilogue: int = kernels.EPI_NONE, scatter=None) -> bool:
+           out: torch.Tensor, n_rows: int, epilogue: int = kernels.EPI_NONE, scatter=None,
+           tile_best: Optional[TileBest] = None) -> bool:
     """out[:n_rows] = a[:n_rows] @ w.T (+ bias) with the epilogue.
 
     On the bfloat16 path up to 64 rows (fewer for a very wide output) go to the decode step's MFMA kernels (reading the residual
@@ -138,6 +151,16 @@ def linear(ctx, a: Union[torch.Tensor, LazyNorm], w: torch.Tensor, bias: Optiona
         a = a.tensor(ctx)      # the kernels below read plain residual rows
     fast = w.dtype == torch.bfloat16 and not ctx.exact and ctx.dtype == torch.bfloat16
     wide_out = w.shape[0] >= WIDE_OUT and n_rows * w.shape[1] > WIDE_OUT_DECODE_WORK
+    if (tile_best is not None and fast and n_rows <= 16 and not wide_out and epilogue == kernels.EPI_NONE
+            and scatter is None and w.shape[0] % 16 == 0 and w.shape[1] % 32 == 0
+            and not kernels.linear_skinny_partials(n_rows, w.shape[0], w.shape[1], False, epilogue)):
+        rows = out.shape[0]
+        tile_best.values = ctx.workspace.get("tile_best_values", rows, w.shape[0] // 16, torch.float32)
+        tile_best.columns = ctx.workspace.get("tile_best_columns", rows, w.shape[0] // 16, torch.int32)
+        if kernels.linear_head_best(as_tensor(ctx, a), w, bias, out, n_rows, tile_best.values, tile_best.columns,
+                                    tile_best.limit, w_packed=packed_weight(w)):
+            tile_best.filled = True
+            return False
     if fast and n_rows <= 64 and not wide_out:
         epi = kernels.SK_EPI_QKV if scatter is not None else epilogue
         if (isinstance(a, LazyNorm) and getattr(a.norm, "fusable_layer_norm", False) and a._tensor is None

@@ -196,3 +196,6 @@ class StepContext:
     lead_cap: int = 0            # padded steps: the decoding requests' tokens lie among the first lead_cap
     # sums that are still to be added to the residual stream (ops.residual.PendingSums); None: it is plain
     pending: Optional[Any] = None
+    # set by a caller that will choose greedily among the logits: an ops.linear.TileBest, which the
+    # head fills beside the logits if its kernel can
+    tile_best: Optional[Any] = None

@@ -61,4 +61,4 @@ class LinearHead(Part):
         return {"weight": WeightRequest((self.vocab_size, self.width), MATRIX)}
 
     def forward(self, ctx: StepContext, h: torch.Tensor, logits: torch.Tensor, n_rows: int) -> None:
-        linear(ctx, h, self.weight, None, logits, n_rows)
+        linear(ctx, h, self.weight, None, logits, n_rows, tile_best=ctx.tile_best)

@@ -16,11 +16,12 @@ class Sampler:
             raise ValueError("real_vocab_size must lie in 1..vocab_size")
         self.engine_seed = int(engine_seed)
 
-    def sample(self, logits: torch.Tensor, arena, n_rows: int, advance=None) -> torch.Tensor:
+    def sample(self, logits: torch.Tensor, arena, n_rows: int, advance=None, tile_best=None) -> torch.Tensor:
         """Writes one token per logits row into arena.tokens_out, using the arena's per-row sampling
         arrays.  Returns arena.tokens_out.  advance = (page_sizes, history): after a decode-only
         step, also turn the arena's device arrays into those of the next step and append the
-        tokens to history [steps, rows] (see kernels.sample)."""
+        tokens to history [steps, rows] (see kernels.sample).  tile_best: an ops.linear.TileBest that
+        the head has filled for these logits with this sampler's real_vocab as its limit."""
         d = arena.d
         adv = None
         if advance is not None:
@@ -30,5 +31,7 @@ class Sampler:
                    d["block_tables"].view(arena.n_groups, arena.r_cap, arena.max_blocks), page_sizes, history,
                    d["history_pos"])
         kernels.sample(logits, n_rows, self.real_vocab, d["temperature"], d["top_k"], d["top_p"], d["seeds"],
-                       d["out_index"], self.engine_seed, arena.tokens_out, advance=adv)
+                       d["out_index"], self.engine_seed, arena.tokens_out, advance=adv,
+                       tile_best=(tile_best.values, tile_best.columns)
+                       if tile_best is not None and tile_best.filled and tile_best.limit == self.real_vocab else None)
         return arena.tokens_out

@@ -95,7 +95,7 @@ def test_many_requests_decode_from_padded_graphs(model_folders, dtype, n_req):
         assert exact >= 0.9 * sum(news)
 
 
-@pytest.mark.parametrize("shape,n_req", [("50M", 8), ("small", 20), ("xl", 64)])
+@pytest.mark.parametrize("shape,n_req", [("50M", 8), ("50M", 3), ("small", 20), ("xl", 64)])
 def test_real_widths_decode_through_graphs_and_bursts(tmp_path, shape, n_req):
     """The benchmarked shapes through the engine itself (padded graphs, bursts of steps fed on the
     device): every greedy choice is the plain implementation's argmax up to the logits' tolerance."""
@@ -113,6 +113,8 @@ def test_real_widths_decode_through_graphs_and_bursts(tmp_path, shape, n_req):
                                                         dtype="bfloat16"))
     got = engine.generate(prompts, SamplingParams(max_tokens=n_new, temperature=0.0))
     assert engine.stats()["graph_steps"] >= n_new - 4
+    # up to 16 rows of a vocabulary of whole tiles choose from the bests that the head leaves per tile
+    assert all(g.tile_best_used == (shape == "50M" and n_req <= 16) for g in engine._graphs.values())
     pcfg, w = P.read_model_folder(folder)
     exact = total = 0
     for prompt, tokens in list(zip(prompts, got))[::max(1, n_req // 8)]:      # a sample of the requests: the plain model is slow

@@ -699,6 +699,75 @@ def test_greedy_ties_at_every_distance_and_rows_that_are_not_aligned():
         assert got == want and got[0] == 11 and got[1] == real - 1 and got[-1] == 5
 
 
+@pytest.mark.parametrize("rows,n_out,k_dim,limit,packed,bias", [(1, 1008, 96, 1001, True, False), (5, 50304, 512, 50257, True, False),
+                                                             (16, 208, 64, 208, False, True), (8, 4096, 1600, 4090, True, True),
+                                                             (3, 2000, 768, 1999, False, False)])
+def test_head_leaves_the_best_column_of_every_tile_and_greedy_rows_choose_from_them(rows, n_out, k_dim, limit, packed, bias):
+    """The logits are those of the plain product; every tile's best is the plain argmax over the
+    tile's columns below the limit (the lowest column among equals: two rows of the matrix are the
+    same, inside a tile and across tiles); and greedy rows that read the tiles' bests choose what
+    they choose from the logits themselves, beside seeded rows that still read the logits."""
+    g = torch.Generator().manual_seed(rows * 7 + n_out)
+    a = rnd(g, rows, k_dim, dtype="bfloat16")
+    w = rnd(g, n_out, k_dim, dtype="bfloat16", scale=0.1)
+    w[17] = w[21]                          # equal logits within a tile
+    w[n_out - 40] = w[3]                   # and in two tiles far apart
+    a[0] = (w[3].float() * 8).bfloat16()   # row 0 points at them: its largest logits are the equal pair
+    if rows > 1:
+        a[-1] = (w[n_out - 1].float() * 8).bfloat16()   # the last row's largest logit lies past the limit (if limit < n_out)
+    b = rnd(g, n_out, scale=0.1) if bias else None
+    if bias:
+        b[17], b[n_out - 40] = b[21], b[3]
+    out = torch.full((rows, n_out), float("nan"), device=DEV)
+    tiles = n_out // 16
+    bv = torch.full((rows + 2, tiles), float("nan"), device=DEV)
+    bi = torch.full((rows + 2, tiles), -3, dtype=torch.int32, device=DEV)
+    wd = w.to(DEV)
+    assert kernels.linear_head_best(a.to(DEV), wd, None if b is None else b.to(DEV), out, rows, bv, bi, limit,
+                                    w_packed=kernels.pack_weight(wd) if packed else None)
+    want = _linear_want(a, w, b, kernels.EPI_NONE, None)
+    helpers.assert_close(out, want, "bfloat16", "head")
+    # the tiles' bests are exact statements about the logits that were stored
+    got = out.cpu()
+    masked = got.clone()
+    masked[:, limit:] = -float("inf")
+    per_tile = masked.view(rows, tiles, 16)
+    want_val, want_off = per_tile.max(dim=2)
+    first = (per_tile == want_val.unsqueeze(2)).int().argmax(dim=2)     # the lowest column among equals
+    want_idx = first + 16 * torch.arange(tiles).unsqueeze(0)
+    live = torch.isfinite(want_val)       # a tile wholly past the limit holds -inf and no column
+    assert torch.equal(bv[:rows].cpu()[live], want_val[live])
+    assert torch.equal(bi[:rows].cpu()[live].long(), want_idx[live])
+    assert (bv[:rows].cpu()[~live] == -float("inf")).all()
+    assert torch.isnan(bv[rows:]).all() and (bi[rows:] == -3).all()
+    # choosing from them
+    temps = [0.0] * rows
+    if rows > 2:
+        temps[1] = 0.8
+    tk = torch.tensor(temps, device=DEV)
+    seeds = torch.arange(rows, dtype=torch.int64, device=DEV)
+    idx = torch.zeros(rows, dtype=torch.int32, device=DEV)
+    from_logits = torch.full((rows,), -1, dtype=torch.int32, device=DEV)
+    from_tiles = torch.full((rows,), -1, dtype=torch.int32, device=DEV)
+    kernels.sample(out, rows, limit, tk, None, None, seeds, idx, 5, from_logits)
+    kernels.sample(out, rows, limit, tk, None, None, seeds, idx, 5, from_tiles, tile_best=(bv, bi))
+    assert torch.equal(from_logits, from_tiles)
+    plain = [P.plain_sample(got[r].numpy(), 0.0, None, None, 0.0, limit)[0] for r in range(rows) if temps[r] == 0.0]
+    assert [t for t, temp in zip(from_tiles.cpu().tolist(), temps) if temp == 0.0] == plain
+    assert from_tiles[0].item() == 3 and from_tiles[-1].item() < limit
+
+
+def test_head_with_tile_bests_refuses_what_its_kernel_does_not_take():
+    g = torch.Generator().manual_seed(4)
+    for rows, n_out, k_dim in ((17, 208, 64), (4, 200, 64), (4, 208, 48)):
+        a, w = rnd(g, rows, k_dim, dtype="bfloat16").to(DEV), rnd(g, n_out, k_dim, dtype="bfloat16").to(DEV)
+        out = torch.zeros(rows, n_out, device=DEV)
+        tiles = max(n_out // 16, 1)
+        bv, bi = torch.zeros(rows, tiles, device=DEV), torch.zeros(rows, tiles, dtype=torch.int32, device=DEV)
+        assert not kernels.linear_head_best(a, w, None, out, rows, bv, bi, n_out)
+        assert (out == 0).all()
+
+
 def test_sampling_prepares_the_next_decode_step_on_the_device():
     """Greedy and seeded rows; two cache groups with pages of 4 and 8 slots; a padded row is left alone;
     a position past the block table's end gets slot -1."""
