@@ -107,8 +107,11 @@ FOLD_MAX_ROWS = 32
 FOLD_MAX_OUT = 4096
 # ... except at few rows, where the LayerNorm kernel's own launch costs more than the conversion
 # (the GPT-2-XL shape, outputs of 4800 and 6400: 957 us a step of 24 layers against 1062 at one
-# row, 1361 against 1399 at 16 rows, 1923 against 1741 at 32)
+# row, 1361 against 1399 at 16 rows, 1923 against 1741 at 32), but not under an output as wide as a
+# vocabulary: every one of its thousands of workgroups would norm the rows again ([50257 x 1600] at
+# one row: 43.5 us with the fold, 30.0 without, and the LayerNorm kernel takes 3)
 FOLD_ANY_OUT_MAX_ROWS = 16
+FOLD_ANY_OUT_MAX_OUT = 8192
 # A very wide output (the head, 8192 columns and more) goes to the decode kernel while rows x inner
 # size stays within this, and to the tiled kernel beyond: that one streams the matrix at nearly the
 # same rate whatever the rows (50304 x 512: 10.2 us at 1 row, 11.4 at 32, 14.0 at 64), the decode
@@ -164,7 +167,8 @@ def linear(ctx, a: Union[torch.Tensor, LazyNorm], w: torch.Tensor, bias: Optiona
     if fast and n_rows <= 64 and not wide_out:
         epi = kernels.SK_EPI_QKV if scatter is not None else epilogue
         if (isinstance(a, LazyNorm) and getattr(a.norm, "fusable_layer_norm", False) and a._tensor is None
-                and (w.shape[0] <= FOLD_MAX_OUT or n_rows <= FOLD_ANY_OUT_MAX_ROWS)
+                and (w.shape[0] <= FOLD_MAX_OUT
+                     or (n_rows <= FOLD_ANY_OUT_MAX_ROWS and w.shape[0] <= FOLD_ANY_OUT_MAX_OUT))
                 and (n_rows <= FOLD_MAX_ROWS or kernels.linear_skinny_row_groups(n_rows, w.shape[0], w.shape[1]))):
             wf, colsum, bias_f = folded_layer_norm(a.norm, w, bias)
             if kernels.linear_skinny(None, wf, bias_f, out, n_rows, epi, ln_x=a.x, ln_colsum=colsum,
