@@ -25,6 +25,8 @@ struct FusedResidual {
 };
 
 #define FUSED_MAX_WIDTH 512    // wider rows bring more parts than a reader can add up on its way in
+#define RESIDUAL_MAX_WIDTH 4096  // the widest row that the kernels which only add a pending residual up (LayerNorm,
+                                 // settle) take: a workgroup's threads hold four values each
 #define FUSED_GROUP_PARTS 4    // parts of a row that one thread of a workgroup adds up
 #define FUSED_THREADS 1024
 #define FUSED_WAVES 16

@@ -869,6 +869,8 @@ __global__ __launch_bounds__(FUSED_THREADS) void residual_layernorm_kernel(Fused
   const float4 gain4 = reinterpret_cast<const float4*>(gain)[vc];
   const float4 beta4 = fd_keep4(beta != nullptr, reinterpret_cast<const float4*>(beta ? beta : gain)[vc]);
   const float4 xv = fd_row_sum<false>(res, V, G, L, xs);
+  // (this workgroup is the row's only reader in this launch: the sum may go where the base was)
+  if (res.settled && tid < V) reinterpret_cast<float4*>(res.settled + row * width)[tid] = xv;
   const float4 y = fd_row_norm(xv, V, width, eps, gain4, beta4, mean_s, var_s);
   if (tid < V) {
     OT* orow = out + (long)i * width;
@@ -898,8 +900,8 @@ __global__ __launch_bounds__(256) void residual_settle_kernel(FusedResidual res,
 
 // What every launcher checks of a residual that is still a sum.  tables_ok: the kernel can look the
 // rows up in the token and position tables itself.
-static int check_residual(const FusedResidual& r, int width, bool tables_ok) {
-  if (width <= 0 || (width % 32) != 0 || width > FUSED_MAX_WIDTH) return MGPT_ERR_BAD_SHAPE;
+static int check_residual(const FusedResidual& r, int width, bool tables_ok, int max_width = FUSED_MAX_WIDTH) {
+  if (width <= 0 || (width % 32) != 0 || width > max_width) return MGPT_ERR_BAD_SHAPE;
   if (!r.base) {
     if (!tables_ok || r.n_parts != 0) return MGPT_ERR_BAD_SHAPE;
     if (!r.tok_table || !r.ids || (r.pos_table && !r.positions)) return MGPT_ERR_NULL;
@@ -922,6 +924,12 @@ static FusedResidual make_residual(const float* base, const float* partials, int
   r.tok_table = (const bf16_t*)tok_table; r.pos_table = (const bf16_t*)pos_table; r.ids = ids;
   r.positions = positions; r.settled = settled;
   return r;
+}
+
+// Most parts of a pending residual of this width that mgpt_residual_layernorm takes (0: the width is not taken).
+extern "C" int mgpt_residual_parts_limit(int width) {
+  if (width <= 0 || (width % 32) != 0 || width > RESIDUAL_MAX_WIDTH) return 0;
+  return group_parts_limit(width);
 }
 
 // Most parts of a pending residual of this width that the fused kernels take (0: the width is not taken).
@@ -1039,17 +1047,19 @@ extern "C" int mgpt_fused_mlp_parts(int hidden) {
   return (hidden > 0 && (hidden % FUSED_MLP_SLICE) == 0) ? hidden / FUSED_MLP_SLICE : 0;
 }
 
-// out[i] = LayerNorm of row rows[i] (or i) of a residual that is still a sum (with a base); out float32 or bfloat16
+// out[i] = LayerNorm of row rows[i] (or i) of a residual that is still a sum (with a base); out float32 or
+// bfloat16.  settled (optional; may be the base): the rows' sums are stored there as well, row by row
+// as named by rows[].  Widths up to RESIDUAL_MAX_WIDTH, at most mgpt_residual_parts_limit(width) parts.
 extern "C" int mgpt_residual_layernorm(const float* base, const float* partials, int n_parts, long part_stride,
                                        const void* tok_table, const void* pos_table, const int* ids,
                                        const int* token_positions, const float* gain, const float* beta,
                                        float eps, const int* rows, void* out, int out_dtype, int n_rows, int width,
-                                       hipStream_t stream) {
+                                       float* settled, hipStream_t stream) {
   if (n_rows == 0) return MGPT_OK;
   if (!gain || !out) return MGPT_ERR_NULL;
   const FusedResidual r = make_residual(base, partials, n_parts, part_stride, tok_table, pos_table, ids,
-                                        token_positions, nullptr);
-  int rc = check_residual(r, width, false);
+                                        token_positions, settled);
+  int rc = check_residual(r, width, false, RESIDUAL_MAX_WIDTH);
   if (rc != MGPT_OK) return rc;
   if (n_rows < 0 || n_parts > group_parts_limit(width) || (((size_t)out | (size_t)gain | (size_t)beta) & 15) != 0)
     return MGPT_ERR_BAD_SHAPE;
@@ -1072,7 +1082,7 @@ extern "C" int mgpt_residual_settle(const float* base, const float* partials, in
   if (!settled) return MGPT_ERR_NULL;
   const FusedResidual r = make_residual(base, partials, n_parts, part_stride, tok_table, pos_table, ids,
                                         token_positions, settled);
-  int rc = check_residual(r, width, false);
+  int rc = check_residual(r, width, false, RESIDUAL_MAX_WIDTH);
   if (rc != MGPT_OK) return rc;
   if (n_rows < 0) return MGPT_ERR_BAD_SHAPE;
   const long total = (long)n_rows * (width / 4);

@@ -62,8 +62,8 @@ int mgpt_fused_mlp_decode(const float* base, const float* partials, int n_parts,
 // fused_decode.hip
 int mgpt_residual_layernorm(const float* base, const float* partials, int n_parts, long part_stride, const
     void* tok_table, const void* pos_table, const int* ids, const int* token_positions, const float* gain,
-    const float* beta, float eps, const int* rows, void* out, int out_dtype, int n_rows, int width,
-    hipStream_t stream);
+    const float* beta, float eps, const int* rows, void* out, int out_dtype, int n_rows, int width, float*
+    settled, hipStream_t stream);
 // fused_decode.hip
 int mgpt_residual_settle(const float* base, const float* partials, int n_parts, long part_stride, const void*
     tok_table, const void* pos_table, const int* ids, const int* token_positions, float* settled, int n_rows,
@@ -93,6 +93,9 @@ int mgpt_linear_skinny(const void* act, long lda, const float* x, const int* row
 int mgpt_linear_head_best(const void* act, long lda, const float* x, const int* rows, const float* colsum,
     float eps, const void* w, const void* w_packed, const float* bias, float* out, long ldo, int n_rows, int
     n_out, int k_dim, float* best_val, int* best_idx, int best_limit, hipStream_t stream);
+// linear_decode_rows.hip
+int mgpt_linear_decode_parts(const void* act, long lda, const void* w, const void* w_packed, const float* bias,
+    float* partials, int n_rows, int n_out, int k_dim, hipStream_t stream);
 // sampling.hip
 int mgpt_sample(const float* logits, long ld, int n_rows, int vocab, int real_vocab, const float* temperature,
     const int* top_k, const float* top_p, const uint64_t* request_seed, const int* out_index, uint64_t
@@ -129,5 +132,6 @@ int mgpt_sample_advance(const float* logits, long ld, int n_rows, int vocab, int
   X(mgpt_linear_mfma_qkv) \
   X(mgpt_linear_skinny) \
   X(mgpt_linear_head_best) \
+  X(mgpt_linear_decode_parts) \
   X(mgpt_sample) \
   X(mgpt_sample_advance)

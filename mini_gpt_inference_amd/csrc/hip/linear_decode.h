@@ -69,7 +69,7 @@ __global__ __launch_bounds__(256) void linear_decode_kernel(SkinnyArgs a) {
     for (int i = 0; i < 4; ++i) old4[t][i] = 0.f;
   }
   OT* const out = reinterpret_cast<OT*>(a.out);
-  if (col_writer && !SPLIT) {
+  if (col_writer && (!SPLIT || (a.bias_in_part0 && part == 0))) {
     if (VEC) {
       if (a.bias != nullptr) {
         const float4 b4 = *reinterpret_cast<const float4*>(a.bias + oc);
@@ -232,7 +232,9 @@ __global__ __launch_bounds__(256) void linear_decode_kernel(SkinnyArgs a) {
     for (int t = 0; t < NT; ++t) {
       if (!row_ok[t]) continue;
       float* prow = a.partials + ((long)part * a.n_rows + r0 + t * 16) * a.n_out + oc;
-      *reinterpret_cast<float4*>(prow) = make_float4(acc[t][0], acc[t][1], acc[t][2], acc[t][3]);
+      // (the bias is zero unless this part carries it)
+      *reinterpret_cast<float4*>(prow) = make_float4(acc[t][0] + bias4[0], acc[t][1] + bias4[1], acc[t][2] + bias4[2],
+                                                     acc[t][3] + bias4[3]);
     }
     return;
   }

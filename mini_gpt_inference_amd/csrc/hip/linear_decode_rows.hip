@@ -1,5 +1,6 @@
 // linear_decode.h's kernel for 17 to 64 rows: two to four tiles of 16 rows share the W a lane loads.
 #include "linear_decode.h"
+#include "launchers.h"
 
 template <int NT>
 static int launch_tiles(const SkinnyArgs& a, int epilogue, int out_dtype, hipStream_t s) {
@@ -89,15 +90,22 @@ __global__ __launch_bounds__(256) void linear_partials_epilogue_kernel(
   }
 }
 
+// the first of the split's two kernels: every workgroup's sums to a.partials
 template <int NT>
-static int launch_split(const SkinnyArgs& a0, int epilogue, int out_dtype, hipStream_t s) {
-  SkinnyArgs a = a0;
-  a.k_parts = LDR_PARTS;
+static int launch_split_parts(const SkinnyArgs& a, hipStream_t s) {
   const int per = (a.k_dim / 32 / LDR_PARTS + 3) / 4;
   dim3 grid((a.n_out / 16) * LDR_PARTS);
   if (per <= 4) hipLaunchKernelGGL((linear_decode_kernel<NT, 4, false, SK_EPI_NONE, float, true, true>), grid, dim3(256), 0, s, a);
   else hipLaunchKernelGGL((linear_decode_kernel<NT, 8, false, SK_EPI_NONE, float, true, true>), grid, dim3(256), 0, s, a);
-  int rc = mgpt_last_error();
+  return mgpt_last_error();
+}
+
+template <int NT>
+static int launch_split(const SkinnyArgs& a0, int epilogue, int out_dtype, hipStream_t s) {
+  SkinnyArgs a = a0;
+  a.k_parts = LDR_PARTS;
+  a.bias_in_part0 = 0;
+  int rc = launch_split_parts<NT>(a, s);
   if (rc != MGPT_OK) return rc;
   dim3 egrid((a.n_rows * (a.n_out / 4) + 255) / 256);
 #define LDR_EPI(E, OT) \
@@ -110,6 +118,35 @@ static int launch_split(const SkinnyArgs& a0, int epilogue, int out_dtype, hipSt
 #undef LDR_EPI
   return mgpt_last_error();
 }
+
+// The split's first kernel alone: partials[p][row][column], p < mgpt_linear_decode_parts_count(), are
+// the sums over the p-th quarter of the inner size, the first with the bias added, and nobody adds
+// them up here: the caller leaves them to whoever reads the sum next (a residual stream kept as
+// base + parts, fused_decode.h).  Takes what mgpt_linear_decode_partials(..., SK_EPI_RESIDUAL) splits
+// (bfloat16 rows, up to 64 of them); partials must hold that many floats.  MGPT_ERR_BAD_SHAPE otherwise.
+extern "C" int mgpt_linear_decode_parts(const void* act, long lda, const void* w, const void* w_packed,
+                                        const float* bias, float* partials, int n_rows, int n_out, int k_dim,
+                                        hipStream_t stream) {
+  if (n_rows == 0 || n_out == 0) return MGPT_OK;
+  if (!act || !w || !partials) return MGPT_ERR_NULL;
+  if (n_rows < 0 || lda < k_dim || (lda % 8) != 0 ||
+      ((((size_t)act) | ((size_t)w) | ((size_t)w_packed) | ((size_t)bias) | ((size_t)partials)) & 15) != 0 ||
+      mgpt_linear_decode_partials(n_rows, n_out, k_dim, false, SK_EPI_RESIDUAL, 0) <= 0)
+    return MGPT_ERR_BAD_SHAPE;
+  SkinnyArgs a = {};
+  a.act = (const bf16_t*)act; a.lda = lda; a.w = (const bf16_t*)w; a.w_packed = (const bf16_t*)w_packed;
+  a.bias = bias; a.out = partials; a.ldo = n_out; a.n_rows = n_rows; a.n_out = n_out; a.k_dim = k_dim;
+  a.ksplit = 1; a.partials = partials; a.k_parts = LDR_PARTS; a.bias_in_part0 = 1; a.rows_per_group = 16;
+  switch ((n_rows + 15) / 16) {
+    case 1: return launch_split_parts<1>(a, stream);
+    case 2: return launch_split_parts<2>(a, stream);
+    case 3: return launch_split_parts<3>(a, stream);
+    case 4: return launch_split_parts<4>(a, stream);
+    default: return MGPT_ERR_BAD_SHAPE;
+  }
+}
+
+extern "C" int mgpt_linear_decode_parts_count() { return LDR_PARTS; }
 
 int mgpt_launch_linear_decode_rows(const SkinnyArgs& a, int epilogue, int out_dtype, hipStream_t stream) {
   const int nt = (a.n_rows + 15) / 16;

@@ -34,6 +34,7 @@ struct SkinnyArgs {
   // partials[part][row][column] and a second kernel adds them and applies the epilogue
   float* partials;
   int k_parts;
+  int bias_in_part0;  // with the split: the first part carries the bias (nobody adds it afterwards)
   // more than 16 rows in linear_decode.hip: 0 = the launcher chooses, SK_ROWS_SHARE_W = one workgroup
   // per column tile takes all rows, SK_ROWS_GROUPS = one workgroup per column tile and 16 rows
   int rows_mode;

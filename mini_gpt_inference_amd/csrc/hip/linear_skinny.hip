@@ -356,6 +356,7 @@ static int linear_skinny_launch(const void* act, long lda, const float* x, const
   a.slot_mapping = slot_mapping; a.q_width = q_width; a.kv_width = kv_width; a.head_dim = head_dim;
   a.n_kv_head = n_kv_head; a.page_size = page_size;
   a.best_val = best_val; a.best_idx = best_idx; a.best_limit = best_limit;
+  a.bias_in_part0 = 0;
   // room for the parts of a split over workgroups, if the caller brought enough of it
   a.k_parts = 1;
   a.rows_mode = ((mode & 0xFF) == SK_ROWS_SHARE_W || (mode & 0xFF) == SK_ROWS_GROUPS) ? (mode & 0xFF) : 0;

@@ -10,7 +10,7 @@ from __future__ import annotations
 
 import contextlib
 import ctypes
-from typing import Optional
+from typing import Dict, Optional
 
 import torch
 
@@ -433,6 +433,36 @@ def linear_head_best(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tens
     return True
 
 
+def linear_decode_parts(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], partials: torch.Tensor,
+                        n_rows: int, w_packed: Optional[torch.Tensor] = None) -> int:
+    """The split product's first half alone: partials[p, :n_rows] (float32 [parts, n_rows, out], dense)
+    = a[:n_rows] @ w[:, stretch p of the inner size].T, the first with the bias added; nobody adds them
+    up.  Returns the number of parts, or 0, having launched nothing, for a shape that linear_skinny
+    would not split (linear_skinny_partials(n_rows, out, inner, False, EPI_RESIDUAL) == 0)."""
+    n_out, k_dim = w.shape
+    if (w.dtype != torch.bfloat16 or a.dtype != torch.bfloat16 or a.stride(0) % 8 or a.data_ptr() % 16
+            or not linear_skinny_partials(n_rows, n_out, k_dim, False, EPI_RESIDUAL)):
+        return 0
+    parts = int(library.kernels().mgpt_linear_decode_parts_count())
+    _need_cuda(a, w, bias, partials, w_packed)
+    _need(w.is_contiguous(), "weight must be dense [out, in]")
+    _need(a.dim() == 2 and a.stride(1) == 1 and a.shape[1] == k_dim and a.shape[0] >= n_rows,
+          "activation must be [>=n_rows, inner] with unit inner stride")
+    _need(bias is None or (bias.dtype == torch.float32 and bias.numel() == n_out and bias.data_ptr() % 16 == 0),
+          "bias must be aligned float32 [out]")
+    _need(partials.dtype == torch.float32 and partials.is_contiguous() and partials.data_ptr() % 16 == 0
+          and tuple(partials.shape) == (parts, n_rows, n_out), f"partials must be dense float32 [{parts}, n_rows, out]")
+    if w_packed is not None:
+        _need(w_packed.dtype == torch.bfloat16 and w_packed.is_contiguous() and w_packed.numel() == n_out * k_dim
+              and w_packed.data_ptr() % 16 == 0, "w_packed must be pack_weight(w)")
+    rc = library.kernels().mgpt_linear_decode_parts(_ptr(a), a.stride(0), _ptr(w), _ptr(w_packed), _ptr(bias),
+                                                    _ptr(partials), n_rows, n_out, k_dim, _stream())
+    if rc == -2:
+        return 0
+    _check(rc, "linear_decode_parts")
+    return parts
+
+
 def linear_skinny_row_groups(n_rows: int, n_out: int, k_dim: int) -> bool:
     """Whether linear_skinny, left to choose, gives every 16 of these rows workgroups of their own
     (a folded LayerNorm then costs a workgroup what it costs at 16 rows)."""
@@ -764,14 +794,33 @@ def fused_mlp_decode(pending, settled: torch.Tensor, gain: torch.Tensor, beta: O
     return True
 
 
+RESIDUAL_MAX_WIDTH = 4096
+_RESIDUAL_PARTS_LIMIT: Dict[int, int] = {}
+
+
+def residual_parts_limit(width: int) -> int:
+    """Most parts of a pending residual of this width that residual_layer_norm adds up (0: the width
+    is not taken).  Wider than the fused kernels take: a row up to RESIDUAL_MAX_WIDTH."""
+    hit = _RESIDUAL_PARTS_LIMIT.get(width)
+    if hit is None:
+        hit = _RESIDUAL_PARTS_LIMIT[width] = int(library.kernels().mgpt_residual_parts_limit(int(width)))
+    return hit
+
+
 def residual_layer_norm(pending, gain: torch.Tensor, beta: Optional[torch.Tensor], eps: float,
-                        rows: Optional[torch.Tensor], out: torch.Tensor, n_rows: int) -> bool:
-    """out[i] = LayerNorm of row rows[i] (or i) of a residual that is still a sum.  False if the
-    width is not taken."""
+                        rows: Optional[torch.Tensor], out: torch.Tensor, n_rows: int,
+                        settled: Optional[torch.Tensor] = None) -> bool:
+    """out[i] = LayerNorm of row rows[i] (or i) of a residual that is still a sum.  With `settled`
+    (float32 rows; may be the sum's base itself) the rows' sums are stored there too.  False if
+    the width is not taken."""
     width = gain.numel()
-    if width % 32 or width > FUSED_MAX_WIDTH or pending.base is None or pending.n_parts > fused_parts_limit(width):
+    if width % 32 or width > RESIDUAL_MAX_WIDTH or pending.base is None or pending.n_parts > residual_parts_limit(width):
         return False
-    _need_cuda(gain, beta, rows, out)
+    _need_cuda(gain, beta, rows, out, settled)
+    _need(settled is None or (settled.dtype == torch.float32 and settled.is_contiguous() and settled.shape[1] == width
+                              and settled.shape[0] >= (n_rows if rows is None else 0) and settled.data_ptr() % 16 == 0),
+          "the settled rows must be dense float32 of the residual's width")
+    _need(settled is None or rows is None, "settling through a row gather is not supported")
     args = _residual_args(pending, width)
     _need(gain.dtype == torch.float32 and (beta is None or (beta.dtype == torch.float32 and beta.numel() == width)),
           "gain and beta must be float32 [width]")
@@ -781,7 +830,7 @@ def residual_layer_norm(pending, gain: torch.Tensor, beta: Optional[torch.Tensor
     else:
         _need_i32("rows", rows, n_rows)
     rc = library.kernels().mgpt_residual_layernorm(*args, _ptr(gain), _ptr(beta), float(eps), _ptr(rows), _ptr(out),
-                                                   _dtype_code(out), n_rows, width, _stream())
+                                                   _dtype_code(out), n_rows, width, _ptr(settled), _stream())
     if rc == -2:
         return False
     _check(rc, "residual_layer_norm")
@@ -792,7 +841,7 @@ def residual_settle(pending, settled: torch.Tensor, n_rows: int) -> bool:
     """settled[:n_rows] = the rows of a residual that is still a sum (settled may be its base).
     False if the width is not taken."""
     width = settled.shape[1]
-    if width % 32 or width > FUSED_MAX_WIDTH or pending.base is None:
+    if width % 32 or width > RESIDUAL_MAX_WIDTH or pending.base is None:
         return False
     _need_cuda(settled)
     args = _residual_args(pending, width)

@@ -139,7 +139,10 @@ def _declare_optional(lib: ctypes.CDLL) -> None:
         "mgpt_fused_attention_decode": [P, P, I, L, P, P, P, P, P, P, P, F, P, P, P, P, P, L, P, P, P, P, I, P, P,
                                         I, I, I, I, I, I, F, P],
         "mgpt_fused_mlp_decode": [P, P, I, L, P, P, P, P, P, P, P, F, P, P, P, P, P, L, I, I, I, P],
-        "mgpt_residual_layernorm": [P, P, I, L, P, P, P, P, P, P, F, P, P, I, I, I, P],
+        "mgpt_residual_layernorm": [P, P, I, L, P, P, P, P, P, P, F, P, P, I, I, I, P, P],
+        "mgpt_residual_parts_limit": [I],
+        "mgpt_linear_decode_parts": [P, L, P, P, P, P, I, I, I, P],
+        "mgpt_linear_decode_parts_count": [],
         "mgpt_residual_settle": [P, P, I, L, P, P, P, P, P, I, I, P],
         "mgpt_fused_parts_limit": [I],
     }

@@ -24,12 +24,17 @@ class LazyNorm:
             h = ctx.workspace.get(self.buffer, self.n_rows, self.x.shape[1], ctx.dtype)
             pending = getattr(ctx, "pending", None)
             if pending is not None:
-                # the residual is still a sum: a LayerNorm adds it up on its way in, anything else
-                # needs plain rows first
+                # the residual is still a sum: a LayerNorm adds it up on its way in (and, where it
+                # goes over all the step's rows, stores the sums: the residual is plain again),
+                # anything else needs plain rows first
                 norm = self.norm
-                if not (getattr(norm, "fusable_layer_norm", False)
+                all_rows = self.rows is None and self.n_rows >= ctx.n_rows
+                if (getattr(norm, "fusable_layer_norm", False)
                         and kernels.residual_layer_norm(pending, norm.weight, norm.bias, norm.eps, self.rows, h,
-                                                        self.n_rows)):
+                                                        self.n_rows, settled=self.x if all_rows else None)):
+                    if all_rows:
+                        ctx.pending = None
+                else:
                     residual.settle(ctx, self.x, ctx.n_rows)
                     pending = None
             if pending is None:
@@ -135,6 +140,50 @@ class TileBest:
         self.values: Optional[torch.Tensor] = None
         self.columns: Optional[torch.Tensor] = None
         self.filled = False
+
+
+# A split product's parts are left pending for rows this wide, or this many: the LayerNorm kernel
+# that then adds them up is one workgroup per row, and for one narrow row costs more than the
+# kernel that adds the parts plus the folded LayerNorm it replaces (decode steps on one box, us:
+# width 768: 296 against 284 at one row, 333 against 336 at 8, 365 against 369 at 16; width 1600:
+# 1748 against 1768, 2049 against 2102, 2439 against 2554)
+LEAVE_PARTS_MIN_WIDTH = 1024
+LEAVE_PARTS_MIN_ROWS = 8
+
+
+def plain_residual(ctx, h, x: torch.Tensor) -> None:
+    """Makes the residual rows x plain for a part that reads or adds to them with ordinary kernels.
+    If they are still a sum and h is the LayerNorm of them that the part is about to read, that
+    LayerNorm is computed now: its kernel adds the sum up and stores it on the way."""
+    if getattr(ctx, "pending", None) is None:
+        return
+    if isinstance(h, LazyNorm) and h.x is x and h._tensor is None:
+        h.tensor(ctx)
+    residual.settle(ctx, x, ctx.n_rows)
+
+
+def linear_add(ctx, a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], x: torch.Tensor, n_rows: int,
+               may_leave_parts: bool = False) -> None:
+    """x[:n_rows] += a[:n_rows] @ w.T (+ bias), x the float32 residual stream.
+
+    may_leave_parts: the caller and whoever reads x next know of ctx.pending.  Then a product whose
+    long inner size is split over workgroups anyway (few rows, few column tiles) leaves the
+    workgroups' sums as the parts of a pending residual instead of running a second kernel that adds
+    them into x; the LayerNorm that reads x next adds them up (LazyNorm.tensor)."""
+    if (may_leave_parts and getattr(ctx, "pending", None) is None and not ctx.exact and ctx.dtype == torch.bfloat16
+            and w.dtype == torch.bfloat16 and a.dtype == torch.bfloat16 and 0 < n_rows <= 64 and n_rows == ctx.n_rows
+            and x.is_contiguous() and x.shape[1] == w.shape[0]
+            and (w.shape[0] >= LEAVE_PARTS_MIN_WIDTH or n_rows >= LEAVE_PARTS_MIN_ROWS)
+            and kernels.residual_parts_limit(w.shape[0]) >= 4
+            and kernels.linear_skinny_partials(n_rows, w.shape[0], w.shape[1], False, kernels.EPI_RESIDUAL)):
+        buf = ctx.workspace.get("residual_parts", 4 * n_rows, w.shape[0], torch.float32)
+        parts = buf[:4 * n_rows].view(4, n_rows, w.shape[0])
+        n_parts = kernels.linear_decode_parts(a, w, bias, parts, n_rows, w_packed=packed_weight(w))
+        if n_parts:
+            assert n_parts == 4
+            ctx.pending = residual.PendingSums(x, parts, n_parts)
+            return
+    linear(ctx, a, w, bias, x, n_rows, kernels.EPI_RESIDUAL)
 
 
 def linear(ctx, a: Union[torch.Tensor, LazyNorm], w: torch.Tensor, bias: Optional[torch.Tensor],

@@ -7,7 +7,7 @@ from typing import Dict
 import torch
 
 from ..ops import kernels, residual
-from ..ops.linear import LazyNorm, linear, packed_weight
+from ..ops.linear import LazyNorm, linear, linear_add, packed_weight, plain_residual
 from .base import MATRIX, Part, StepContext, VECTOR, WeightRequest, register_feed_forward
 
 _ACTIVATIONS = {"gelu_tanh": kernels.EPI_GELU}
@@ -76,8 +76,10 @@ class DenseMLP(FeedForward):
     def forward_add(self, ctx: StepContext, h: torch.Tensor, x: torch.Tensor) -> None:
         if self._forward_add_fused(ctx, h, x):
             return
-        residual.settle(ctx, x, ctx.n_rows)
+        plain_residual(ctx, h, x)
         n = ctx.n_rows
         u = ctx.workspace.get("ff_hidden", n, self.hidden, ctx.dtype)
         linear(ctx, h, self.fc_weight, self.fc_bias, u, n, _ACTIVATIONS[self.activation])
-        linear(ctx, u, self.proj_weight, self.proj_bias, x, n, kernels.EPI_RESIDUAL)
+        # (a caller that hands over a LazyNorm of x itself knows that x may be left as a sum)
+        linear_add(ctx, u, self.proj_weight, self.proj_bias, x, n,
+                   may_leave_parts=isinstance(h, LazyNorm) and h.x is x)

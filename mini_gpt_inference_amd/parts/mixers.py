@@ -8,7 +8,7 @@ import torch
 
 from ..ops import attention as attention_ops
 from ..ops import kernels, residual
-from ..ops.linear import LazyNorm, linear, packed_weight
+from ..ops.linear import LazyNorm, linear, linear_add, packed_weight, plain_residual
 from .base import (CacheBinding, KVNeed, MATRIX, Part, StateNeed, StepContext, VECTOR, WeightRequest,
                    register_mixer)
 from .positions import PositionEncoding
@@ -104,7 +104,7 @@ class PagedCausalAttention(Mixer):
                     position: PositionEncoding) -> None:
         if self._forward_add_fused(ctx, h, x, binding, position):
             return
-        residual.settle(ctx, x, ctx.n_rows)
+        plain_residual(ctx, h, x)
         n = ctx.n_rows
         total = self.q_width + 2 * self.kv_width
         qkv = ctx.workspace.get("qkv", n, total, ctx.dtype)
@@ -122,4 +122,5 @@ class PagedCausalAttention(Mixer):
                              group.slot_mapping, n)
         y = ctx.workspace.get("attn_out", n, self.q_width, ctx.dtype)
         attention_ops.paged_attention(ctx, qkv, y, k_pool, v_pool, group, self.n_head, self.scale, self.window)
-        linear(ctx, y, self.proj_weight, self.proj_bias, x, n, kernels.EPI_RESIDUAL)
+        linear_add(ctx, y, self.proj_weight, self.proj_bias, x, n,
+                   may_leave_parts=isinstance(h, LazyNorm) and h.x is x)

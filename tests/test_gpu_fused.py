@@ -175,7 +175,8 @@ def test_fused_mlp_decode(case):
 
 
 @pytest.mark.parametrize("out_dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("c,parts,bias", [(512, 32, True), (96, 3, False), (64, 0, True), (320, 12, True), (32, 100, True)])
+@pytest.mark.parametrize("c,parts,bias", [(512, 32, True), (96, 3, False), (64, 0, True), (320, 12, True), (32, 100, True),
+                                          (768, 20, True), (1600, 4, True), (1600, 8, False), (4096, 4, True), (2080, 0, True)])
 def test_residual_layer_norm_and_settle(c, parts, bias, out_dtype):
     g = torch.Generator().manual_seed(300 + c)
     rows = 7
@@ -191,13 +192,92 @@ def test_residual_layer_norm_and_settle(c, parts, bias, out_dtype):
     out2 = torch.full((4, c), float("nan"), dtype=tdt, device=DEV)
     assert kernels.residual_layer_norm(pending, dev(gain), dev(beta), 1e-5, i32(pick), out2, 4)
     helpers.assert_close(out2, want[pick], out_dtype, "LayerNorm of chosen rows of a pending residual")
+    # the LayerNorm that goes over all rows can store the sums on its way: into another array ...
+    out3 = torch.full((rows, c), float("nan"), dtype=tdt, device=DEV)
+    stored = torch.full((rows + 2, c), float("nan"), device=DEV)
+    assert kernels.residual_layer_norm(pending, dev(gain), dev(beta), 1e-5, None, out3, rows, settled=stored)
+    assert torch.equal(out3, out)
+    helpers.assert_close(stored[:rows], true, "float32", "sums stored by the LayerNorm")
+    assert torch.isnan(stored[rows:]).all()
     # the sum itself: into another array, and into the base
     settled = torch.full((rows + 2, c), float("nan"), device=DEV)
     assert kernels.residual_settle(pending, settled, rows)
     helpers.assert_close(settled[:rows], true, "float32", "settle")
     assert torch.isnan(settled[rows:]).all()
+    # ... and into the base itself (a workgroup is the only reader of its row)
+    keep = pending.base.clone()
+    out4 = torch.full((rows, c), float("nan"), dtype=tdt, device=DEV)
+    assert kernels.residual_layer_norm(pending, dev(gain), dev(beta), 1e-5, None, out4, rows, settled=pending.base)
+    assert torch.equal(out4, out) and torch.equal(pending.base[:rows], stored[:rows])
+    pending.base.copy_(keep)
     assert kernels.residual_settle(pending, pending.base, rows)
     helpers.assert_close(pending.base[:rows], true, "float32", "settle in place")
+
+
+def test_residual_kernels_say_which_widths_and_parts_they_take():
+    assert kernels.residual_parts_limit(512) == 32 and kernels.residual_parts_limit(1600) == 8
+    assert kernels.residual_parts_limit(4096) == 4 and kernels.residual_parts_limit(4128) == 0
+    assert kernels.residual_parts_limit(1616) == 0          # no multiple of 32
+    g = torch.Generator().manual_seed(9)
+    for c, parts in ((1600, 9), (4128, 1), (1616, 1)):
+        base = rnd(g, 2, c).to(DEV)
+        pending = PendingSums(base, rnd(g, parts, 2, c).to(DEV), parts)
+        out = torch.full((2, c), 7.0, device=DEV)
+        assert not kernels.residual_layer_norm(pending, torch.ones(c, device=DEV), None, 1e-5, None, out, 2)
+        assert (out == 7.0).all()
+
+
+@pytest.mark.parametrize("rows,n_out,k_dim,bias,packed", [(1, 1600, 6400, True, True), (8, 768, 3072, True, True),
+                                                        (16, 512, 4096, False, False), (40, 1600, 6400, True, True),
+                                                        (5, 96, 3072, True, False)])
+def test_split_product_left_as_parts_of_a_pending_residual(rows, n_out, k_dim, bias, packed):
+    """The split product's first kernel alone: its parts (the first carries the bias) add up to the
+    plain product, in the order of k to the very bits that the two-kernel product stores; and the
+    residual LayerNorm that reads base + parts gives the LayerNorm of x + product."""
+    g = torch.Generator().manual_seed(rows + n_out)
+    a = bf(rnd(g, rows, k_dim))
+    w = bf(rnd(g, n_out, k_dim, scale=0.03))
+    b = rnd(g, n_out) if bias else None
+    x = rnd(g, rows + 1, n_out, scale=2.0)
+    x[rows:] = float("nan")
+    dev = lambda t: None if t is None else t.to(DEV)
+    wd = dev(w)
+    need = kernels.linear_skinny_partials(rows, n_out, k_dim, False, kernels.EPI_RESIDUAL)
+    assert need == 4 * rows * n_out
+    parts = torch.full((4, rows, n_out), float("nan"), device=DEV)
+    wp = kernels.pack_weight(wd) if packed else None
+    assert kernels.linear_decode_parts(dev(a), wd, dev(b), parts, rows, w_packed=wp) == 4
+    want = P.plain_linear(a.double(), w.double(), None if b is None else b.double())
+    helpers.assert_close(parts.sum(0), want, "bfloat16", "sum of the parts")
+    # the same sums as the product that adds them up itself (parts in the order of k, then the bias)
+    two = torch.zeros(rows, n_out, device=DEV)
+    scratch = torch.zeros(need, device=DEV)
+    assert kernels.linear_skinny(dev(a), wd, dev(b), two, rows, kernels.EPI_NONE, partials=scratch, w_packed=wp)
+    raw = scratch.view(4, rows, n_out)
+    assert torch.equal(parts[1:], raw[1:])
+    if b is None:
+        assert torch.equal(parts[0], raw[0])
+    else:
+        assert torch.equal(parts[0], raw[0] + dev(b))
+    # read as a pending residual
+    pending = PendingSums(dev(x), parts, 4)
+    gain, beta = 1 + 0.1 * rnd(g, n_out), rnd(g, n_out, scale=0.1)
+    out = torch.full((rows, n_out), float("nan"), dtype=torch.bfloat16, device=DEV)
+    assert kernels.residual_layer_norm(pending, dev(gain), dev(beta), 1e-5, None, out, rows, settled=pending.base)
+    true = x[:rows].double() + want
+    helpers.assert_close(pending.base[:rows], true, "bfloat16", "x + product")
+    assert torch.isnan(pending.base[rows:]).all()
+    helpers.assert_close(out, P.plain_layer_norm(pending.base[:rows].double().cpu(), gain.double(), beta.double(), 1e-5),
+                         "bfloat16", "LayerNorm of x + product")
+
+
+def test_split_parts_are_refused_where_the_product_is_not_split():
+    g = torch.Generator().manual_seed(2)
+    for rows, n_out, k_dim in ((4, 512, 2048), (4, 4096, 4096), (70, 512, 4096)):
+        a, w = bf(rnd(g, rows, k_dim)).to(DEV), bf(rnd(g, n_out, k_dim)).to(DEV)
+        parts = torch.full((4, rows, n_out), 7.0, device=DEV)
+        assert kernels.linear_decode_parts(a, w, None, parts, rows) == 0
+        assert (parts == 7.0).all()
 
 
 def test_fused_kernels_refuse_what_they_cannot_do():
@@ -217,7 +297,7 @@ def test_fused_kernels_refuse_what_they_cannot_do():
                                             out, 2, f)
         torch.cuda.synchronize()
         assert bool((out == 7.0).all()) and bool((settled == 7.0).all())
-        if c % 32 or c > 512 or parts > 32:
+        if c % 32 or parts > kernels.residual_parts_limit(c):      # (this kernel alone takes rows up to 4096 wide)
             assert not kernels.residual_layer_norm(pending, torch.ones(c, device=DEV), None, 1e-5, None,
                                                    torch.zeros(2, c, device=DEV), 2)
     # attention: two key/value heads under four query heads, and a head size of 48
