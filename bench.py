@@ -394,11 +394,19 @@ def write_report(path, record, samples):
                                  cwd=os.path.dirname(os.path.abspath(__file__))).stdout.strip()
         except Exception:
             sha = ""
+    # what identifies the code where there is no history: the digest of the native sources and flags
+    # that the loaded kernel library was built from
+    from mini_gpt_inference_amd.csrc import build
+    try:
+        with open(build.KERNEL_LIB + ".digest", encoding="ascii") as fh:
+            kernels_digest = fh.read().strip()
+    except OSError:
+        kernels_digest = ""
     report = {"record": record,
               "ms_per_step": {"median": quart[1] * 1e3, "q1": quart[0] * 1e3, "q3": quart[2] * 1e3,
                               "calls": len(per_step)},
               "samples": [[n, sec] for n, sec in samples],
-              "environment": {"git": sha, "torch": torch.__version__, "hip": torch.version.hip,
+              "environment": {"git": sha, "kernel_sources_sha256": kernels_digest, "torch": torch.__version__, "hip": torch.version.hip,
                               "device": torch.cuda.get_device_name(0)}}
     with open(path, "w", encoding="utf-8") as fh:
         json.dump(report, fh, indent=1)
