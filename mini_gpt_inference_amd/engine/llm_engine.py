@@ -6,6 +6,7 @@ or from a configuration and a seed.
 
 from __future__ import annotations
 
+import contextlib
 import shutil
 import tempfile
 import time
@@ -17,8 +18,9 @@ import torch
 from ..cache.kv_store import KVStore
 from ..cache.manager import CacheManager, GroupGeometry, plan_group_pages
 from ..config.engine_config import EngineConfig, SamplingParams
-from ..ops import kernels
+from ..ops import kernels, library
 from ..ops.linear import TileBest
+from ..ops.plan import LaunchPlan
 from ..parts.base import Workspace
 from ..sampling.sampler import Sampler
 from ..weights.loader import load_model
@@ -52,17 +54,24 @@ class _GraphedDecode:
         self.burst_graph: Optional[torch.cuda.CUDAGraph] = None
         self.shape: Optional[StepShape] = None   # of the last single step; launch geometry for captures
         self.kernels_per_step = 0                # kernels that the captured step launches
+        self.plan: Optional[LaunchPlan] = None   # the step's launches, recorded at its one eager run
         self.tile_best_used = False              # greedy rows choose from what the head left per tile
 
-    def _launch(self, shape: StepShape) -> None:
+    def _launch(self, shape: StepShape, record: bool = False) -> None:
+        """The step's kernels (model and sampling) through the model's Python.  record: keep the
+        launches as a plan, from which the captures make them again without the Python."""
         ctx = self.runner.context(self.arena, shape, padded=True, workspace=self.workspace)
         # launch geometry must not depend on this step's lengths: size it for the longest sequence
         ctx.max_seq_len = self.runner.max_positions or ctx.max_seq_len
         ctx.tile_best = TileBest(self.sampler.real_vocab)
-        with kernels.pinned_stream():
+        launched = kernels.launches
+        with kernels.pinned_stream(), (library.record() if record else contextlib.nullcontext()) as launches:
             logits = self.runner.model.forward(ctx)
             self.sampler.sample(logits, self.arena, self.cap, advance=(self.runner.page_sizes, self.history),
                                 tile_best=ctx.tile_best)
+        self.kernels_per_step = kernels.launches - launched
+        if record:
+            self.plan = LaunchPlan(launches)
         self.tile_best_used = ctx.tile_best.filled
 
     def _capture(self, shape: StepShape, times: int) -> torch.cuda.CUDAGraph:
@@ -70,13 +79,15 @@ class _GraphedDecode:
         graph = torch.cuda.CUDAGraph()
         side = torch.cuda.Stream()
         side.wait_stream(torch.cuda.current_stream())
-        launched = kernels.launches
         with torch.cuda.stream(side):
             graph.capture_begin()
             try:
                 for _ in range(times):
-                    self._launch(shape)
-                self.kernels_per_step = (kernels.launches - launched) // times
+                    if self.plan is not None:
+                        with kernels.pinned_stream():
+                            self.plan.run()
+                    else:
+                        self._launch(shape)
             except BaseException:
                 # never leave the stream capturing: the graph object's destructor synchronizes the
                 # device, which a stream that is still capturing turns into an abort of the process
@@ -96,7 +107,7 @@ class _GraphedDecode:
         self.arena.upload()
         if self.graph is None:
             # once eagerly, so that every workspace buffer exists before capture
-            self._launch(shape)
+            self._launch(shape, record=self.runner.plan_steps)
             torch.cuda.synchronize()
             self.workspace.frozen = True
             self.graph = self._capture(shape, 1)
