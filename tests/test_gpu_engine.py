@@ -130,6 +130,40 @@ def test_real_widths_decode_through_graphs_and_bursts(tmp_path, shape, n_req):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("seed", range(6))
+def test_drawn_configurations_generate_through_graphs_and_bursts(tmp_path, seed, dtype):
+    """Configurations drawn from a seed (every size and option varies), a drawn number of requests:
+    greedy generation through the entry point, its decode steps from graphs and bursts (and, in
+    bfloat16 at widths that take them, the fused kernels), gives the plain implementation's tokens."""
+    from safetensors.torch import save_file
+    from mini_gpt_inference_amd.config.model_config import write_config_json
+    from mini_gpt_inference_amd.weights.random_init import random_tensors
+    from test_gpu_replay import _drawn_configuration
+    cfg = _drawn_configuration(seed + 20)
+    folder = str(tmp_path / f"drawn{seed}")
+    os.makedirs(folder)
+    write_config_json(folder, cfg)
+    save_file({k: v.contiguous() for k, v in random_tensors(cfg, seed, torch.bfloat16, 4.0).items()},
+              os.path.join(folder, "model.safetensors"))
+    rng = np.random.default_rng(seed)
+    n_req, n_new = int(rng.integers(1, 10)), 20
+    prompts = [helpers.random_ids(rng, cfg.vocab_size, int(n)) for n in rng.integers(1, cfg.block_size - n_new, n_req)]
+    page = int(rng.choice([4, 8, 16]))
+    pages = n_req * (-(-cfg.block_size // page))
+    engine = LLMEngine.from_folder(folder, EngineConfig(block_size=page, num_blocks=pages, max_batch_size=n_req,
+                                                        dtype=dtype))
+    got = engine.generate(prompts, SamplingParams(max_tokens=n_new, temperature=0.0))
+    assert engine.stats()["graph_steps"] >= n_new - 4
+    assert engine.cache.check() == 0 and engine.cache.num_free_pages() == pages
+    if dtype == "float32":
+        assert got == _plain_greedy(folder, prompts, n_new)
+    else:
+        for prompt, tokens in zip(prompts, got):
+            assert len(tokens) == n_new
+            _assert_greedy_within_tolerance(folder, prompt, tokens, dtype)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_chunked_mixed_and_whole_prompt_policies_give_the_same_tokens(model_folders, dtype):
     prompts = _prompts("B", [1, 9, 33, 64, 100], seed=2)
     sp = SamplingParams(max_tokens=16, temperature=0.0)

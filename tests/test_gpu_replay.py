@@ -78,6 +78,46 @@ def test_head_sizes_that_are_no_power_of_two(model_folders, name, dtype, way):
     assert replayer.cache.check() == 0 and replayer.cache.num_free_pages() == replayer.num_pages
 
 
+def _drawn_configuration(seed):
+    """A configuration drawn from the seed: every size and option of the architecture varies."""
+    from mini_gpt_inference_amd import GPTConfig
+    rng = np.random.default_rng(1000 + seed)
+    head = int(rng.choice([16, 32, 48, 64, 80, 128]))
+    heads = int(rng.integers(1, 7 if head <= 64 else 4))
+    return GPTConfig("gpt2-mini", n_layer=int(rng.integers(1, 4)), n_embd=head * heads, n_head=heads,
+                     vocab_size=int(rng.integers(50, 700)), block_size=int(rng.choice([64, 96, 160, 256])),
+                     bias=bool(rng.integers(0, 2)), layer_norm_eps=float(rng.choice([1e-6, 1e-5, 1e-3])))
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("seed", range(8))
+def test_drawn_configurations_mixed_with_page_reuse(tmp_path, seed, dtype):
+    """Configurations nobody chose by hand (head sizes 16 to 128, one to six heads, any vocabulary,
+    with and without biases), requests of drawn lengths, mixed steps, a tight poisoned pool of drawn
+    page size: whichever kernels the sizes select, the logits are the plain implementation's."""
+    from safetensors.torch import save_file
+    from mini_gpt_inference_amd.config.model_config import write_config_json
+    from mini_gpt_inference_amd.weights.random_init import random_tensors
+    cfg = _drawn_configuration(seed)
+    folder = str(tmp_path / f"drawn{seed}")
+    os.makedirs(folder)
+    write_config_json(folder, cfg)
+    save_file({k: v.contiguous() for k, v in random_tensors(cfg, seed, torch.bfloat16, 4.0).items()},
+              os.path.join(folder, "model.safetensors"))
+    rng = np.random.default_rng(seed)
+    page_size = int(rng.choice([2, 4, 8, 16, 32]))
+    lengths = [int(n) for n in rng.integers(1, cfg.block_size + 1, 5)]
+    reqs = {f"r{i}": helpers.random_ids(rng, cfg.vocab_size, n) for i, n in enumerate(lengths)}
+    pcfg, w = P.read_model_folder(folder)
+    plan = helpers.plan_mixed(reqs, np.random.default_rng(seed + 50))
+    replayer = TraceReplayer(folder, dtype, plan.tight_tokens(page_size), page_size=page_size, poison=True)
+    got = plan.assemble(helpers.run_plan_in_process(replayer, plan), {r: len(t) for r, t in reqs.items()},
+                        cfg.vocab_size)
+    for rid, ids in reqs.items():
+        helpers.assert_close(got[rid], P.plain_forward(w, pcfg, ids).numpy(), dtype, f"{cfg} {dtype} {rid}")
+    assert replayer.cache.check() == 0 and replayer.cache.num_free_pages() == replayer.num_pages
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_cuts_agree_with_each_other_bit_for_bit_in_32_bit(model_folders, dtype):
     """On the 32-bit path the order of every sum depends only on a token's position, so all ways of
