@@ -234,7 +234,7 @@ __global__ __launch_bounds__(FUSED_THREADS) void fused_attention_decode_kernel(F
   static_assert(FUSED_WAVES * D <= POOL_FLOATS, "the pool holds the waves' sums of attention");
   __shared__ __align__(16) float pool[POOL_FLOATS];
   __shared__ __align__(16) bf16_t act_s[FUSED_MAX_WIDTH];
-  __shared__ float mean_s[FUSED_WAVES], var_s[FUSED_WAVES];
+  __shared__ __align__(16) float gain_s[FUSED_MAX_WIDTH], beta_s[FUSED_MAX_WIDTH];
   __shared__ __align__(16) bf16_t q_s[D];
   __shared__ __align__(16) bf16_t k_s[D];
   __shared__ __align__(16) bf16_t v_s[D];
@@ -292,6 +292,7 @@ __global__ __launch_bounds__(FUSED_THREADS) void fused_attention_decode_kernel(F
         part[u] = reinterpret_cast<const float4*>(a.res.partials + p * a.res.part_stride)[(long)n * V + vq];
     }
   }
+  // the LayerNorm's gain and bias go through LDS to the wave that will norm the row
   const int vc = tid < V ? tid : 0;
   float4 gain4 = make_float4(0.f, 0.f, 0.f, 0.f), beta4 = make_float4(0.f, 0.f, 0.f, 0.f);
   if (tid < V) {
@@ -323,78 +324,88 @@ __global__ __launch_bounds__(FUSED_THREADS) void fused_attention_decode_kernel(F
     const long tile_ = (long)(tt_ / (D / 16)) * tiles_per_part + h * (D / 16) + (tt_ % (D / 16));           \
     wv[tt_][i_] = fd_packed(a.wqkv, tile_, KS, i_ < nks ? ks0 + i_ : 0, lane);                              \
   }
-  FA_LOAD_W(0)
-  if (qr < 0) return;  // a token of the padding (the whole workgroup)
-  FD_STAMP_AFTER(16, piece.x);
-
-  // ---- the residual row's sum and LayerNorm
-  if (!TABLES) {
-#pragma unroll
-    for (int u = 0; u < FUSED_GROUP_PARTS; ++u) piece = fd_add4(piece, part[u]);
-  }
-  if (gq < G) reinterpret_cast<float4*>(xs)[gq * V + vq] = piece;
-  fd_barrier();
-  FD_STAMP(17);
-  FA_LOAD_W(1)
-  float4 xv = make_float4(0.f, 0.f, 0.f, 0.f);
-  if (tid < V) {
-    // groups beyond the parts hold zeros: only the groups that had something are read
-    const int used = TABLES ? 1 : min(G, max(a.res.n_parts, 1));
-    xv = reinterpret_cast<const float4*>(xs)[tid];
-#pragma unroll 8
-    for (int q = 1; q < used; ++q) xv = fd_add4(xv, reinterpret_cast<const float4*>(xs)[q * V + tid]);
-    if (h == 0 && a.res.settled) reinterpret_cast<float4*>(a.res.settled + (long)n * C)[tid] = xv;
-  }
-  const int waves_used = (V + 63) >> 6;  // the waves that hold the row
-  {
-    const float ws = wave_sum(fd_sum4(xv));
-    if (lane == 0) mean_s[wave] = ws;
-  }
-  fd_barrier();
-  FD_STAMP(18);
-  FA_LOAD_W(2)
-  float mean = 0.f;
-  for (int w = 0; w < waves_used; ++w) mean += mean_s[w];
-  mean /= (float)C;
-  float4 dv = make_float4(0.f, 0.f, 0.f, 0.f);
-  if (tid < V) dv = make_float4(xv.x - mean, xv.y - mean, xv.z - mean, xv.w - mean);
-  {
-    const float wq = wave_sum((dv.x * dv.x + dv.y * dv.y) + (dv.z * dv.z + dv.w * dv.w));
-    if (lane == 0) var_s[wave] = wq;
-  }
-  fd_barrier();
-  FD_STAMP(19);
-  FA_LOAD_W(3)
-#undef FA_LOAD_W
   // keys and values of the first pass: their addresses need the block table and the position only
   const int kv_end = qpos;  // the keys before the token's own
   const int page_mask = (1 << a.page_shift) - 1;
   const unsigned int lane_off = ((unsigned int)(h << a.page_shift) * D + dg * 8) * 2u;
   uint4 kraw[NI], vraw[NI];
   const int c00 = wave * CHUNK;
-  if (c00 < kv_end) {  // the same in all lanes of a wave
+#define FA_LOAD_KV                                                                                                    \
+  if (c00 < kv_end) { /* the same in all lanes of a wave */                                                          \
+    _Pragma("unroll") for (int i = 0; i < NI; ++i) {                                                                 \
+      const int j_ = c00 + i * KPI + sub;                                                                            \
+      const bool follow_ = j_ < kv_end && (unsigned int)page0[i] < (unsigned int)a.num_pages;                        \
+      const unsigned int row_off_ = ((unsigned int)page0[i] * a.page_bytes) + (unsigned int)(j_ & page_mask) * (D * 2u); \
+      const unsigned int off_ = follow_ ? row_off_ + lane_off : 0u;                                                  \
+      kraw[i] = *reinterpret_cast<const uint4*>(reinterpret_cast<const char*>(a.kpool) + off_);                      \
+      vraw[i] = *reinterpret_cast<const uint4*>(reinterpret_cast<const char*>(a.vpool) + off_);                      \
+    }                                                                                                                \
+  }
+  FA_LOAD_W(0)
+  if (qr < 0) return;  // a token of the padding (the whole workgroup)
+  FD_STAMP_AFTER(16, piece.x);
+
+  // ---- the residual row's sum: every group of threads its parts, then the first wave all groups
+  if (!TABLES) {
 #pragma unroll
-    for (int i = 0; i < NI; ++i) {
-      const int j = c00 + i * KPI + sub;
-      const bool follow = j < kv_end && (unsigned int)page0[i] < (unsigned int)a.num_pages;
-      const unsigned int row_off = ((unsigned int)page0[i] * a.page_bytes) + (unsigned int)(j & page_mask) * (D * 2u);
-      const unsigned int off = follow ? row_off + lane_off : 0u;
-      kraw[i] = *reinterpret_cast<const uint4*>(reinterpret_cast<const char*>(a.kpool) + off);
-      vraw[i] = *reinterpret_cast<const uint4*>(reinterpret_cast<const char*>(a.vpool) + off);
+    for (int u = 0; u < FUSED_GROUP_PARTS; ++u) piece = fd_add4(piece, part[u]);
+  }
+  if (gq < G) reinterpret_cast<float4*>(xs)[gq * V + vq] = piece;
+  if (tid < V) {
+    reinterpret_cast<float4*>(gain_s)[tid] = gain4;
+    reinterpret_cast<float4*>(beta_s)[tid] = beta4;
+  }
+  fd_barrier();
+  FD_STAMP(17);
+  // every wave sends for the rest of its weights and for its keys and values; then the first wave
+  // norms the row (LDS and arithmetic only) while the others wait at the next barrier
+  FA_LOAD_W(1)
+  FA_LOAD_W(2)
+  FA_LOAD_W(3)
+  FA_LOAD_KV
+#undef FA_LOAD_W
+#undef FA_LOAD_KV
+  if (wave == 0) {
+    float4 xv[2];
+    xv[0] = xv[1] = make_float4(0.f, 0.f, 0.f, 0.f);
+    // ---- LayerNorm, within one wave: no barrier between the sums
+    // groups beyond the parts hold zeros: only the groups that had something are read
+    const int used = TABLES ? 1 : min(G, max(a.res.n_parts, 1));
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      const int v = lane + 64 * u;
+      if (v < V) {
+        xv[u] = reinterpret_cast<const float4*>(xs)[v];
+#pragma unroll 8
+        for (int q = 1; q < used; ++q) xv[u] = fd_add4(xv[u], reinterpret_cast<const float4*>(xs)[q * V + v]);
+        // the row as it stands, stored by the first head's workgroup for the kernels behind this one
+        if (h == 0 && a.res.settled) reinterpret_cast<float4*>(a.res.settled + (long)n * C)[v] = xv[u];
+      }
+    }
+    const float mean = wave_sum(fd_sum4(xv[0]) + fd_sum4(xv[1])) / (float)C;
+    float4 dv[2];
+    float sq = 0.f;
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      const bool in = lane + 64 * u < V;
+      dv[u] = in ? make_float4(xv[u].x - mean, xv[u].y - mean, xv[u].z - mean, xv[u].w - mean)
+                 : make_float4(0.f, 0.f, 0.f, 0.f);
+      sq += (dv[u].x * dv[u].x + dv[u].y * dv[u].y) + (dv[u].z * dv[u].z + dv[u].w * dv[u].w);
+    }
+    const float rstd = 1.0f / sqrtf(wave_sum(sq) / (float)C + a.eps);
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      const int v = lane + 64 * u;
+      if (v < V) {
+        const float4 gn = reinterpret_cast<const float4*>(gain_s)[v], bt4 = reinterpret_cast<const float4*>(beta_s)[v];
+        uint2 pk;
+        pk.x = pack_bf16x2(dv[u].x * rstd * gn.x + bt4.x, dv[u].y * rstd * gn.y + bt4.y);
+        pk.y = pack_bf16x2(dv[u].z * rstd * gn.z + bt4.z, dv[u].w * rstd * gn.w + bt4.w);
+        reinterpret_cast<uint2*>(act_s)[v] = pk;
+      }
     }
   }
-  {
-    float var = 0.f;
-    for (int w = 0; w < waves_used; ++w) var += var_s[w];
-    const float rstd = 1.0f / sqrtf(var / (float)C + a.eps);
-    if (tid < V) {
-      uint2 pk;
-      pk.x = pack_bf16x2(dv.x * rstd * gain4.x + beta4.x, dv.y * rstd * gain4.y + beta4.y);
-      pk.y = pack_bf16x2(dv.z * rstd * gain4.z + beta4.z, dv.w * rstd * gain4.w + beta4.w);
-      reinterpret_cast<uint2*>(act_s)[tid] = pk;
-    }
-  }
-  fd_barrier();  // also: everybody has read the row's partial sums, whose place the waves' sums take now
+  fd_barrier();  // also: the row's partial sums are read, their place takes the waves' sums now
   FD_STAMP(1);
 
   // ---- q, k, v of this head: every wave a stretch of k over all the row tiles; the waves' sums
