@@ -212,10 +212,10 @@ struct FusedAttnArgs {
   float scale_log2e;
 };
 
-// Sixteen waves a workgroup: a compute unit takes in about 200 KB a microsecond when sixteen waves
-// each have up to sixteen loads of 16 bytes a lane in flight, and half of that with eight waves
-// that have twice as many each.  A wave therefore holds few loads at a time, and a lane at most
-// 128 registers.
+// Sixteen waves a workgroup: a compute unit issues a wave's 16-byte-a-lane load about every 6 ns
+// (170 KB a microsecond) when sixteen waves each have up to sixteen of them in flight, and half of
+// that with eight waves that have twice as many each.  A wave therefore holds few loads at a time,
+// and a lane at most 128 registers.
 template <int D, bool TABLES>
 __global__ __launch_bounds__(FUSED_THREADS) void fused_attention_decode_kernel(FusedAttnArgs a) {
   constexpr int T = 3 * D / 16;                  // row tiles of this head's q, k and v
@@ -254,11 +254,12 @@ __global__ __launch_bounds__(FUSED_THREADS) void fused_attention_decode_kernel(F
 
   FD_STAMP(0);
   // ---- The prologue.  A compute unit issues a wave's 16-byte loads at about a kilobyte every
-  // ten clocks, and a barrier lets a wave pass only when every other wave has issued what stands
-  // before it: the weights' loads (most of the traffic) are therefore dealt out in four pieces
-  // between the barriers of the residual row's sum and LayerNorm, which need the row's loads only
-  // and happen while the pieces are on their way.  A wave's loads come back in order: the step's
-  // numbers and the row first, keys and values last.
+  // twelve clocks, and a barrier lets a wave pass only when every other wave has issued what
+  // stands before it: only a quarter of the weights' loads stand before the barrier at which the
+  // row's partial sums meet (the row's loads of the last waves would otherwise wait behind all the
+  // weights of the first: measured, 1.6 us a layer slower); the rest, and the keys and values, are
+  // sent for behind it, while the first wave norms the row.  A wave's loads come back in order:
+  // the step's numbers and the row first, keys and values last.
   const int qr = a.q_req[n];
   const int qpos = a.positions[n];
   const int slot = a.slot_mapping[n];
@@ -315,7 +316,7 @@ __global__ __launch_bounds__(FUSED_THREADS) void fused_attention_decode_kernel(F
   const int ks0 = wave * per;
   const int nks = max(0, min(per, KS - ks0));
   const int tiles_per_part = a.n_head * (D / 16);
-  constexpr int NW = TG * SMAX;  // loads of the weights' first pass, dealt out in four pieces
+  constexpr int NW = TG * SMAX;  // loads of the weights' first pass: a quarter before the first barrier, the rest behind it
   static_assert(NW % 4 == 0, "four pieces");
   bf16x8_t wv[TG][SMAX];
 #define FA_LOAD_W(piece_no)                                                                                 \
