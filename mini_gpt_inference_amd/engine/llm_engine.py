@@ -106,10 +106,14 @@ class _GraphedDecode:
         self.history_base = 0
         self.arena.upload()
         if self.graph is None:
-            # once eagerly, so that every workspace buffer exists before capture
-            self._launch(shape, record=self.runner.plan_steps)
+            # once eagerly, so that every workspace buffer and every derived copy of a matrix exists
+            # before capture; then once more, counted and recorded: the step as every later one runs
+            self._launch(shape)
             torch.cuda.synchronize()
             self.workspace.frozen = True
+            self.arena.upload()
+            self._launch(shape, record=self.runner.plan_steps)
+            torch.cuda.synchronize()
             self.graph = self._capture(shape, 1)
             # the eager launch above did this step's work and moved the device arrays on to the
             # next step: upload this step's again
