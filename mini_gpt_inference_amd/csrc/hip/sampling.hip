@@ -146,21 +146,54 @@ struct AdvanceArgs {
   int history_rows, history_stride;
 };
 
-__device__ __forceinline__ void finish_row(int row, int token, int* out_tokens, const AdvanceArgs& adv) {
+// What the row's first thread reads for that, asked for at the kernel's start: none of it depends on the
+// token, and two of the loads depend on each other (the position, then the block table's entry), so
+// behind the choice they would be two trips to memory more.
+#define SAMPLE_ADV_GROUPS 4   // cache groups whose slots are looked up ahead; more are looked up at the end
+struct AdvanceAhead {
+  bool live;
+  int pos, seq_len, out_index, history_pos;
+  int slot[SAMPLE_ADV_GROUPS];
+};
+
+__device__ __forceinline__ int advance_slot(int row, int pos, int g, const AdvanceArgs& adv) {
+  const int ps = adv.page_sizes[g];
+  const int idx = pos / ps;
+  const int page = idx < adv.max_blocks ? adv.block_tables[((long)g * adv.r_stride + row) * adv.max_blocks + idx] : -1;
+  return page >= 0 ? page * ps + pos % ps : -1;
+}
+
+__device__ __forceinline__ AdvanceAhead look_ahead(int row, const AdvanceArgs& adv) {
+  AdvanceAhead a;
+  a.live = adv.token_ids != nullptr && adv.q_req[row] >= 0;
+  a.pos = a.seq_len = a.out_index = a.history_pos = 0;
+#pragma unroll
+  for (int g = 0; g < SAMPLE_ADV_GROUPS; ++g) a.slot[g] = -1;
+  if (!a.live) return a;
+  a.pos = adv.positions[row] + 1;
+  a.seq_len = adv.seq_lens[row] + 1;
+  a.out_index = adv.out_index[row] + 1;
+  a.history_pos = adv.history_pos[row];
+#pragma unroll
+  for (int g = 0; g < SAMPLE_ADV_GROUPS; ++g)
+    if (g < adv.n_groups) a.slot[g] = advance_slot(row, a.pos, g, adv);
+  return a;
+}
+
+__device__ __forceinline__ void finish_row(int row, int token, int* out_tokens, const AdvanceArgs& adv,
+                                           const AdvanceAhead& ahead) {
   out_tokens[row] = token;
-  if (adv.token_ids == nullptr || adv.q_req[row] < 0) return;
+  if (!ahead.live) return;
   adv.token_ids[row] = token;
-  const int pos = adv.positions[row] + 1;
-  adv.positions[row] = pos;
-  adv.seq_lens[row] += 1;
-  adv.out_index[row] += 1;
-  for (int g = 0; g < adv.n_groups; ++g) {
-    const int ps = adv.page_sizes[g];
-    const int idx = pos / ps;
-    const int page = idx < adv.max_blocks ? adv.block_tables[((long)g * adv.r_stride + row) * adv.max_blocks + idx] : -1;
-    adv.slot_mapping[(long)g * adv.n_stride + row] = page >= 0 ? page * ps + pos % ps : -1;
-  }
-  const int j = adv.history_pos[row];
+  adv.positions[row] = ahead.pos;
+  adv.seq_lens[row] = ahead.seq_len;
+  adv.out_index[row] = ahead.out_index;
+#pragma unroll
+  for (int g = 0; g < SAMPLE_ADV_GROUPS; ++g)
+    if (g < adv.n_groups) adv.slot_mapping[(long)g * adv.n_stride + row] = ahead.slot[g];
+  for (int g = SAMPLE_ADV_GROUPS; g < adv.n_groups; ++g)
+    adv.slot_mapping[(long)g * adv.n_stride + row] = advance_slot(row, ahead.pos, g, adv);
+  const int j = ahead.history_pos;
   if (j < adv.history_rows) adv.history[(long)j * adv.history_stride + row] = token;
   adv.history_pos[row] = j + 1;
 }
@@ -178,6 +211,9 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
   __shared__ int chosen;
 
   const int row = blockIdx.x, tid = threadIdx.x;
+  AdvanceAhead ahead;
+  ahead.live = false;
+  if (tid == 0) ahead = look_ahead(row, adv);
   const float* lg = logits + (long)row * ld;
   const int nv = real_vocab < vocab ? real_vocab : vocab;
   const float temp = temperature[row];
@@ -256,7 +292,7 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
       best_i = tid < SAMPLE_WAVES ? red_i[tid] : 0x7fffffff;
       argmax_rows16(best, best_i);
     }
-    if (tid == 0) finish_row(row, best_i == 0x7fffffff ? 0 : best_i, out_tokens, adv);
+    if (tid == 0) finish_row(row, best_i == 0x7fffffff ? 0 : best_i, out_tokens, adv, ahead);
     return;
   }
 
@@ -361,7 +397,7 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
       c = 0;
       for (int i = 0; i < SAMPLE_WAVES; ++i) c = max(c, red_i[i]);
     }
-    finish_row(row, c, out_tokens, adv);
+    finish_row(row, c, out_tokens, adv, ahead);
   }
 }
 
