@@ -21,12 +21,55 @@
 #pragma once
 #include "linear_skinny.h"
 
+// DPP row_shl:n: lane l of a row of 16 gets the value of lane l + n (0 from past the row's end)
+template <int N>
+__device__ __forceinline__ unsigned int ld_shl(unsigned int v) {
+  return N == 0 ? v : (unsigned int)__builtin_amdgcn_update_dpp(0, (int)v, 0x100 + (N == 0 ? 1 : N), 0xf, 0xf, false);
+}
+__device__ __forceinline__ float ld_shl_f(float v, int n) {
+  switch (n) {
+    case 1: return __uint_as_float(ld_shl<1>(__float_as_uint(v)));
+    case 2: return __uint_as_float(ld_shl<2>(__float_as_uint(v)));
+    case 4: return __uint_as_float(ld_shl<4>(__float_as_uint(v)));
+    default: return __uint_as_float(ld_shl<8>(__float_as_uint(v)));
+  }
+}
+// the 8 rounded values of a k step, taken from the lane FEW * j further on in the row
+template <int FEW>
+__device__ __forceinline__ bf16x8_t ld_row_shl(bf16x8_t v, int j) {
+  typedef __attribute__((__vector_size__(4 * sizeof(unsigned int)))) unsigned int u32x4_t;
+  const u32x4_t s = __builtin_bit_cast(u32x4_t, v);
+  u32x4_t r = s;
+#define LD_CASE(J)                                                                                   \
+  case J:                                                                                            \
+    if (FEW * J < 16)                                                                                \
+      r = (u32x4_t){ld_shl<(FEW * J < 16 ? FEW * J : 0)>(s[0]), ld_shl<(FEW * J < 16 ? FEW * J : 0)>(s[1]), \
+                    ld_shl<(FEW * J < 16 ? FEW * J : 0)>(s[2]), ld_shl<(FEW * J < 16 ? FEW * J : 0)>(s[3])}; \
+    break;
+  switch (j) {
+    LD_CASE(1) LD_CASE(2) LD_CASE(3) LD_CASE(4) LD_CASE(5) LD_CASE(6) LD_CASE(7) LD_CASE(8)
+    LD_CASE(9) LD_CASE(10) LD_CASE(11) LD_CASE(12) LD_CASE(13) LD_CASE(14) LD_CASE(15)
+    default: break;
+  }
+#undef LD_CASE
+  return __builtin_bit_cast(bf16x8_t, r);
+}
+
 // VEC: n_out is a multiple of 16 and bias, column sums and output rows are aligned for vectors of
 // four; otherwise every access of the epilogue is a single element with its own bound check.
 // SPLIT: k is also split over a.k_parts workgroups per column tile; each stores its raw sums to
 // a.partials (no LayerNorm, no epilogue: linear_partials_epilogue_kernel finishes the job).
-template <int NT, int SMAX, bool LN, int EPI, typename OT, bool VEC, bool SPLIT = false>
+// FEW (with LN and one tile; 1, 2, 4 or 8, at least the rows of a group): the residual rows are
+// loaded by all sixteen lanes of a lane row, not only by the FEW that hold a row: lane r + FEW j
+// loads the j-th of 16 / FEW k steps of row r, rounds it and adds up its statistics, and the row's
+// own lane takes the rounded values over with a DPP shift.  A load instruction costs the compute
+// unit the same whether four of its lanes are live or all: at one row that is 2 instead of 26 of
+// them for an inner size of 1600 ([6400 x 1600] at one row: the LayerNorm's share of the kernel
+// falls from 2.2 to 0.6 us).  0: every lane loads what it multiplies.
+template <int NT, int SMAX, bool LN, int EPI, typename OT, bool VEC, bool SPLIT = false, int FEW = 0>
 __global__ __launch_bounds__(256) void linear_decode_kernel(SkinnyArgs a) {
+  static_assert(FEW == 0 || (LN && NT == 1 && !SPLIT && (FEW == 1 || FEW == 2 || FEW == 4 || FEW == 8)),
+                "rows packed into a load: one tile, with the LayerNorm, 1, 2, 4 or 8 rows");
   __shared__ float red[3 * NT * 6 * 64];  // waves 1..3: per row tile four sums and two statistics per lane
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // the same in all lanes: branches on it are scalar
@@ -113,10 +156,23 @@ __global__ __launch_bounds__(256) void linear_decode_kernel(SkinnyArgs a) {
     x0[t] = sd[t] = sq[t] = 0.f;
     // the shift of a row: the median of three of its values, so that one channel that stands far
     // out (residual streams have such) does not become the shift
-    if (LN && row_ok[t]) {
+    if (LN && FEW == 0 && row_ok[t]) {
       const float* xr = a.x + (long)src[t] * K;
       x0[t] = __builtin_amdgcn_fmed3f(xr[0], xr[K >> 1], xr[K - 1]);
     }
+  }
+  // FEW: the row this lane loads for (fr of the group) and which of a batch's k steps (fj)
+  constexpr int FJ = FEW > 0 ? 16 / FEW : 1;
+  const int fr = FEW > 0 ? (lrow & (FEW - 1)) : 0, fj = FEW > 0 ? lrow / (FEW > 0 ? FEW : 1) : 0;
+  const float* frow_x = a.x;
+  bool f_ok = false;
+  if (FEW > 0) {
+    const int frow = (int)blockIdx.y * rpg + fr;
+    f_ok = fr < rpg && frow < a.n_rows;
+    const int fsrc = f_ok ? (a.rows != nullptr ? a.rows[frow] : frow) : 0;
+    frow_x = a.x + (long)fsrc * K;
+    // (the lane that holds the row is its first loader: fj = 0, fr = lrow)
+    if (f_ok) x0[0] = __builtin_amdgcn_fmed3f(frow_x[0], frow_x[K >> 1], frow_x[K - 1]);
   }
   // W as it is (a wave's load is sixteen rows' 64 bytes), or packed so that it is 1 KB in one piece
   const bf16_t* wp = a.w_packed ? a.w_packed + (((long)(o0 >> 4) * (K >> 5) + (kb >> 5)) * 64 + lane) * 8
@@ -127,7 +183,42 @@ __global__ __launch_bounds__(256) void linear_decode_kernel(SkinnyArgs a) {
 #pragma unroll
     for (int i = 0; i < SMAX; ++i)
       wv[i] = *reinterpret_cast<const bf16x8_t*>(wp + (s0 + i < steps ? s0 + i : 0) * w_step);
-    if (LN) {
+    if (LN && FEW > 0) {
+      // a batch of FJ k steps per pair of loads: this lane loads step b * FJ + fj of the pass
+      constexpr int NB = (SMAX + FJ - 1) / FJ;
+      bf16x8_t packed[NB];
+#pragma unroll
+      for (int b = 0; b < NB; ++b) {
+        const int st = s0 + b * FJ + fj;
+        const bool live = f_ok && st < steps && b * FJ + fj < SMAX;
+        float4 lo = make_float4(0.f, 0.f, 0.f, 0.f), hi = lo;
+        if (live) {
+          const float4* p = reinterpret_cast<const float4*>(frow_x + kb + g * 8 + st * 32);
+          lo = p[0];
+          hi = p[1];
+        }
+        const float xs0 = x0[0];
+        const float f[8] = {lo.x - xs0, lo.y - xs0, lo.z - xs0, lo.w - xs0, hi.x - xs0, hi.y - xs0, hi.z - xs0, hi.w - xs0};
+        typedef __attribute__((__vector_size__(4 * sizeof(unsigned int)))) unsigned int u32x4_t;
+        u32x4_t pk = {pack_bf16x2(f[0], f[1]), pack_bf16x2(f[2], f[3]), pack_bf16x2(f[4], f[5]), pack_bf16x2(f[6], f[7])};
+        if (!live) pk = (u32x4_t){0u, 0u, 0u, 0u};
+        packed[b] = __builtin_bit_cast(bf16x8_t, pk);
+        if (live) {
+#pragma unroll
+          for (int e = 0; e < 8; ++e) {
+            sd[0] += f[e];
+            sq[0] = fmaf(f[e], f[e], sq[0]);
+          }
+        }
+      }
+      // the row's own lane (lrow < FEW) takes step i from the lane that loaded it
+#pragma unroll
+      for (int i = 0; i < SMAX; ++i) {
+        constexpr int dummy = 0;
+        (void)dummy;
+        av[0][i] = ld_row_shl<FEW>(packed[i / FJ], i % FJ);
+      }
+    } else if (LN) {
       float4 lo[NT][SMAX], hi[NT][SMAX];
 #pragma unroll
       for (int t = 0; t < NT; ++t) {
@@ -185,6 +276,14 @@ __global__ __launch_bounds__(256) void linear_decode_kernel(SkinnyArgs a) {
 #pragma unroll
         for (int t = 0; t < NT; ++t) acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wv[i], av[t][i], acc[t], 0, 0, 0);
       }
+  }
+  if (LN && FEW > 0) {
+    // the loaders of a row lie FEW lanes apart: their sums meet in the row's own lane
+#pragma unroll
+    for (int n = FEW; n < 16; n <<= 1) {
+      sd[0] += ld_shl_f(sd[0], n);
+      sq[0] += ld_shl_f(sq[0], n);
+    }
   }
   if (LN) {
     // the four lanes that share a row hold parts of its sums
@@ -308,10 +407,10 @@ __global__ __launch_bounds__(256) void linear_decode_kernel(SkinnyArgs a) {
   }
 }
 
-template <int NT, int SMAX, bool LN, bool VEC>
+template <int NT, int SMAX, bool LN, bool VEC, int FEW = 0>
 static int launch_decode_epi(const SkinnyArgs& a, int epi, int out_dtype, dim3 grid, hipStream_t s) {
 #define LD_LAUNCH(E, OT) \
-  hipLaunchKernelGGL((linear_decode_kernel<NT, SMAX, LN, E, OT, VEC>), grid, dim3(256), 0, s, a)
+  hipLaunchKernelGGL((linear_decode_kernel<NT, SMAX, LN, E, OT, VEC, false, FEW>), grid, dim3(256), 0, s, a)
   if (epi == SK_EPI_NONE && out_dtype == MGPT_BF16) LD_LAUNCH(SK_EPI_NONE, bf16_t);
   else if (epi == SK_EPI_NONE && out_dtype == MGPT_F32) LD_LAUNCH(SK_EPI_NONE, float);
   else if (epi == SK_EPI_GELU && out_dtype == MGPT_BF16) LD_LAUNCH(SK_EPI_GELU, bf16_t);

@@ -10,9 +10,18 @@ int mgpt_launch_linear_decode_rows(const SkinnyArgs& a, int epilogue, int out_dt
 template <int SMAX>
 static int launch_one_tile(const SkinnyArgs& a, int epilogue, int out_dtype, dim3 grid, hipStream_t s) {
   const bool ln = a.x != nullptr;
-  if (decode_vec_ok(a))
+  if (decode_vec_ok(a)) {
+    if (ln) {
+      // few rows to a workgroup: the residual rows loaded by all lanes of a lane row (FEW in linear_decode.h)
+      const int rows = a.rows_per_group < a.n_rows ? a.rows_per_group : a.n_rows;
+      if (rows <= 1) return launch_decode_epi<1, SMAX, true, true, 1>(a, epilogue, out_dtype, grid, s);
+      if (rows <= 2) return launch_decode_epi<1, SMAX, true, true, 2>(a, epilogue, out_dtype, grid, s);
+      if (rows <= 4) return launch_decode_epi<1, SMAX, true, true, 4>(a, epilogue, out_dtype, grid, s);
+      if (rows <= 8) return launch_decode_epi<1, SMAX, true, true, 8>(a, epilogue, out_dtype, grid, s);
+    }
     return ln ? launch_decode_epi<1, SMAX, true, true>(a, epilogue, out_dtype, grid, s)
               : launch_decode_epi<1, SMAX, false, true>(a, epilogue, out_dtype, grid, s);
+  }
   return ln ? launch_decode_epi<1, SMAX, true, false>(a, epilogue, out_dtype, grid, s)
             : launch_decode_epi<1, SMAX, false, false>(a, epilogue, out_dtype, grid, s);
 }

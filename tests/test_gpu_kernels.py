@@ -254,7 +254,9 @@ def test_linear_mfma_chooses_the_largest_tiles_for_a_large_problem():
 @pytest.mark.parametrize("n,k,o,ln_bias,gather", [(8, 512, 1536, True, False), (3, 96, 503, False, True),
                                                   (40, 80, 257, True, True), (64, 2048, 64, False, False), (64, 512, 2048, True, False), (33, 768, 96, True, True),
                                                   (17, 1600, 48, True, False), (16, 1600, 130, True, True),
-                                                  (1, 160, 48, False, False), (5, 768, 2050, True, True)])
+                                                  (1, 160, 48, False, False), (5, 768, 2050, True, True),
+                                                  (2, 1024, 272, True, True), (4, 1600, 144, False, True), (7, 512, 80, True, True),
+                                                  (1, 1600, 4800, True, True), (8, 2048, 96, True, True)])
 def test_linear_skinny_through_a_folded_layer_norm(n, k, o, ln_bias, gather, general):
     g = torch.Generator().manual_seed(4)
     x = rnd(g, 70, k, scale=2.0) + 0.5
@@ -287,15 +289,16 @@ def test_linear_skinny_through_a_folded_layer_norm(n, k, o, ln_bias, gather, gen
             helpers.assert_close(out_m[:n], P.plain_linear(h, w.double(), bias.double()), "bfloat16",
                                  f"LN + skinny, rows mode {mode}")
             assert torch.isnan(out_m[n:]).all(), "rows beyond n_rows were written"
-        outs = []
-        for rpg in (16, 4, 2):
+        for rpg in (16, 8, 4, 2, 1):
             out_g = torch.full((n + 1, o), float("nan"), dtype=torch.float32, device=DEV)
             assert kernels.linear_skinny(None, wf, bias_f, out_g, n, kernels.EPI_NONE, ln_x=x.to(DEV),
                                          ln_colsum=colsum, ln_eps=1e-5, ln_rows=i32(rows) if gather else None,
                                          rows_mode=kernels.ROWS_GROUPS, rows_per_group=rpg)
-            outs.append(out_g)
-        assert torch.equal(outs[0][:n], outs[1][:n]) and torch.equal(outs[0][:n], outs[2][:n])
-        assert torch.isnan(outs[2][n:]).all(), "rows beyond n_rows were written"
+            # the rows' statistics are summed in an order that follows the rows of a workgroup,
+            # so the results agree to rounding, not bit by bit
+            helpers.assert_close(out_g[:n], P.plain_linear(h, w.double(), bias.double()), "bfloat16",
+                                 f"LN + skinny, {rpg} rows to a workgroup")
+            assert torch.isnan(out_g[n:]).all(), "rows beyond n_rows were written"
 
 
 @pytest.mark.parametrize("general", [False, True])
