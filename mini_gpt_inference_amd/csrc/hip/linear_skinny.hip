@@ -328,6 +328,8 @@ static int linear_skinny_launch(const void* act, long lda, const float* x, const
   const bool ln = x != nullptr;
   if (ln && !colsum) return MGPT_ERR_NULL;
   if (!ln && (lda < k_dim || (lda % 8) != 0)) return MGPT_ERR_BAD_SHAPE;
+  // rows and matrix are loaded 16 bytes at a time
+  if (((((size_t)act) | ((size_t)x) | ((size_t)w) | ((size_t)w_packed)) & 15) != 0) return MGPT_ERR_BAD_SHAPE;
   if (epilogue == SK_EPI_QKV) {
     if (!kpool || !vpool || !slot_mapping) return MGPT_ERR_NULL;
     if (head_dim <= 0 || (head_dim % 4) != 0 || (q_width % 4) != 0 || q_width + 2 * kv_width != n_out ||
