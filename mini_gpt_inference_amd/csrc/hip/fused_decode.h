@@ -30,4 +30,5 @@ struct FusedResidual {
 #define FUSED_GROUP_PARTS 4    // parts of a row that one thread of a workgroup adds up
 #define FUSED_THREADS 1024
 #define FUSED_WAVES 16
+#define FUSED_ATTN_ONE_TOKEN_WGS 256  // (token, head) pairs up to which the attention kernel gives each a workgroup of its own
 #define FUSED_MLP_SLICE 64     // hidden units of the feed-forward that one workgroup owns

@@ -1,6 +1,7 @@
 // The fused kernels of a decode step with few rows (bfloat16): two kernels a layer.
 //
-//  * fused_attention_decode_kernel, one workgroup per (token, head): adds up the residual row that
+//  * fused_attention_decode_kernel, one workgroup per head and token (or two or four neighbouring
+//    tokens, in steps of many rows): adds up the residual row that
 //    the kernels before it left as a sum (fused_decode.h), LayerNorm, this head's query, key and
 //    value (src/minigpt_infer/model.py:43,49-53), the key and value into their page
 //    (src/minigpt_infer/cache/paged.py:125-137), attention over the request's pages and the new
@@ -207,7 +208,7 @@ struct FusedAttnArgs {
   int max_blocks;
   const int* positions;
   const int* q_req;
-  int width, n_head, page_shift, num_pages;
+  int n_rows, width, n_head, page_shift, num_pages;
   unsigned int page_bytes;
   float scale_log2e;
 };
@@ -216,7 +217,11 @@ struct FusedAttnArgs {
 // (170 KB a microsecond) when sixteen waves each have up to sixteen of them in flight, and half of
 // that with eight waves that have twice as many each.  A wave therefore holds few loads at a time,
 // and a lane at most 128 registers.
-template <int D, bool TABLES>
+// TK: tokens of a workgroup (the same head of TK neighbouring tokens).  The projections of all of
+// them come out of the same matrix loads (a token a column of the MFMA's output); each token's
+// attention follows in turn.  More tokens a workgroup pay where the step has more (token, head)
+// pairs than the machine has compute units.
+template <int D, bool TABLES, int TK = 1>
 __global__ __launch_bounds__(FUSED_THREADS) void fused_attention_decode_kernel(FusedAttnArgs a) {
   constexpr int T = 3 * D / 16;                  // row tiles of this head's q, k and v
   constexpr int TG = T < 12 ? T : 12;            // of them in flight together
@@ -227,30 +232,32 @@ __global__ __launch_bounds__(FUSED_THREADS) void fused_attention_decode_kernel(F
   constexpr int CHUNK = NI * KPI;                // keys of a wave in one pass
   constexpr int NK2 = D <= 32 ? 1 : D / 32;      // k steps of the projection that hold this head's columns
   constexpr int TP2 = 4 / NK2 > 0 ? 4 / NK2 : 1; // its row tiles per wave whose loads are in flight together
-  // one pool for what is never alive together: the row's partial sums, then the waves' sums of
-  // q, k, v, then attention's partial results
-  constexpr int POOL_FLOATS = FUSED_WAVES * T * 16 > 4096 ? FUSED_WAVES * T * 16 : 4096;
-  static_assert(FUSED_WAVES * T * 16 <= POOL_FLOATS, "the pool holds the waves' sums of q, k, v");
-  static_assert(FUSED_WAVES * D <= POOL_FLOATS, "the pool holds the waves' sums of attention");
-  __shared__ __align__(16) float pool[POOL_FLOATS];
-  __shared__ __align__(16) bf16_t act_s[FUSED_MAX_WIDTH];
+  // one pool for what is never alive together: the rows' partial sums, then the waves' sums of
+  // q, k, v, then attention's partial results; a stretch of it per token
+  constexpr int POOL_ONE = FUSED_WAVES * T * 16 > 4096 ? FUSED_WAVES * T * 16 : 4096;
+  static_assert(FUSED_WAVES * T * 16 <= POOL_ONE, "the pool holds the waves' sums of q, k, v");
+  static_assert(FUSED_WAVES * D <= POOL_ONE, "the pool holds the waves' sums of attention");
+  static_assert(TK >= 1 && TK <= 4 && 3 * D * TK <= FUSED_THREADS, "a thread per value of q, k, v of every token");
+  __shared__ __align__(16) float pool[POOL_ONE * TK];
+  __shared__ __align__(16) bf16_t act_s[TK * FUSED_MAX_WIDTH];
   __shared__ __align__(16) float gain_s[FUSED_MAX_WIDTH], beta_s[FUSED_MAX_WIDTH];
-  __shared__ __align__(16) bf16_t q_s[D];
-  __shared__ __align__(16) bf16_t k_s[D];
-  __shared__ __align__(16) bf16_t v_s[D];
-  __shared__ __align__(16) bf16_t y_s[D];
+  __shared__ __align__(16) float bproj_s[FUSED_MAX_WIDTH];  // the projection's bias (first head only)
+  __shared__ __align__(16) bf16_t q_s[TK * D];
+  __shared__ __align__(16) bf16_t k_s[TK * D];
+  __shared__ __align__(16) bf16_t v_s[TK * D];
+  __shared__ __align__(16) bf16_t y_s[TK * D];
   __shared__ float m_s[FUSED_WAVES];
   __shared__ float l_s[FUSED_WAVES];
-  float* const xs = pool;
   float* const red_s = pool;
   float* const acc_s = pool;
 
-  const int h = blockIdx.x, n = blockIdx.y;
+  const int h = blockIdx.x, n0 = blockIdx.y * TK;
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int lrow = lane & 15, g = lane >> 4;
   const int sub = lane / LPK, dg = lane % LPK;
   const int C = a.width, KS = C >> 5, V = C >> 2;
+  const int ltok = TK == 1 ? 0 : lrow % TK;  // the token whose column of an MFMA this lane holds
 
   FD_STAMP(0);
   // ---- The prologue.  A compute unit issues a wave's 16-byte loads at about a kilobyte every
@@ -260,58 +267,82 @@ __global__ __launch_bounds__(FUSED_THREADS) void fused_attention_decode_kernel(F
   // weights of the first: measured, 1.6 us a layer slower); the rest, and the keys and values, are
   // sent for behind it, while the first wave norms the row.  A wave's loads come back in order:
   // the step's numbers and the row first, keys and values last.
-  const int qr = a.q_req[n];
-  const int qpos = a.positions[n];
-  const int slot = a.slot_mapping[n];
-  const int* bt = a.block_tables + (long)n * a.max_blocks;  // a decode-only step: token n is request n
+  // (a token beyond the step's rows repeats the workgroup's first and stores nothing, like a token of
+  // the padding; a decode-only step: token n is request n)
+  int tokn[TK], qpos[TK], slot[TK];
+  bool ok[TK];
+  const int* bt[TK];
+  bool any = false;
+#pragma unroll
+  for (int t = 0; t < TK; ++t) {
+    const bool in = n0 + t < a.n_rows;
+    tokn[t] = in ? n0 + t : n0;
+    ok[t] = in && a.q_req[tokn[t]] >= 0;
+    any = any || ok[t];
+    qpos[t] = a.positions[tokn[t]];
+    slot[t] = a.slot_mapping[tokn[t]];
+    bt[t] = a.block_tables + (long)tokn[t] * a.max_blocks;
+  }
+  // attention: the waves are dealt out to the tokens, WPT neighbouring waves each
+  constexpr int WPT = FUSED_WAVES / TK;
+  const int wt = wave / WPT, ww = wave - wt * WPT;  // this wave's token, and its place among the token's waves
+  int my_qpos = qpos[0];
+  bool my_ok = ok[0];
+  const int* my_bt = bt[0];
+#pragma unroll
+  for (int t = 1; t < TK; ++t)
+    if (wt == t) {
+      my_qpos = qpos[t];
+      my_ok = ok[t];
+      my_bt = bt[t];
+    }
+  const int c00 = ww * CHUNK;
   int page0[NI];
 #pragma unroll
   for (int i = 0; i < NI; ++i) {
-    const int e = (wave * CHUNK + i * KPI + sub) >> a.page_shift;
-    page0[i] = bt[e < a.max_blocks ? e : a.max_blocks - 1];
+    const int e = (c00 + i * KPI + sub) >> a.page_shift;
+    page0[i] = my_bt[e < a.max_blocks ? e : a.max_blocks - 1];
   }
-  // the row: V vectors of four; the threads form G groups of V, group q adds up the parts q, q + G, ...
+  // a row: V vectors of four; the threads form G groups of V, group q adds up the parts q, q + G, ...
   // (group 0 the base as well)
   const int G = FUSED_THREADS / V;
   const int gq = tid / V, vq = tid - gq * V;
-  float4 piece = make_float4(0.f, 0.f, 0.f, 0.f);
-  float4 part[FUSED_GROUP_PARTS];
-  if (TABLES) {
-    if (gq == 0) {
-      const uint2 t = reinterpret_cast<const uint2*>(a.res.tok_table)[(long)a.res.ids[n] * V + vq];
-      piece = fd_bf16x4(t);
-      if (a.res.pos_table)
-        piece = fd_add4(piece, fd_bf16x4(reinterpret_cast<const uint2*>(a.res.pos_table)[(long)a.res.positions[n] * V + vq]));
-    }
-  } else {
-    if (gq == 0) piece = reinterpret_cast<const float4*>(a.res.base)[(long)n * V + vq];
+  float4 piece[TK];
+  float4 part[TK][FUSED_GROUP_PARTS];
 #pragma unroll
-    for (int u = 0; u < FUSED_GROUP_PARTS; ++u) {
-      part[u] = make_float4(0.f, 0.f, 0.f, 0.f);
-      const int p = gq + u * G;
-      if (gq < G && p < a.res.n_parts)
-        part[u] = reinterpret_cast<const float4*>(a.res.partials + p * a.res.part_stride)[(long)n * V + vq];
+  for (int t = 0; t < TK; ++t) {
+    piece[t] = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (TABLES) {
+      if (gq == 0) {
+        const uint2 tr = reinterpret_cast<const uint2*>(a.res.tok_table)[(long)a.res.ids[tokn[t]] * V + vq];
+        piece[t] = fd_bf16x4(tr);
+        if (a.res.pos_table)
+          piece[t] = fd_add4(piece[t], fd_bf16x4(reinterpret_cast<const uint2*>(
+                                           a.res.pos_table)[(long)a.res.positions[tokn[t]] * V + vq]));
+      }
+    } else {
+      if (gq == 0) piece[t] = reinterpret_cast<const float4*>(a.res.base)[(long)tokn[t] * V + vq];
+#pragma unroll
+      for (int u = 0; u < FUSED_GROUP_PARTS; ++u) {
+        part[t][u] = make_float4(0.f, 0.f, 0.f, 0.f);
+        const int p = gq + u * G;
+        if (gq < G && p < a.res.n_parts)
+          part[t][u] = reinterpret_cast<const float4*>(a.res.partials + p * a.res.part_stride)[(long)tokn[t] * V + vq];
+      }
     }
   }
-  // the LayerNorm's gain and bias go through LDS to the wave that will norm the row
-  const int vc = tid < V ? tid : 0;
-  float4 gain4 = make_float4(0.f, 0.f, 0.f, 0.f), beta4 = make_float4(0.f, 0.f, 0.f, 0.f);
-  if (tid < V) {
-    gain4 = reinterpret_cast<const float4*>(a.gain)[vc];
-    if (a.beta) beta4 = reinterpret_cast<const float4*>(a.beta)[vc];
-  }
-  // what the epilogues add: this thread's bias of q, k or v, and (first head) the projection's
+  // the LayerNorm's gain and bias go through LDS to the waves that will norm the rows, and so does
+  // what the last epilogue adds (first head: the projection's bias); a group of threads each
+  const bool proj_bias = h == 0 && a.bproj != nullptr;
+  float4 gb4 = make_float4(0.f, 0.f, 0.f, 0.f);
+  if (gq == 0) gb4 = reinterpret_cast<const float4*>(a.gain)[vq];
+  else if (gq == 1 && a.beta) gb4 = reinterpret_cast<const float4*>(a.beta)[vq];
+  else if (gq == 2 && proj_bias) gb4 = reinterpret_cast<const float4*>(a.bproj)[vq];
+  // what the epilogue of q, k, v adds: this thread's bias
+  const int qt = tid / (3 * D), qi = tid - qt * (3 * D);  // this thread's token and value among its q, k, v
   float qkv_bias = 0.f;
-  if (tid < 3 * D && a.bqkv) qkv_bias = a.bqkv[(tid / D) * a.n_head * D + h * D + tid % D];
+  if (qt < TK && a.bqkv) qkv_bias = a.bqkv[(qi / D) * a.n_head * D + h * D + qi % D];
   const int n_tiles2 = C >> 4;
-  float4 proj_bias[TP2];
-#pragma unroll
-  for (int j = 0; j < TP2; ++j) {
-    proj_bias[j] = make_float4(0.f, 0.f, 0.f, 0.f);
-    const int tile = wave + FUSED_WAVES * j;
-    if (h == 0 && a.bproj && lrow == 0 && tile < n_tiles2)
-      proj_bias[j] = *reinterpret_cast<const float4*>(a.bproj + tile * 16 + g * 4);
-  }
   const int per = (KS + FUSED_WAVES - 1) / FUSED_WAVES;  // k steps of a wave
   const int ks0 = wave * per;
   const int nks = max(0, min(per, KS - ks0));
@@ -325,14 +356,14 @@ __global__ __launch_bounds__(FUSED_THREADS) void fused_attention_decode_kernel(F
     const long tile_ = (long)(tt_ / (D / 16)) * tiles_per_part + h * (D / 16) + (tt_ % (D / 16));           \
     wv[tt_][i_] = fd_packed(a.wqkv, tile_, KS, i_ < nks ? ks0 + i_ : 0, lane);                              \
   }
-  // keys and values of the first pass: their addresses need the block table and the position only
-  const int kv_end = qpos;  // the keys before the token's own
+  // keys and values of a token's first pass: their addresses need the block table and the position only
+  // (kv_end: the keys before the token's own)
   const int page_mask = (1 << a.page_shift) - 1;
   const unsigned int lane_off = ((unsigned int)(h << a.page_shift) * D + dg * 8) * 2u;
   uint4 kraw[NI], vraw[NI];
-  const int c00 = wave * CHUNK;
+  const int kv_end = my_qpos;
 #define FA_LOAD_KV                                                                                                    \
-  if (c00 < kv_end) { /* the same in all lanes of a wave */                                                          \
+  if (my_ok && c00 < kv_end) { /* the same in all lanes of a wave */                                                 \
     _Pragma("unroll") for (int i = 0; i < NI; ++i) {                                                                 \
       const int j_ = c00 + i * KPI + sub;                                                                            \
       const bool follow_ = j_ < kv_end && (unsigned int)page0[i] < (unsigned int)a.num_pages;                        \
@@ -343,30 +374,39 @@ __global__ __launch_bounds__(FUSED_THREADS) void fused_attention_decode_kernel(F
     }                                                                                                                \
   }
   FA_LOAD_W(0)
-  if (qr < 0) return;  // a token of the padding (the whole workgroup)
-  FD_STAMP_AFTER(16, piece.x);
+  if (!any) return;  // tokens of the padding only (the whole workgroup)
+  FD_STAMP_AFTER(16, piece[0].x);
 
-  // ---- the residual row's sum: every group of threads its parts, then the first wave all groups
-  if (!TABLES) {
+  // ---- the residual rows' sums: every group of threads its parts, then a wave per row all groups
 #pragma unroll
-    for (int u = 0; u < FUSED_GROUP_PARTS; ++u) piece = fd_add4(piece, part[u]);
+  for (int t = 0; t < TK; ++t) {
+    if (!TABLES) {
+#pragma unroll
+      for (int u = 0; u < FUSED_GROUP_PARTS; ++u) piece[t] = fd_add4(piece[t], part[t][u]);
+    }
+    if (gq < G) reinterpret_cast<float4*>(pool + t * POOL_ONE)[gq * V + vq] = piece[t];
   }
-  if (gq < G) reinterpret_cast<float4*>(xs)[gq * V + vq] = piece;
-  if (tid < V) {
-    reinterpret_cast<float4*>(gain_s)[tid] = gain4;
-    reinterpret_cast<float4*>(beta_s)[tid] = beta4;
-  }
+  if (gq < 3) reinterpret_cast<float4*>(gq == 0 ? gain_s : gq == 1 ? beta_s : bproj_s)[vq] = gb4;
   fd_barrier();
   FD_STAMP(17);
-  // every wave sends for the rest of its weights and for its keys and values; then the first wave
-  // norms the row (LDS and arithmetic only) while the others wait at the next barrier
+  // every wave sends for the rest of its weights and for its keys and values; then the first waves
+  // norm a row each (LDS and arithmetic only) while the others wait at the next barrier
   FA_LOAD_W(1)
   FA_LOAD_W(2)
   FA_LOAD_W(3)
   FA_LOAD_KV
 #undef FA_LOAD_W
 #undef FA_LOAD_KV
-  if (wave == 0) {
+  if (wave < TK) {
+    const float* xs = pool + wave * POOL_ONE;
+    int row = tokn[0];
+    bool row_ok = ok[0];
+#pragma unroll
+    for (int t = 1; t < TK; ++t)
+      if (wave == t) {
+        row = tokn[t];
+        row_ok = ok[t];
+      }
     float4 xv[2];
     xv[0] = xv[1] = make_float4(0.f, 0.f, 0.f, 0.f);
     // ---- LayerNorm, within one wave: no barrier between the sums
@@ -380,7 +420,7 @@ __global__ __launch_bounds__(FUSED_THREADS) void fused_attention_decode_kernel(F
 #pragma unroll 8
         for (int q = 1; q < used; ++q) xv[u] = fd_add4(xv[u], reinterpret_cast<const float4*>(xs)[q * V + v]);
         // the row as it stands, stored by the first head's workgroup for the kernels behind this one
-        if (h == 0 && a.res.settled) reinterpret_cast<float4*>(a.res.settled + (long)n * C)[v] = xv[u];
+        if (h == 0 && row_ok && a.res.settled) reinterpret_cast<float4*>(a.res.settled + (long)row * C)[v] = xv[u];
       }
     }
     const float mean = wave_sum(fd_sum4(xv[0]) + fd_sum4(xv[1])) / (float)C;
@@ -402,15 +442,15 @@ __global__ __launch_bounds__(FUSED_THREADS) void fused_attention_decode_kernel(F
         uint2 pk;
         pk.x = pack_bf16x2(dv[u].x * rstd * gn.x + bt4.x, dv[u].y * rstd * gn.y + bt4.y);
         pk.y = pack_bf16x2(dv[u].z * rstd * gn.z + bt4.z, dv[u].w * rstd * gn.w + bt4.w);
-        reinterpret_cast<uint2*>(act_s)[v] = pk;
+        reinterpret_cast<uint2*>(act_s + wave * FUSED_MAX_WIDTH)[v] = pk;
       }
     }
   }
-  fd_barrier();  // also: the row's partial sums are read, their place takes the waves' sums now
+  fd_barrier();  // also: the rows' partial sums are read, their place takes the waves' sums now
   FD_STAMP(1);
 
   // ---- q, k, v of this head: every wave a stretch of k over all the row tiles; the waves' sums
-  // meet in LDS (every column of the MFMA's output holds the one token: the lanes of column 0 speak)
+  // meet in LDS (column c of the MFMA's output holds token c mod TK: the lanes of the first TK columns speak)
   for (int s0 = 0, first = 1;; first = 0) {
 #pragma unroll
     for (int grp = 0; grp < NG; ++grp) {
@@ -426,15 +466,16 @@ __global__ __launch_bounds__(FUSED_THREADS) void fused_attention_decode_kernel(F
       bf16x8_t b[SMAX];
 #pragma unroll
       for (int i = 0; i < SMAX; ++i)
-        b[i] = *reinterpret_cast<const bf16x8_t*>(act_s + (s0 + i < nks ? ks0 + s0 + i : 0) * 32 + g * 8);
+        b[i] = *reinterpret_cast<const bf16x8_t*>(act_s + ltok * FUSED_MAX_WIDTH +
+                                                  (s0 + i < nks ? ks0 + s0 + i : 0) * 32 + g * 8);
 #pragma unroll
       for (int tt = 0; tt < TG; ++tt) {
         f32x4_t acc = (f32x4_t){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int i = 0; i < SMAX; ++i)
           if (s0 + i < nks) acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wv[tt][i], b[i], acc, 0, 0, 0);
-        if (lrow == 0) {
-          float4* r = reinterpret_cast<float4*>(red_s + (wave * T + grp * TG + tt) * 16 + g * 4);
+        if (lrow < TK) {
+          float4* r = reinterpret_cast<float4*>(red_s + ((lrow * FUSED_WAVES + wave) * T + grp * TG + tt) * 16 + g * 4);
           float4 v = make_float4(acc[0], acc[1], acc[2], acc[3]);
           if (s0 > 0) v = fd_add4(v, *r);
           *r = v;
@@ -456,19 +497,23 @@ __global__ __launch_bounds__(FUSED_THREADS) void fused_attention_decode_kernel(F
   }
   fd_barrier();
   FD_STAMP(2);
-  if (tid < 3 * D) {
+  if (qt < TK) {
     float v = 0.f;
 #pragma unroll
-    for (int w = 0; w < FUSED_WAVES; ++w) v += red_s[w * T * 16 + tid];
-    const int part = tid / D, d = tid - part * D;
+    for (int w = 0; w < FUSED_WAVES; ++w) v += red_s[(qt * FUSED_WAVES + w) * T * 16 + qi];
+    const int part = qi / D, d = qi - part * D;
     const bf16_t b = float_to_bf16(v + qkv_bias);
     if (part == 0) {
-      q_s[d] = b;
+      q_s[qt * D + d] = b;
     } else {
-      (part == 1 ? k_s : v_s)[d] = b;
-      if (slot >= 0) {
-        const long page = slot >> a.page_shift;
-        const int off = slot & page_mask;
+      (part == 1 ? k_s : v_s)[qt * D + d] = b;
+      int my_slot = -1;
+#pragma unroll
+      for (int t = 0; t < TK; ++t)
+        if (qt == t && ok[t]) my_slot = slot[t];
+      if (my_slot >= 0) {
+        const long page = my_slot >> a.page_shift;
+        const int off = my_slot & page_mask;
         const long dst = ((((page * a.n_head + h) << a.page_shift) + off) * (long)D) + d;
         (part == 1 ? a.kpool : a.vpool)[dst] = b;
       }
@@ -477,106 +522,110 @@ __global__ __launch_bounds__(FUSED_THREADS) void fused_attention_decode_kernel(F
   fd_barrier();  // also: the waves' sums are read, their place takes attention's partial results
   FD_STAMP(3);
 
-  // ---- attention over the keys before the token's own (from the pages) and its own (from LDS)
-  const uint4 qraw = *reinterpret_cast<const uint4*>(q_s + dg * 8);
+  // ---- attention: each token's waves over the keys before the token's own (from the pages); the
+  // token's first wave its own as well (from LDS)
   float m = -INFINITY, l = 0.f;
   float acc[8];
 #pragma unroll
   for (int e = 0; e < 8; ++e) acc[e] = 0.f;
-  for (int c_base = 0; c_base < kv_end; c_base += CHUNK * FUSED_WAVES) {
-    const int c0 = c_base + wave * CHUNK;
-    if (c_base > 0 && c0 < kv_end) {
-      int page[NI];
+  if (my_ok) {
+    const uint4 qraw = *reinterpret_cast<const uint4*>(q_s + wt * D + dg * 8);
+    for (int c_base = 0; c_base < kv_end; c_base += CHUNK * WPT) {
+      const int c0 = c_base + c00;
+      if (c_base > 0 && c0 < kv_end) {
+        int page[NI];
+#pragma unroll
+        for (int i = 0; i < NI; ++i) {
+          const int e = (c0 + i * KPI + sub) >> a.page_shift;
+          page[i] = my_bt[e < a.max_blocks ? e : a.max_blocks - 1];
+        }
+#pragma unroll
+        for (int i = 0; i < NI; ++i) {
+          const int j = c0 + i * KPI + sub;
+          const bool follow = j < kv_end && (unsigned int)page[i] < (unsigned int)a.num_pages;
+          const unsigned int row_off = ((unsigned int)page[i] * a.page_bytes) + (unsigned int)(j & page_mask) * (D * 2u);
+          const unsigned int off = follow ? row_off + lane_off : 0u;
+          kraw[i] = *reinterpret_cast<const uint4*>(reinterpret_cast<const char*>(a.kpool) + off);
+          vraw[i] = *reinterpret_cast<const uint4*>(reinterpret_cast<const char*>(a.vpool) + off);
+        }
+      }
+      if (__builtin_amdgcn_readfirstlane(c0 >= kv_end)) continue;
+      bool valid[NI];
 #pragma unroll
       for (int i = 0; i < NI; ++i) {
-        const int e = (c0 + i * KPI + sub) >> a.page_shift;
-        page[i] = bt[e < a.max_blocks ? e : a.max_blocks - 1];
+        valid[i] = c0 + i * KPI + sub < kv_end;
+        if (!valid[i]) vraw[i] = make_uint4(0, 0, 0, 0);  // its weight is 0, but 0 * NaN is not
       }
+      float s[NI];
+      float cmax = -INFINITY;
 #pragma unroll
       for (int i = 0; i < NI; ++i) {
-        const int j = c0 + i * KPI + sub;
-        const bool follow = j < kv_end && (unsigned int)page[i] < (unsigned int)a.num_pages;
-        const unsigned int row_off = ((unsigned int)page[i] * a.page_bytes) + (unsigned int)(j & page_mask) * (D * 2u);
-        const unsigned int off = follow ? row_off + lane_off : 0u;
-        kraw[i] = *reinterpret_cast<const uint4*>(reinterpret_cast<const char*>(a.kpool) + off);
-        vraw[i] = *reinterpret_cast<const uint4*>(reinterpret_cast<const char*>(a.vpool) + off);
+        float dot = fd_dot2(qraw.x, kraw[i].x, 0.f);
+        dot = fd_dot2(qraw.y, kraw[i].y, dot);
+        dot = fd_dot2(qraw.z, kraw[i].z, dot);
+        dot = fd_dot2(qraw.w, kraw[i].w, dot);
+        dot = fd_group_sum<LPK>(dot) * a.scale_log2e;
+        s[i] = valid[i] ? dot : -INFINITY;
+        cmax = fmaxf(cmax, s[i]);
+      }
+      const float m_new = fmaxf(m, wave_max(cmax));
+      if (m_new != -INFINITY) {  // the same in all lanes; false only while the wave has seen no key
+        const float alpha = __builtin_amdgcn_exp2f(m - m_new);  // m = -inf: 0
+        l *= alpha;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc[e] *= alpha;
+        m = m_new;
+#pragma unroll
+        for (int i = 0; i < NI; i += 2) {
+          const float pa = __builtin_amdgcn_exp2f(s[i] - m_new), pb = __builtin_amdgcn_exp2f(s[i + 1] - m_new);
+          l += pa + pb;
+          const unsigned int pp = pack_bf16x2(pa, pb);
+          const unsigned int va[4] = {vraw[i].x, vraw[i].y, vraw[i].z, vraw[i].w};
+          const unsigned int vb[4] = {vraw[i + 1].x, vraw[i + 1].y, vraw[i + 1].z, vraw[i + 1].w};
+#pragma unroll
+          for (int w = 0; w < 4; ++w) {
+            // (va.low half, vb.low half) and (va.high half, vb.high half): channel 2w and 2w+1 of both keys
+            const unsigned int lo = __builtin_amdgcn_perm(vb[w], va[w], 0x05040100u);
+            const unsigned int hi = __builtin_amdgcn_perm(vb[w], va[w], 0x07060302u);
+            acc[2 * w] = fd_dot2(pp, lo, acc[2 * w]);
+            acc[2 * w + 1] = fd_dot2(pp, hi, acc[2 * w + 1]);
+          }
+        }
       }
     }
-    if (__builtin_amdgcn_readfirstlane(c0 >= kv_end)) continue;
-    bool valid[NI];
-#pragma unroll
-    for (int i = 0; i < NI; ++i) {
-      valid[i] = c0 + i * KPI + sub < kv_end;
-      if (!valid[i]) vraw[i] = make_uint4(0, 0, 0, 0);  // its weight is 0, but 0 * NaN is not
-    }
-    float s[NI];
-    float cmax = -INFINITY;
-#pragma unroll
-    for (int i = 0; i < NI; ++i) {
-      float dot = fd_dot2(qraw.x, kraw[i].x, 0.f);
-      dot = fd_dot2(qraw.y, kraw[i].y, dot);
-      dot = fd_dot2(qraw.z, kraw[i].z, dot);
-      dot = fd_dot2(qraw.w, kraw[i].w, dot);
+    if (ww == 0) {
+      // the token's own key and value: its first wave takes them in, that wave's first key group holds the weight
+      const uint4 kk = *reinterpret_cast<const uint4*>(k_s + wt * D + dg * 8);
+      const uint4 vv = *reinterpret_cast<const uint4*>(v_s + wt * D + dg * 8);
+      float dot = fd_dot2(qraw.x, kk.x, 0.f);
+      dot = fd_dot2(qraw.y, kk.y, dot);
+      dot = fd_dot2(qraw.z, kk.z, dot);
+      dot = fd_dot2(qraw.w, kk.w, dot);
       dot = fd_group_sum<LPK>(dot) * a.scale_log2e;
-      s[i] = valid[i] ? dot : -INFINITY;
-      cmax = fmaxf(cmax, s[i]);
-    }
-    const float m_new = fmaxf(m, wave_max(cmax));
-    if (m_new != -INFINITY) {  // the same in all lanes; false only while the wave has seen no key
-      const float alpha = __builtin_amdgcn_exp2f(m - m_new);  // m = -inf: 0
+      const float m_new = fmaxf(m, dot);
+      const float alpha = __builtin_amdgcn_exp2f(m - m_new);
       l *= alpha;
 #pragma unroll
       for (int e = 0; e < 8; ++e) acc[e] *= alpha;
       m = m_new;
-#pragma unroll
-      for (int i = 0; i < NI; i += 2) {
-        const float pa = __builtin_amdgcn_exp2f(s[i] - m_new), pb = __builtin_amdgcn_exp2f(s[i + 1] - m_new);
-        l += pa + pb;
-        const unsigned int pp = pack_bf16x2(pa, pb);
-        const unsigned int va[4] = {vraw[i].x, vraw[i].y, vraw[i].z, vraw[i].w};
-        const unsigned int vb[4] = {vraw[i + 1].x, vraw[i + 1].y, vraw[i + 1].z, vraw[i + 1].w};
+      const float p = __builtin_amdgcn_exp2f(dot - m_new);
+      if (sub == 0) {
+        l += p;
+        const unsigned int pp = pack_bf16x2(p, 0.f);
+        const unsigned int vw[4] = {vv.x, vv.y, vv.z, vv.w};
 #pragma unroll
         for (int w = 0; w < 4; ++w) {
-          // (va.low half, vb.low half) and (va.high half, vb.high half): channel 2w and 2w+1 of both keys
-          const unsigned int lo = __builtin_amdgcn_perm(vb[w], va[w], 0x05040100u);
-          const unsigned int hi = __builtin_amdgcn_perm(vb[w], va[w], 0x07060302u);
-          acc[2 * w] = fd_dot2(pp, lo, acc[2 * w]);
-          acc[2 * w + 1] = fd_dot2(pp, hi, acc[2 * w + 1]);
+          acc[2 * w] = fd_dot2(pp, vw[w] & 0xffffu, acc[2 * w]);
+          acc[2 * w + 1] = fd_dot2(pp, vw[w] >> 16, acc[2 * w + 1]);
         }
-      }
-    }
-  }
-  if (wave == 0) {
-    // the token's own key and value: the first wave takes them in, its first key group holds the weight
-    const uint4 kk = *reinterpret_cast<const uint4*>(k_s + dg * 8);
-    const uint4 vv = *reinterpret_cast<const uint4*>(v_s + dg * 8);
-    float dot = fd_dot2(qraw.x, kk.x, 0.f);
-    dot = fd_dot2(qraw.y, kk.y, dot);
-    dot = fd_dot2(qraw.z, kk.z, dot);
-    dot = fd_dot2(qraw.w, kk.w, dot);
-    dot = fd_group_sum<LPK>(dot) * a.scale_log2e;
-    const float m_new = fmaxf(m, dot);
-    const float alpha = __builtin_amdgcn_exp2f(m - m_new);
-    l *= alpha;
-#pragma unroll
-    for (int e = 0; e < 8; ++e) acc[e] *= alpha;
-    m = m_new;
-    const float p = __builtin_amdgcn_exp2f(dot - m_new);
-    if (sub == 0) {
-      l += p;
-      const unsigned int pp = pack_bf16x2(p, 0.f);
-      const unsigned int vw[4] = {vv.x, vv.y, vv.z, vv.w};
-#pragma unroll
-      for (int w = 0; w < 4; ++w) {
-        acc[2 * w] = fd_dot2(pp, vw[w] & 0xffffu, acc[2 * w]);
-        acc[2 * w + 1] = fd_dot2(pp, vw[w] >> 16, acc[2 * w + 1]);
       }
     }
   }
   FD_STAMP(4);
 
   // ---- merge: first across the key groups of a wave (lanes that differ above the LPK lanes of a
-  // key: the maximum is the wave's already, so the sums simply add), then across the waves in LDS
+  // key: the maximum is the wave's already, so the sums simply add), then across a token's waves in LDS
+  // (the waves of a token that stores nothing leave zeros)
   l = fd_sum_over_keys<LPK>(l);
 #pragma unroll
   for (int e = 0; e < 8; ++e) acc[e] = fd_sum_over_keys<LPK>(acc[e]);
@@ -590,16 +639,18 @@ __global__ __launch_bounds__(FUSED_THREADS) void fused_attention_decode_kernel(F
     dst[1] = make_float4(acc[4], acc[5], acc[6], acc[7]);
   }
   fd_barrier();
-  if (tid < D) {
-    float mx = m_s[0];
+  if (tid < D * TK) {
+    const int t = tid / D, d = tid - t * D;
+    const int w0 = t * WPT;
+    float mx = m_s[w0];
 #pragma unroll
-    for (int w = 1; w < FUSED_WAVES; ++w) mx = fmaxf(mx, m_s[w]);
+    for (int w = 1; w < WPT; ++w) mx = fmaxf(mx, m_s[w0 + w]);
     float av = 0.f, lt = 0.f;
 #pragma unroll
-    for (int w = 0; w < FUSED_WAVES; ++w) {
-      const float f = __builtin_amdgcn_exp2f(m_s[w] - mx);  // a wave without keys: exp2(-inf) = 0, and its sums are 0
-      av = fmaf(acc_s[w * D + tid], f, av);
-      lt = fmaf(l_s[w], f, lt);
+    for (int w = 0; w < WPT; ++w) {
+      const float f = __builtin_amdgcn_exp2f(m_s[w0 + w] - mx);  // a wave without keys: exp2(-inf) = 0, and its sums are 0
+      av = fmaf(acc_s[(w0 + w) * D + d], f, av);
+      lt = fmaf(l_s[w0 + w], f, lt);
     }
     y_s[tid] = float_to_bf16(av / lt);
   }
@@ -613,9 +664,13 @@ __global__ __launch_bounds__(FUSED_THREADS) void fused_attention_decode_kernel(F
 #pragma unroll
     for (int i = 0; i < NK2; ++i) {
       const int idx0 = (ks_b + i) * 32 + g * 8 - h * D;  // where this lane's 8 values of k lie in the head
-      yb[i] = (idx0 >= 0 && idx0 < D) ? *reinterpret_cast<const bf16x8_t*>(y_s + idx0) : zero8;
+      yb[i] = (idx0 >= 0 && idx0 < D) ? *reinterpret_cast<const bf16x8_t*>(y_s + ltok * D + idx0) : zero8;
     }
-    float* orow = a.out_partials + h * a.out_part_stride + (long)n * C;
+    bool store = false;
+#pragma unroll
+    for (int t = 0; t < TK; ++t)
+      if (lrow == t) store = ok[t];
+    float* orow = a.out_partials + h * a.out_part_stride + (long)(n0 + (lrow < TK ? lrow : 0)) * C;
     for (int pass = 0;; ++pass) {
 #pragma unroll
       for (int j = 0; j < TP2; ++j) {
@@ -624,11 +679,10 @@ __global__ __launch_bounds__(FUSED_THREADS) void fused_attention_decode_kernel(F
           f32x4_t o = (f32x4_t){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
           for (int i = 0; i < NK2; ++i) o = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w2[j][i], yb[i], o, 0, 0, 0);
-          if (lrow == 0) {
+          if (store) {
             const int oc = tile * 16 + g * 4;
             float4 v = make_float4(o[0], o[1], o[2], o[3]);
-            if (pass == 0) v = fd_add4(v, proj_bias[j]);
-            else if (h == 0 && a.bproj) v = fd_add4(v, *reinterpret_cast<const float4*>(a.bproj + oc));
+            if (proj_bias) v = fd_add4(v, *reinterpret_cast<const float4*>(bproj_s + oc));
             *reinterpret_cast<float4*>(orow + oc) = v;
           }
         }
@@ -988,16 +1042,29 @@ extern "C" int mgpt_fused_attention_decode(
   a.out_partials = out_partials; a.out_part_stride = out_part_stride;
   a.kpool = (bf16_t*)kpool; a.vpool = (bf16_t*)vpool; a.slot_mapping = slot_mapping;
   a.block_tables = block_tables; a.max_blocks = max_blocks; a.positions = positions; a.q_req = q_req;
-  a.width = width; a.n_head = n_head; a.page_shift = page_shift; a.num_pages = num_pages;
+  a.n_rows = n_rows; a.width = width; a.n_head = n_head; a.page_shift = page_shift; a.num_pages = num_pages;
   a.page_bytes = (unsigned int)(n_head * page_size * head_dim * 2);
   a.scale_log2e = scale * 1.4426950408889634f;
-  // the head is the fast index: the workgroups of a head (one per token) then land on the same
-  // XCD when the number of heads is a multiple of 8, and share its copy of the head's weights
-  dim3 grid(n_head, n_rows), block(FUSED_THREADS);
-#define FA_LAUNCH(DD)                                                                                     \
-  do {                                                                                                    \
-    if (base) hipLaunchKernelGGL((fused_attention_decode_kernel<DD, false>), grid, block, 0, stream, a);  \
-    else hipLaunchKernelGGL((fused_attention_decode_kernel<DD, true>), grid, block, 0, stream, a);        \
+  // the head is the fast index: the workgroups of a head then land on the same XCD when the number
+  // of heads is a multiple of 8, and share its copy of the head's weights.  Two tokens a workgroup
+  // from where one a workgroup would be more workgroups than compute units, four from where two would
+  // (heads of 128 keep to two: four tokens' q, k, v are more values than the workgroup has threads).
+  const long pairs = (long)n_rows * n_head;
+  int tk = pairs > 2 * FUSED_ATTN_ONE_TOKEN_WGS ? 4 : pairs > FUSED_ATTN_ONE_TOKEN_WGS ? 2 : 1;
+  if (tk == 4 && head_dim > 64) tk = 2;
+  dim3 grid(n_head, (n_rows + tk - 1) / tk), block(FUSED_THREADS);
+#define FA_LAUNCH(DD)                                                                                           \
+  do {                                                                                                          \
+    if (tk == 4) {                                                                                              \
+      if (base) hipLaunchKernelGGL((fused_attention_decode_kernel<(DD > 64 ? 64 : DD), false, 4>), grid, block, 0, stream, a);   \
+      else hipLaunchKernelGGL((fused_attention_decode_kernel<(DD > 64 ? 64 : DD), true, 4>), grid, block, 0, stream, a);         \
+    } else if (tk == 2) {                                                                                              \
+      if (base) hipLaunchKernelGGL((fused_attention_decode_kernel<DD, false, 2>), grid, block, 0, stream, a);   \
+      else hipLaunchKernelGGL((fused_attention_decode_kernel<DD, true, 2>), grid, block, 0, stream, a);         \
+    } else {                                                                                                    \
+      if (base) hipLaunchKernelGGL((fused_attention_decode_kernel<DD, false, 1>), grid, block, 0, stream, a);   \
+      else hipLaunchKernelGGL((fused_attention_decode_kernel<DD, true, 1>), grid, block, 0, stream, a);         \
+    }                                                                                                           \
   } while (0)
   switch (head_dim) {
     case 16: FA_LAUNCH(16); break;

@@ -21,11 +21,13 @@ import torch
 
 from . import kernels
 
-# most rows of a decode-only step that go through the fused kernels (one workgroup per token and
-# head re-reads the head's weights from the L2: beyond this the kernels that share a matrix
-# among the rows are faster; the 50.9M model's step takes 184 us against 203 at 32 rows, 282
-# against 256 at 48)
-FUSED_MAX_ROWS = 32
+# most rows of a decode-only step that go through the fused kernels.  A workgroup of the attention
+# kernel takes one token of a head, two from where that would be more workgroups than compute units
+# and four from where two would, so that a head's weights are read once for them; the 50.9M model's
+# step against the kernels that share a matrix among all rows: 228 us against 243 at 40 rows, 243 /
+# 263 at 64, 353 / 440 at 96, 371 / 456 at 128 (context 170); 336 / 368 at 64 and 569 / 650 at 128
+# (context 740).  Steps of more rows than this are not replayed from graphs either.
+FUSED_MAX_ROWS = 128
 
 
 @dataclass

@@ -50,6 +50,17 @@ ATTN_CASES = [
     dict(c=256, h=2, d=128, page=32, ctx=[40, 600], parts=0, bias=True),
     dict(c=320, h=5, d=64, page=16, ctx=[77, 0, 300], parts=12, bias=False),
     dict(c=128, h=6, d=32, page=2, ctx=[9, 64], parts=1, bias=True),     # heads * head size wider than the model
+    # more (token, head) pairs than compute units: two tokens a workgroup (more than 256 pairs) or four
+    # (more than 512; heads of 128 keep to two); workgroups of real tokens and padded ones, and of
+    # padded tokens only
+    dict(c=512, h=8, d=64, page=16, ctx=[(7 * i * i + 3 * i) % 600 for i in range(45)], parts=8, bias=True, pad=3),
+    dict(c=96, h=3, d=32, page=8, ctx=[(5 * i * i + i) % 300 for i in range(90)], parts=3, bias=False, pad=1),
+    dict(c=64, h=4, d=16, page=4, ctx=[(11 * i * i) % 1100 for i in range(70)], parts=4, bias=True, pad=2),
+    dict(c=256, h=2, d=128, page=32, ctx=[(3 * i * i + 2) % 400 for i in range(131)], parts=0, bias=True, pad=1),
+    dict(c=512, h=8, d=64, page=16, ctx=[(7 * i * i + 3 * i) % 530 for i in range(65)], parts=32, bias=True, pad=6),
+    dict(c=64, h=4, d=16, page=4, ctx=[(13 * i * i) % 270 for i in range(141)], parts=4, bias=False, pad=1),
+    dict(c=96, h=3, d=32, page=8, ctx=[(5 * i * i + 7 * i) % 200 for i in range(175)], parts=2, bias=True, pad=3),
+    dict(c=256, h=2, d=128, page=32, ctx=[(3 * i) % 40 for i in range(259)], parts=1, bias=True, pad=1),
 ]
 
 
@@ -60,7 +71,8 @@ def test_fused_attention_decode(case, tables):
     c, h, d, page, ctxs = spec["c"], spec["h"], spec["d"], spec["page"], spec["ctx"]
     g = torch.Generator().manual_seed(100 + case)
     n = len(ctxs)
-    rows = n + 1                                  # one padded token behind the real ones
+    pad = spec.get("pad", 1)
+    rows = n + pad                                # padded tokens behind the real ones
     qw = h * d
     gain, beta = 1 + 0.1 * rnd(g, c), rnd(g, c, scale=0.1)
     wqkv, wproj = bf(rnd(g, 3 * qw, c, scale=c ** -0.5)), bf(rnd(g, c, qw, scale=qw ** -0.5))
@@ -70,10 +82,10 @@ def test_fused_attention_decode(case, tables):
         vocab, n_pos = 61, max(ctxs) + 1
         tok, pos = bf(rnd(g, vocab, c)), bf(rnd(g, n_pos, c, scale=0.5))
         ids = torch.randint(0, vocab, (rows,), generator=g)
-        pending = PendingSums(None, None, 0, (tok.to(DEV), pos.to(DEV), i32(ids), i32(ctxs + [0])))
+        pending = PendingSums(None, None, 0, (tok.to(DEV), pos.to(DEV), i32(ids), i32(ctxs + [0] * pad)))
         true = tok.double()[ids[:n]] + pos.double()[ctxs]
     else:
-        pending, true = _pending(g, n, c, spec["parts"], extra_rows=1)
+        pending, true = _pending(g, n, c, spec["parts"], extra_rows=pad)
     # the cache: every request's earlier keys and values in pages handed out in a shuffled order
     max_blocks = max(-(-(x + 1) // page) for x in ctxs) + 1
     n_pages = sum(-(-(x + 1) // page) for x in ctxs) + 3
@@ -115,13 +127,13 @@ def test_fused_attention_decode(case, tables):
     kp_d, vp_d = kp.to(DEV), vp.to(DEV)
     took = kernels.fused_attention_decode(
         pending, settled, dev(gain), dev(beta), eps, kernels.pack_weight(wqkv.to(DEV)), dev(bqkv),
-        kernels.pack_weight(wproj.to(DEV)), dev(bproj), out, kp_d, vp_d, i32(slots + [-1]), bt.to(DEV),
-        i32(ctxs + [0]), i32(list(range(n)) + [-1]), rows, h, scale)
+        kernels.pack_weight(wproj.to(DEV)), dev(bproj), out, kp_d, vp_d, i32(slots + [-1] * pad), bt.to(DEV),
+        i32(ctxs + [0] * pad), i32(list(range(n)) + [-1] * pad), rows, h, scale)
     assert took
     torch.cuda.synchronize()
     helpers.assert_close(settled[:n], true, "float32", "the settled rows")
     helpers.assert_close(out[:, :n].sum(0), want, "bfloat16", f"fused attention case {case}")
-    assert torch.isnan(out[:, n]).all() and torch.isnan(settled[n]).all(), "the padded token's rows were written"
+    assert torch.isnan(out[:, n:]).all() and torch.isnan(settled[n:]).all(), "the padded tokens' rows were written"
     for r, ctx in enumerate(ctxs):                 # the token's key and value are in its page, nothing else changed
         page_i, off = slots[r] // page, slots[r] % page
         _, k, v = P.plain_split_heads(qkv[r:r + 1], h)
