@@ -199,6 +199,7 @@ struct FusedAttnArgs {
   const float* bqkv;   // or null
   const bf16_t* wproj;  // packed [width rows, n_head * D]
   const float* bproj;   // or null
+  const bf16_t* normed; // NORMED kernels: the rows after their LayerNorm, [rows][width]; the residual is not read
   float* out_partials;  // [n_head][part_rows][width]
   long out_part_stride;
   bf16_t* kpool;
@@ -218,11 +219,16 @@ struct FusedAttnArgs {
 // that with eight waves that have twice as many each.  A wave therefore holds few loads at a time,
 // and a lane at most 128 registers.
 // TK: tokens of a workgroup (the same head of TK neighbouring tokens).  The projections of all of
-// them come out of the same matrix loads (a token a column of the MFMA's output); each token's
-// attention follows in turn.  More tokens a workgroup pay where the step has more (token, head)
-// pairs than the machine has compute units.
-template <int D, bool TABLES, int TK = 1>
+// them come out of the same matrix loads (a token a column of the MFMA's output), and the waves are
+// dealt out to the tokens for attention.  More tokens a workgroup pay where the step has more
+// (token, head) pairs than the machine has compute units.
+// NORMED: the rows come normed, in bfloat16 (a.normed): every head's workgroup adding up the same
+// pending parts of its tokens is, at many rows, more traffic between the XCDs than everything else
+// the kernel reads (32 parts of 2 KB a token, eight heads: the first barrier passed after 12 us at
+// 128 rows), so a LayerNorm kernel before this one adds them up once.
+template <int D, bool TABLES, int TK = 1, bool NORMED = false>
 __global__ __launch_bounds__(FUSED_THREADS) void fused_attention_decode_kernel(FusedAttnArgs a) {
+  static_assert(!(NORMED && TABLES), "normed rows are no table rows");
   constexpr int T = 3 * D / 16;                  // row tiles of this head's q, k and v
   constexpr int TG = T < 12 ? T : 12;            // of them in flight together
   constexpr int NG = T / TG;
@@ -309,10 +315,17 @@ __global__ __launch_bounds__(FUSED_THREADS) void fused_attention_decode_kernel(F
   const int gq = tid / V, vq = tid - gq * V;
   float4 piece[TK];
   float4 part[TK][FUSED_GROUP_PARTS];
+  uint2 normed4 = make_uint2(0u, 0u);  // NORMED: group t of the threads brings token t's row
+  if (NORMED) {
+#pragma unroll
+    for (int t = 0; t < TK; ++t)
+      if (gq == t) normed4 = reinterpret_cast<const uint2*>(a.normed)[(long)tokn[t] * V + vq];
+  }
 #pragma unroll
   for (int t = 0; t < TK; ++t) {
     piece[t] = make_float4(0.f, 0.f, 0.f, 0.f);
-    if (TABLES) {
+    if (NORMED) {
+    } else if (TABLES) {
       if (gq == 0) {
         const uint2 tr = reinterpret_cast<const uint2*>(a.res.tok_table)[(long)a.res.ids[tokn[t]] * V + vq];
         piece[t] = fd_bf16x4(tr);
@@ -335,8 +348,8 @@ __global__ __launch_bounds__(FUSED_THREADS) void fused_attention_decode_kernel(F
   // what the last epilogue adds (first head: the projection's bias); a group of threads each
   const bool proj_bias = h == 0 && a.bproj != nullptr;
   float4 gb4 = make_float4(0.f, 0.f, 0.f, 0.f);
-  if (gq == 0) gb4 = reinterpret_cast<const float4*>(a.gain)[vq];
-  else if (gq == 1 && a.beta) gb4 = reinterpret_cast<const float4*>(a.beta)[vq];
+  if (gq == 0 && !NORMED) gb4 = reinterpret_cast<const float4*>(a.gain)[vq];
+  else if (gq == 1 && !NORMED && a.beta) gb4 = reinterpret_cast<const float4*>(a.beta)[vq];
   else if (gq == 2 && proj_bias) gb4 = reinterpret_cast<const float4*>(a.bproj)[vq];
   // what the epilogue of q, k, v adds: this thread's bias
   const int qt = tid / (3 * D), qi = tid - qt * (3 * D);  // this thread's token and value among its q, k, v
@@ -375,77 +388,87 @@ __global__ __launch_bounds__(FUSED_THREADS) void fused_attention_decode_kernel(F
   }
   FA_LOAD_W(0)
   if (!any) return;  // tokens of the padding only (the whole workgroup)
-  FD_STAMP_AFTER(16, piece[0].x);
+  if (NORMED) {
+    // everything is sent for at once; the rows go to LDS as they are
+    FA_LOAD_W(1)
+    FA_LOAD_W(2)
+    FA_LOAD_W(3)
+    FA_LOAD_KV
+    if (gq < TK) reinterpret_cast<uint2*>(act_s + gq * FUSED_MAX_WIDTH)[vq] = normed4;
+    if (gq == 2 && proj_bias) reinterpret_cast<float4*>(bproj_s)[vq] = gb4;
+  } else {
+    FD_STAMP_AFTER(16, piece[0].x);
 
-  // ---- the residual rows' sums: every group of threads its parts, then a wave per row all groups
+    // ---- the residual rows' sums: every group of threads its parts, then a wave per row all groups
 #pragma unroll
-  for (int t = 0; t < TK; ++t) {
-    if (!TABLES) {
+    for (int t = 0; t < TK; ++t) {
+      if (!TABLES) {
 #pragma unroll
-      for (int u = 0; u < FUSED_GROUP_PARTS; ++u) piece[t] = fd_add4(piece[t], part[t][u]);
+        for (int u = 0; u < FUSED_GROUP_PARTS; ++u) piece[t] = fd_add4(piece[t], part[t][u]);
+      }
+      if (gq < G) reinterpret_cast<float4*>(pool + t * POOL_ONE)[gq * V + vq] = piece[t];
     }
-    if (gq < G) reinterpret_cast<float4*>(pool + t * POOL_ONE)[gq * V + vq] = piece[t];
+    if (gq < 3) reinterpret_cast<float4*>(gq == 0 ? gain_s : gq == 1 ? beta_s : bproj_s)[vq] = gb4;
+    fd_barrier();
+    FD_STAMP(17);
+    // every wave sends for the rest of its weights and for its keys and values; then the first waves
+    // norm a row each (LDS and arithmetic only) while the others wait at the next barrier
+    FA_LOAD_W(1)
+    FA_LOAD_W(2)
+    FA_LOAD_W(3)
+    FA_LOAD_KV
+    if (wave < TK) {
+      const float* xs = pool + wave * POOL_ONE;
+      int row = tokn[0];
+      bool row_ok = ok[0];
+#pragma unroll
+      for (int t = 1; t < TK; ++t)
+        if (wave == t) {
+          row = tokn[t];
+          row_ok = ok[t];
+        }
+      float4 xv[2];
+      xv[0] = xv[1] = make_float4(0.f, 0.f, 0.f, 0.f);
+      // ---- LayerNorm, within one wave: no barrier between the sums
+      // groups beyond the parts hold zeros: only the groups that had something are read
+      const int used = TABLES ? 1 : min(G, max(a.res.n_parts, 1));
+#pragma unroll
+      for (int u = 0; u < 2; ++u) {
+        const int v = lane + 64 * u;
+        if (v < V) {
+          xv[u] = reinterpret_cast<const float4*>(xs)[v];
+#pragma unroll 8
+          for (int q = 1; q < used; ++q) xv[u] = fd_add4(xv[u], reinterpret_cast<const float4*>(xs)[q * V + v]);
+          // the row as it stands, stored by the first head's workgroup for the kernels behind this one
+          if (h == 0 && row_ok && a.res.settled) reinterpret_cast<float4*>(a.res.settled + (long)row * C)[v] = xv[u];
+        }
+      }
+      const float mean = wave_sum(fd_sum4(xv[0]) + fd_sum4(xv[1])) / (float)C;
+      float4 dv[2];
+      float sq = 0.f;
+#pragma unroll
+      for (int u = 0; u < 2; ++u) {
+        const bool in = lane + 64 * u < V;
+        dv[u] = in ? make_float4(xv[u].x - mean, xv[u].y - mean, xv[u].z - mean, xv[u].w - mean)
+                   : make_float4(0.f, 0.f, 0.f, 0.f);
+        sq += (dv[u].x * dv[u].x + dv[u].y * dv[u].y) + (dv[u].z * dv[u].z + dv[u].w * dv[u].w);
+      }
+      const float rstd = 1.0f / sqrtf(wave_sum(sq) / (float)C + a.eps);
+#pragma unroll
+      for (int u = 0; u < 2; ++u) {
+        const int v = lane + 64 * u;
+        if (v < V) {
+          const float4 gn = reinterpret_cast<const float4*>(gain_s)[v], bt4 = reinterpret_cast<const float4*>(beta_s)[v];
+          uint2 pk;
+          pk.x = pack_bf16x2(dv[u].x * rstd * gn.x + bt4.x, dv[u].y * rstd * gn.y + bt4.y);
+          pk.y = pack_bf16x2(dv[u].z * rstd * gn.z + bt4.z, dv[u].w * rstd * gn.w + bt4.w);
+          reinterpret_cast<uint2*>(act_s + wave * FUSED_MAX_WIDTH)[v] = pk;
+        }
+      }
+    }
   }
-  if (gq < 3) reinterpret_cast<float4*>(gq == 0 ? gain_s : gq == 1 ? beta_s : bproj_s)[vq] = gb4;
-  fd_barrier();
-  FD_STAMP(17);
-  // every wave sends for the rest of its weights and for its keys and values; then the first waves
-  // norm a row each (LDS and arithmetic only) while the others wait at the next barrier
-  FA_LOAD_W(1)
-  FA_LOAD_W(2)
-  FA_LOAD_W(3)
-  FA_LOAD_KV
 #undef FA_LOAD_W
 #undef FA_LOAD_KV
-  if (wave < TK) {
-    const float* xs = pool + wave * POOL_ONE;
-    int row = tokn[0];
-    bool row_ok = ok[0];
-#pragma unroll
-    for (int t = 1; t < TK; ++t)
-      if (wave == t) {
-        row = tokn[t];
-        row_ok = ok[t];
-      }
-    float4 xv[2];
-    xv[0] = xv[1] = make_float4(0.f, 0.f, 0.f, 0.f);
-    // ---- LayerNorm, within one wave: no barrier between the sums
-    // groups beyond the parts hold zeros: only the groups that had something are read
-    const int used = TABLES ? 1 : min(G, max(a.res.n_parts, 1));
-#pragma unroll
-    for (int u = 0; u < 2; ++u) {
-      const int v = lane + 64 * u;
-      if (v < V) {
-        xv[u] = reinterpret_cast<const float4*>(xs)[v];
-#pragma unroll 8
-        for (int q = 1; q < used; ++q) xv[u] = fd_add4(xv[u], reinterpret_cast<const float4*>(xs)[q * V + v]);
-        // the row as it stands, stored by the first head's workgroup for the kernels behind this one
-        if (h == 0 && row_ok && a.res.settled) reinterpret_cast<float4*>(a.res.settled + (long)row * C)[v] = xv[u];
-      }
-    }
-    const float mean = wave_sum(fd_sum4(xv[0]) + fd_sum4(xv[1])) / (float)C;
-    float4 dv[2];
-    float sq = 0.f;
-#pragma unroll
-    for (int u = 0; u < 2; ++u) {
-      const bool in = lane + 64 * u < V;
-      dv[u] = in ? make_float4(xv[u].x - mean, xv[u].y - mean, xv[u].z - mean, xv[u].w - mean)
-                 : make_float4(0.f, 0.f, 0.f, 0.f);
-      sq += (dv[u].x * dv[u].x + dv[u].y * dv[u].y) + (dv[u].z * dv[u].z + dv[u].w * dv[u].w);
-    }
-    const float rstd = 1.0f / sqrtf(wave_sum(sq) / (float)C + a.eps);
-#pragma unroll
-    for (int u = 0; u < 2; ++u) {
-      const int v = lane + 64 * u;
-      if (v < V) {
-        const float4 gn = reinterpret_cast<const float4*>(gain_s)[v], bt4 = reinterpret_cast<const float4*>(beta_s)[v];
-        uint2 pk;
-        pk.x = pack_bf16x2(dv[u].x * rstd * gn.x + bt4.x, dv[u].y * rstd * gn.y + bt4.y);
-        pk.y = pack_bf16x2(dv[u].z * rstd * gn.z + bt4.z, dv[u].w * rstd * gn.w + bt4.w);
-        reinterpret_cast<uint2*>(act_s + wave * FUSED_MAX_WIDTH)[v] = pk;
-      }
-    }
-  }
   fd_barrier();  // also: the rows' partial sums are read, their place takes the waves' sums now
   FD_STAMP(1);
 
@@ -1005,14 +1028,27 @@ extern "C" int mgpt_fused_parts_limit(int width) {
   return a < b ? a : b;
 }
 
+// Tokens that a workgroup of the attention kernel takes in a step of n_rows rows: two from where one
+// a workgroup would be more workgroups than compute units, four from where two would (heads of 128
+// keep to two: four tokens' q, k, v are more values than the workgroup has threads).
+extern "C" int mgpt_fused_attention_tokens(int n_rows, int n_head, int head_dim) {
+  const long pairs = (long)n_rows * n_head;
+  const int tk = pairs > 2 * FUSED_ATTN_ONE_TOKEN_WGS ? 4 : pairs > FUSED_ATTN_ONE_TOKEN_WGS ? 2 : 1;
+  return (tk == 4 && head_dim > 64) ? 2 : tk;
+}
+
 // The attention half of a layer for the single tokens of a decode-only step (token n is request n or,
 // with q_req[n] < 0, padding).  Refuses (MGPT_ERR_BAD_SHAPE) head sizes other than 16, 32, 64, 128,
 // widths beyond FUSED_MAX_WIDTH or no multiple of 32, n_head * head_dim no multiple of 32, pages that
 // are no power of two, pools of 4 GiB or more, more parts than mgpt_fused_parts_limit.
 // out_partials gets n_head parts.
+// Where mgpt_fused_attention_tokens(...) is more than one and the rows are no table rows, the rows
+// must come normed as well (normed: bfloat16 [rows][width], the LayerNorm of base; base then has no
+// parts, and nothing is stored to settled); with one token a workgroup normed is not read.
 extern "C" int mgpt_fused_attention_decode(
     const float* base, const float* partials, int n_parts, long part_stride, const void* tok_table,
-    const void* pos_table, const int* ids, const int* token_positions, float* settled, const float* gain,
+    const void* pos_table, const int* ids, const int* token_positions, float* settled, const void* normed,
+    const float* gain,
     const float* beta, float eps, const void* wqkv_packed, const float* bqkv, const void* wproj_packed,
     const float* bproj, float* out_partials, long out_part_stride, void* kpool, void* vpool,
     const int* slot_mapping, const int* block_tables, int max_blocks, const int* positions, const int* q_req,
@@ -1037,8 +1073,11 @@ extern "C" int mgpt_fused_attention_decode(
   if (page_shift < 0) return MGPT_ERR_BAD_SHAPE;
   const long pool_bytes = (long)num_pages * n_head * page_size * head_dim * 2;
   if (pool_bytes >= (1L << 32)) return MGPT_ERR_BAD_SHAPE;
+  const int tk = mgpt_fused_attention_tokens(n_rows, n_head, head_dim);
+  if (tk > 1 && base && (!normed || n_parts != 0 || (((size_t)normed) & 7) != 0)) return MGPT_ERR_BAD_SHAPE;
   a.gain = gain; a.beta = beta; a.eps = eps;
   a.wqkv = (const bf16_t*)wqkv_packed; a.bqkv = bqkv; a.wproj = (const bf16_t*)wproj_packed; a.bproj = bproj;
+  a.normed = (const bf16_t*)normed;
   a.out_partials = out_partials; a.out_part_stride = out_part_stride;
   a.kpool = (bf16_t*)kpool; a.vpool = (bf16_t*)vpool; a.slot_mapping = slot_mapping;
   a.block_tables = block_tables; a.max_blocks = max_blocks; a.positions = positions; a.q_req = q_req;
@@ -1046,20 +1085,16 @@ extern "C" int mgpt_fused_attention_decode(
   a.page_bytes = (unsigned int)(n_head * page_size * head_dim * 2);
   a.scale_log2e = scale * 1.4426950408889634f;
   // the head is the fast index: the workgroups of a head then land on the same XCD when the number
-  // of heads is a multiple of 8, and share its copy of the head's weights.  Two tokens a workgroup
-  // from where one a workgroup would be more workgroups than compute units, four from where two would
-  // (heads of 128 keep to two: four tokens' q, k, v are more values than the workgroup has threads).
-  const long pairs = (long)n_rows * n_head;
-  int tk = pairs > 2 * FUSED_ATTN_ONE_TOKEN_WGS ? 4 : pairs > FUSED_ATTN_ONE_TOKEN_WGS ? 2 : 1;
-  if (tk == 4 && head_dim > 64) tk = 2;
+  // of heads is a multiple of 8, and share its copy of the head's weights
   dim3 grid(n_head, (n_rows + tk - 1) / tk), block(FUSED_THREADS);
 #define FA_LAUNCH(DD)                                                                                           \
   do {                                                                                                          \
+    constexpr int D4 = DD > 64 ? 64 : DD; /* (heads of 128 never come with four tokens) */                      \
     if (tk == 4) {                                                                                              \
-      if (base) hipLaunchKernelGGL((fused_attention_decode_kernel<(DD > 64 ? 64 : DD), false, 4>), grid, block, 0, stream, a);   \
-      else hipLaunchKernelGGL((fused_attention_decode_kernel<(DD > 64 ? 64 : DD), true, 4>), grid, block, 0, stream, a);         \
-    } else if (tk == 2) {                                                                                              \
-      if (base) hipLaunchKernelGGL((fused_attention_decode_kernel<DD, false, 2>), grid, block, 0, stream, a);   \
+      if (base) hipLaunchKernelGGL((fused_attention_decode_kernel<D4, false, 4, true>), grid, block, 0, stream, a); \
+      else hipLaunchKernelGGL((fused_attention_decode_kernel<D4, true, 4>), grid, block, 0, stream, a);         \
+    } else if (tk == 2) {                                                                                       \
+      if (base) hipLaunchKernelGGL((fused_attention_decode_kernel<DD, false, 2, true>), grid, block, 0, stream, a); \
       else hipLaunchKernelGGL((fused_attention_decode_kernel<DD, true, 2>), grid, block, 0, stream, a);         \
     } else {                                                                                                    \
       if (base) hipLaunchKernelGGL((fused_attention_decode_kernel<DD, false, 1>), grid, block, 0, stream, a);   \

@@ -48,8 +48,8 @@ int mgpt_pack_weight(const void* w, void* packed, int n_out, int k_dim, hipStrea
 // fused_decode.hip
 int mgpt_fused_attention_decode(const float* base, const float* partials, int n_parts, long part_stride, const
     void* tok_table, const void* pos_table, const int* ids, const int* token_positions, float* settled, const
-    float* gain, const float* beta, float eps, const void* wqkv_packed, const float* bqkv, const void*
-    wproj_packed, const float* bproj, float* out_partials, long out_part_stride, void* kpool, void* vpool,
+    void* normed, const float* gain, const float* beta, float eps, const void* wqkv_packed, const float* bqkv,
+    const void* wproj_packed, const float* bproj, float* out_partials, long out_part_stride, void* kpool, void* vpool,
     const int* slot_mapping, const int* block_tables, int max_blocks, const int* positions, const int* q_req,
     int n_rows, int width, int n_head, int head_dim, int page_size, int num_pages, float scale, hipStream_t
     stream);

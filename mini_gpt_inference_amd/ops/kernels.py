@@ -701,17 +701,26 @@ def _residual_rows(pending) -> int:
     return rows
 
 
-def fused_attention_decode(pending, settled: torch.Tensor, gain: torch.Tensor, beta: Optional[torch.Tensor],
+def fused_attention_tokens(n_rows: int, n_head: int, head_dim: int) -> int:
+    """Tokens that a workgroup of fused_attention_decode takes in a step of n_rows rows.  With more
+    than one, rows that are no table rows must be handed over normed."""
+    return int(library.kernels().mgpt_fused_attention_tokens(int(n_rows), int(n_head), int(head_dim)))
+
+
+def fused_attention_decode(pending, settled: Optional[torch.Tensor], gain: torch.Tensor, beta: Optional[torch.Tensor],
                            eps: float, wqkv_packed: torch.Tensor, bqkv: Optional[torch.Tensor],
                            wproj_packed: torch.Tensor, bproj: Optional[torch.Tensor], out_partials: torch.Tensor,
                            k_pool: torch.Tensor, v_pool: torch.Tensor, slot_mapping: torch.Tensor,
                            block_tables: torch.Tensor, positions: torch.Tensor, q_req: torch.Tensor, n_rows: int,
-                           n_head: int, scale: float) -> bool:
+                           n_head: int, scale: float, normed: Optional[torch.Tensor] = None) -> bool:
     """LayerNorm, one head's q/k/v, cache write, attention and that head's share of the output
     projection, for the single tokens of a decode-only step: out_partials[h, n] is head h's share
     of what token n adds to the residual.  The residual comes as a sum (pending), whose value is
-    stored to `settled` on the way.  False, having launched nothing, if the kernel does not take
-    the shape."""
+    stored to `settled` on the way.  In a step of so many rows that a workgroup takes several
+    tokens (fused_attention_tokens), rows that are no table rows come normed instead (`normed`:
+    bfloat16 [rows, width], the LayerNorm of the plain rows `pending.base`; nothing is stored to
+    `settled`, which may be None).  False, having launched nothing, if the kernel does not take the
+    shape."""
     width = gain.numel()
     _need_cuda(settled, gain, beta, wqkv_packed, bqkv, wproj_packed, bproj, out_partials, k_pool, v_pool,
                slot_mapping, block_tables, positions, q_req)
@@ -723,11 +732,20 @@ def fused_attention_decode(pending, settled: torch.Tensor, gain: torch.Tensor, b
     if (n_kv_head != n_head or head_dim not in (16, 32, 64, 128) or width % 32 or width > FUSED_MAX_WIDTH
             or q_width % 32 or page_size & (page_size - 1) or pending.n_parts > fused_parts_limit(width)):
         return False
+    use_normed = pending.base is not None and fused_attention_tokens(n_rows, n_head, head_dim) > 1
+    if use_normed and (normed is None or pending.n_parts):
+        return False
     args = _residual_args(pending, width)
     _need(_residual_rows(pending) >= n_rows, "the pending residual holds fewer rows than the step")
-    _need(settled.dtype == torch.float32 and settled.is_contiguous() and settled.shape[1] == width
-          and settled.shape[0] >= n_rows and (pending.base is None or settled.data_ptr() != pending.base.data_ptr()),
-          "the settled rows need a dense float32 array of their own")
+    if use_normed:
+        _need_cuda(normed)
+        _need(normed.dtype == torch.bfloat16 and normed.is_contiguous() and normed.dim() == 2
+              and normed.shape[1] == width and normed.shape[0] >= n_rows, "normed rows must be dense bfloat16 [>=rows, width]")
+    else:
+        _need(settled is not None and settled.dtype == torch.float32 and settled.is_contiguous()
+              and settled.shape[1] == width and settled.shape[0] >= n_rows
+              and (pending.base is None or settled.data_ptr() != pending.base.data_ptr()),
+              "the settled rows need a dense float32 array of their own")
     for name, t, numel in (("gain", gain, width), ("beta", beta, width), ("qkv bias", bqkv, 3 * q_width),
                            ("projection bias", bproj, width)):
         _need(t is None or (t.dtype == torch.float32 and t.numel() == numel), f"{name} must be float32 [{numel}]")
@@ -744,7 +762,8 @@ def fused_attention_decode(pending, settled: torch.Tensor, gain: torch.Tensor, b
     _need_i32("positions", positions, n_rows)
     _need_i32("q_req", q_req, n_rows)
     rc = library.kernels().mgpt_fused_attention_decode(
-        *args, _ptr(settled), _ptr(gain), _ptr(beta), float(eps), _ptr(wqkv_packed), _ptr(bqkv), _ptr(wproj_packed),
+        *args, None if use_normed else _ptr(settled), _ptr(normed) if use_normed else None, _ptr(gain), _ptr(beta),
+        float(eps), _ptr(wqkv_packed), _ptr(bqkv), _ptr(wproj_packed),
         _ptr(bproj), _ptr(out_partials), out_partials.stride(0), _ptr(k_pool), _ptr(v_pool), _ptr(slot_mapping),
         _ptr(block_tables), block_tables.shape[1], _ptr(positions), _ptr(q_req), n_rows, width, n_head, head_dim,
         page_size, num_pages, float(scale), _stream())

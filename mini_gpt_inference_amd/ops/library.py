@@ -136,8 +136,9 @@ def _declare_optional(lib: ctypes.CDLL) -> None:
         "mgpt_linear_mfma_qkv": [P, L, P, P, P, L, I, I, I, P, P, P, I, I, I, I, I, I, P],
         "mgpt_prefill_attention_bf16": [P, L, P, L, P, P, P, I, P, P, I, I, I, I, I, I, F, I, I, P],
         # a residual that is still a sum: base, partials, n_parts, part_stride, token table, position table, ids, positions
-        "mgpt_fused_attention_decode": [P, P, I, L, P, P, P, P, P, P, P, F, P, P, P, P, P, L, P, P, P, P, I, P, P,
+        "mgpt_fused_attention_decode": [P, P, I, L, P, P, P, P, P, P, P, P, F, P, P, P, P, P, L, P, P, P, P, I, P, P,
                                         I, I, I, I, I, I, F, P],
+        "mgpt_fused_attention_tokens": [I, I, I],
         "mgpt_fused_mlp_decode": [P, P, I, L, P, P, P, P, P, P, P, F, P, P, P, P, P, L, I, I, I, P],
         "mgpt_residual_layernorm": [P, P, I, L, P, P, P, P, P, P, F, P, P, I, I, I, P, P],
         "mgpt_residual_parts_limit": [I],

@@ -24,8 +24,8 @@ from . import kernels
 # most rows of a decode-only step that go through the fused kernels.  A workgroup of the attention
 # kernel takes one token of a head, two from where that would be more workgroups than compute units
 # and four from where two would, so that a head's weights are read once for them; the 50.9M model's
-# step against the kernels that share a matrix among all rows: 228 us against 243 at 40 rows, 243 /
-# 263 at 64, 353 / 440 at 96, 371 / 456 at 128 (context 170); 336 / 368 at 64 and 569 / 650 at 128
+# step against the kernels that share a matrix among all rows: 222 us against 243 at 40 rows, 242 /
+# 264 at 64, 311 / 438 at 96, 330 / 455 at 128 (context 170); 340 / 367 at 64 and 530 / 647 at 128
 # (context 740).  Steps of more rows than this are not replayed from graphs either.
 FUSED_MAX_ROWS = 128
 

@@ -76,8 +76,9 @@ class PagedCausalAttention(Mixer):
                            position: PositionEncoding) -> bool:
         """A decode-only step of few rows: one kernel from the residual (as the kernels before left
         it: a sum) through LayerNorm, projections, cache write and attention to this mixer's
-        addition to the residual, left as one partial sum per head.  False, with nothing launched,
-        where that kernel does not apply."""
+        addition to the residual, left as one partial sum per head.  False where that kernel does
+        not apply (with nothing launched but, in a step of many rows, the LayerNorm that the other
+        path needs as well)."""
         if not (isinstance(h, LazyNorm) and h._tensor is None and h.rows is None and h.x is x
                 and getattr(h.norm, "fusable_layer_norm", False) and residual.usable(ctx, self.width, self.n_head)
                 and binding.writes and not position.rotates and self.window == 0
@@ -89,15 +90,24 @@ class PagedCausalAttention(Mixer):
             return False
         n = ctx.n_rows
         group = ctx.groups[binding.group]
+        # In a step of so many rows that a workgroup takes several tokens, every head's workgroup
+        # adding up its tokens' pending parts would be most of the kernel's traffic: the LayerNorm
+        # kernel adds them up once (x is plain after it) and hands the rows over normed.
+        normed = None
+        table_rows = ctx.pending is not None and ctx.pending.base is None
+        if not table_rows and kernels.fused_attention_tokens(n, self.n_head, self.head_dim) > 1:
+            normed = h.tensor(ctx)
+            if ctx.pending is not None:
+                return False
         pending, settled = residual.take(ctx, x)
         parts = ctx.workspace.get("attention_parts", self.n_head * n, self.width, torch.float32) \
             [:self.n_head * n].view(self.n_head, n, self.width)
         if not kernels.fused_attention_decode(
                 pending, settled, h.norm.weight, h.norm.bias, h.norm.eps, wqkv, self.qkv_bias, wproj, self.proj_bias,
                 parts, group.k_pools[binding.index], group.v_pools[binding.index], group.slot_mapping,
-                group.block_tables, ctx.positions, ctx.q_req, n, self.n_head, self.scale):
+                group.block_tables, ctx.positions, ctx.q_req, n, self.n_head, self.scale, normed=normed):
             return False
-        ctx.pending = residual.PendingSums(settled, parts, self.n_head)
+        ctx.pending = residual.PendingSums(x if normed is not None else settled, parts, self.n_head)
         return True
 
     def forward_add(self, ctx: StepContext, h: torch.Tensor, x: torch.Tensor, binding: CacheBinding,

@@ -86,6 +86,25 @@ def test_fused_attention_decode(case, tables):
         true = tok.double()[ids[:n]] + pos.double()[ctxs]
     else:
         pending, true = _pending(g, n, c, spec["parts"], extra_rows=pad)
+    # many (token, head) pairs: a workgroup takes several tokens, and rows that are no table rows come normed
+    several = kernels.fused_attention_tokens(rows, h, d) > 1
+    assert several == (rows * h > 256)
+    normed = None
+    if several and not tables:
+        assert not kernels.fused_attention_decode(          # the pending parts are refused, nothing is launched
+            pending, torch.zeros(rows, c, device=DEV), gain.to(DEV), beta.to(DEV), eps,
+            torch.zeros(3 * qw * c, dtype=torch.bfloat16, device=DEV), None,
+            torch.zeros(c * qw, dtype=torch.bfloat16, device=DEV), None, torch.zeros(h, rows, c, device=DEV),
+            torch.zeros(4, h, page, d, dtype=torch.bfloat16, device=DEV),
+            torch.zeros(4, h, page, d, dtype=torch.bfloat16, device=DEV), i32([-1] * rows),
+            torch.zeros(rows, 4, dtype=torch.int32, device=DEV), i32([0] * rows), i32([-1] * rows), rows, h, scale)
+        plain_rows = torch.full((rows, c), float("nan"))
+        plain_rows[:n] = true.float()
+        true = plain_rows[:n].double()
+        pending = PendingSums(plain_rows.to(DEV), None, 0)
+        normed = torch.full((rows, c), float("nan"), dtype=torch.bfloat16)
+        normed[:n] = bf(P.plain_layer_norm(true, gain.double(), beta.double(), eps))
+        normed = normed.to(DEV)
     # the cache: every request's earlier keys and values in pages handed out in a shuffled order
     max_blocks = max(-(-(x + 1) // page) for x in ctxs) + 1
     n_pages = sum(-(-(x + 1) // page) for x in ctxs) + 3
@@ -128,10 +147,13 @@ def test_fused_attention_decode(case, tables):
     took = kernels.fused_attention_decode(
         pending, settled, dev(gain), dev(beta), eps, kernels.pack_weight(wqkv.to(DEV)), dev(bqkv),
         kernels.pack_weight(wproj.to(DEV)), dev(bproj), out, kp_d, vp_d, i32(slots + [-1] * pad), bt.to(DEV),
-        i32(ctxs + [0] * pad), i32(list(range(n)) + [-1] * pad), rows, h, scale)
+        i32(ctxs + [0] * pad), i32(list(range(n)) + [-1] * pad), rows, h, scale, normed=normed)
     assert took
     torch.cuda.synchronize()
-    helpers.assert_close(settled[:n], true, "float32", "the settled rows")
+    if normed is None:
+        helpers.assert_close(settled[:n], true, "float32", "the settled rows")
+    else:
+        assert torch.isnan(settled).all(), "rows that came normed are not stored again"
     helpers.assert_close(out[:, :n].sum(0), want, "bfloat16", f"fused attention case {case}")
     assert torch.isnan(out[:, n:]).all() and torch.isnan(settled[n:]).all(), "the padded tokens' rows were written"
     for r, ctx in enumerate(ctxs):                 # the token's key and value are in its page, nothing else changed
