@@ -324,8 +324,8 @@ __global__ __launch_bounds__(FUSED_THREADS) void fused_attention_decode_kernel(F
 #pragma unroll
   for (int t = 0; t < TK; ++t) {
     piece[t] = make_float4(0.f, 0.f, 0.f, 0.f);
-    if (NORMED) {
-    } else if (TABLES) {
+    if (NORMED) continue;
+    if (TABLES) {
       if (gq == 0) {
         const uint2 tr = reinterpret_cast<const uint2*>(a.res.tok_table)[(long)a.res.ids[tokn[t]] * V + vq];
         piece[t] = fd_bf16x4(tr);
@@ -1030,11 +1030,14 @@ extern "C" int mgpt_fused_parts_limit(int width) {
 
 // Tokens that a workgroup of the attention kernel takes in a step of n_rows rows: two from where one
 // a workgroup would be more workgroups than compute units, four from where two would (heads of 128
-// keep to two: four tokens' q, k, v are more values than the workgroup has threads).
+// keep to two: four tokens' q, k, v are more values than the workgroup has threads).  0: more rows
+// than the kernel takes (more workgroups than compute units even so: the kernels that share a matrix
+// among all rows are faster there).
 extern "C" int mgpt_fused_attention_tokens(int n_rows, int n_head, int head_dim) {
   const long pairs = (long)n_rows * n_head;
-  const int tk = pairs > 2 * FUSED_ATTN_ONE_TOKEN_WGS ? 4 : pairs > FUSED_ATTN_ONE_TOKEN_WGS ? 2 : 1;
-  return (tk == 4 && head_dim > 64) ? 2 : tk;
+  const int most = head_dim > 64 ? 2 : 4;
+  if (pairs > (long)most * FUSED_ATTN_ONE_TOKEN_WGS) return 0;
+  return pairs > 2 * FUSED_ATTN_ONE_TOKEN_WGS ? 4 : pairs > FUSED_ATTN_ONE_TOKEN_WGS ? 2 : 1;
 }
 
 // The attention half of a layer for the single tokens of a decode-only step (token n is request n or,
@@ -1074,6 +1077,7 @@ extern "C" int mgpt_fused_attention_decode(
   const long pool_bytes = (long)num_pages * n_head * page_size * head_dim * 2;
   if (pool_bytes >= (1L << 32)) return MGPT_ERR_BAD_SHAPE;
   const int tk = mgpt_fused_attention_tokens(n_rows, n_head, head_dim);
+  if (tk == 0) return MGPT_ERR_BAD_SHAPE;
   if (tk > 1 && base && (!normed || n_parts != 0 || (((size_t)normed) & 7) != 0)) return MGPT_ERR_BAD_SHAPE;
   a.gain = gain; a.beta = beta; a.eps = eps;
   a.wqkv = (const bf16_t*)wqkv_packed; a.bqkv = bqkv; a.wproj = (const bf16_t*)wproj_packed; a.bproj = bproj;

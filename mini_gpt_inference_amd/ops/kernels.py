@@ -703,7 +703,8 @@ def _residual_rows(pending) -> int:
 
 def fused_attention_tokens(n_rows: int, n_head: int, head_dim: int) -> int:
     """Tokens that a workgroup of fused_attention_decode takes in a step of n_rows rows.  With more
-    than one, rows that are no table rows must be handed over normed."""
+    than one, rows that are no table rows must be handed over normed; 0: the kernel does not take so
+    many rows."""
     return int(library.kernels().mgpt_fused_attention_tokens(int(n_rows), int(n_head), int(head_dim)))
 
 
@@ -732,8 +733,9 @@ def fused_attention_decode(pending, settled: Optional[torch.Tensor], gain: torch
     if (n_kv_head != n_head or head_dim not in (16, 32, 64, 128) or width % 32 or width > FUSED_MAX_WIDTH
             or q_width % 32 or page_size & (page_size - 1) or pending.n_parts > fused_parts_limit(width)):
         return False
-    use_normed = pending.base is not None and fused_attention_tokens(n_rows, n_head, head_dim) > 1
-    if use_normed and (normed is None or pending.n_parts):
+    tokens = fused_attention_tokens(n_rows, n_head, head_dim)
+    use_normed = pending.base is not None and tokens > 1
+    if tokens == 0 or (use_normed and (normed is None or pending.n_parts)):
         return False
     args = _residual_args(pending, width)
     _need(_residual_rows(pending) >= n_rows, "the pending residual holds fewer rows than the step")

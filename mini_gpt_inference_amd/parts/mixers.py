@@ -95,7 +95,10 @@ class PagedCausalAttention(Mixer):
         # kernel adds them up once (x is plain after it) and hands the rows over normed.
         normed = None
         table_rows = ctx.pending is not None and ctx.pending.base is None
-        if not table_rows and kernels.fused_attention_tokens(n, self.n_head, self.head_dim) > 1:
+        tokens = kernels.fused_attention_tokens(n, self.n_head, self.head_dim)
+        if tokens == 0:
+            return False
+        if not table_rows and tokens > 1:
             normed = h.tensor(ctx)
             if ctx.pending is not None:
                 return False

@@ -60,7 +60,7 @@ ATTN_CASES = [
     dict(c=512, h=8, d=64, page=16, ctx=[(7 * i * i + 3 * i) % 530 for i in range(65)], parts=32, bias=True, pad=6),
     dict(c=64, h=4, d=16, page=4, ctx=[(13 * i * i) % 270 for i in range(141)], parts=4, bias=False, pad=1),
     dict(c=96, h=3, d=32, page=8, ctx=[(5 * i * i + 7 * i) % 200 for i in range(175)], parts=2, bias=True, pad=3),
-    dict(c=256, h=2, d=128, page=32, ctx=[(3 * i) % 40 for i in range(259)], parts=1, bias=True, pad=1),
+    dict(c=256, h=2, d=128, page=32, ctx=[(3 * i) % 40 for i in range(253)], parts=1, bias=True, pad=1),
 ]
 
 
@@ -320,6 +320,9 @@ def test_fused_kernels_refuse_what_they_cannot_do():
     and nothing is written."""
     assert kernels.fused_parts_limit(512) == 32 and kernels.fused_parts_limit(544) == 0
     assert kernels.fused_parts_limit(48) == 0 and kernels.fused_parts_limit(64) >= 128
+    # rows: up to four tokens a workgroup (two with heads of 128) and 256 workgroups a head's share
+    assert [kernels.fused_attention_tokens(r, 8, 64) for r in (1, 32, 33, 64, 65, 128, 129)] == [1, 1, 2, 2, 4, 4, 0]
+    assert [kernels.fused_attention_tokens(r, 2, 128) for r in (128, 129, 256, 257)] == [1, 2, 2, 0]
     g = torch.Generator().manual_seed(5)
     for c, f, parts in [(544, 2176, 2), (48, 192, 2), (512, 2048, 33), (512, 2000, 2)]:
         base = rnd(g, 2, c).to(DEV)
