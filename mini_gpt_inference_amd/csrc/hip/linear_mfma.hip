@@ -117,7 +117,13 @@ constexpr int MM_GROUP = 4;         // row tiles per block of tiles
 
 // WTM x WTN: 16-wide tiles per wave along the rows of the activations and along the rows of W;
 // WVM x WVN: waves in a workgroup along the same.
-template <int WTM, int WTN, int WVM, int WVN, int EPI, typename OT>
+// AHEAD: steps whose chunks are on their way from memory beyond the one that is being put into LDS
+// (1: the schedule described above).  With few tiles of few rows over a large matrix that has to
+// come from memory, a step's MFMAs are over long before the chunks of the step after next arrive
+// (a 64 x 64 tile: 8 MFMAs a wave and step against a microsecond or more), and the product takes
+// a memory round trip every two steps; more steps in flight, each in registers of its own, take that
+// wait apart.
+template <int WTM, int WTN, int WVM, int WVN, int EPI, typename OT, int AHEAD = 1>
 __global__ __launch_bounds__(64 * WVM * WVN) void linear_mfma_kernel(
     const bf16_t* __restrict__ act, long lda, const bf16_t* __restrict__ w,
     const float* __restrict__ bias, OT* __restrict__ out, long ldo, int n_rows, int n_out, int k_dim,
@@ -162,7 +168,7 @@ __global__ __launch_bounds__(64 * WVM * WVN) void linear_mfma_kernel(
   const bf16x8_t zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
   // What a thread stages per step: PA chunks of the activations' slice and PW of W's, each 16 bytes.
   constexpr int ITEMS = PA + PW;
-  bf16x8_t gv[ITEMS];
+  bf16x8_t gv[AHEAD][ITEMS];
   // rows past the end are read from the last row: their results are never stored
   const bf16_t* gp[ITEMS];
 #pragma unroll
@@ -177,14 +183,15 @@ __global__ __launch_bounds__(64 * WVM * WVN) void linear_mfma_kernel(
   }
   // A chunk that lies beyond the stretch's end (in its last, partial step) is read from the stretch's start instead
   // and counts as zero when it is stored: the select then waits for no load.
-  auto load_item = [&](int p, int step) {
+  // (set: which of the AHEAD sets of registers; a constant wherever these are called)
+  auto load_item = [&](int p, int step, int set = 0) {
     const int k0 = step * MM_BK;
-    gv[p] = *reinterpret_cast<const bf16x8_t*>(gp[p] + (k0 + sk + 8 <= k_len ? k0 : -sk));
+    gv[set][p] = *reinterpret_cast<const bf16x8_t*>(gp[p] + (k0 + sk + 8 <= k_len ? k0 : -sk));
   };
-  auto store_item = [&](int p, int step, int buf) {
+  auto store_item = [&](int p, int step, int buf, int set = 0) {
     bf16_t* dst = p < PA ? as_base + buf * (BM * MM_LD) + p * RPP * MM_LD
                          : ws_base + buf * (BN * MM_LD) + (p - PA) * RPP * MM_LD;
-    *reinterpret_cast<bf16x8_t*>(dst + s_lds) = step * MM_BK + sk + 8 <= k_len ? gv[p] : zero8;
+    *reinterpret_cast<bf16x8_t*>(dst + s_lds) = step * MM_BK + sk + 8 <= k_len ? gv[set][p] : zero8;
   };
 
   f32x4_t acc[WTN][WTM];  // [column tile of W][row tile of activations]
@@ -202,7 +209,10 @@ __global__ __launch_bounds__(64 * WVM * WVN) void linear_mfma_kernel(
   // Spread between the groups, the thread puts the next step's chunks (loaded during the step
   // before this one) into the other LDS buffer and sends for those of the step after: LDS takes
   // writes at half the rate of reads, and all at once they would hold every wave up.
-  auto k_step = [&](int s, auto store_next, auto load_after) {
+  // store_next / load_after: a compile-time yes or no; set: the registers that hold step s + 1 and
+  // take step s + 1 + AHEAD
+  auto k_step = [&](int s, auto store_next, auto load_after, auto set_c) {
+    constexpr int set = decltype(set_c)::value;
     const int buf = s & 1;
     const bf16_t* as = as_base + buf * (BM * MM_LD) + (wr + lrow) * MM_LD;
     const bf16_t* ws = ws_base + buf * (BN * MM_LD) + (wc + lrow) * MM_LD;
@@ -230,8 +240,8 @@ __global__ __launch_bounds__(64 * WVM * WVN) void linear_mfma_kernel(
       }
 #pragma unroll
       for (int p = g * ITEMS / GROUPS; p < (g + 1) * ITEMS / GROUPS; ++p) {
-        if (decltype(store_next)::value) store_item(p, s + 1, buf ^ 1);
-        if (decltype(load_after)::value) load_item(p, s + 2);
+        if (decltype(store_next)::value) store_item(p, s + 1, buf ^ 1, set);
+        if (decltype(load_after)::value) load_item(p, s + 1 + AHEAD, set);
       }
       // the compiler's scheduler would move each read down to its use again
       __builtin_amdgcn_sched_barrier(0);
@@ -244,6 +254,7 @@ __global__ __launch_bounds__(64 * WVM * WVN) void linear_mfma_kernel(
   };
   using yes = std::integral_constant<bool, true>;
   using no = std::integral_constant<bool, false>;
+  using set0 = std::integral_constant<int, 0>;
 
   // The first two steps' chunks are sent for together, the first step's into registers of their own
   // (free before the loop needs them for MFMA operands): one trip to memory before the first MFMA
@@ -252,9 +263,11 @@ __global__ __launch_bounds__(64 * WVM * WVN) void linear_mfma_kernel(
     bf16x8_t first[ITEMS];
 #pragma unroll
     for (int p = 0; p < ITEMS; ++p) first[p] = *reinterpret_cast<const bf16x8_t*>(gp[p] + (sk + 8 <= k_len ? 0 : -sk));
-    if (k_steps > 1) {
+    if (AHEAD > 1 || k_steps > 1) {
 #pragma unroll
-      for (int p = 0; p < ITEMS; ++p) load_item(p, 1);
+      for (int j = 1; j <= AHEAD; ++j)
+#pragma unroll
+        for (int p = 0; p < ITEMS; ++p) load_item(p, j, j - 1);
     }
 #pragma unroll
     for (int p = 0; p < ITEMS; ++p) {
@@ -264,9 +277,24 @@ __global__ __launch_bounds__(64 * WVM * WVN) void linear_mfma_kernel(
   }
   __syncthreads();
   int s = 0;
-  for (; s + 2 < k_steps; ++s) k_step(s, yes{}, yes{});
-  if (s + 1 < k_steps) k_step(s++, yes{}, no{});
-  k_step(s, no{}, no{});
+  if constexpr (AHEAD == 1) {
+    for (; s + 2 < k_steps; ++s) k_step(s, yes{}, yes{}, set0{});
+    if (s + 1 < k_steps) k_step(s++, yes{}, no{}, set0{});
+    k_step(s, no{}, no{}, set0{});
+  } else {
+    // Step s + 1 lies in set s mod AHEAD: the sets take turns, AHEAD steps a round, in whole rounds
+    // and without a branch (where control flow joins the compiler waits for every load in flight):
+    // a step beyond the last multiplies the zeros that stand in for chunks beyond the stretch's
+    // end, and its loads read the stretch's start.
+    auto round = [&](auto... set_c) { ((k_step(s, yes{}, yes{}, set_c), ++s), ...); };
+    while (s < k_steps) {
+      if constexpr (AHEAD == 2) round(std::integral_constant<int, 0>{}, std::integral_constant<int, 1>{});
+      else if constexpr (AHEAD == 3) round(std::integral_constant<int, 0>{}, std::integral_constant<int, 1>{},
+                                           std::integral_constant<int, 2>{});
+      else round(std::integral_constant<int, 0>{}, std::integral_constant<int, 1>{}, std::integral_constant<int, 2>{},
+                 std::integral_constant<int, 3>{});
+    }
+  }
 
   // lane holds out[row0 + wr + j*16 + (lane & 15)][col0 + wc + i*16 + (lane >> 4)*4 + e], e = 0..3
   const bool vec = (n_out & 3) == 0 && (ldo & 3) == 0 && (((size_t)out | (size_t)bias) & 15) == 0;
@@ -368,12 +396,13 @@ __global__ __launch_bounds__(64 * WVM * WVN) void linear_mfma_kernel(
   }
 }
 
-template <int WTM, int WTN, int WVM, int WVN, int EPI, typename OT>
+template <int WTM, int WTN, int WVM, int WVN, int EPI, typename OT, int AHEAD>
 int launch_one(const void* act, long lda, const void* w, const float* bias, void* out, long ldo, int n_rows,
                int n_out, int k_dim, int k_parts, long part_stride, const MfmaScatter& sc, hipStream_t stream) {
+  static_assert(AHEAD >= 1 && AHEAD <= 4, "sets of staging registers");
   constexpr int BM = WVM * WTM * 16, BN = WVN * WTN * 16;
   constexpr size_t lds_bytes = 2ul * (BM + BN) * MM_LD * sizeof(bf16_t);
-  auto kernel = linear_mfma_kernel<WTM, WTN, WVM, WVN, EPI, OT>;
+  auto kernel = linear_mfma_kernel<WTM, WTN, WVM, WVN, EPI, OT, AHEAD>;
   static bool allowed = false;  // more LDS than a kernel gets without asking
   if (!allowed) {
     const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
@@ -389,13 +418,13 @@ int launch_one(const void* act, long lda, const void* w, const float* bias, void
   return mgpt_last_error();
 }
 
-template <int WTM, int WTN, int WVM, int WVN>
+template <int WTM, int WTN, int WVM, int WVN, int AHEAD = 1>
 int launch_shape(const void* act, long lda, const void* w, const float* bias, void* out, int out_dtype, long ldo,
                  int n_rows, int n_out, int k_dim, int epilogue, int k_parts, long part_stride,
                  const MfmaScatter& sc, hipStream_t stream) {
-#define MM_LAUNCH(E, OT)                                                                                     \
-  return launch_one<WTM, WTN, WVM, WVN, E, OT>(act, lda, w, bias, out, ldo, n_rows, n_out, k_dim, k_parts, \
-                                               part_stride, sc, stream)
+#define MM_LAUNCH(E, OT)                                                                                            \
+  return launch_one<WTM, WTN, WVM, WVN, E, OT, AHEAD>(act, lda, w, bias, out, ldo, n_rows, n_out, k_dim, k_parts, \
+                                                      part_stride, sc, stream)
   if (epilogue == MM_EPI_NONE && out_dtype == MGPT_BF16) MM_LAUNCH(MM_EPI_NONE, bf16_t);
   if (epilogue == MM_EPI_NONE && out_dtype == MGPT_F32) MM_LAUNCH(MM_EPI_NONE, float);
   if (epilogue == MM_EPI_GELU && out_dtype == MGPT_BF16) MM_LAUNCH(MM_EPI_GELU, bf16_t);
@@ -410,6 +439,7 @@ constexpr int MM_SHAPES = 5;
 constexpr int MM_TILE_ROWS[MM_SHAPES] = {256, 128, 128, 64, 32};
 constexpr int MM_TILE_COLS[MM_SHAPES] = {256, 256, 64, 64, 32};
 constexpr int MM_MAX_PARTS = 8;
+constexpr int MM_AHEAD = 4;  // steps on their way from memory in the variant for few tiles over a large matrix
 
 long tiles_of(int shape, int n_rows, int n_out) {
   return (long)((n_rows + MM_TILE_ROWS[shape] - 1) / MM_TILE_ROWS[shape]) *
@@ -540,6 +570,14 @@ int launch_any(int shape, int k_parts, const void* act, long lda, const void* w,
   if (n_rows == 0 || n_out == 0) return MGPT_OK;
   if (!act || !w || !out) return MGPT_ERR_NULL;
   if (!shapes_ok(act, lda, w, out, ldo, n_rows, n_out, k_dim)) return MGPT_ERR_BAD_SHAPE;
+  // shapes MM_SHAPES and MM_SHAPES + 1: the two smallest tiles with more steps on their way from memory
+  int ahead = 0;  // 0: chosen below
+  if (shape >= MM_SHAPES && shape < MM_SHAPES + 2) {
+    shape -= 2;
+    ahead = MM_AHEAD;
+  } else if (shape >= 0) {
+    ahead = 1;
+  }
   const bool forced = k_parts > 1;
   if (shape < 0 && k_parts == 0 && partials) {
     choose_split(n_rows, n_out, k_dim, epilogue, &shape, &k_parts);
@@ -548,6 +586,15 @@ int launch_any(int shape, int k_parts, const void* act, long lda, const void* w,
   if (shape < 0) shape = choose_shape(n_rows, n_out);
   if (shape >= MM_SHAPES) return MGPT_ERR_BAD_SHAPE;
   if (k_parts == 0) k_parts = 1;
+  if (ahead == 0) {
+    // Few tiles of few rows over a long enough stretch: the workgroups are too few to hide a trip to
+    // memory behind one another.  Measured over matrices that come from memory, 32 x 32 tiles, 40-64
+    // rows: [4800 x 1600] 9.8-10.0 us against 10.8, [6400 x 1600] 10.7-11.9 against 15.6, [1600 x 1600]
+    // 8.4 against 10.3, [4096 x 1024] 6.3 against 7.6; from a hundred rows on nothing is gained.
+    const int steps = (k_dim + MM_BK - 1) / MM_BK;
+    ahead = (shape == 4 && n_rows <= 64 && steps / k_parts >= 12 && tiles_of(4, n_rows, n_out) * k_parts <= 1024)
+                ? MM_AHEAD : 1;
+  }
   if (k_parts > 1) {
     k_parts = used_parts(k_dim, k_parts > MM_MAX_PARTS ? MM_MAX_PARTS : k_parts);
     const bool fits = partials && (long)k_parts * n_rows * n_out <= partials_floats &&
@@ -568,8 +615,12 @@ int launch_any(int shape, int k_parts, const void* act, long lda, const void* w,
     case 0: rc = launch_shape<8, 4, 2, 4>(MM_ARGS); break;  // 256 x 256, eight waves of 128 x 64
     case 1: rc = launch_shape<4, 4, 2, 4>(MM_ARGS); break;  // 128 x 256, eight waves of 64 x 64
     case 2: rc = launch_shape<4, 2, 2, 2>(MM_ARGS); break;  // 128 x 64, four waves of 64 x 32
-    case 3: rc = launch_shape<2, 2, 2, 2>(MM_ARGS); break;  // 64 x 64, four waves of 32 x 32
-    case 4: rc = launch_shape<1, 1, 2, 2>(MM_ARGS); break;  // 32 x 32, four waves of 16 x 16
+    case 3:  // 64 x 64, four waves of 32 x 32
+      rc = ahead > 1 ? launch_shape<2, 2, 2, 2, MM_AHEAD>(MM_ARGS) : launch_shape<2, 2, 2, 2>(MM_ARGS);
+      break;
+    case 4:  // 32 x 32, four waves of 16 x 16
+      rc = ahead > 1 ? launch_shape<1, 1, 2, 2, MM_AHEAD>(MM_ARGS) : launch_shape<1, 1, 2, 2>(MM_ARGS);
+      break;
   }
 #undef MM_ARGS
   if (rc != MGPT_OK || !split) return rc;
@@ -608,7 +659,7 @@ extern "C" int mgpt_linear_mfma_shape(int shape, int k_parts, const void* act, l
                                       const float* bias, void* out, int out_dtype, long ldo, int n_rows,
                                       int n_out, int k_dim, int epilogue, float* partials, long partials_floats,
                                       hipStream_t stream) {
-  if (epilogue == MM_EPI_QKV || shape >= MM_SHAPES || k_parts < 0) return MGPT_ERR_BAD_SHAPE;
+  if (epilogue == MM_EPI_QKV || shape >= MM_SHAPES + 2 || k_parts < 0) return MGPT_ERR_BAD_SHAPE;
   MfmaScatter sc = {};
   return launch_any(shape, k_parts, act, lda, w, bias, out, out_dtype, ldo, n_rows, n_out, k_dim, epilogue,
                     partials, partials_floats, sc, stream);

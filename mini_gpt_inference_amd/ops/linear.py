@@ -124,6 +124,17 @@ FOLD_ANY_OUT_MAX_OUT = 8192
 # row (9.4, 16.4, 28.5 us; at an inner size of 1600 it is behind from 4 rows on).
 WIDE_OUT = 8192
 WIDE_OUT_DECODE_WORK = 8192
+# The decode kernel's time grows with the rows (every workgroup loads all of them for its 16 output
+# columns), the tiled kernel's hardly: under a large matrix with a wide output the tiled kernel (32 x
+# 32 tiles, several steps on their way from memory) is ahead from 17 rows on.  Matrices from memory,
+# decode kernel against tiled: [4800 x 1600] 8.5 / 8.5 us at 16 rows, 10.6 / 8.5 at 24, 11.7 / 8.5 at
+# 32, 18.8 / 10.0 at 64; [6400 x 1600] 9.3 / 9.1, 11.4 / 9.3, 12.7 / 9.3, 19.8 / 12.0; under smaller
+# matrices the decode kernel stays ahead up to 64 rows ([3072 x 768] 5.0 / 5.6 at 32, 6.2 / 5.6 at
+# 64; [1600 x 1600] 5.8 / 8.4 and 8.0 / 8.4), and a long inner size under a narrow output is split
+# over workgroups by either.
+TILED_FROM_ROWS = 17
+TILED_MIN_OUT = 4096
+TILED_MIN_MATRIX = 6_000_000
 
 
 def as_tensor(ctx, a: Union[torch.Tensor, LazyNorm]) -> torch.Tensor:
@@ -213,7 +224,9 @@ def linear(ctx, a: Union[torch.Tensor, LazyNorm], w: torch.Tensor, bias: Optiona
                                     tile_best.limit, w_packed=packed_weight(w)):
             tile_best.filled = True
             return False
-    if fast and n_rows <= 64 and not wide_out:
+    tiled = (n_rows >= TILED_FROM_ROWS and w.shape[0] >= TILED_MIN_OUT
+             and w.shape[0] * w.shape[1] >= TILED_MIN_MATRIX)
+    if fast and n_rows <= 64 and not wide_out and not tiled:
         epi = kernels.SK_EPI_QKV if scatter is not None else epilogue
         if (isinstance(a, LazyNorm) and getattr(a.norm, "fusable_layer_norm", False) and a._tensor is None
                 and (w.shape[0] <= FOLD_MAX_OUT
