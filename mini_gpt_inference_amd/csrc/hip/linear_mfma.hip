@@ -653,7 +653,8 @@ extern "C" int mgpt_linear_mfma(const void* act, long lda, const void* w, const 
 }
 
 // The same product with the tile shape given (0 = 256 x 256, 1 = 128 x 256, 2 = 128 x 64,
-// 3 = 64 x 64, 4 = 32 x 32; negative: chosen) and the number of stretches of the inner size given
+// 3 = 64 x 64, 4 = 32 x 32, 5 and 6 = 64 x 64 and 32 x 32 with four steps on their way from memory;
+// negative: chosen) and the number of stretches of the inner size given
 // (k_parts as for launch_any above), instead of chosen by the size: for tests and measurements.
 extern "C" int mgpt_linear_mfma_shape(int shape, int k_parts, const void* act, long lda, const void* w,
                                       const float* bias, void* out, int out_dtype, long ldo, int n_rows,
@@ -677,7 +678,7 @@ extern "C" int mgpt_linear_mfma_qkv(const void* act, long lda, const void* w, co
   if (!kpool || !vpool || !slot_mapping) return MGPT_ERR_NULL;
   if (head_dim <= 0 || (head_dim % 4) != 0 || (q_width % 4) != 0 || q_width + 2 * kv_width != n_out ||
       kv_width != n_kv_head * head_dim || page_size <= 0 || (n_out % 4) != 0 || (ldo % 4) != 0 ||
-      (((size_t)out | (size_t)bias) & 15) != 0 || shape >= MM_SHAPES)
+      (((size_t)out | (size_t)bias) & 15) != 0 || shape >= MM_SHAPES + 2)
     return MGPT_ERR_BAD_SHAPE;
   MfmaScatter sc = {(bf16_t*)kpool, (bf16_t*)vpool, slot_mapping, q_width, kv_width, head_dim, n_kv_head, page_size};
   return launch_any(shape, 1, act, lda, w, bias, out, MGPT_BF16, ldo, n_rows, n_out, k_dim, MM_EPI_QKV, nullptr, 0, sc,

@@ -178,13 +178,16 @@ def test_linear_mfma(n, k, o, epi, o_dt):
     helpers.assert_close(out2[:n - 3], _linear_want(a, w, None, epi, prev)[:n - 3], "bfloat16", "mfma partial rows")
 
 
-@pytest.mark.parametrize("n,k,o", [(300, 80, 257), (513, 512, 520), (256, 2048, 256), (1000, 48, 130), (70, 64, 1030)])
+@pytest.mark.parametrize("n,k,o", [(300, 80, 257), (513, 512, 520), (256, 2048, 256), (1000, 48, 130), (70, 64, 1030),
+                                   (40, 1616, 272)])
 @pytest.mark.parametrize("epi,o_dt", [(kernels.EPI_NONE, "bfloat16"), (kernels.EPI_NONE, "float32"),
                                       (kernels.EPI_GELU, "bfloat16"), (kernels.EPI_RESIDUAL, "float32")])
-@pytest.mark.parametrize("shape", [0, 1, 2, 3, 4])
+@pytest.mark.parametrize("shape", [0, 1, 2, 3, 4, 5, 6])
 def test_linear_mfma_each_tile_shape(n, k, o, epi, o_dt, shape):
     """Each tile shape forced at sizes that cut its tiles everywhere: rows and columns past the end, an
-    inner size that ends inside a step, several tiles each way."""
+    inner size that ends inside a step, several tiles each way.  Shapes 5 and 6: the 64 x 64 and 32 x 32
+    tiles with four steps on their way from memory, in whole rounds of four (inner sizes of 1, 2, 8, 26
+    and 32 steps: rounds that end beyond the last step)."""
     g = torch.Generator().manual_seed(16)
     a, w, bias = rnd(g, n, k, dtype="bfloat16"), rnd(g, o, k, dtype="bfloat16", scale=k ** -0.5), rnd(g, o)
     prev = rnd(g, n + 2, o, dtype=o_dt)
@@ -195,7 +198,8 @@ def test_linear_mfma_each_tile_shape(n, k, o, epi, o_dt, shape):
 
 
 @pytest.mark.parametrize("n,k,o,shape,parts", [(100, 2048, 96, 4, 4), (70, 1040, 132, 3, 2), (300, 6400, 64, 3, 8),
-                                                (33, 576, 40, 4, 3), (130, 1600, 260, 2, 4)])
+                                                (33, 576, 40, 4, 3), (130, 1600, 260, 2, 4), (64, 1600, 528, 6, 2),
+                                                (50, 3200, 96, 5, 4), (48, 6400, 1600, None, 0)])
 @pytest.mark.parametrize("epi,o_dt", [(kernels.EPI_NONE, "bfloat16"), (kernels.EPI_NONE, "float32"),
                                       (kernels.EPI_GELU, "bfloat16"), (kernels.EPI_RESIDUAL, "float32")])
 def test_linear_mfma_split_along_the_inner_size(n, k, o, shape, parts, epi, o_dt):
@@ -205,7 +209,12 @@ def test_linear_mfma_split_along_the_inner_size(n, k, o, shape, parts, epi, o_dt
     a, w, bias = rnd(g, n, k, dtype="bfloat16"), rnd(g, o, k, dtype="bfloat16", scale=k ** -0.5), rnd(g, o)
     prev = rnd(g, n + 2, o, dtype=o_dt)
     out = prev.clone().to(DEV)
+    if shape is None:      # what the library chooses by itself: a split, 32 x 32 tiles, four steps in flight
+        assert kernels.linear_mfma_partials(n, o, k, epi) > 0
+        parts = kernels.linear_mfma_partials(n, o, k, epi) // (n * o)
     scratch = torch.full((parts * n * o + 8,), float("nan"), device=DEV)
+    if shape is None:
+        parts = None
     assert kernels.linear_mfma(a.to(DEV), w.to(DEV), bias.to(DEV), out, n, epi, shape=shape, k_parts=parts,
                                partials=scratch)
     helpers.assert_close(out[:n], _linear_want(a, w, bias, epi, prev[:n]), "bfloat16", f"split {parts} of {k}")
@@ -216,8 +225,9 @@ def test_linear_mfma_split_along_the_inner_size(n, k, o, shape, parts, epi, o_dt
                                partials=scratch)
     assert torch.equal(out, out2)
     # a buffer that is too small is refused when the split is forced, and not used when it is not
-    assert not kernels.linear_mfma(a.to(DEV), w.to(DEV), bias.to(DEV), out2, n, epi, shape=shape, k_parts=parts,
-                                   partials=scratch[:16])
+    if shape is not None:
+        assert not kernels.linear_mfma(a.to(DEV), w.to(DEV), bias.to(DEV), out2, n, epi, shape=shape, k_parts=parts,
+                                       partials=scratch[:16])
 
 
 def test_linear_mfma_splits_by_itself_when_tiles_are_few_and_the_inner_size_long():
@@ -424,12 +434,14 @@ def test_linear_skinny_few_rows_with_a_long_inner_size_split_over_workgroups(n, 
     helpers.assert_close(whole[:n], want[:n], "bfloat16", "unsplit")
 
 
-@pytest.mark.parametrize("n,shape", [(70, None), (300, 3), (1100, 2), (300, 1), (520, 0)])
-def test_linear_mfma_stores_keys_and_values(n, shape):
-    """The tiled kernel's fused QKV product: the tile shape chosen by the size and each larger one forced;
+@pytest.mark.parametrize("n,shape,k", [(70, None, 96), (300, 3, 96), (1100, 2, 96), (300, 1, 96), (520, 0, 96),
+                                       (40, None, 832), (60, 6, 96), (33, 5, 1024)])
+def test_linear_mfma_stores_keys_and_values(n, shape, k):
+    """The tiled kernel's fused QKV product: the tile shape chosen by the size and each larger one forced
+    (at 40 rows over 13 steps the library takes the variant with four steps in flight by itself);
     groups of heads; padded rows (slot -1) leave the pools alone."""
     g = torch.Generator().manual_seed(15)
-    k, h, hk, d, page = 96, 6, 2, 16, 8
+    h, hk, d, page = 6, 2, 16, 8
     pages = n // page + 3
     qw, kvw = h * d, hk * d
     a, w, bias = rnd(g, n, k, dtype="bfloat16"), rnd(g, qw + 2 * kvw, k, dtype="bfloat16", scale=0.2), rnd(g, qw + 2 * kvw)
