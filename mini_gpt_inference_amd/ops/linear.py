@@ -130,11 +130,21 @@ WIDE_OUT_DECODE_WORK = 8192
 # decode kernel against tiled: [4800 x 1600] 8.5 / 8.5 us at 16 rows, 10.6 / 8.5 at 24, 11.7 / 8.5 at
 # 32, 18.8 / 10.0 at 64; [6400 x 1600] 9.3 / 9.1, 11.4 / 9.3, 12.7 / 9.3, 19.8 / 12.0; under smaller
 # matrices the decode kernel stays ahead up to 64 rows ([3072 x 768] 5.0 / 5.6 at 32, 6.2 / 5.6 at
-# 64; [1600 x 1600] 5.8 / 8.4 and 8.0 / 8.4), and a long inner size under a narrow output is split
-# over workgroups by either.
+# 64; [1600 x 1600] 5.8 / 8.4 and 8.0 / 8.4).  A long inner size under a narrow output is split over
+# workgroups by either; there the tiled kernel with its joining kernel is ahead from 33 rows on
+# ([1600 x 6400]: the decode kernel's first half alone, its sums left pending, 20.0 us at 64 rows, the
+# tiled pair 15.1; at 32 rows about 11.5 against 12.7).
 TILED_FROM_ROWS = 17
 TILED_MIN_OUT = 4096
 TILED_MIN_MATRIX = 6_000_000
+TILED_ANY_OUT_FROM_ROWS = 33
+
+
+def tiled_at_few_rows(n_rows: int, w: torch.Tensor) -> bool:
+    """Whether a product of at most 64 rows goes to the tiled kernel rather than the decode kernel."""
+    if w.shape[0] * w.shape[1] < TILED_MIN_MATRIX:
+        return False
+    return n_rows >= TILED_ANY_OUT_FROM_ROWS or (n_rows >= TILED_FROM_ROWS and w.shape[0] >= TILED_MIN_OUT)
 
 
 def as_tensor(ctx, a: Union[torch.Tensor, LazyNorm]) -> torch.Tensor:
@@ -183,7 +193,7 @@ def linear_add(ctx, a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tenso
     them into x; the LayerNorm that reads x next adds them up (LazyNorm.tensor)."""
     if (may_leave_parts and getattr(ctx, "pending", None) is None and not ctx.exact and ctx.dtype == torch.bfloat16
             and w.dtype == torch.bfloat16 and a.dtype == torch.bfloat16 and 0 < n_rows <= 64 and n_rows == ctx.n_rows
-            and x.is_contiguous() and x.shape[1] == w.shape[0]
+            and not tiled_at_few_rows(n_rows, w) and x.is_contiguous() and x.shape[1] == w.shape[0]
             and (w.shape[0] >= LEAVE_PARTS_MIN_WIDTH or n_rows >= LEAVE_PARTS_MIN_ROWS)
             and kernels.residual_parts_limit(w.shape[0]) >= 4
             and kernels.linear_skinny_partials(n_rows, w.shape[0], w.shape[1], False, kernels.EPI_RESIDUAL)):
@@ -224,9 +234,7 @@ def linear(ctx, a: Union[torch.Tensor, LazyNorm], w: torch.Tensor, bias: Optiona
                                     tile_best.limit, w_packed=packed_weight(w)):
             tile_best.filled = True
             return False
-    tiled = (n_rows >= TILED_FROM_ROWS and w.shape[0] >= TILED_MIN_OUT
-             and w.shape[0] * w.shape[1] >= TILED_MIN_MATRIX)
-    if fast and n_rows <= 64 and not wide_out and not tiled:
+    if fast and n_rows <= 64 and not wide_out and not tiled_at_few_rows(n_rows, w):
         epi = kernels.SK_EPI_QKV if scatter is not None else epilogue
         if (isinstance(a, LazyNorm) and getattr(a.norm, "fusable_layer_norm", False) and a._tensor is None
                 and (w.shape[0] <= FOLD_MAX_OUT
