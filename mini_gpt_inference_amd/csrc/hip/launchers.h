@@ -72,6 +72,8 @@ int mgpt_residual_settle(const float* base, const float* partials, int n_parts, 
 int mgpt_linear_generic(const void* A, int a_dtype, long lda, const void* W, int w_dtype, const float* bias,
     void* out, int out_dtype, long ldo, int n_rows, int n_out, int k_dim, int epilogue, hipStream_t stream);
 // linear_mfma.hip
+int mgpt_linear_mfma_parts(const void* act, long lda, const void* w, const float* bias, float* partials,
+                           long partials_floats, int n_rows, int n_out, int k_dim, hipStream_t stream);
 int mgpt_linear_mfma(const void* act, long lda, const void* w, const float* bias, void* out, int out_dtype,
     long ldo, int n_rows, int n_out, int k_dim, int epilogue, float* partials, long partials_floats,
     hipStream_t stream);
@@ -128,6 +130,7 @@ int mgpt_sample_advance(const float* logits, long ld, int n_rows, int vocab, int
   X(mgpt_residual_settle) \
   X(mgpt_linear_generic) \
   X(mgpt_linear_mfma) \
+  X(mgpt_linear_mfma_parts) \
   X(mgpt_linear_mfma_shape) \
   X(mgpt_linear_mfma_qkv) \
   X(mgpt_linear_skinny) \

@@ -160,6 +160,7 @@ __global__ __launch_bounds__(64 * WVM * WVN) void linear_mfma_kernel(
   const int k_begin = part * k_per;
   const int k_len = k_dim - k_begin < k_per ? k_dim - k_begin : k_per;
   out += part * part_stride;
+  if (part != 0) bias = nullptr;  // of a product split along k, the first stretch's sums carry the bias (if any is given)
   const int wr = (wave / WVN) * (WTM * 16), wc = (wave % WVN) * (WTN * 16);
   const int lrow = lane & 15;
 
@@ -564,9 +565,11 @@ bool shapes_ok(const void* act, long lda, const void* w, const void* out, long l
 // shape < 0: chosen by the size.  k_parts: 0 = chosen by the size, together with the shape, if
 // `partials` holds enough floats (else unsplit; with a given shape unsplit too), 1 = unsplit,
 // more = that many stretches (refused if the buffer is too small).
+// leave_parts: the stretches' sums stay in `partials` ([parts][n_rows][n_out], the first with the
+// bias), no second kernel joins them; *leave_parts gets the number of parts, 0 if the product is not split.
 int launch_any(int shape, int k_parts, const void* act, long lda, const void* w, const float* bias, void* out,
                int out_dtype, long ldo, int n_rows, int n_out, int k_dim, int epilogue, float* partials,
-               long partials_floats, const MfmaScatter& sc, hipStream_t stream) {
+               long partials_floats, const MfmaScatter& sc, hipStream_t stream, int* leave_parts = nullptr) {
   if (n_rows == 0 || n_out == 0) return MGPT_OK;
   if (!act || !w || !out) return MGPT_ERR_NULL;
   if (!shapes_ok(act, lda, w, out, ldo, n_rows, n_out, k_dim)) return MGPT_ERR_BAD_SHAPE;
@@ -605,8 +608,12 @@ int launch_any(int shape, int k_parts, const void* act, long lda, const void* w,
     }
   }
   const bool split = k_parts > 1;
+  if (leave_parts) {
+    *leave_parts = split ? k_parts : 0;
+    if (!split) return MGPT_OK;  // nothing launched: the caller takes another way
+  }
   void* dst = split ? (void*)partials : out;
-  const float* b = split ? nullptr : bias;
+  const float* b = (split && !leave_parts) ? nullptr : bias;
   const int dt = split ? MGPT_F32 : out_dtype, epi = split ? MM_EPI_NONE : epilogue;
   const long ld = split ? n_out : ldo, stride = split ? (long)n_rows * n_out : 0;
 #define MM_ARGS act, lda, w, b, dst, dt, ld, n_rows, n_out, k_dim, epi, k_parts, stride, sc, stream
@@ -623,7 +630,7 @@ int launch_any(int shape, int k_parts, const void* act, long lda, const void* w,
       break;
   }
 #undef MM_ARGS
-  if (rc != MGPT_OK || !split) return rc;
+  if (rc != MGPT_OK || !split || leave_parts) return rc;
   return launch_join(partials, k_parts, bias, out, out_dtype, ldo, n_rows, n_out, epilogue, stream);
 }
 
@@ -636,6 +643,21 @@ extern "C" long mgpt_linear_mfma_partials(int n_rows, int n_out, int k_dim, int 
   int shape, parts;
   choose_split(n_rows, n_out, k_dim, epilogue, &shape, &parts);
   return parts > 1 ? (long)used_parts(k_dim, parts) * n_rows * n_out : 0;
+}
+
+// The first half of a split product alone: partials[p][n][o] = the sum over stretch p of the inner
+// size (+ bias[o] in p = 0), p < mgpt_linear_mfma_partials(n_rows, n_out, k_dim, residual epilogue) /
+// (n_rows * n_out), for a caller that adds the parts up itself (a pending residual: fused_decode.h).
+// MGPT_ERR_BAD_SHAPE, with nothing launched, if the product would not be split or the buffer is too small.
+extern "C" int mgpt_linear_mfma_parts(const void* act, long lda, const void* w, const float* bias, float* partials,
+                                      long partials_floats, int n_rows, int n_out, int k_dim, hipStream_t stream) {
+  if (!partials) return MGPT_ERR_NULL;
+  MfmaScatter sc = {};
+  int parts = 0;
+  const int rc = launch_any(-1, 0, act, lda, w, bias, partials, MGPT_F32, n_out, n_rows, n_out, k_dim, MM_EPI_RESIDUAL,
+                            partials, partials_floats, sc, stream, &parts);
+  if (rc != MGPT_OK) return rc;
+  return parts > 1 ? MGPT_OK : MGPT_ERR_BAD_SHAPE;
 }
 
 // act: [n_rows, k_dim] bfloat16 with row stride lda (a multiple of 8, 16-byte aligned base);

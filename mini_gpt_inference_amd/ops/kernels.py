@@ -559,6 +559,33 @@ def linear_mfma_partials(n_rows: int, n_out: int, k_dim: int, epilogue: int) -> 
     return hit
 
 
+def linear_mfma_parts(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], partials: torch.Tensor,
+                      n_rows: int) -> bool:
+    """The tiled product's first half alone where it splits the inner size: partials[p, :n_rows]
+    (float32 [parts, n_rows, out], dense, parts = linear_mfma_partials(n_rows, out, inner, EPI_RESIDUAL)
+    // (n_rows * out)) = a[:n_rows] @ w[:, stretch p].T, the first with the bias added; nobody adds
+    them up.  False, having launched nothing, where the product would not be split."""
+    n_out, k_dim = w.shape
+    need = linear_mfma_partials(n_rows, n_out, k_dim, EPI_RESIDUAL)
+    if (not need or w.dtype != torch.bfloat16 or a.dtype != torch.bfloat16 or a.stride(0) % 8 or a.data_ptr() % 16
+            or w.data_ptr() % 16 or k_dim % 16):
+        return False
+    parts = need // (n_rows * n_out)
+    _need_cuda(a, w, bias, partials)
+    _need(w.is_contiguous(), "weight must be dense [out, in]")
+    _need(a.dim() == 2 and a.stride(1) == 1 and a.shape[1] == k_dim and a.shape[0] >= n_rows,
+          "activation must be [>=n_rows, inner] with unit inner stride")
+    _need(bias is None or (bias.dtype == torch.float32 and bias.numel() == n_out), "bias must be float32 [out]")
+    _need(partials.dtype == torch.float32 and partials.is_contiguous() and partials.data_ptr() % 16 == 0
+          and tuple(partials.shape) == (parts, n_rows, n_out), f"partials must be dense float32 [{parts}, n_rows, out]")
+    rc = library.kernels().mgpt_linear_mfma_parts(_ptr(a), a.stride(0), _ptr(w), _ptr(bias), _ptr(partials),
+                                                  partials.numel(), n_rows, n_out, k_dim, _stream())
+    if rc == -2:
+        return False
+    _check(rc, "linear_mfma_parts")
+    return True
+
+
 def linear_mfma(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor,
                 n_rows: int, epilogue: int, scatter=None, shape: Optional[int] = None,
                 partials: Optional[torch.Tensor] = None, k_parts: Optional[int] = None) -> bool:

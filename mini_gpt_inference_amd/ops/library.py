@@ -133,6 +133,7 @@ def _declare_optional(lib: ctypes.CDLL) -> None:
         "mgpt_linear_mfma": [P, L, P, P, P, I, L, I, I, I, I, P, L, P],
         "mgpt_linear_mfma_shape": [I, I, P, L, P, P, P, I, L, I, I, I, I, P, L, P],
         "mgpt_linear_mfma_partials": [I, I, I, I],
+        "mgpt_linear_mfma_parts": [P, L, P, P, P, L, I, I, I, P],
         "mgpt_linear_mfma_qkv": [P, L, P, P, P, L, I, I, I, P, P, P, I, I, I, I, I, I, P],
         "mgpt_prefill_attention_bf16": [P, L, P, L, P, P, P, I, P, P, I, I, I, I, I, I, F, I, I, P],
         # a residual that is still a sum: base, partials, n_parts, part_stride, token table, position table, ids, positions

@@ -191,10 +191,20 @@ def linear_add(ctx, a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tenso
     long inner size is split over workgroups anyway (few rows, few column tiles) leaves the
     workgroups' sums as the parts of a pending residual instead of running a second kernel that adds
     them into x; the LayerNorm that reads x next adds them up (LazyNorm.tensor)."""
-    if (may_leave_parts and getattr(ctx, "pending", None) is None and not ctx.exact and ctx.dtype == torch.bfloat16
-            and w.dtype == torch.bfloat16 and a.dtype == torch.bfloat16 and 0 < n_rows <= 64 and n_rows == ctx.n_rows
-            and not tiled_at_few_rows(n_rows, w) and x.is_contiguous() and x.shape[1] == w.shape[0]
-            and (w.shape[0] >= LEAVE_PARTS_MIN_WIDTH or n_rows >= LEAVE_PARTS_MIN_ROWS)
+    leave = (may_leave_parts and getattr(ctx, "pending", None) is None and not ctx.exact
+             and ctx.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and a.dtype == torch.bfloat16
+             and 0 < n_rows <= 64 and n_rows == ctx.n_rows and x.is_contiguous() and x.shape[1] == w.shape[0])
+    if leave and tiled_at_few_rows(n_rows, w):
+        # the tiled kernel's split: its stretches' sums are the parts (2 to 8 of them)
+        need = kernels.linear_mfma_partials(n_rows, w.shape[0], w.shape[1], kernels.EPI_RESIDUAL)
+        n_parts = need // (n_rows * w.shape[0])
+        if 1 < n_parts <= kernels.residual_parts_limit(w.shape[0]):
+            buf = ctx.workspace.get("residual_parts", n_parts * n_rows, w.shape[0], torch.float32)
+            parts = buf[:n_parts * n_rows].view(n_parts, n_rows, w.shape[0])
+            if kernels.linear_mfma_parts(a, w, bias, parts, n_rows):
+                ctx.pending = residual.PendingSums(x, parts, n_parts)
+                return
+    elif (leave and (w.shape[0] >= LEAVE_PARTS_MIN_WIDTH or n_rows >= LEAVE_PARTS_MIN_ROWS)
             and kernels.residual_parts_limit(w.shape[0]) >= 4
             and kernels.linear_skinny_partials(n_rows, w.shape[0], w.shape[1], False, kernels.EPI_RESIDUAL)):
         buf = ctx.workspace.get("residual_parts", 4 * n_rows, w.shape[0], torch.float32)

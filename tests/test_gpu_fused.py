@@ -305,6 +305,49 @@ def test_split_product_left_as_parts_of_a_pending_residual(rows, n_out, k_dim, b
                          "bfloat16", "LayerNorm of x + product")
 
 
+@pytest.mark.parametrize("rows,n_out,k_dim,bias", [(48, 1600, 6400, True), (64, 1600, 6400, False), (33, 768, 3072, True),
+                                                   (100, 512, 4096, True)])
+def test_tiled_split_left_as_parts_of_a_pending_residual(rows, n_out, k_dim, bias):
+    """The tiled product's first kernel alone where it splits the inner size: its parts (the first
+    carries the bias) add up to the plain product, to the very bits of the product that joins them
+    itself; the residual LayerNorm that reads base + parts gives the LayerNorm of x + product."""
+    g = torch.Generator().manual_seed(rows + n_out)
+    a = bf(rnd(g, rows, k_dim))
+    w = bf(rnd(g, n_out, k_dim, scale=0.03))
+    b = rnd(g, n_out) if bias else None
+    x = rnd(g, rows + 1, n_out, scale=2.0)
+    x[rows:] = float("nan")
+    dev = lambda t: None if t is None else t.to(DEV)
+    wd = dev(w)
+    need = kernels.linear_mfma_partials(rows, n_out, k_dim, kernels.EPI_RESIDUAL)
+    n_parts = need // (rows * n_out)
+    assert n_parts > 1 and need == n_parts * rows * n_out
+    parts = torch.full((n_parts, rows, n_out), float("nan"), device=DEV)
+    assert kernels.linear_mfma_parts(dev(a), wd, dev(b), parts, rows)
+    want = P.plain_linear(a.double(), w.double(), None if b is None else b.double())
+    helpers.assert_close(parts.sum(0), want, "bfloat16", "sum of the parts")
+    joined = torch.zeros(rows, n_out, device=DEV)
+    scratch = torch.zeros(need, device=DEV)
+    assert kernels.linear_mfma(dev(a), wd, dev(b), joined, rows, kernels.EPI_NONE, partials=scratch)
+    raw = scratch.view(n_parts, rows, n_out)
+    assert torch.equal(parts[1:], raw[1:])
+    helpers.assert_close(parts[0], raw[0].double().cpu() + (0 if b is None else b.double()), "float32", "the first part")
+    # read as a pending residual
+    pending = PendingSums(dev(x), parts, n_parts)
+    gain, beta = 1 + 0.1 * rnd(g, n_out), rnd(g, n_out, scale=0.1)
+    out = torch.full((rows, n_out), float("nan"), dtype=torch.bfloat16, device=DEV)
+    assert kernels.residual_layer_norm(pending, dev(gain), dev(beta), 1e-5, None, out, rows, settled=pending.base)
+    true = x[:rows].double() + want
+    helpers.assert_close(pending.base[:rows], true, "bfloat16", "x + product")
+    assert torch.isnan(pending.base[rows:]).all()
+    helpers.assert_close(out, P.plain_layer_norm(pending.base[:rows].double().cpu(), gain.double(), beta.double(), 1e-5),
+                         "bfloat16", "LayerNorm of x + product")
+    # a product that the tiled kernel does not split leaves no parts
+    small = torch.full((2, rows, 4096), 7.0, device=DEV)
+    assert not kernels.linear_mfma_parts(dev(a)[:, :512].contiguous(), bf(rnd(g, 4096, 512)).to(DEV), None, small, rows)
+    assert bool((small == 7.0).all())
+
+
 def test_split_parts_are_refused_where_the_product_is_not_split():
     g = torch.Generator().manual_seed(2)
     for rows, n_out, k_dim in ((4, 512, 2048), (4, 4096, 4096), (70, 512, 4096)):
