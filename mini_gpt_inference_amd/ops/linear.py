@@ -170,6 +170,7 @@ class TileBest:
 # 1748 against 1768, 2049 against 2102, 2439 against 2554)
 LEAVE_PARTS_MIN_WIDTH = 1024
 LEAVE_PARTS_MIN_ROWS = 8
+LEAVE_PARTS_MAX_ROWS = 256     # (the tiled kernel's split; the decode kernel's ends at its 64 rows)
 
 
 def plain_residual(ctx, h, x: torch.Tensor) -> None:
@@ -193,7 +194,8 @@ def linear_add(ctx, a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tenso
     them into x; the LayerNorm that reads x next adds them up (LazyNorm.tensor)."""
     leave = (may_leave_parts and getattr(ctx, "pending", None) is None and not ctx.exact
              and ctx.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and a.dtype == torch.bfloat16
-             and 0 < n_rows <= 64 and n_rows == ctx.n_rows and x.is_contiguous() and x.shape[1] == w.shape[0])
+             and 0 < n_rows <= LEAVE_PARTS_MAX_ROWS and n_rows == ctx.n_rows and x.is_contiguous()
+             and x.shape[1] == w.shape[0])
     if leave and tiled_at_few_rows(n_rows, w):
         # the tiled kernel's split: its stretches' sums are the parts (2 to 8 of them)
         need = kernels.linear_mfma_partials(n_rows, w.shape[0], w.shape[1], kernels.EPI_RESIDUAL)
@@ -204,7 +206,7 @@ def linear_add(ctx, a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tenso
             if kernels.linear_mfma_parts(a, w, bias, parts, n_rows):
                 ctx.pending = residual.PendingSums(x, parts, n_parts)
                 return
-    elif (leave and (w.shape[0] >= LEAVE_PARTS_MIN_WIDTH or n_rows >= LEAVE_PARTS_MIN_ROWS)
+    elif (leave and n_rows <= 64 and (w.shape[0] >= LEAVE_PARTS_MIN_WIDTH or n_rows >= LEAVE_PARTS_MIN_ROWS)
             and kernels.residual_parts_limit(w.shape[0]) >= 4
             and kernels.linear_skinny_partials(n_rows, w.shape[0], w.shape[1], False, kernels.EPI_RESIDUAL)):
         buf = ctx.workspace.get("residual_parts", 4 * n_rows, w.shape[0], torch.float32)
