@@ -590,13 +590,14 @@ int launch_any(int shape, int k_parts, const void* act, long lda, const void* w,
   if (shape >= MM_SHAPES) return MGPT_ERR_BAD_SHAPE;
   if (k_parts == 0) k_parts = 1;
   if (ahead == 0) {
-    // Few tiles of few rows over a long enough stretch: the workgroups are too few to hide a trip to
+    // Few small tiles over a long enough stretch: the workgroups are too few to hide a trip to
     // memory behind one another.  Measured over matrices that come from memory, 32 x 32 tiles, 40-64
     // rows: [4800 x 1600] 9.8-10.0 us against 10.8, [6400 x 1600] 10.7-11.9 against 15.6, [1600 x 1600]
-    // 8.4 against 10.3, [4096 x 1024] 6.3 against 7.6; from a hundred rows on nothing is gained.
+    // 8.4 against 10.3 (and 8.6 / 10.5 at 136 rows, 250 tiles), [4096 x 1024] 6.3 against 7.6; with more
+    // than two such workgroups a compute unit nothing is gained ([4800 x 1600] at 136 rows, 750 tiles:
+    // 12.8 against 11.7).
     const int steps = (k_dim + MM_BK - 1) / MM_BK;
-    ahead = (shape == 4 && n_rows <= 64 && steps / k_parts >= 12 && tiles_of(4, n_rows, n_out) * k_parts <= 1024)
-                ? MM_AHEAD : 1;
+    ahead = (shape == 4 && steps / k_parts >= 12 && tiles_of(4, n_rows, n_out) * k_parts <= 512) ? MM_AHEAD : 1;
   }
   if (k_parts > 1) {
     k_parts = used_parts(k_dim, k_parts > MM_MAX_PARTS ? MM_MAX_PARTS : k_parts);
