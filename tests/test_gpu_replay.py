@@ -385,12 +385,13 @@ def test_real_family_sizes_mixed_with_page_reuse(tmp_path_factory, shape, dtype)
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("n_req", [8, 17, 40, 64])
+@pytest.mark.parametrize("n_req", [8, 17, 40, 64, 100, 128])
 @pytest.mark.parametrize("shape", ["small", "xl", "50M"])
 def test_real_family_sizes_many_requests_decoding(tmp_path_factory, shape, dtype, n_req):
-    """Decode steps of 8, 17, 40 and 64 requests at the real widths, as logits: the decode products
+    """Decode steps of 8 to 128 requests at the real widths, as logits: the decode products
     change kernels with the rows and the matrix's size (rows dealt out in groups, the inner size
-    split over workgroups, the head's hand-over to the tiled kernel, the fused kernels of few rows).
+    split over workgroups and its sums left pending, the hand-over to the tiled kernel, the fused
+    kernels with one, two and four tokens a workgroup).
     The same step comes several times, so the later ones are graph replays."""
     folder, cfg, pcfg, w = _family_model(tmp_path_factory, shape)
     rng = np.random.default_rng(100 + n_req)
