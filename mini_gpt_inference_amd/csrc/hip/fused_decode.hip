@@ -389,11 +389,11 @@ __global__ __launch_bounds__(FUSED_THREADS) void fused_attention_decode_kernel(F
   FA_LOAD_W(0)
   if (!any) return;  // tokens of the padding only (the whole workgroup)
   if (NORMED) {
-    // everything is sent for at once; the rows go to LDS as they are
+    // all of the weights are sent for at once; the rows go to LDS as they are.  The keys and values
+    // wait for the block table's entries: they are sent for behind the barrier, which then does not.
     FA_LOAD_W(1)
     FA_LOAD_W(2)
     FA_LOAD_W(3)
-    FA_LOAD_KV
     if (gq < TK) reinterpret_cast<uint2*>(act_s + gq * FUSED_MAX_WIDTH)[vq] = normed4;
     if (gq == 2 && proj_bias) reinterpret_cast<float4*>(bproj_s)[vq] = gb4;
   } else {
@@ -467,9 +467,10 @@ __global__ __launch_bounds__(FUSED_THREADS) void fused_attention_decode_kernel(F
       }
     }
   }
+  fd_barrier();  // also: the rows' partial sums are read, their place takes the waves' sums now
+  if (NORMED) FA_LOAD_KV
 #undef FA_LOAD_W
 #undef FA_LOAD_KV
-  fd_barrier();  // also: the rows' partial sums are read, their place takes the waves' sums now
   FD_STAMP(1);
 
   // ---- q, k, v of this head: every wave a stretch of k over all the row tiles; the waves' sums
