@@ -64,8 +64,9 @@ __device__ __forceinline__ bf16x8_t ld_row_shl(bf16x8_t v, int j) {
 // loads the j-th of 16 / FEW k steps of row r, rounds it and adds up its statistics, and the row's
 // own lane takes the rounded values over with a DPP shift.  A load instruction costs the compute
 // unit the same whether four of its lanes are live or all: at one row that is 2 instead of 26 of
-// them for an inner size of 1600 ([6400 x 1600] at one row: the LayerNorm's share of the kernel
-// falls from 2.2 to 0.6 us).  0: every lane loads what it multiplies.
+// them for an inner size of 1600 ([6400 x 1600] at one row: 6.9 us with the LayerNorm against 6.9
+// over rows that are normed already, where it was 2.2 us more; at 8 rows 9.9 against 7.9).  0: every
+// lane loads what it multiplies.
 template <int NT, int SMAX, bool LN, int EPI, typename OT, bool VEC, bool SPLIT = false, int FEW = 0>
 __global__ __launch_bounds__(256) void linear_decode_kernel(SkinnyArgs a) {
   static_assert(FEW == 0 || (LN && NT == 1 && !SPLIT && (FEW == 1 || FEW == 2 || FEW == 4 || FEW == 8)),
@@ -213,11 +214,7 @@ __global__ __launch_bounds__(256) void linear_decode_kernel(SkinnyArgs a) {
       }
       // the row's own lane (lrow < FEW) takes step i from the lane that loaded it
 #pragma unroll
-      for (int i = 0; i < SMAX; ++i) {
-        constexpr int dummy = 0;
-        (void)dummy;
-        av[0][i] = ld_row_shl<FEW>(packed[i / FJ], i % FJ);
-      }
+      for (int i = 0; i < SMAX; ++i) av[0][i] = ld_row_shl<FEW>(packed[i / FJ], i % FJ);
     } else if (LN) {
       float4 lo[NT][SMAX], hi[NT][SMAX];
 #pragma unroll

@@ -141,7 +141,8 @@ TILED_ANY_OUT_FROM_ROWS = 33
 
 
 def tiled_at_few_rows(n_rows: int, w: torch.Tensor) -> bool:
-    """Whether a product of at most 64 rows goes to the tiled kernel rather than the decode kernel."""
+    """Whether a product of few rows (the decode kernel takes up to 64; linear_add asks for up to
+    LEAVE_PARTS_MAX_ROWS) goes to the tiled kernel rather than the decode kernel."""
     if w.shape[0] * w.shape[1] < TILED_MIN_MATRIX:
         return False
     return n_rows >= TILED_ANY_OUT_FROM_ROWS or (n_rows >= TILED_FROM_ROWS and w.shape[0] >= TILED_MIN_OUT)
