@@ -271,8 +271,8 @@ __global__ __launch_bounds__(FUSED_THREADS) void fused_attention_decode_kernel(F
   // stands before it: only a quarter of the weights' loads stand before the barrier at which the
   // row's partial sums meet (the row's loads of the last waves would otherwise wait behind all the
   // weights of the first: measured, 1.6 us a layer slower); the rest, and the keys and values, are
-  // sent for behind it, while the first wave norms the row.  A wave's loads come back in order:
-  // the step's numbers and the row first, keys and values last.
+  // sent for behind it, while the first waves norm a row each.  A wave's loads come back in order:
+  // the step's numbers and the rows first, keys and values last.
   // (a token beyond the step's rows repeats the workgroup's first and stores nothing, like a token of
   // the padding; a decode-only step: token n is request n)
   int tokn[TK], qpos[TK], slot[TK];
