@@ -717,6 +717,14 @@ def _residual_args(pending, width: int):
             _ptr(positions))
 
 
+def _overlap(a: Optional[torch.Tensor], b: Optional[torch.Tensor]) -> bool:
+    """Whether two tensors' bytes overlap."""
+    if a is None or b is None or not a.numel() or not b.numel():
+        return False
+    a0, b0 = a.data_ptr(), b.data_ptr()
+    return a0 < b0 + b.numel() * b.element_size() and b0 < a0 + a.numel() * a.element_size()
+
+
 def _residual_rows(pending) -> int:
     """Rows that every array of a pending residual holds."""
     rows = 1 << 30
@@ -786,6 +794,9 @@ def fused_attention_decode(pending, settled: Optional[torch.Tensor], gain: torch
     _need(out_partials.dtype == torch.float32 and out_partials.dim() == 3 and out_partials.is_contiguous()
           and out_partials.shape[0] >= n_head and out_partials.shape[1] >= n_rows and out_partials.shape[2] == width,
           "out_partials must be dense float32 [>=heads, >=rows, width]")
+    # a workgroup adds the pending sums up while others of the launch already store theirs
+    _need(not (pending.n_parts and _overlap(out_partials, pending.partials)),
+          "out_partials must not be the array that holds the pending sums")
     _need(block_tables.dtype == torch.int32 and block_tables.dim() == 2 and block_tables.is_contiguous()
           and block_tables.shape[0] >= n_rows, "block_tables must be dense int32 [>=rows, blocks]")
     _need_i32("slot_mapping", slot_mapping, n_rows)
@@ -834,6 +845,8 @@ def fused_mlp_decode(pending, settled: torch.Tensor, gain: torch.Tensor, beta: O
     _need(out_partials.dtype == torch.float32 and out_partials.dim() == 3 and out_partials.is_contiguous()
           and out_partials.shape[0] >= parts and out_partials.shape[1] >= n_rows and out_partials.shape[2] == width,
           "out_partials must be dense float32 [>=hidden/64, >=rows, width]")
+    _need(not (pending.n_parts and _overlap(out_partials, pending.partials)),
+          "out_partials must not be the array that holds the pending sums")
     rc = library.kernels().mgpt_fused_mlp_decode(
         *args, _ptr(settled), _ptr(gain), _ptr(beta), float(eps), _ptr(wfc_packed), _ptr(bfc), _ptr(wproj_packed),
         _ptr(bproj), _ptr(out_partials), out_partials.stride(0), n_rows, width, hidden, _stream())

@@ -57,6 +57,22 @@ def take(ctx, x: torch.Tensor) -> Tuple[PendingSums, torch.Tensor]:
     return pending, (twin_of(ctx, x) if on_x else x)
 
 
+def parts_buffer(ctx, name: str, n_parts: int, n_rows: int, width: int) -> torch.Tensor:
+    """Where a kernel leaves its n_parts partial sums [n_parts, n_rows, width].  Every part kind has
+    two arrays under its name and takes the one that does not hold the sums still pending: the kernel
+    adds those up in its prologue while other workgroups of the same launch already store theirs, so
+    two parts of one kind in a row (two attention mixers, two feed-forwards) must not share one."""
+    def get(suffix: str) -> torch.Tensor:
+        return ctx.workspace.get(name + suffix, n_parts * n_rows, width, torch.float32)[:n_parts * n_rows] \
+            .view(n_parts, n_rows, width)
+    buf = get("")
+    pending = ctx.pending
+    if pending is not None and pending.partials is not None \
+            and pending.partials.untyped_storage().data_ptr() == buf.untyped_storage().data_ptr():
+        buf = get("_second")
+    return buf
+
+
 def settle(ctx, x: torch.Tensor, n_rows: int) -> None:
     """Makes x[:n_rows] plain: adds up what is pending into it."""
     pending = ctx.pending

@@ -65,8 +65,7 @@ class DenseMLP(FeedForward):
         if ctx.pending is not None and ctx.pending.base is None:
             residual.settle(ctx, x, n)      # table rows: this kernel reads residual rows only
         pending, settled = residual.take(ctx, x)
-        parts = ctx.workspace.get("feed_forward_parts", parts_n * n, self.width, torch.float32) \
-            [:parts_n * n].view(parts_n, n, self.width)
+        parts = residual.parts_buffer(ctx, "feed_forward_parts", parts_n, n, self.width)
         if not kernels.fused_mlp_decode(pending, settled, h.norm.weight, h.norm.bias, h.norm.eps, wfc, self.fc_bias,
                                         wproj, self.proj_bias, parts, n, self.hidden):
             return False

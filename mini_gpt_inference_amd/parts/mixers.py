@@ -103,8 +103,7 @@ class PagedCausalAttention(Mixer):
             if ctx.pending is not None:
                 return False
         pending, settled = residual.take(ctx, x)
-        parts = ctx.workspace.get("attention_parts", self.n_head * n, self.width, torch.float32) \
-            [:self.n_head * n].view(self.n_head, n, self.width)
+        parts = residual.parts_buffer(ctx, "attention_parts", self.n_head, n, self.width)
         if not kernels.fused_attention_decode(
                 pending, settled, h.norm.weight, h.norm.bias, h.norm.eps, wqkv, self.qkv_bias, wproj, self.proj_bias,
                 parts, group.k_pools[binding.index], group.v_pools[binding.index], group.slot_mapping,

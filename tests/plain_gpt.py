@@ -110,8 +110,9 @@ def plain_block(x: torch.Tensor, w: Dict[str, torch.Tensor], prefix: str, n_head
     return x
 
 
-def plain_forward(w: Dict[str, torch.Tensor], cfg: dict, ids: Sequence[int]) -> torch.Tensor:
-    """Whole-sequence forward, logits at every position [T, V]
+def plain_forward(w: Dict[str, torch.Tensor], cfg: dict, ids: Sequence[int],
+                  rows: Optional[Sequence[int]] = None) -> torch.Tensor:
+    """Whole-sequence forward, logits at every position [T, V], or at the positions `rows` only
     (src/minigpt_infer/reference.py:105-114; tied head: reference.py:89-90)."""
     ids_t = torch.as_tensor(list(ids), dtype=torch.long)
     if ids_t.numel() > cfg["block_size"]:
@@ -121,6 +122,8 @@ def plain_forward(w: Dict[str, torch.Tensor], cfg: dict, ids: Sequence[int]) -> 
     for layer in range(cfg["n_layer"]):
         x = plain_block(x, w, f"blocks.{layer}.", cfg["n_head"], eps)
     x = plain_layer_norm(x, w["ln_f.weight"], w.get("ln_f.bias"), eps)
+    if rows is not None:
+        x = x[list(rows)]
     return x @ w["tok_emb.weight"].t()
 
 

@@ -306,7 +306,9 @@ def test_split_product_left_as_parts_of_a_pending_residual(rows, n_out, k_dim, b
 
 
 @pytest.mark.parametrize("rows,n_out,k_dim,bias", [(48, 1600, 6400, True), (64, 1600, 6400, False), (33, 768, 3072, True),
-                                                   (100, 512, 4096, True)])
+                                                   (100, 512, 4096, True), (129, 1600, 6400, True),
+                                                   (200, 1600, 6400, False), (256, 1600, 6400, True),
+                                                   (160, 768, 3072, True), (256, 768, 3072, False)])
 def test_tiled_split_left_as_parts_of_a_pending_residual(rows, n_out, k_dim, bias):
     """The tiled product's first kernel alone where it splits the inner size: its parts (the first
     carries the bias) add up to the plain product, to the very bits of the product that joins them

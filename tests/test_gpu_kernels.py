@@ -477,7 +477,10 @@ def test_linear_skinny_refuses_what_it_cannot_do():
 class PagedCase:
     """Random requests with part of their tokens already cached, laid out in scattered pages."""
 
-    def __init__(self, seq_lens, q_lens, h, hk, d, page, dtype, seed=0, poison=True):
+    def __init__(self, seq_lens, q_lens, h, hk, d, page, dtype, seed=0, poison=True, spikes=()):
+        """spikes: (request, query index within the step, key position, head): that query and that key
+        are made long and parallel, so that this one score stands out among hundreds and the query's
+        output is that key's value; a kernel that misses the key, or takes another for it, shows."""
         g = torch.Generator().manual_seed(seed)
         self.h, self.hk, self.d, self.page = h, hk, d, page
         self.seq_lens, self.q_lens = seq_lens, q_lens
@@ -486,6 +489,12 @@ class PagedCase:
         self.k = [rnd(g, s, hk, d, dtype=dtype) for s in seq_lens]
         self.v = [rnd(g, s, hk, d, dtype=dtype) for s in seq_lens]
         self.q = [rnd(g, ql, h, d, dtype=dtype) for ql in q_lens]
+        for r, qi, key, head in spikes:
+            assert key <= seq_lens[r] - q_lens[r] + qi, "a query sees no later key"
+            u = torch.randn(d, generator=g)
+            u = (3.0 * math.sqrt(d) * u / u.norm()).to(TDT[dtype])      # |u|^2 = 9 d: the score is 9 d * scale
+            self.q[r][qi, head] = u
+            self.k[r][key, head // (h // hk)] = u
         fill = float("nan") if poison else 0.0
         kp = torch.full((n_pages, hk, page, d), fill, dtype=TDT[dtype])
         vp = kp.clone()
@@ -572,6 +581,54 @@ def test_prefill_attention_with_many_tiles(d, window):
     assert kernels.prefill_attention_bf16(c.q_flat, out, c.kp, c.vp, c.bt, c.cu, c.sl, len(lens), max(c.q_lens),
                                           c.h, scale, window)
     helpers.assert_close(out, c.want(scale, window), "bfloat16", f"many tiles, head size {d}")
+
+
+LONG_PREFILL_CASES = {
+    # the benchmarked prefill step: two whole prompts of 1,024 tokens, 8 heads of 64 (256 query tiles:
+    # two wave groups split every 256 keys), and the same with more than 320 tiles (one wave group)
+    "2x1024-d64": dict(seq_lens=[1024, 1024], q_lens=[1024, 1024], h=8, hk=8, d=64, page=16),
+    "3x1024-d64": dict(seq_lens=[1024, 1000, 1024], q_lens=[1024, 1000, 1024], h=8, hk=8, d=64, page=16),
+    "1x1024-d128": dict(seq_lens=[1024], q_lens=[1024], h=4, hk=4, d=128, page=16),
+    "6x1024-d128": dict(seq_lens=[1024] * 6, q_lens=[1024] * 6, h=4, hk=2, d=128, page=32),
+    # portions of 64 to 512 tokens over 512 and 900 cached keys, few tiles and many
+    "portions-d64": dict(seq_lens=[576, 1024, 1024, 964], q_lens=[64, 124, 512, 64], h=8, hk=8, d=64, page=16),
+    "portions-d64-many": dict(seq_lens=[576, 1024, 1024, 964], q_lens=[64, 124, 512, 64], h=32, hk=8, d=64, page=16),
+    "portions-d128": dict(seq_lens=[1024, 612, 1000], q_lens=[512, 100, 100], h=4, hk=4, d=128, page=8),
+    "portions-d128-many": dict(seq_lens=[1024, 612, 1000], q_lens=[512, 100, 100], h=32, hk=4, d=128, page=8),
+}
+
+
+@pytest.mark.parametrize("name", sorted(LONG_PREFILL_CASES))
+def test_prefill_attention_at_the_benchmarked_lengths(name):
+    """The MFMA tile kernel with whole prompts of 1,024 tokens and with portions over 512 and 900
+    cached keys, head sizes 64 and 128, in both of its modes (two wave groups that split every 256
+    keys while the step has at most 320 query tiles, one wave group beyond), pages scattered over a
+    NaN-poisoned pool.  Random scores alone are nearly flat over so many keys: in every request a
+    few queries get one key that stands out (the first key, one a few blocks back, the last key of a
+    128-key block, the query's own), and the query's output must be that key's value."""
+    spec = LONG_PREFILL_CASES[name]
+    tiles = sum(-(-q // 64) for q in spec["q_lens"]) * spec["h"]
+    assert (tiles > 320) == (name.startswith(("3x", "6x")) or name.endswith("many")), tiles
+    spikes = []
+    for r, (s, ql) in enumerate(zip(spec["seq_lens"], spec["q_lens"])):
+        first = s - ql
+        for j, (qi, key) in enumerate([(ql - 1, 0), (ql - 1 - 7, max(first + ql - 8 - 300, 1)), (ql // 2, 127),
+                                       (ql // 3, first + ql // 3), (1, first + 1), (ql - 2, 383)]):
+            if key <= first + qi:
+                spikes.append((r, qi, key, (r + j) % spec["h"]))
+    assert len({(r, key) for r, _, key, _ in spikes}) == len({(r, qi) for r, qi, _, _ in spikes}) == len(spikes)
+    c = PagedCase(**spec, dtype="bfloat16", seed=len(name), spikes=spikes)
+    scale = 1.0 / math.sqrt(c.d)
+    out = torch.full((c.n, c.h * c.d), float("nan"), dtype=torch.bfloat16, device=DEV)
+    assert kernels.prefill_attention_bf16(c.q_flat, out, c.kp, c.vp, c.bt, c.cu, c.sl, len(c.seq_lens),
+                                          max(c.q_lens), c.h, scale, 0)
+    want = c.want(scale, 0)
+    helpers.assert_close(out, want, "bfloat16", name)
+    # the spiked queries really are decided by one key (so the comparison above pins the lookup)
+    offs = np.concatenate([[0], np.cumsum(c.q_lens)])
+    for r, qi, key, head in spikes:
+        row = want[offs[r] + qi, head * c.d:(head + 1) * c.d]
+        helpers.assert_close(row, c.v[r][key, head // (c.h // c.hk)].double(), "bfloat16", f"{name}: spike {r, qi, key}")
 
 
 @pytest.mark.parametrize("window", [0, 20])

@@ -687,3 +687,111 @@ def test_a_toy_arrangement_with_one_norm_and_two_mixers(dtype):
             done[i] += q
     for i in range(2):
         helpers.assert_close(torch.cat(got[i]), want[i], dtype, f"parallel block, request {i}")
+
+
+# ----------------------------------------------------------------------------- two parts of one kind in a row
+@register_arrangement("toy_twice")
+class ToyTwice(Arrangement):
+    """x += attention_a(norm_a(x)); x += attention_b(norm_b(x)); x += ff_a(norm_c(x)); x += ff_b(norm_d(x)):
+    two mixers of one kind and two feed-forwards of one kind follow each other, each reading the
+    residual as the one before left it (in a decode step of few rows: as sums still pending)."""
+
+    takes_pending_residual = True
+    graph_safe = True
+    plan_safe = True
+    roles = ("norm_a", "attention_a", "norm_b", "attention_b", "norm_c", "ff_a", "norm_d", "ff_b")
+
+    def __init__(self, width: int) -> None:
+        self.width = int(width)
+
+    def run(self, ctx, x, parts, bindings, position) -> None:
+        n = ctx.n_rows
+        for norm, mixer in (("norm_a", "attention_a"), ("norm_b", "attention_b")):
+            parts[mixer].forward_add(ctx, LazyNorm(parts[norm], x, n), x, bindings[mixer], position)
+        for norm, ff in (("norm_c", "ff_a"), ("norm_d", "ff_b")):
+            parts[ff].forward_add(ctx, LazyNorm(parts[norm], x, n), x)
+
+
+TW_C, TW_H, TW_D, TW_HID = 128, 4, 32, 192
+
+
+def _twice_spec():
+    a, b = (_attn_layer(i, TW_C, TW_H, TW_H, TW_D, 0, 1 / math.sqrt(TW_D), TW_HID, EPS) for i in (0, 1))
+    layer = LayerSpec(PartSpec("toy_twice", {"width": TW_C}),
+                      parts={"norm_a": ("norm", a.norm1), "attention_a": ("mixer", a.mixer),
+                             "norm_b": ("norm", b.norm1), "attention_b": ("mixer", b.mixer),
+                             "norm_c": ("norm", a.norm2), "ff_a": ("feed_forward", a.feed_forward),
+                             "norm_d": ("norm", b.norm2), "ff_b": ("feed_forward", b.feed_forward)})
+    return ModelSpec(width=TW_C, vocab_size=V,
+                     embedding=PartSpec("token_embedding", {"vocab_size": V, "width": TW_C}, {"weight": "emb.w"}),
+                     position=PartSpec("learned_absolute", {"max_positions": 50, "width": TW_C}, {"weight": "pos.w"}),
+                     layers=(layer,), order=(LayerRun(0), LayerRun(0)), final_norm=_norm("nf.", TW_C, EPS),
+                     head=PartSpec("linear_head", {"vocab_size": V, "width": TW_C, "tied": True}, {"weight": "emb.w"}),
+                     max_positions=50)
+
+
+def _plain_twice_model(w, ids):
+    x = P.plain_embed(torch.tensor(ids), w["emb.w"].double(), w["pos.w"].double())
+    for _ in range(2):
+        for p in ("L0.", "L1."):
+            a, _kv = _pl_attn(_pl_norm(x, w, p + "n1.", EPS), w, p, TW_H, TW_H, 1 / math.sqrt(TW_D), 0)
+            x = x + a
+        for p in ("L0.", "L1."):
+            x = x + _pl_mlp(_pl_norm(x, w, p + "n2.", EPS), w, p)
+    return _pl_norm(x, w, "nf.", EPS) @ w["emb.w"].double().t()
+
+
+@pytest.mark.parametrize("n_req", [1, 3, 40])
+def test_two_fused_parts_of_one_kind_in_a_row_keep_their_sums_apart(n_req):
+    """Decode steps of few rows through the fused kernels with two attention mixers and two
+    feed-forwards one behind the other: the second of a kind adds up the first one's pending sums
+    while its workgroups store their own, so the two must not share an array; the logits are the
+    plain model's, and the kernel wrapper refuses an output that is the pending sums' array."""
+    from mini_gpt_inference_amd.ops import kernels as K, residual as R
+
+    model = DecoderModel(_twice_spec())
+    assert model.graph_safe and model.plan_safe
+    weights = _random_weights(model, 33)
+    _bind(model, weights, "bfloat16")
+    rng = np.random.default_rng(n_req)
+    steps = 5
+    reqs = [rng.integers(0, V, int(rng.integers(1, 7)) + steps).tolist() for _ in range(n_req)]
+    want = [_plain_twice_model(weights, ids).numpy() for ids in reqs]
+    runner, cache = _runner(model, "bfloat16", num_pages=4 * n_req + 8, max_requests=n_req)
+    slots = [cache.acquire_slot() for _ in reqs]
+    heads = [len(r) - steps for r in reqs]
+    for s, r in zip(slots, reqs):
+        assert cache.reserve(s, len(r))
+    runner.step(slots, [0] * n_req, heads, sum((r[:h] for r, h in zip(reqs, heads)), []), [])
+    seen = []
+    launch = K.fused_attention_decode
+
+    def spy(pending, settled, *args, **kwargs):
+        out_partials = args[7]
+        seen.append((None if pending.partials is None else pending.partials.data_ptr(), out_partials.data_ptr()))
+        return launch(pending, settled, *args, **kwargs)
+
+    K.fused_attention_decode = spy
+    try:
+        for j in range(steps):
+            got = runner.step(slots, [h + j for h in heads], [1] * n_req, [r[h + j] for r, h in zip(reqs, heads)],
+                              list(range(n_req)))
+            ref = np.stack([wv[h + j] for wv, h in zip(want, heads)])
+            helpers.assert_close(got, ref, "bfloat16", f"{n_req} requests, decode step {j}")
+    finally:
+        K.fused_attention_decode = launch
+    assert seen, "the fused attention kernel did not run"
+    assert all(a != b for a, b in seen)
+    if n_req <= 3:      # one token a workgroup: the second mixer reads the first one's sums
+        assert any(a is not None for a, _ in seen)
+    # and the wrapper itself refuses the shared array
+    from mini_gpt_inference_amd.ops.linear import packed_weight
+
+    ff, norm = model.layers[0].parts["ff_a"], model.layers[0].parts["norm_c"]
+    n_parts = TW_HID // 64
+    x = torch.zeros(n_req, TW_C, device=DEV)
+    parts = torch.zeros(n_parts, n_req, TW_C, device=DEV)
+    with pytest.raises(K.KernelError, match="pending sums"):
+        K.fused_mlp_decode(R.PendingSums(x, parts, n_parts), torch.zeros_like(x), norm.weight, norm.bias, norm.eps,
+                           packed_weight(ff.fc_weight), ff.fc_bias, packed_weight(ff.proj_weight), ff.proj_bias,
+                           parts, n_req, TW_HID)

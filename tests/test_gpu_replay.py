@@ -385,10 +385,40 @@ def test_real_family_sizes_mixed_with_page_reuse(tmp_path_factory, shape, dtype)
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("n_req", [8, 17, 40, 64, 100, 128])
+@pytest.mark.parametrize("cut", ["whole", "halves"])
+def test_the_benchmarked_prefill_step(tmp_path_factory, dtype, cut):
+    """The prefill step that the benchmark times: two prompts of 1,024 tokens at the 50.9M model's
+    widths in one step (and the same prompts as two steps of 512 + 512 over the cache), logits at a
+    prompt's first, middle and last positions, against the plain implementation (the reference
+    compares a prompt's prefill logits with its oracle, tests/test_cache.py:30-49; a portion's queries
+    see the cached keys and their own up to themselves, src/minigpt_infer/batch.py:202-227)."""
+    folder, cfg, pcfg, w = _family_model(tmp_path_factory, "50M")
+    rng = np.random.default_rng(77)
+    prompts = [helpers.random_ids(rng, cfg.vocab_size, 1024) for _ in range(2)]
+    rep = TraceReplayer(folder, dtype, 2048, poison=True)
+    if cut == "whole":
+        steps = [([p for p in prompts], [0, 511, 1023])]
+    else:
+        steps = [([p[:512] for p in prompts], [0, 511]), ([p[512:] for p in prompts], [0, 511])]
+    got, positions, base = [], [], 0
+    for i, (portions, rows) in enumerate(steps):
+        out = rep.run_step({"step": i, "entries": [{"id": f"p{j}", "tokens": t, "want": rows}
+                                                   for j, t in enumerate(portions)], "end": []})
+        got.append(out.clone().view(2, len(rows), -1))
+        positions += [base + r for r in rows]
+        base += len(portions[0])
+    got = torch.cat(got, dim=1)
+    for j, prompt in enumerate(prompts):
+        want = P.plain_forward(w, pcfg, prompt, rows=positions)
+        helpers.assert_close(got[j], want, dtype, f"prompt {j}, {cut}, positions {positions}")
+    assert rep.cache.num_free_pages() == 0, "the pool was meant to be exactly the two prompts"
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("n_req", [8, 17, 40, 64, 100, 128, 200, 256])
 @pytest.mark.parametrize("shape", ["small", "xl", "50M"])
 def test_real_family_sizes_many_requests_decoding(tmp_path_factory, shape, dtype, n_req):
-    """Decode steps of 8 to 128 requests at the real widths, as logits: the decode products
+    """Decode steps of 8 to 256 requests at the real widths, as logits: the decode products
     change kernels with the rows and the matrix's size (rows dealt out in groups, the inner size
     split over workgroups and its sums left pending, the hand-over to the tiled kernel, the fused
     kernels with one, two and four tokens a workgroup).
