@@ -1,9 +1,18 @@
-"""One registry from an architecture's name to how its model is built."""
+"""One registry from an architecture's name to how its model is built.
+
+An architecture is a module under models/ that calls register_architecture once.  Every module
+found there is imported when a name is first looked up, so adding an architecture is adding a
+file; nothing here names one.  What the framework asks of an architecture's typed configuration
+is little: an attribute `architecture` that holds the registered name (config.json carries it
+under the same key), and the two conversions below.
+"""
 
 from __future__ import annotations
 
+import importlib
+import pkgutil
 from dataclasses import dataclass
-from typing import Any, Callable, Dict, List, Mapping, Tuple
+from typing import Any, Callable, Dict, List, Mapping, Set, Tuple
 
 
 @dataclass(frozen=True)
@@ -13,9 +22,12 @@ class Architecture:
     model_spec: Callable[[Any], Any]                        # typed config -> parts.model.ModelSpec
     init_plan: Callable[[Any], List[Tuple[str, Tuple[int, ...], str, float]]]
     # init_plan: (tensor name, shape, rule, scale) in the order tensors are drawn in random-weights mode
+    config_to_json: Callable[[Any], Mapping[str, Any]] = lambda config: config.to_json_dict()
+    # typed config -> the dict that config.json holds (flat; carries "architecture": name)
 
 
 _ARCHITECTURES: Dict[str, Architecture] = {}
+_SCANNED: Set[str] = set()      # modules under models/ imported so far
 
 
 def register_architecture(arch: Architecture) -> None:
@@ -25,14 +37,15 @@ def register_architecture(arch: Architecture) -> None:
 
 
 def get_architecture(name: str) -> Architecture:
-    _load_builtin()
+    if name not in _ARCHITECTURES:
+        _load_models()
     if name not in _ARCHITECTURES:
         raise KeyError(f"unknown architecture {name!r}; registered: {sorted(_ARCHITECTURES)}")
     return _ARCHITECTURES[name]
 
 
 def architecture_names() -> List[str]:
-    _load_builtin()
+    _load_models()
     return sorted(_ARCHITECTURES)
 
 
@@ -44,5 +57,22 @@ def architecture_of(raw_config: Mapping[str, Any]) -> Architecture:
     return get_architecture(name)
 
 
-def _load_builtin() -> None:
-    from ..models import gpt2_mini  # noqa: F401  (registers itself)
+def architecture_of_config(config: Any) -> Architecture:
+    """The architecture of a typed configuration: the one its `architecture` attribute names."""
+    name = getattr(config, "architecture", None)
+    if not isinstance(name, str):
+        raise TypeError(f"{type(config).__name__} has no attribute 'architecture' that names its architecture")
+    return get_architecture(name)
+
+
+def _load_models() -> None:
+    """Imports every module of the models package that has not been imported yet (each registers
+    itself).  The package's search path is read anew at every call: a module that appears later, or
+    a folder appended to models.__path__, is found at the next lookup of an unknown name."""
+    from .. import models
+
+    for info in pkgutil.iter_modules(models.__path__):
+        if info.name.startswith("_") or info.name in _SCANNED:
+            continue
+        _SCANNED.add(info.name)
+        importlib.import_module(f"{models.__name__}.{info.name}")

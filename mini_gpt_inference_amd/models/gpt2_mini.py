@@ -12,15 +12,78 @@ embedding with no bias (model.py:128-130).
 from __future__ import annotations
 
 import math
-from typing import List, Tuple
+from dataclasses import asdict, dataclass, fields
+from typing import Any, List, Mapping, Tuple
 
-from ..config.model_config import GPTConfig
+from ..config.model_config import ConfigError
 from ..config.registry import Architecture, register_architecture
 from ..parts.base import PartSpec
 from ..parts.model import LayerRun, LayerSpec, ModelSpec
 
 NAME = "gpt2-mini"
 MLP_RATIO = 4   # src/minigpt_infer/model.py:96
+
+# Keys a config.json may carry that the engine reads past: the reference forces dropout to 0 at
+# inference (src/minigpt_infer/loader.py:58).
+_IGNORED_KEYS = {"dropout", "model_type", "torch_dtype"}
+
+
+@dataclass(frozen=True)
+class GPTConfig:
+    """The architecture's typed configuration, read from its own config.json keys: the fields of the
+    reference's GPTConfig dataclass (src/minigpt_infer/config.py:10-18; model.py:118-130).
+    layer_norm_eps is added because the reference leaves it at nn.LayerNorm's default
+    (model.py:107,109,127) and a model folder has to be able to say otherwise."""
+
+    architecture: str
+    n_layer: int
+    n_embd: int
+    n_head: int
+    vocab_size: int
+    block_size: int          # rows of the learned position table = most positions
+    bias: bool               # biases on every Linear and every LayerNorm
+    layer_norm_eps: float = 1e-5
+
+    def __post_init__(self) -> None:
+        for name in ("n_layer", "n_embd", "n_head", "vocab_size", "block_size"):
+            value = getattr(self, name)
+            if not isinstance(value, int) or isinstance(value, bool) or value <= 0:
+                raise ConfigError(f"{name} must be a positive integer, got {value!r}")
+        if not isinstance(self.bias, bool):
+            raise ConfigError(f"bias must be true or false, got {self.bias!r}")
+        if not (isinstance(self.layer_norm_eps, float) and self.layer_norm_eps > 0.0):
+            raise ConfigError(f"layer_norm_eps must be a positive float, got {self.layer_norm_eps!r}")
+        # src/minigpt_infer/model.py:39
+        if self.n_embd % self.n_head != 0:
+            raise ConfigError(
+                f"n_embd ({self.n_embd}) is not divisible by n_head ({self.n_head})"
+            )
+
+    @property
+    def head_dim(self) -> int:
+        return self.n_embd // self.n_head
+
+    def to_json_dict(self) -> dict[str, Any]:
+        return asdict(self)
+
+    @classmethod
+    def from_json_dict(cls, raw: Mapping[str, Any]) -> "GPTConfig":
+        known = {f.name for f in fields(cls)}
+        data = dict(raw)
+        if "architecture" not in data and "model_type" in data:
+            data["architecture"] = data["model_type"]
+        unknown = sorted(k for k in data if k not in known and k not in _IGNORED_KEYS
+                         and not k.startswith("_"))
+        if unknown:
+            raise ConfigError(f"config.json has keys this architecture does not know: {unknown}")
+        required = [f.name for f in fields(cls) if f.name != "layer_norm_eps"]
+        missing = [k for k in required if k not in data]
+        if missing:
+            raise ConfigError(f"config.json lacks required keys: {missing}")
+        kwargs = {k: data[k] for k in known if k in data}
+        if "layer_norm_eps" in kwargs:
+            kwargs["layer_norm_eps"] = float(kwargs["layer_norm_eps"])
+        return cls(**kwargs)
 
 
 def _w(prefix: str, has_bias: bool, /, **names: str) -> dict:
@@ -103,4 +166,4 @@ def init_plan(cfg: GPTConfig) -> List[Tuple[str, Tuple[int, ...], str, float]]:
     return plan
 
 
-register_architecture(Architecture(NAME, GPTConfig.from_json_dict, model_spec, init_plan))
+register_architecture(Architecture(NAME, GPTConfig.from_json_dict, model_spec, init_plan, GPTConfig.to_json_dict))

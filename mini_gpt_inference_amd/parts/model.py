@@ -104,6 +104,49 @@ class CacheLayout:
         return [next(iter(b.values())) if len(b) == 1 else None for b in self.run_bindings]
 
 
+@dataclass(frozen=True)
+class KVRun:
+    """One mixer of one run that reads keys and values."""
+    n_head: int
+    n_kv_head: int
+    head_dim: int
+    window: int
+
+
+@dataclass(frozen=True)
+class ModelCost:
+    """What a step of the model has to read and to compute, taken from its parts and its order (for
+    measurements against the machine's peaks; a dense model: every token goes through every matrix)."""
+    whole_tensor_bytes: int       # tensors that a step reads whole (matrices, gains, biases; a table only where a
+                                  # part also multiplies by it, as a tied head does), each once
+    table_row_bytes: int          # bytes a token reads from the tables that are looked up by row only
+    run_matrix_elements: int      # matrix elements a token goes through in the layers, over all runs of the order
+    head_matrix_elements: int     # matrix elements a wanted logit row goes through behind the last run
+    kv_runs: Tuple[KVRun, ...]    # every (run, mixer) that reads keys and values, its own cache or another run's
+
+    def step_read_bytes(self, n_tokens: int, context_lens, cache_itemsize: int) -> float:
+        """Bytes that a step of n_tokens single tokens has to read when request i has context_lens[i]
+        keys to look at (its own included): every whole tensor once, the tokens' table rows, and
+        for every run that attends the keys and values in its reach."""
+        kv = 0.0
+        for run in self.kv_runs:
+            for c in context_lens:
+                reach = min(c, run.window) if run.window else c
+                kv += reach * 2 * run.n_kv_head * run.head_dim * cache_itemsize
+        return self.whole_tensor_bytes + n_tokens * self.table_row_bytes + kv
+
+    def prompt_flops(self, prompt_lens, n_logit_rows: int) -> float:
+        """Multiply-adds times two of whole prompts in one step: the matrices for every token, causal
+        attention (scores and weighted values for the keys a query sees), the head for the wanted rows."""
+        n = sum(prompt_lens)
+        flops = 2.0 * n * self.run_matrix_elements + 2.0 * n_logit_rows * self.head_matrix_elements
+        for run in self.kv_runs:
+            for t in prompt_lens:
+                seen = sum(min(i + 1, run.window) if run.window else i + 1 for i in range(t))
+                flops += 4.0 * seen * run.n_head * run.head_dim
+        return flops
+
+
 class _Layer:
     """The built parts of a layer, by role (also as attributes)."""
 
@@ -184,6 +227,41 @@ class DecoderModel:
             loaded += tensor.numel() * tensor.element_size()
             derived += derived_bytes(tensor)
         return loaded, derived
+
+    def cost(self) -> ModelCost:
+        """The model's bytes and multiply-adds per step, from the bound tensors and the order of runs."""
+        bound = getattr(self, "_bound", None)
+        if bound is None:
+            raise RuntimeError("cost() needs the model's tensors (bind)")
+        whole, by_row = set(), set()
+        for part, spec in self._named_parts():
+            for local, req in part.weight_requests().items():
+                (by_row if req.role == "table" else whole).add(spec.weights[local])
+        by_row -= whole
+        size = lambda name: bound[name].numel() * bound[name].element_size()
+        row_bytes = sum(size(name) // bound[name].shape[0] for name in by_row)
+
+        def matrices(part: Part) -> int:
+            total = 0
+            for req in part.weight_requests().values():
+                if req.role == "matrix":
+                    n = 1
+                    for dim in req.shape:
+                        n *= dim
+                    total += n
+            return total
+
+        run_elements, kv_runs = 0, []
+        for run in self.spec.order:
+            layer = self.layers[run.layer]
+            for part in layer.parts.values():
+                run_elements += matrices(part)
+                need = part.cache_need() if hasattr(part, "cache_need") else None
+                if isinstance(need, KVNeed):
+                    kv_runs.append(KVRun(int(getattr(part, "n_head", need.n_kv_head)), need.n_kv_head,
+                                         need.head_dim, need.window))
+        return ModelCost(sum(size(name) for name in whole), row_bytes, run_elements, matrices(self.head),
+                         tuple(kv_runs))
 
     # ------------------------------------------------------------------ cache
     def _plan_cache(self) -> CacheLayout:

@@ -16,14 +16,14 @@ import torch
 from safetensors.torch import save_file
 
 from ..config.model_config import write_config_json
-from ..config.registry import get_architecture
+from ..config.registry import architecture_of_config
 from .loader import WEIGHTS_FILE
 
 
 def random_tensors(config, seed: int, dtype: torch.dtype = torch.bfloat16, std_scale: float = 1.0
                    ) -> Dict[str, torch.Tensor]:
     """std_scale multiplies every standard deviation of the plan (gains stay centred on one)."""
-    arch = get_architecture(config.architecture)
+    arch = architecture_of_config(config)
     gen = torch.Generator(device="cpu")
     gen.manual_seed(int(seed))
     tensors: Dict[str, torch.Tensor] = {}
