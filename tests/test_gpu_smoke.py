@@ -40,7 +40,7 @@ def test_bench_prints_one_record_with_the_agreed_fields():
     came from a graph."""
     import json
     proc = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--steps", "20", "--warmup", "5",
-                           "--layers", "2", "--no-extras"], capture_output=True, text=True, timeout=300)
+                           "--layers", "2", "--no-extras", "--blocks", "13"], capture_output=True, text=True, timeout=300)
     assert proc.returncode == 0, proc.stderr[-2000:]
     lines = [line for line in proc.stdout.splitlines() if line.startswith("{")]
     assert len(lines) == 1
@@ -49,6 +49,9 @@ def test_bench_prints_one_record_with_the_agreed_fields():
                 "vs_baseline", "dtype", "data", "config", "roofline"):
         assert key in rec, key
     assert rec["n_gpus"] == 1 and rec["steps"] == 20 and rec["warmup"] == 5 and rec["value"] > 0
+    # 256 generated tokens hold 12 blocks of 20 steps behind 5 of warm-up: the 13th block needs new requests
+    assert rec["blocks"] == 24 and rec["iqr_ms"] >= 0 and rec["config"]["generated"] == 256
+    assert 128 + 5 + 1 < rec["config"]["mean_context"] < 128 + 256
     assert rec["config"]["hip_graph"] is True and 0 < rec["kernels_per_step"] < 40
     assert rec["config"]["n_layer"] == 2 and rec["config"]["n_layer_full"] == 8      # fewer layers are named
     assert len(rec["config"]) <= 20 and not any(isinstance(v, (dict, list)) for v in rec["config"].values())
