@@ -99,7 +99,6 @@ def decode_run(args, batch, steps, warmup, dtype, min_blocks):
     rng = np.random.default_rng(0)
     sched = engine.scheduler
     blocks, contexts, stretches_all = [], [], []
-    captures = None
 
     def run_decode_steps(n):
         """engine.step() until exactly n more decode steps have run (a call may run a burst of them)."""
@@ -126,7 +125,6 @@ def decode_run(args, batch, steps, warmup, dtype, min_blocks):
         assert per_round >= 1
         torch.cuda.synchronize()
         before = engine.stats()
-        captures = before["graph_captures"] if captures is None else captures
         for _ in range(per_round):
             engine.stretch_times = stretches = []
             t0 = time.perf_counter()
@@ -140,7 +138,7 @@ def decode_run(args, batch, steps, warmup, dtype, min_blocks):
             done += steps
             stretches_all += [(n, t1 - t_prev) for (_, t_prev), (n, t1) in zip(stretches, stretches[1:])]
         after = engine.stats()
-        assert after["graph_captures"] == captures, "a HIP graph was recorded inside the timed steps"
+        assert after["graph_captures"] == before["graph_captures"], "a HIP graph was recorded inside the timed steps"
         if not args.no_graph:
             assert after["graph_steps"] - before["graph_steps"] == per_round * steps, \
                 "a timed step did not come from a graph"
