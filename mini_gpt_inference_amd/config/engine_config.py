@@ -40,6 +40,10 @@ class EngineConfig:
                                      # device is at work
     decode_ahead: bool = True        # before the host waits for a chain's last tokens it plans and enqueues
                                      # the next chain, whose tokens the next step() call returns
+    derived_weight_bytes: Optional[int] = None   # most device memory for the copies of matrices that the decode
+                                     # kernels make at first use (packed for their loads, folded with a
+                                     # LayerNorm: up to 1.5 times the weights); None = no bound, 0 = no copies:
+                                     # the decode steps then read the matrices as loaded, more slowly
     seed: int = 0                    # engine-wide sampler seed
     real_vocab_size: Optional[int] = None  # ids at or above it are never sampled
                                            # (src/minigpt_infer/tokenizer.py:37-46)
@@ -53,6 +57,8 @@ class EngineConfig:
             raise ValueError("max_num_batched_tokens must be positive")
         if self.decode_burst < 1 or self.decode_chain < 1:
             raise ValueError("decode_burst and decode_chain must be at least 1")
+        if self.derived_weight_bytes is not None and self.derived_weight_bytes < 0:
+            raise ValueError("derived_weight_bytes must be >= 0")
         if self.prefill_chunk < 0:
             raise ValueError("prefill_chunk must be >= 0")
         if self.evict not in ("newest", "newest_other"):

@@ -31,26 +31,6 @@ __device__ __forceinline__ void fd_barrier() {
   asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
 }
 
-#ifdef FD_TRACE
-// time stamps (100 MHz) of the first workgroup's first thread, for measurements of where a kernel's time goes
-__device__ unsigned long long fd_trace_buf[64];
-#define FD_STAMP(k)                                                                  \
-  do {                                                                               \
-    if (blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x == 0) fd_trace_buf[k] = wall_clock64(); \
-  } while (0)
-// a stamp once the value v has arrived in its register
-#define FD_STAMP_AFTER(k, v)              \
-  do {                                    \
-    asm volatile("" ::"v"(v) : "memory"); \
-    FD_STAMP(k);                          \
-  } while (0)
-extern "C" int mgpt_fd_trace(unsigned long long* host) {
-  return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(fd_trace_buf), sizeof(fd_trace_buf));
-}
-#else
-#define FD_STAMP(k)
-#define FD_STAMP_AFTER(k, v)
-#endif
 
 template <int CTRL>
 __device__ __forceinline__ float fd_dpp(float v) {
@@ -265,7 +245,6 @@ __global__ __launch_bounds__(FUSED_THREADS) void fused_attention_decode_kernel(F
   const int C = a.width, KS = C >> 5, V = C >> 2;
   const int ltok = TK == 1 ? 0 : lrow % TK;  // the token whose column of an MFMA this lane holds
 
-  FD_STAMP(0);
   // ---- The prologue.  A compute unit issues a wave's 16-byte loads at about a kilobyte every
   // twelve clocks, and a barrier lets a wave pass only when every other wave has issued what
   // stands before it: only a quarter of the weights' loads stand before the barrier at which the
@@ -397,7 +376,6 @@ __global__ __launch_bounds__(FUSED_THREADS) void fused_attention_decode_kernel(F
     if (gq < TK) reinterpret_cast<uint2*>(act_s + gq * FUSED_MAX_WIDTH)[vq] = normed4;
     if (gq == 2 && proj_bias) reinterpret_cast<float4*>(bproj_s)[vq] = gb4;
   } else {
-    FD_STAMP_AFTER(16, piece[0].x);
 
     // ---- the residual rows' sums: every group of threads its parts, then a wave per row all groups
 #pragma unroll
@@ -410,7 +388,6 @@ __global__ __launch_bounds__(FUSED_THREADS) void fused_attention_decode_kernel(F
     }
     if (gq < 3) reinterpret_cast<float4*>(gq == 0 ? gain_s : gq == 1 ? beta_s : bproj_s)[vq] = gb4;
     fd_barrier();
-    FD_STAMP(17);
     // every wave sends for the rest of its weights and for its keys and values; then the first waves
     // norm a row each (LDS and arithmetic only) while the others wait at the next barrier
     FA_LOAD_W(1)
@@ -471,7 +448,6 @@ __global__ __launch_bounds__(FUSED_THREADS) void fused_attention_decode_kernel(F
   if (NORMED) FA_LOAD_KV
 #undef FA_LOAD_W
 #undef FA_LOAD_KV
-  FD_STAMP(1);
 
   // ---- q, k, v of this head: every wave a stretch of k over all the row tiles; the waves' sums
   // meet in LDS (column c of the MFMA's output holds token c mod TK: the lanes of the first TK columns speak)
@@ -520,7 +496,6 @@ __global__ __launch_bounds__(FUSED_THREADS) void fused_attention_decode_kernel(F
     for (int i = 0; i < NK2; ++i) w2[j][i] = fd_packed(a.wproj, tile < n_tiles2 ? tile : 0, KS2, ks_b + i, lane);
   }
   fd_barrier();
-  FD_STAMP(2);
   if (qt < TK) {
     float v = 0.f;
 #pragma unroll
@@ -544,7 +519,6 @@ __global__ __launch_bounds__(FUSED_THREADS) void fused_attention_decode_kernel(F
     }
   }
   fd_barrier();  // also: the waves' sums are read, their place takes attention's partial results
-  FD_STAMP(3);
 
   // ---- attention: each token's waves over the keys before the token's own (from the pages); the
   // token's first wave its own as well (from LDS)
@@ -645,7 +619,6 @@ __global__ __launch_bounds__(FUSED_THREADS) void fused_attention_decode_kernel(F
       }
     }
   }
-  FD_STAMP(4);
 
   // ---- merge: first across the key groups of a wave (lanes that differ above the LPK lanes of a
   // key: the maximum is the wave's already, so the sums simply add), then across a token's waves in LDS
@@ -679,7 +652,6 @@ __global__ __launch_bounds__(FUSED_THREADS) void fused_attention_decode_kernel(F
     y_s[tid] = float_to_bf16(av / lt);
   }
   fd_barrier();
-  FD_STAMP(5);
 
   // ---- this head's share of the output projection: row tiles dealt out to the waves
   {
@@ -720,7 +692,6 @@ __global__ __launch_bounds__(FUSED_THREADS) void fused_attention_decode_kernel(F
       }
     }
   }
-  FD_STAMP(6);
 }
 
 struct FusedMlpArgs {
@@ -767,7 +738,6 @@ __global__ __launch_bounds__(FUSED_THREADS) void fused_mlp_decode_kernel(FusedMl
   const int xs_bytes = FUSED_WAVES * C * 4 > FM_RED_BYTES ? FUSED_WAVES * C * 4 : FM_RED_BYTES;
   bf16_t* act_s = reinterpret_cast<bf16_t*>(smem + xs_bytes);
 
-  FD_STAMP(8);
   // ---- loads in the order in which their data is needed: this wave's share of a residual row,
   // then the weights of both products (the second product's behind the barrier that the rows'
   // sums need: a wave passes a barrier only when all others have issued what stands before it)
@@ -873,7 +843,6 @@ __global__ __launch_bounds__(FUSED_THREADS) void fused_mlp_decode_kernel(FusedMl
     }
   }
   fd_barrier();
-  FD_STAMP(9);
 
   // ---- first product: a wave one row tile of the slice over its stretch of k
   // (a column of the MFMA beyond the workgroup's rows repeats its first row and is never stored)
@@ -895,7 +864,6 @@ __global__ __launch_bounds__(FUSED_THREADS) void fused_mlp_decode_kernel(FusedMl
   // (the rows' sums were read before the last barrier: their place takes the waves' sums of the product)
   *reinterpret_cast<float4*>(red + ((kq * FM_TS + tt) * 64 + lane) * 4) = make_float4(acc[0], acc[1], acc[2], acc[3]);
   fd_barrier();
-  FD_STAMP(10);
   {
     // a thread one hidden unit of one row: the waves' sums in the order of k, bias, GELU
     const int t2 = tid >> 8, ln = (tid >> 2) & 63, i4 = tid & 3;
@@ -906,7 +874,6 @@ __global__ __launch_bounds__(FUSED_THREADS) void fused_mlp_decode_kernel(FusedMl
     g_s[(ln & 15) * FM_GS + o] = float_to_bf16(gelu_tanh_fast(v + fc_bias));
   }
   fd_barrier();
-  FD_STAMP(11);
 
   // ---- the slice's share of the second product: row tiles dealt out to the waves
   bf16x8_t yb[FM_NK2];
@@ -939,7 +906,6 @@ __global__ __launch_bounds__(FUSED_THREADS) void fused_mlp_decode_kernel(FusedMl
       for (int i = 0; i < FM_NK2; ++i) w2[q][i] = fd_packed(a.wproj, tile < n_tiles2 ? tile : 0, KS2, j * FM_NK2 + i, lane);
     }
   }
-  FD_STAMP(12);
 }
 
 // out[i] = LayerNorm(row rows[i] (or i) of a residual that is still a sum); a workgroup a row

@@ -41,10 +41,12 @@ __global__ __launch_bounds__(256) void linear_generic_kernel(
   const WT* wp = W + (long)wrow * k_dim + lk;
 
   for (int k0 = 0; k0 < k_dim; k0 += BK) {
+    // an inner size that is no multiple of the stage ends in zeros: fma(0, 0, acc) leaves acc as it is
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      As[lk + i][lrow] = a_ok ? to_float<AT>(ap[k0 + i]) : 0.f;
-      Ws[lk + i][lrow] = w_ok ? to_float<WT>(wp[k0 + i]) : 0.f;
+      const bool k_ok = k0 + lk + i < k_dim;
+      As[lk + i][lrow] = (a_ok && k_ok) ? to_float<AT>(ap[k0 + i]) : 0.f;
+      Ws[lk + i][lrow] = (w_ok && k_ok) ? to_float<WT>(wp[k0 + i]) : 0.f;
     }
     __syncthreads();
 #pragma unroll
@@ -107,10 +109,10 @@ __global__ __launch_bounds__(256) void linear_generic_rows_kernel(
   const WT* wp = W + (long)(col0 + r) * k_dim + sk;
   float acc = 0.f;
   for (int k0 = 0; k0 < k_dim; k0 += ROWS_BK) {
-    const int kmax = k_dim - k0 < ROWS_BK ? k_dim - k0 : ROWS_BK;   // a multiple of 16, so of 4
-    const bool k_ok = sk < kmax;
+    const int kmax = k_dim - k0 < ROWS_BK ? k_dim - k0 : ROWS_BK;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
+      const bool k_ok = sk + i < kmax;
       As[r][sk + i] = (a_ok && k_ok) ? to_float<AT>(ap[k0 + i]) : 0.f;
       Ws[r][sk + i] = (w_ok && k_ok) ? to_float<WT>(wp[k0 + i]) : 0.f;
     }
@@ -172,13 +174,13 @@ static int launch_out(const void* A, long lda, const void* W, const float* bias,
 }
 
 // A: [n_rows, k_dim] with row stride lda; W: [n_out, k_dim] dense; out: [n_rows, n_out] with row
-// stride ldo.  k_dim must be a multiple of 16.
+// stride ldo.  Any inner size.
 extern "C" int mgpt_linear_generic(const void* A, int a_dtype, long lda, const void* W, int w_dtype,
                                    const float* bias, void* out, int out_dtype, long ldo, int n_rows,
                                    int n_out, int k_dim, int epilogue, hipStream_t stream) {
   if (n_rows == 0 || n_out == 0) return MGPT_OK;
   if (!A || !W || !out) return MGPT_ERR_NULL;
-  if (n_rows < 0 || n_out < 0 || k_dim <= 0 || (k_dim % BK) != 0 || lda < k_dim || ldo < n_out)
+  if (n_rows < 0 || n_out < 0 || k_dim <= 0 || lda < k_dim || ldo < n_out)
     return MGPT_ERR_BAD_SHAPE;
   if ((n_rows + TILE - 1) / TILE > 65535) return MGPT_ERR_TOO_LARGE;
   if (a_dtype == MGPT_F32 && w_dtype == MGPT_F32)

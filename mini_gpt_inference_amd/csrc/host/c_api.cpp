@@ -284,4 +284,7 @@ int mgpt_sched_copy_output(void* sv, int id, int* out, int cap) {
 
 void mgpt_sched_forget_finished(void* sv) { static_cast<Scheduler*>(sv)->forget_finished(); }
 
+// request records that the scheduler holds now (waiting, running, and finished ones not yet forgotten)
+int mgpt_sched_num_records(void* sv) { return static_cast<Scheduler*>(sv)->num_records(); }
+
 }  // extern "C"

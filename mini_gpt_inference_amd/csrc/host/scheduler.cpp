@@ -37,16 +37,25 @@ int Scheduler::add_request(const int* prompt, int n_prompt, int max_tokens, int 
     if (cache_->pages_needed(g, n_prompt + max_tokens - 1) > cache_->group(g).num_pages)
       return ERR_NEVER_FITS;
   auto r = std::make_unique<Request>();
-  r->id = (int)requests_.size();
+  // the id of a forgotten request is used again, so that a scheduler that serves for a long time
+  // holds as many records as it has live requests
+  if (!free_ids_.empty()) {
+    r->id = free_ids_.back();
+    free_ids_.pop_back();
+  } else {
+    r->id = (int)requests_.size();
+    requests_.emplace_back();
+  }
   r->prompt.assign(prompt, prompt + n_prompt);
   r->max_tokens = max_tokens;
   r->eot = eot;
   r->temperature = temperature;
   r->top_k = top_k;
   r->top_p = top_p;
-  r->seed = has_seed ? seed : (uint64_t)r->id;
+  r->seed = has_seed ? seed : num_added_;     // a stream of its own per arrival
+  ++num_added_;
   const int id = r->id;
-  requests_.push_back(std::move(r));
+  requests_[id] = std::move(r);
   waiting_.push_back(id);
   return id;
 }
@@ -268,12 +277,12 @@ const std::vector<StepOutput>& Scheduler::commit_burst(const int* tokens, int k,
 }
 
 void Scheduler::forget_finished() {
+  // not while a burst's tokens are still to come: its entries name requests that may have ended
+  if (pending_ > 0) return;
   for (auto& r : requests_)
     if (r && r->status == FINISHED) {
-      r->prompt.clear();
-      r->prompt.shrink_to_fit();
-      r->output.clear();
-      r->output.shrink_to_fit();
+      free_ids_.push_back(r->id);
+      r.reset();
     }
 }
 

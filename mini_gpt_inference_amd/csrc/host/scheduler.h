@@ -116,8 +116,9 @@ class Scheduler {
   long num_prompt_tokens = 0;  // scheduled as part of a portion of more than one token or an unfinished prompt
   long num_decode_tokens = 0;
 
-  // drops the records of finished requests (their ids are not reused)
+  // drops the records of finished requests; their ids are given to later requests
   void forget_finished();
+  int num_records() const { return (int)requests_.size() - (int)free_ids_.size(); }
 
  private:
   Request* get(int id);
@@ -129,7 +130,9 @@ class Scheduler {
 
   CacheManager* cache_;
   SchedulerConfig cfg_;
-  std::vector<std::unique_ptr<Request>> requests_;  // index = id
+  std::vector<std::unique_ptr<Request>> requests_;  // index = id; null = forgotten
+  std::vector<int> free_ids_;                        // ids of forgotten requests
+  uint64_t num_added_ = 0;
   std::deque<int> waiting_;
   std::vector<int> running_;  // admission order
   std::vector<StepEntry> entries_;

@@ -174,7 +174,8 @@ class LLMEngine:
         self.store = KVStore(layout, geometry, engine_config.max_batch_size, self.dtype, self.device)
         max_positions = model.spec.max_positions
         self.runner = ModelRunner(model, self.cache, self.store, self.dtype, self.device, max_positions,
-                                  graph_steps=engine_config.use_graph)
+                                  graph_steps=engine_config.use_graph,
+                                  derived_weight_bytes=engine_config.derived_weight_bytes)
         self.scheduler = Scheduler(
             self.cache, engine_config.max_batch_size,
             max(engine_config.max_num_batched_tokens, engine_config.max_batch_size),

@@ -186,4 +186,11 @@ class Scheduler:
         return buf[:got].tolist()
 
     def forget_finished(self) -> None:
+        """Drops the records of finished requests (not while tokens of planned decode steps are still
+        to be handed in); their ids go to later requests."""
         self._lib.mgpt_sched_forget_finished(self._h)
+
+    @property
+    def num_records(self) -> int:
+        """Request records held now: waiting, running, and finished ones not yet forgotten."""
+        return int(self._lib.mgpt_sched_num_records(self._h))

@@ -19,6 +19,7 @@ import torch
 from ..cache.kv_store import KVStore
 from ..cache.manager import CacheManager
 from ..ops import kernels, library
+from ..ops.linear import CopyBudget
 from ..ops.plan import LaunchPlan
 from ..parts.base import GroupView, StepContext, Workspace, WorkspaceFrozen
 from ..parts.model import DecoderModel
@@ -158,8 +159,10 @@ class ModelRunner:
     CAPTURE_AT = 3     # a shape is captured when it comes for the third time (capturing costs a step's launches again)
 
     def __init__(self, model: DecoderModel, cache: CacheManager, store: KVStore, dtype: torch.dtype,
-                 device: torch.device, max_positions: Optional[int], graph_steps: bool = True) -> None:
+                 device: torch.device, max_positions: Optional[int], graph_steps: bool = True,
+                 derived_weight_bytes: Optional[int] = None) -> None:
         self.model, self.cache, self.store = model, cache, store
+        self.copy_budget = CopyBudget(derived_weight_bytes)     # what copies of matrices made at first use may take
         self.dtype, self.device = dtype, device
         self.exact = dtype == torch.float32
         self.max_positions = max_positions
@@ -168,7 +171,7 @@ class ModelRunner:
         self.graph_steps = graph_steps and device.type == "cuda" and model.graph_safe
         self.plan_steps = device.type == "cuda" and model.plan_safe      # launches recorded and made again from C++
         self.num_planned_steps = 0        # steps whose launches came from a recorded plan
-        self._step_graphs: Dict[Tuple, _StepGraph] = {}     # by exact shape; emptied when it has MAX_STEP_GRAPHS
+        self._step_graphs: Dict[Tuple, _StepGraph] = {}     # by exact shape, least recently used first; at most MAX_STEP_GRAPHS
         self._bucket_graphs: Dict[Tuple, _StepGraph] = {}   # by capacities: as many as there are buckets
         self.num_replayed_steps = 0
         self.num_graph_captures = 0       # HIP graphs recorded so far, decode steps' and other steps'
@@ -267,7 +270,7 @@ class ModelRunner:
             decode_only=False if bucket else shape.max_q_len <= 1,
             host_q_lens=None if bucket else shape.q_lens, host_ctx_lens=None if bucket else shape.ctx_lens,
             host_state_slots=None if bucket else shape.slots, exact=self.exact, padded=padded,
-            lead_cap=lead_cap or 0)
+            lead_cap=lead_cap or 0, copy_budget=self.copy_budget)
 
     def run(self, arena: StepArena, shape: StepShape) -> torch.Tensor:
         """Uploads the arena and runs the model.  Returns float32 logits [n_logits, vocab] (in the
@@ -328,11 +331,13 @@ class ModelRunner:
         return logits
 
     def _entry(self, key: Tuple) -> _StepGraph:
-        entry = self._step_graphs.get(key)
+        entry = self._step_graphs.pop(key, None)
         if entry is None:
-            if len(self._step_graphs) >= self.MAX_STEP_GRAPHS:
-                self._step_graphs.clear()
-            entry = self._step_graphs[key] = _StepGraph()
+            while len(self._step_graphs) >= self.MAX_STEP_GRAPHS:
+                # the shape that has not come for the longest time goes, the others keep their graphs
+                del self._step_graphs[next(iter(self._step_graphs))]
+            entry = _StepGraph()
+        self._step_graphs[key] = entry      # the dict keeps insertion order: the newest use is last
         return entry
 
     def _live(self, entry: _StepGraph, arena: StepArena) -> bool:

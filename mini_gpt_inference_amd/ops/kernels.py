@@ -145,7 +145,6 @@ def linear_generic(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor
           f"activation must be [>=n_rows, {k_dim}] with unit inner stride")
     _need(out.dim() == 2 and out.stride(1) == 1 and out.shape[1] == n_out and out.shape[0] >= n_rows,
           f"output must be [>=n_rows, {n_out}] with unit inner stride")
-    _need(k_dim % 16 == 0, f"inner size {k_dim} is not a multiple of 16")
     _need(bias is None or (bias.dtype == torch.float32 and bias.numel() == n_out), "bias must be float32 [out]")
     rc = library.kernels().mgpt_linear_generic(
         _ptr(a), _dtype_code(a), a.stride(0), _ptr(w), _dtype_code(w), _ptr(bias), _ptr(out), _dtype_code(out),

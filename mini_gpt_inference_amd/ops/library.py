@@ -196,6 +196,8 @@ def host() -> ctypes.CDLL:
         lib.mgpt_sched_counter.restype = c_long
         lib.mgpt_sched_forget_finished.argtypes = [P]
         lib.mgpt_sched_forget_finished.restype = None
+        lib.mgpt_sched_num_records.argtypes = [P]
+        lib.mgpt_sched_num_records.restype = I
         _host = lib
     return _host
 

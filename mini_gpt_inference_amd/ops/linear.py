@@ -82,23 +82,53 @@ def derived_bytes(w: torch.Tensor) -> int:
     return total
 
 
-def folded_layer_norm(norm, w: torch.Tensor, bias: Optional[torch.Tensor]):
+class CopyBudget:
+    """Device memory that derived copies of matrices may still take (EngineConfig.derived_weight_bytes).
+    A copy that does not fit is not made: its matrix is then read as it was loaded (row-major through
+    the decode kernels, its LayerNorm by the LayerNorm kernel), slower and with the same results up
+    to rounding."""
+
+    def __init__(self, limit: Optional[int]) -> None:
+        self.limit = limit          # None: no bound
+        self.used = 0
+
+    def take(self, n_bytes: int) -> bool:
+        if self.limit is not None and self.used + n_bytes > self.limit:
+            return False
+        self.used += n_bytes
+        return True
+
+
+def _budget(ctx) -> Optional[CopyBudget]:
+    return getattr(ctx, "copy_budget", None) if ctx is not None else None
+
+
+def folded_layer_norm(norm, w: torch.Tensor, bias: Optional[torch.Tensor], ctx=None):
     """(folded matrix, column sums, folded bias): the matrix with the LayerNorm's gain and bias
-    folded in, made once per (norm, matrix, bias)."""
+    folded in, made once per (norm, matrix, bias).  None if the step's budget for copies has no
+    room for it."""
     key = ("folded", norm.weight.data_ptr(), 0 if norm.bias is None else norm.bias.data_ptr(),
            0 if bias is None else bias.data_ptr())
     d = _derived(w)
     hit = d.get(key)
     if hit is None:
+        budget = _budget(ctx)
+        if budget is not None and not budget.take(w.numel() * w.element_size() + 8 * w.shape[0]):
+            return None
         hit = d[key] = kernels.fold_layer_norm(w, norm.weight, norm.bias, bias)
     return hit
 
 
-def packed_weight(w: torch.Tensor) -> Optional[torch.Tensor]:
+def packed_weight(w: torch.Tensor, ctx=None) -> Optional[torch.Tensor]:
     """The matrix in the layout the decode kernel reads fastest, made once per matrix (at its first
-    decode step, before any graph is captured)."""
+    decode step, before any graph is captured).  None if the kernel's layout does not take the
+    shape, or if the step's budget for copies has no room for it."""
     d = _derived(w)
     if "packed" not in d:
+        budget = _budget(ctx)
+        if budget is not None and w.shape[1] % 32 == 0 \
+                and not budget.take(-(-w.shape[0] // 16) * 16 * w.shape[1] * w.element_size()):
+            return None         # (not remembered: a later step never has more room, but a test may lift the bound)
         d["packed"] = kernels.pack_weight(w)
     return d["packed"]
 
@@ -196,7 +226,7 @@ def linear_add(ctx, a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tenso
     leave = (may_leave_parts and getattr(ctx, "pending", None) is None and not ctx.exact
              and ctx.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and a.dtype == torch.bfloat16
              and 0 < n_rows <= LEAVE_PARTS_MAX_ROWS and n_rows == ctx.n_rows and x.is_contiguous()
-             and x.shape[1] == w.shape[0])
+             and x.shape[1] == w.shape[0] and w.shape[1] % 16 == 0)
     if leave and tiled_at_few_rows(n_rows, w):
         # the tiled kernel's split: its stretches' sums are the parts (2 to 8 of them)
         need = kernels.linear_mfma_partials(n_rows, w.shape[0], w.shape[1], kernels.EPI_RESIDUAL)
@@ -212,7 +242,7 @@ def linear_add(ctx, a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tenso
             and kernels.linear_skinny_partials(n_rows, w.shape[0], w.shape[1], False, kernels.EPI_RESIDUAL)):
         buf = ctx.workspace.get("residual_parts", 4 * n_rows, w.shape[0], torch.float32)
         parts = buf[:4 * n_rows].view(4, n_rows, w.shape[0])
-        n_parts = kernels.linear_decode_parts(a, w, bias, parts, n_rows, w_packed=packed_weight(w))
+        n_parts = kernels.linear_decode_parts(a, w, bias, parts, n_rows, w_packed=packed_weight(w, ctx))
         if n_parts:
             assert n_parts == 4
             ctx.pending = residual.PendingSums(x, parts, n_parts)
@@ -235,7 +265,8 @@ def linear(ctx, a: Union[torch.Tensor, LazyNorm], w: torch.Tensor, bias: Optiona
         return scatter is not None
     if isinstance(a, LazyNorm) and getattr(ctx, "pending", None) is not None:
         a = a.tensor(ctx)      # the kernels below read plain residual rows
-    fast = w.dtype == torch.bfloat16 and not ctx.exact and ctx.dtype == torch.bfloat16
+    # (the MFMA kernels take inner sizes in steps of 16; any other goes to the general kernel)
+    fast = w.dtype == torch.bfloat16 and not ctx.exact and ctx.dtype == torch.bfloat16 and w.shape[1] % 16 == 0
     wide_out = w.shape[0] >= WIDE_OUT and n_rows * w.shape[1] > WIDE_OUT_DECODE_WORK
     if (tile_best is not None and fast and n_rows <= 16 and not wide_out and epilogue == kernels.EPI_NONE
             and scatter is None and w.shape[0] % 16 == 0 and w.shape[1] % 32 == 0
@@ -244,7 +275,7 @@ def linear(ctx, a: Union[torch.Tensor, LazyNorm], w: torch.Tensor, bias: Optiona
         tile_best.values = ctx.workspace.get("tile_best_values", rows, w.shape[0] // 16, torch.float32)
         tile_best.columns = ctx.workspace.get("tile_best_columns", rows, w.shape[0] // 16, torch.int32)
         if kernels.linear_head_best(as_tensor(ctx, a), w, bias, out, n_rows, tile_best.values, tile_best.columns,
-                                    tile_best.limit, w_packed=packed_weight(w)):
+                                    tile_best.limit, w_packed=packed_weight(w, ctx)):
             tile_best.filled = True
             return False
     if fast and n_rows <= 64 and not wide_out and not tiled_at_few_rows(n_rows, w):
@@ -253,17 +284,19 @@ def linear(ctx, a: Union[torch.Tensor, LazyNorm], w: torch.Tensor, bias: Optiona
                 and (w.shape[0] <= FOLD_MAX_OUT
                      or (n_rows <= FOLD_ANY_OUT_MAX_ROWS and w.shape[0] <= FOLD_ANY_OUT_MAX_OUT))
                 and (n_rows <= FOLD_MAX_ROWS or kernels.linear_skinny_row_groups(n_rows, w.shape[0], w.shape[1]))):
-            wf, colsum, bias_f = folded_layer_norm(a.norm, w, bias)
-            if kernels.linear_skinny(None, wf, bias_f, out, n_rows, epi, ln_x=a.x, ln_colsum=colsum,
-                                     ln_eps=a.norm.eps, ln_rows=a.rows, scatter=scatter,
-                                     w_packed=packed_weight(wf)):
-                return scatter is not None
+            folded = folded_layer_norm(a.norm, w, bias, ctx)
+            if folded is not None:
+                wf, colsum, bias_f = folded
+                if kernels.linear_skinny(None, wf, bias_f, out, n_rows, epi, ln_x=a.x, ln_colsum=colsum,
+                                         ln_eps=a.norm.eps, ln_rows=a.rows, scatter=scatter,
+                                         w_packed=packed_weight(wf, ctx)):
+                    return scatter is not None
         partials = None
         need = kernels.linear_skinny_partials(n_rows, w.shape[0], w.shape[1], False, epi)
         if need:
             partials = ctx.workspace.get("linear_partials", need, 1, torch.float32)
         if kernels.linear_skinny(as_tensor(ctx, a), w, bias, out, n_rows, epi, scatter=scatter, partials=partials,
-                                 w_packed=packed_weight(w)):
+                                 w_packed=packed_weight(w, ctx)):
             return scatter is not None
     a = as_tensor(ctx, a)
     if fast and scatter is not None and kernels.linear_mfma(a, w, bias, out, n_rows, epilogue, scatter=scatter):

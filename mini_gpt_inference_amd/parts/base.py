@@ -196,6 +196,9 @@ class StepContext:
     lead_cap: int = 0            # padded steps: the decoding requests' tokens lie among the first lead_cap
     # sums that are still to be added to the residual stream (ops.residual.PendingSums); None: it is plain
     pending: Optional[Any] = None
+    # an ops.linear.CopyBudget: device memory that copies of matrices made at first use may still take;
+    # None: no bound
+    copy_budget: Optional[Any] = None
     # set by a caller that will choose greedily among the logits: an ops.linear.TileBest, which the
     # head fills beside the logits if its kernel can
     tile_best: Optional[Any] = None

@@ -58,7 +58,7 @@ class DenseMLP(FeedForward):
                 and self.activation == "gelu_tanh" and self.fc_weight.dtype == torch.bfloat16
                 and self.proj_weight.dtype == torch.bfloat16):
             return False
-        wfc, wproj = packed_weight(self.fc_weight), packed_weight(self.proj_weight)
+        wfc, wproj = packed_weight(self.fc_weight, ctx), packed_weight(self.proj_weight, ctx)
         if wfc is None or wproj is None:
             return False
         n = ctx.n_rows

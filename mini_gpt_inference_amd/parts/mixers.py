@@ -52,8 +52,8 @@ class PagedCausalAttention(Mixer):
         self.has_bias = bool(bias)
         self.scale = float(scale) if scale is not None else self.head_dim ** -0.5
         self.window = int(window)
-        if self.head_dim % 16 != 0 or self.head_dim > 256:
-            raise ValueError(f"head size {self.head_dim}: the kernels take multiples of 16 up to 256")
+        if not 0 < self.head_dim <= 256:
+            raise ValueError(f"head size {self.head_dim}: the kernels take head sizes up to 256")
         if self.n_head % self.n_kv_head != 0:
             raise ValueError("n_head must be a multiple of n_kv_head")
         self.q_width = self.n_head * self.head_dim
@@ -85,7 +85,7 @@ class PagedCausalAttention(Mixer):
                 and self.n_kv_head == self.n_head and self.qkv_weight.dtype == torch.bfloat16
                 and self.proj_weight.dtype == torch.bfloat16):
             return False
-        wqkv, wproj = packed_weight(self.qkv_weight), packed_weight(self.proj_weight)
+        wqkv, wproj = packed_weight(self.qkv_weight, ctx), packed_weight(self.proj_weight, ctx)
         if wqkv is None or wproj is None:
             return False
         n = ctx.n_rows

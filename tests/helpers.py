@@ -25,13 +25,19 @@ CONFIGS: Dict[str, GPTConfig] = {
                    layer_norm_eps=1e-4),
     "D": GPTConfig("gpt2-mini", n_layer=1, n_embd=80, n_head=1, vocab_size=77, block_size=200, bias=False,
                    layer_norm_eps=1e-5),
+    # head sizes that are no multiple of 16 (40, 12) and widths that are none either: the
+    # architecture takes any n_embd that n_head divides (src/minigpt_infer/model.py:39-41)
+    "E": GPTConfig("gpt2-mini", n_layer=2, n_embd=40, n_head=1, vocab_size=99, block_size=72, bias=True,
+                   layer_norm_eps=1e-5),
+    "F": GPTConfig("gpt2-mini", n_layer=2, n_embd=36, n_head=3, vocab_size=150, block_size=80, bias=False,
+                   layer_norm_eps=1e-6),
     "LONG": GPTConfig("gpt2-mini", n_layer=1, n_embd=48, n_head=1, vocab_size=61, block_size=640, bias=True,
                       layer_norm_eps=1e-3),
 }
-SEEDS = {"A": 0, "B": 1, "C": 3, "D": 4, "LONG": 2}
+SEEDS = {"A": 0, "B": 1, "C": 3, "D": 4, "E": 5, "F": 6, "LONG": 2}
 # The init rule's standard deviations give nearly uniform attention and tiny logits, which hides
 # faults; the tests scale them up so that softmax is peaked and every path carries signal.
-STD_SCALE = {"A": 5.0, "B": 5.0, "C": 4.0, "D": 5.0, "LONG": 6.0}
+STD_SCALE = {"A": 5.0, "B": 5.0, "C": 4.0, "D": 5.0, "E": 6.0, "F": 6.0, "LONG": 6.0}
 
 # Tolerances, fixed before any kernel was measured.  float32: summation order only.  bfloat16:
 # activations and weights carry 8 bits of mantissa (relative 2^-9 per rounding, a handful of

@@ -377,6 +377,26 @@ def test_stats_count_the_weights_and_the_copies_made_of_them(model_folders):
     assert after["derived_weight_bytes"] >= L * (3 * c * c + c * c + 2 * f * c) * 2
 
 
+@pytest.mark.parametrize("limit", [0, 40_000])
+def test_the_copies_of_matrices_stay_within_their_bound(model_folders, limit):
+    """EngineConfig.derived_weight_bytes bounds the copies that the decode kernels make of matrices
+    at first use (0: none at all): the matrices whose copies do not fit are read as loaded, and the
+    tokens are still the plain implementation's argmax up to rounding."""
+    prompts = _prompts("B", [9, 33, 2], seed=6)
+    engine = LLMEngine.from_folder(model_folders["B"], EngineConfig(block_size=8, num_blocks=64, max_batch_size=4,
+                                                                    dtype="bfloat16", derived_weight_bytes=limit))
+    got = engine.generate(prompts, SamplingParams(max_tokens=10, temperature=0.0))
+    stats = engine.stats()
+    assert stats["derived_weight_bytes"] <= limit and (limit == 0 or stats["derived_weight_bytes"] > 0)
+    assert stats["graph_steps"] > 0
+    for prompt, tokens in zip(prompts, got):
+        _assert_greedy_within_tolerance(model_folders["B"], prompt, tokens, "bfloat16")
+    free = LLMEngine.from_folder(model_folders["B"], EngineConfig(block_size=8, num_blocks=64, max_batch_size=4,
+                                                                  dtype="bfloat16"))
+    free.generate(prompts, SamplingParams(max_tokens=10, temperature=0.0))
+    assert free.stats()["derived_weight_bytes"] > 40_000
+
+
 def test_real_vocabulary_bound_is_never_crossed(model_folders):
     engine = LLMEngine.from_folder(model_folders["A"], EngineConfig(block_size=4, num_blocks=32, max_batch_size=4,
                                                                     dtype="float32", real_vocab_size=40))

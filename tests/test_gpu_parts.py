@@ -323,8 +323,9 @@ def test_each_part_alone(dtype):
 
 def test_part_constructors_refuse_what_the_kernels_cannot_do():
     from mini_gpt_inference_amd.parts.base import FEED_FORWARDS, MIXERS
-    with pytest.raises(ValueError, match="multiples of 16"):
-        MIXERS.build(PartSpec("paged_causal_attention", {"width": 40, "n_head": 2, "head_dim": 20, "bias": False}))
+    with pytest.raises(ValueError, match="up to 256"):
+        MIXERS.build(PartSpec("paged_causal_attention", {"width": 544, "n_head": 2, "head_dim": 272, "bias": False}))
+    MIXERS.build(PartSpec("paged_causal_attention", {"width": 40, "n_head": 2, "head_dim": 20, "bias": False}))
     with pytest.raises(ValueError, match="multiple of n_kv_head"):
         MIXERS.build(PartSpec("paged_causal_attention", {"width": 96, "n_head": 6, "head_dim": 16, "bias": False,
                                                          "n_kv_head": 4}))

@@ -18,7 +18,7 @@ from mini_gpt_inference_amd.engine.replay import TraceError, TraceReplayer
 pytestmark = pytest.mark.gpu
 
 LENGTHS = {"A": [5, 17, 30, 64, 41, 23], "B": [1, 9, 33, 64, 100, 128], "C": [2, 96, 40, 71, 18],
-           "D": [200, 3, 130, 77, 150]}
+           "D": [200, 3, 130, 77, 150], "E": [72, 5, 40, 33, 64], "F": [3, 80, 47, 66, 21]}
 
 
 def _requests(name, rng):
@@ -71,6 +71,24 @@ def test_head_sizes_that_are_no_power_of_two(model_folders, name, dtype, way):
     want = _plain_logits(model_folders[name], name, reqs)
     plan = helpers.PLANS[way](reqs, np.random.default_rng(6))
     replayer = TraceReplayer(model_folders[name], dtype, plan.tight_tokens(16), poison=True)
+    got = plan.assemble(helpers.run_plan_in_process(replayer, plan), {r: len(t) for r, t in reqs.items()},
+                        helpers.CONFIGS[name].vocab_size)
+    for rid in reqs:
+        helpers.assert_close(got[rid], want[rid], dtype, f"{name} {dtype} {way} {rid}")
+    assert replayer.cache.check() == 0 and replayer.cache.num_free_pages() == replayer.num_pages
+
+
+@pytest.mark.parametrize("way", ["whole", "tail", "portions", "mixed"])
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["E", "F"])
+def test_head_sizes_and_widths_that_are_no_multiple_of_16(model_folders, name, dtype, way):
+    """n_embd 40 with one head and n_embd 36 with three heads of 12: the architecture takes any width
+    that the heads divide (src/minigpt_infer/model.py:39-41).  The matrix-core kernels refuse such
+    inner sizes and head sizes; the general kernels take them, in both dtypes, cut in every way."""
+    reqs = _requests(name, np.random.default_rng(19))
+    want = _plain_logits(model_folders[name], name, reqs)
+    plan = helpers.PLANS[way](reqs, np.random.default_rng(7))
+    replayer = TraceReplayer(model_folders[name], dtype, plan.tight_tokens(8), page_size=8, poison=True)
     got = plan.assemble(helpers.run_plan_in_process(replayer, plan), {r: len(t) for r, t in reqs.items()},
                         helpers.CONFIGS[name].vocab_size)
     for rid in reqs:

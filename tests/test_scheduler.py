@@ -366,3 +366,53 @@ def test_burst_needs_pages_for_every_step_or_does_not_start():
     free = cm.num_free_pages()
     assert s.plan_burst(8) == 0 and cm.num_free_pages() == free     # 2 free pages, 4 would be needed
     assert s.plan_burst(2) == 2                                      # two more tokens each fit
+
+
+def test_a_scheduler_that_serves_for_long_holds_only_its_live_requests():
+    """Finished requests are forgotten for good: their records go and their ids are given to later
+    requests, so the number of records follows the live requests, not the requests ever served.  A
+    request's default sampling stream is its place in the order of arrival, not its id."""
+    cm, s = make(32, 4, max_batch=4)
+    seen_ids = set()
+    for wave in range(50):
+        ids = [s.add_request([1, 2, 3], 2) for _ in range(3)]
+        seen_ids.update(ids)
+        assert s.num_records <= 3 + 3                       # this wave's and, before forgetting, the last one's
+        while s.has_work():
+            step(s)
+        assert all(s.info(i).status == FINISHED and s.output(i) == [100, 101] for i in ids)
+        s.forget_finished()
+        assert s.num_records == 0
+        for i in ids:
+            with pytest.raises(KeyError):
+                s.info(i)
+    assert len(seen_ids) <= 6, "ids of forgotten requests were not used again"
+    assert cm.num_free_pages() == 32 and cm.check() == 0
+    # a forgotten id among live ones: the others stay what they were
+    a, b = s.add_request([5] * 5, 3), s.add_request([6] * 2, 1)
+    while s.info(b).status != FINISHED:
+        step(s)
+    s.forget_finished()
+    c = s.add_request([7] * 3, 2)
+    assert c == b and s.info(a).status == RUNNING and s.info(c).status == WAITING and s.info(c).prompt_len == 3
+    while s.has_work():
+        step(s)
+    assert s.output(a) == [100, 101, 102] and s.output(c) == [100, 101]
+
+
+def test_records_are_kept_while_a_planned_burst_is_not_all_handed_in():
+    cm, s = make(32, 4, max_batch=2)
+    ids = [s.add_request([1, 2, 3], 9, eot=7) for _ in range(2)]
+    step(s)
+    step(s)
+    k = s.plan_burst(4)
+    assert k == 4
+    tokens = np.full((4, 2), 50, dtype=np.int32)
+    tokens[1, 0] = 7                                   # request 0 meets its end token in the burst's second step
+    s.commit_burst(tokens[:2], 2, last=False)
+    assert s.info(ids[0]).status == FINISHED
+    s.forget_finished()                                # refused: two steps of the burst are still to come
+    assert s.num_records == 2 and s.info(ids[0]).status == FINISHED
+    s.commit_burst(tokens[2:], 2, last=True)
+    s.forget_finished()
+    assert s.num_records == 1 and s.info(ids[1]).status == RUNNING
