@@ -304,7 +304,7 @@ def host_cost_run(args):
     med = lambda runs, i: sorted(r[i] for r in runs)[len(runs) // 2]
     n_kernels = plan_runs[0][1]      # launcher calls (one whose product is split along k is two kernels)
     # the launches alone, without describing the step and uploading its arrays
-    plan = runner._entry((tuple(q_lens), len(rows))).plan
+    plan = runner._entry((tuple(q_lens), len(rows), False)).plan
     alone = []
     for _ in range(args.host_cost_reps):
         torch.cuda.synchronize()

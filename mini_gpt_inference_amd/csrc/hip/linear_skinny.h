@@ -63,13 +63,19 @@ bool mgpt_linear_decode_row_groups(int n_rows, int n_out, int k_dim, int rows_mo
 // mgpt_linear_skinny for callers that cannot allocate device memory and bring no scratch of their
 // own (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  It has
 // no counterpart in the reference.  Where mgpt_linear_skinny would split a long inner size over
-// workgroups (17 to 64 rows, see mgpt_linear_skinny_partials) the partial sums go to an array that
+// workgroups (17 to 64 rows under a matrix too large for groups of rows, and 16 rows or fewer under
+// an inner size of 3072 or more with few column tiles: whenever mgpt_linear_skinny_partials is not
+// zero) the partial sums go to an array that
 // the library itself holds in device memory, MGPT_STATIC_SCRATCH_FLOATS floats (1 MiB) on every GPU
 // the library runs on, until the process ends; a shape that needs more is refused with
 // MGPT_ERR_SCRATCH and nothing is launched.  The call allocates and frees nothing.  Every call on
 // a GPU uses that GPU's one array, so calls that overlap on one GPU (on different streams, or from
 // different threads) race; calls on one stream follow each other and are safe.  Nothing in the
 // array has to start at zero: the first kernel writes every partial sum that the second reads.
+// The array's address on a GPU is asked of the runtime once per GPU (hipGetSymbolAddress), at
+// mgpt_linear_skinny_static_scratch_init() or else inside the first call on that GPU: a caller that
+// captures a stream into a graph calls the init function (with that GPU current) before the capture
+// begins, so that no call inside the capture is the first.
 #define MGPT_STATIC_SCRATCH_FLOATS (4L * 64 * 1024)
 #define MGPT_ERR_SCRATCH (-5)
 extern "C" int mgpt_linear_skinny_static_scratch(
@@ -79,3 +85,5 @@ extern "C" int mgpt_linear_skinny_static_scratch(
     int n_kv_head, int page_size, int mode, hipStream_t stream);
 // the array's size in floats
 extern "C" long mgpt_linear_skinny_static_scratch_floats();
+// resolves the array's address on the current GPU (MGPT_OK, or the runtime's error code); launches nothing
+extern "C" int mgpt_linear_skinny_static_scratch_init();

@@ -463,6 +463,11 @@ static int static_scratch(float** ptr) {
 
 extern "C" long mgpt_linear_skinny_static_scratch_floats() { return MGPT_STATIC_SCRATCH_FLOATS; }
 
+extern "C" int mgpt_linear_skinny_static_scratch_init() {
+  float* p = nullptr;
+  return static_scratch(&p);
+}
+
 extern "C" int mgpt_linear_skinny_static_scratch(
     const void* act, long lda, const float* x, const int* rows, const float* colsum, float eps, const void* w,
     const void* w_packed, const float* bias, void* out, int out_dtype, long ldo, int n_rows, int n_out, int k_dim,

@@ -10,6 +10,7 @@ rectangular (B, T) ForwardBatch with a mask instead and never mixes prompts with
 
 from __future__ import annotations
 
+import os
 from dataclasses import dataclass
 from typing import Dict, List, Optional, Sequence, Tuple
 
@@ -128,6 +129,7 @@ class StepShape:
     q_lens: List[int]
     ctx_lens: List[int]
     slots: List[int]
+    rows_in_order: bool = False     # the wanted logit rows are 0, 1, ..., n_tokens - 1: every token's, in order
 
 
 @dataclass
@@ -171,6 +173,9 @@ class ModelRunner:
         self.graph_steps = graph_steps and device.type == "cuda" and model.graph_safe
         self.plan_steps = device.type == "cuda" and model.plan_safe      # launches recorded and made again from C++
         self.num_planned_steps = 0        # steps whose launches came from a recorded plan
+        # a check for tests and for whoever writes a part: a step whose shape has a plan runs through the
+        # model's Python again and its launches are compared with the plan's (environment MGPT_VERIFY_PLANS=1)
+        self.verify_plans = os.environ.get("MGPT_VERIFY_PLANS", "") not in ("", "0")
         self._step_graphs: Dict[Tuple, _StepGraph] = {}     # by exact shape, least recently used first; at most MAX_STEP_GRAPHS
         self._bucket_graphs: Dict[Tuple, _StepGraph] = {}   # by capacities: as many as there are buckets
         self.num_replayed_steps = 0
@@ -221,7 +226,12 @@ class ModelRunner:
         h["logit_rows"][:m] = rows
         h["logit_rows"][m:] = 0
         q_lens = list(q_lens)
-        return StepShape(n, r, m, max(q_lens, default=0), max_seq, q_lens, list(ctx_lens), list(slots))
+        return StepShape(n, r, m, max(q_lens, default=0), max_seq, q_lens, list(ctx_lens), list(slots),
+                         rows_in_order=self._rows_in_order(arena, n, m))
+
+    @staticmethod
+    def _rows_in_order(arena: StepArena, n: int, m: int) -> bool:
+        return m == n and bool((arena.h["logit_rows"][:m] == np.arange(m, dtype=np.int32)).all())
 
     def check_positions(self, ctx_lens: Sequence[int], q_lens: Sequence[int]) -> int:
         """The longest sequence after the step; refuses positions the model does not have
@@ -239,7 +249,8 @@ class ModelRunner:
         if n and (ids.min() < 0 or ids.max() >= self.vocab_size):
             raise ValueError(f"token id outside 0..{self.vocab_size - 1}")
         max_seq = self.check_positions(ctx_lens, q_lens)
-        return StepShape(n, r, m, max(q_lens, default=0), max_seq, q_lens, ctx_lens, slots)
+        return StepShape(n, r, m, max(q_lens, default=0), max_seq, q_lens, ctx_lens, slots,
+                         rows_in_order=self._rows_in_order(arena, n, m))
 
     # ------------------------------------------------------------------ running
     def context(self, arena: StepArena, shape: StepShape, padded: bool, workspace: Optional[Workspace] = None,
@@ -270,7 +281,7 @@ class ModelRunner:
             decode_only=False if bucket else shape.max_q_len <= 1,
             host_q_lens=None if bucket else shape.q_lens, host_ctx_lens=None if bucket else shape.ctx_lens,
             host_state_slots=None if bucket else shape.slots, exact=self.exact, padded=padded,
-            lead_cap=lead_cap or 0, copy_budget=self.copy_budget)
+            lead_cap=lead_cap or 0, copy_budget=self.copy_budget, logit_rows_in_order=shape.rows_in_order)
 
     def run(self, arena: StepArena, shape: StepShape) -> torch.Tensor:
         """Uploads the arena and runs the model.  Returns float32 logits [n_logits, vocab] (in the
@@ -285,7 +296,7 @@ class ModelRunner:
         if not self.plan_steps and not self.graph_steps:
             with kernels.pinned_stream():
                 return self.model.forward(self.context(arena, shape, padded=False))
-        exact = self._entry((tuple(shape.q_lens), shape.n_logits))
+        exact = self._entry((tuple(shape.q_lens), shape.n_logits, shape.rows_in_order))
         if not self.graph_steps:
             return self._planned_or_recorded(exact, arena, shape)
         if self._live(exact, arena):
@@ -321,7 +332,16 @@ class ModelRunner:
             if not self.plan_steps:
                 return self.model.forward(self.context(arena, shape, padded=False))
             if self._plan_live(entry, arena):
-                entry.plan.run()
+                if self.verify_plans:
+                    # the step through the model's Python once more, which must make the plan's launches
+                    with library.record() as launches:
+                        self.model.forward(self.context(arena, shape, padded=False))
+                    diff = entry.plan.difference(launches)
+                    if diff is not None:
+                        raise RuntimeError("a part that promises plan_safe launched otherwise for a step of the "
+                                           "same shape: " + diff)
+                else:
+                    entry.plan.run()
                 self.num_planned_steps += 1
                 return entry.plan_logits
             with library.record() as launches:

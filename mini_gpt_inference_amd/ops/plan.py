@@ -26,6 +26,12 @@ def _slot(argtype, value) -> int:
     return int(value) & (2 ** 64 - 1)
 
 
+def signature_of(launches: List[tuple]) -> List[tuple]:
+    """(launcher name, its arguments as 64-bit slots) of every recorded launch; the stream, a launcher's
+    last argument, is left out."""
+    return [(name, tuple(_slot(t, v) for t, v in zip(argtypes[:-1], args[:-1]))) for name, argtypes, args in launches]
+
+
 class LaunchPlan:
     def __init__(self, launches: List[tuple]) -> None:
         """launches: what library.record() collected."""
@@ -35,6 +41,7 @@ class LaunchPlan:
         if not self._h:
             raise kernels.KernelError("no memory for a launch plan")
         self.n_kernels = 0
+        self.signature = signature_of(launches)      # what was recorded, for difference()
         for name, argtypes, args in launches:
             slots = (ctypes.c_ulonglong * len(args))(*[_slot(t, v) for t, v in zip(argtypes, args)])
             rc = lib.mgpt_plan_add(self._h, name.encode(), slots, len(args))
@@ -50,6 +57,22 @@ class LaunchPlan:
 
     def __len__(self) -> int:
         return self.n_kernels
+
+    def difference(self, launches: List[tuple]) -> Optional[str]:
+        """None if `launches` (what library.record() collected of another run of the same step shape)
+        are this plan's launches, launcher for launcher and argument for argument; else a line that
+        names the first difference.  A part that promises plan_safe and still takes a launcher's
+        argument from the host's view of the step (a context length, say) shows here."""
+        other = signature_of(launches)
+        for i, (mine, theirs) in enumerate(zip(self.signature, other)):
+            if mine[0] != theirs[0]:
+                return f"launch {i}: the plan has {mine[0]}, this run made {theirs[0]}"
+            for j, (a, b) in enumerate(zip(mine[1], theirs[1])):
+                if a != b:
+                    return f"launch {i} ({mine[0]}): argument {j} was {a:#x} when recorded and is {b:#x} now"
+        if len(self.signature) != len(other):
+            return f"the plan has {len(self.signature)} launches, this run made {len(other)}"
+        return None
 
     def run(self, stream: Optional[int] = None) -> None:
         """Makes the plan's launches on the stream (default: the current one)."""

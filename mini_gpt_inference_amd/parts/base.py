@@ -196,6 +196,8 @@ class StepContext:
     lead_cap: int = 0            # padded steps: the decoding requests' tokens lie among the first lead_cap
     # sums that are still to be added to the residual stream (ops.residual.PendingSums); None: it is plain
     pending: Optional[Any] = None
+    # the host has seen that logit_rows is 0, 1, ..., n_tokens - 1 (every token's logits, in order)
+    logit_rows_in_order: bool = False
     # an ops.linear.CopyBudget: device memory that copies of matrices made at first use may still take;
     # None: no bound
     copy_budget: Optional[Any] = None

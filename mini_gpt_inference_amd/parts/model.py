@@ -335,9 +335,9 @@ class DecoderModel:
         vocab = self.spec.vocab_size
         logits = ws.get("logits", m, -(-vocab // 4) * 4, torch.float32)[:, :vocab]
         if m:
-            # every token of a decode-only step wanted: row i of the logits is token i, and the norm
-            # need not wait for the list of rows before it can send for them
-            rows = None if ctx.decode_only and m == n else ctx.logit_rows
+            # every token's logits wanted, in order (the host has looked at the list): row i of the
+            # logits is token i, and the norm need not wait for the list before it can send for its rows
+            rows = None if ctx.decode_only and m == n and ctx.logit_rows_in_order else ctx.logit_rows
             self.head.forward(ctx, LazyNorm(self.final_norm, x, m, rows=rows, buffer="final_normed"), logits, m)
         ctx.pending = None
         return logits[:m]

@@ -796,3 +796,48 @@ def test_two_fused_parts_of_one_kind_in_a_row_keep_their_sums_apart(n_req):
         K.fused_mlp_decode(R.PendingSums(x, parts, n_parts), torch.zeros_like(x), norm.weight, norm.bias, norm.eps,
                            packed_weight(ff.fc_weight), ff.fc_bias, packed_weight(ff.proj_weight), ff.proj_bias,
                            parts, n_req, TW_HID)
+
+
+# ----------------------------------------------------------------------------- a part that breaks its promise
+from mini_gpt_inference_amd.parts.base import register_norm                 # noqa: E402
+from mini_gpt_inference_amd.parts.norms import LayerNorm                     # noqa: E402
+
+
+@register_norm("toy_norm_that_reads_the_host")
+class ToyNormThatReadsTheHost(LayerNorm):
+    """Promises plan_safe (inherited) and still takes a kernel argument from the host's view of the
+    step: its eps grows with the longest sequence.  The results are right whenever its Python runs;
+    a plan recorded for the shape would replay the eps of the step it was recorded at."""
+
+    fusable_layer_norm = False
+
+    def forward(self, ctx, x, out, n_rows, rows=None):
+        from mini_gpt_inference_amd.ops import kernels as K
+
+        K.layer_norm(x, self.weight, self.bias, out, n_rows, self.eps * ctx.max_seq_len, rows)
+
+
+def test_plan_verification_names_a_part_that_breaks_its_promise():
+    """ModelRunner.verify_plans finds a launcher argument that changed between two steps of one shape."""
+    base = _attn_layer(0, C, H, H, D, 0, 1 / math.sqrt(D), HID, EPS)
+    lying = PartSpec("toy_norm_that_reads_the_host", {"width": C, "eps": EPS, "bias": True},
+                     {"weight": "L0.n2.weight", "bias": "L0.n2.bias"})
+    spec = ModelSpec(width=C, vocab_size=V,
+                     embedding=PartSpec("token_embedding", {"vocab_size": V, "width": C}, {"weight": "emb.w"}),
+                     position=PartSpec("learned_absolute", {"max_positions": 50, "width": C}, {"weight": "pos.w"}),
+                     layers=(LayerSpec(base.arrangement, base.norm1, base.mixer, lying, base.feed_forward),),
+                     order=(LayerRun(0),), final_norm=_norm("nf.", C, EPS),
+                     head=PartSpec("linear_head", {"vocab_size": V, "width": C, "tied": True}, {"weight": "emb.w"}),
+                     max_positions=50)
+    model = DecoderModel(spec)
+    assert model.plan_safe                                   # so it claims
+    _bind(model, _random_weights(model, 8), "float32")
+    runner, cache = _runner(model, "float32")
+    runner.graph_steps = False
+    runner.verify_plans = True
+    slot = cache.acquire_slot()
+    assert cache.reserve(slot, 20)
+    runner.step([slot], [0], [4], [1, 2, 3, 4], [3])
+    runner.step([slot], [4], [1], [5], [0])                  # shape (1,): recorded
+    with pytest.raises(RuntimeError, match="plan_safe.*layer_norm.*argument"):
+        runner.step([slot], [5], [1], [6], [0])              # the same shape one token further: another eps

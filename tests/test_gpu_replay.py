@@ -96,6 +96,30 @@ def test_head_sizes_and_widths_that_are_no_multiple_of_16(model_folders, name, d
     assert replayer.cache.check() == 0 and replayer.cache.num_free_pages() == replayer.num_pages
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_logit_rows_of_a_decode_step_in_any_order(model_folders, dtype):
+    """A decode-only step whose wanted rows are as many as its tokens but not 0, 1, 2 in order (a
+    permutation, a row twice): the logits come in the order asked for, also when the same shape
+    came before with the rows in order (whose graph or plan drops the row list)."""
+    cfg = helpers.CONFIGS["A"]
+    rng = np.random.default_rng(31)
+    seqs = [helpers.random_ids(rng, cfg.vocab_size, n) for n in (9, 14, 6)]
+    pcfg, w = P.read_model_folder(model_folders["A"])
+    want = [P.plain_forward(w, pcfg, s).numpy() for s in seqs]
+    rep = TraceReplayer(model_folders["A"], dtype, 256, poison=True)
+    slots = [rep.cache.acquire_slot() for _ in seqs]
+    for slot, s in zip(slots, seqs):
+        assert rep.cache.reserve(slot, len(s))
+    heads = [3, 5, 2]
+    rep.runner.step(slots, [0, 0, 0], heads, sum((s[:h] for s, h in zip(seqs, heads)), []), [])
+    for j, rows in enumerate([[0, 1, 2], [0, 1, 2], [0, 1, 2], [0, 1, 2], [2, 0, 1], [1, 1, 0], [0, 1, 2], [2, 2, 2]]):
+        ctx = [h + j for h in heads]
+        got = rep.runner.step(slots, ctx, [1, 1, 1], [s[c] for s, c in zip(seqs, ctx)], rows).cpu()
+        ref = np.stack([want[r][ctx[r]] for r in rows])
+        helpers.assert_close(got, ref, dtype, f"step {j}, rows {rows}")
+    assert rep.runner.num_replayed_steps >= 1
+
+
 def _drawn_configuration(seed):
     """A configuration drawn from the seed: every size and option of the architecture varies."""
     from mini_gpt_inference_amd import GPTConfig
@@ -547,6 +571,47 @@ def test_a_shape_seen_before_is_launched_from_its_recorded_plan(model_folders, d
     assert rep.runner.num_planned_steps == before + 6
     for i in range(40, 44):                      # the other request goes on where it stood, from its own plans
         feed(1, "y", other, want_other, i)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_a_plan_holds_what_the_models_python_launches_whatever_the_contexts(model_folders, name, dtype):
+    """A recorded plan is valid for every step of its shape only if no launcher argument comes from the
+    host's view of the step beyond the shape (context lengths, the longest sequence).  With
+    ModelRunner.verify_plans a step whose shape has a plan goes through the model's Python again and
+    its launches are compared with the plan's, argument for argument: shapes with single tokens,
+    portions and both, at growing and very different context lengths."""
+    cfg = helpers.CONFIGS[name]
+    rng = np.random.default_rng(12)
+    seqs = {rid: helpers.random_ids(rng, cfg.vocab_size, cfg.block_size) for rid in "abc"}
+    pcfg, w = P.read_model_folder(model_folders[name])
+    want = {rid: P.plain_forward(w, pcfg, s).numpy() for rid, s in seqs.items()}
+    rep = TraceReplayer(model_folders[name], dtype, 3 * cfg.block_size, poison=True)
+    rep.runner.graph_steps = False
+    rep.runner.verify_plans = True
+    fed = {rid: 0 for rid in seqs}
+
+    def run(parts):
+        entries = [{"id": rid, "tokens": seqs[rid][fed[rid]:fed[rid] + n], "want": [n - 1]} for rid, n in parts]
+        got = rep.run_step({"step": 0, "entries": entries, "end": []}).cpu()
+        for row, (rid, n) in enumerate(parts):
+            helpers.assert_close(got[row], want[rid][fed[rid] + n - 1], dtype, f"{rid} +{n} at {fed[rid]}")
+            fed[rid] += n
+
+    run([("a", 30), ("b", 2)])          # contexts that differ from the start
+    run([("c", 1)])
+    for _ in range(2):                   # the workspace has all its buffers after the first round
+        run([("a", 1), ("b", 1), ("c", 1)])
+        run([("a", 1), ("b", 5)])
+        run([("c", 7)])
+        run([("b", 1)])
+    checked = rep.runner.num_planned_steps
+    for _ in range(4):
+        run([("a", 1), ("b", 1), ("c", 1)])
+        run([("a", 1), ("b", 5)])
+        run([("c", 7)])
+        run([("b", 1)])
+    assert rep.runner.num_planned_steps >= checked + 16
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])

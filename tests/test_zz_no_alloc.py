@@ -84,3 +84,47 @@ def test_static_scratch_entry_point_refuses_what_its_array_cannot_hold():
     assert rc == ERR_SCRATCH
     torch.cuda.synchronize()
     assert bool((out == 7.0).all()), "a refused call launches nothing"
+
+
+def test_static_scratch_at_few_rows_under_a_long_inner_size_and_inside_a_captured_graph():
+    """The split also comes at 16 rows or fewer under a long inner size with few column tiles, and
+    the entry point is meant for code under graph capture: after the init call (which asks the
+    runtime for the array's address outside any capture) a call captured into a graph gives the
+    eager result on every replay, with other work on the array between the replays."""
+    lib = library.kernels()
+    lib.mgpt_linear_skinny_static_scratch_init.restype = ctypes.c_int
+    assert lib.mgpt_linear_skinny_static_scratch_init() == 0
+    n_rows, n_out, k_dim = 8, 1600, 6400
+    assert kernels.linear_skinny_partials(n_rows, n_out, k_dim, False, kernels.EPI_RESIDUAL) > 0
+    few = _both(n_rows, n_out, k_dim, kernels.EPI_RESIDUAL, seed=3)
+    assert torch.equal(few[0], few[1])
+    fn = lib.mgpt_linear_skinny_static_scratch
+    g = torch.Generator(device="cuda").manual_seed(4)
+    act = (torch.randn(n_rows, k_dim, device="cuda", generator=g) * 0.5).to(torch.bfloat16)
+    w = (torch.randn(n_out, k_dim, device="cuda", generator=g) * 0.05).to(torch.bfloat16)
+    out = torch.zeros(n_rows, n_out, device="cuda", dtype=torch.bfloat16)
+
+    def call():
+        stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+        rc = fn(act.data_ptr(), act.stride(0), None, None, None, 0.0, w.data_ptr(), None, None, out.data_ptr(),
+                kernels.BF16, out.stride(0), n_rows, n_out, k_dim, kernels.EPI_NONE, None, None, None, 0, 0, 0, 0, 0,
+                SHARE_W, stream)
+        assert rc == 0, rc
+
+    call()
+    torch.cuda.synchronize()
+    eager = out.clone()
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        graph.capture_begin()
+        call()
+        graph.capture_end()
+    torch.cuda.current_stream().wait_stream(side)
+    for _ in range(3):
+        out.fill_(7.0)
+        _both(64, 512, 2048, kernels.EPI_RESIDUAL, seed=5)      # eager work that leaves other sums in the array
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, eager)
