@@ -839,5 +839,5 @@ def test_plan_verification_names_a_part_that_breaks_its_promise():
     assert cache.reserve(slot, 20)
     runner.step([slot], [0], [4], [1, 2, 3, 4], [3])
     runner.step([slot], [4], [1], [5], [0])                  # shape (1,): recorded
-    with pytest.raises(RuntimeError, match="plan_safe.*layer_norm.*argument"):
+    with pytest.raises(RuntimeError, match="plan_safe.*mgpt_layernorm.*argument"):
         runner.step([slot], [5], [1], [6], [0])              # the same shape one token further: another eps
