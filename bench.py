@@ -58,7 +58,8 @@ def build_engine(args, batch, dtype, raw=None, **engine_options):
     positions = arch.model_spec(cfg).max_positions or args.positions
     options = dict(block_size=args.kv_block, num_blocks=batch * (-(-positions // args.kv_block)) + 8,
                    max_batch_size=max(batch, 2), max_num_batched_tokens=max(4096, batch * args.prompt), dtype=dtype,
-                   use_graph=not args.no_graph, decode_burst=args.burst, decode_chain=args.chain)
+                   use_graph=not args.no_graph, decode_burst=args.burst, decode_chain=args.chain,
+                   derived_weight_bytes=args.derived_weight_bytes)
     options.update(engine_options)
     return LLMEngine.from_random(cfg, seed=0, engine_config=EngineConfig(**options)), cfg, arch
 
@@ -344,6 +345,8 @@ def main(argv=None) -> int:
     ap.add_argument("--prompt", type=int, default=128)
     ap.add_argument("--kv-block", type=int, default=16)
     ap.add_argument("--no-graph", action="store_true")
+    ap.add_argument("--derived-weight-bytes", type=int, default=None,
+                    help="bound for the copies of matrices that the decode kernels make at first use (0 = none)")
     ap.add_argument("--burst", type=int, default=8, help="decode steps captured as one graph (1 = off)")
     ap.add_argument("--chain", type=int, default=4, help="such graphs enqueued before the host waits")
     ap.add_argument("--no-extras", action="store_true", help="skip prefill and the batch 1 / 64 points")
@@ -420,6 +423,7 @@ def main(argv=None) -> int:
         # the timing rule: `value` is from the median block of `steps` decode steps; the quartiles' distance per step
         "blocks": len(run["blocks"]), "iqr_ms": round((q3 - q1) / args.steps * 1e3, 4), "decode_chain": args.chain,
         "kernels_per_step": kernels_per_step(engine, args.batch),
+        "weight_bytes": stats["weight_bytes"], "derived_weight_bytes": stats["derived_weight_bytes"],
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 5)},
     }
