@@ -463,7 +463,13 @@ int choose_shape(int n_rows, int n_out) {
     const long rounds = (t + 255) / 256;
     if (t >= (shape == 0 ? 160 : 140) && 10 * t >= 7 * rounds * 256) return shape;
   }
-  if (tiles_of(2, n_rows, n_out) >= 300) return 2;
+  // 128 x 64 tiles only where their last round of 256 is well filled: 384 of them (2,048 rows under 1,536
+  // columns) leave half the compute units with two tiles and half with one, and 768 tiles of 64 x 64
+  // take 8.4 us where they take 9.2; 512 (under 2,048 columns) take 10.3 against 10.6
+  {
+    const long t = tiles_of(2, n_rows, n_out);
+    if (t >= 300 && 100 * t >= 85 * ((t + 255) / 256) * 256) return 2;
+  }
   if (tiles_of(3, n_rows, n_out) >= 192) return 3;
   return 4;
 }
