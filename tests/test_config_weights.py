@@ -149,3 +149,28 @@ def test_missing_files(tmp_path):
         json.dump(helpers.CONFIGS["A"].to_json_dict(), fh)
     with pytest.raises(WeightError, match="no model.safetensors"):
         load_model(str(tmp_path), "float32", "cpu")
+
+
+def test_the_models_cost_follows_the_architectures_formulas(tmp_path):
+    """DecoderModel.cost() (what bench.py prices a step with) against the GPT-2 formulas written out:
+    every matrix, gain and bias once and the tied table once as the head's matrix; the position
+    table by row; 12 C^2 matrix elements a token and layer; keys and values of every layer."""
+    from mini_gpt_inference_amd.weights.loader import load_model
+
+    cfg = helpers.CONFIGS["A"]
+    folder = write_random_model(str(tmp_path / "m"), cfg, 3)
+    model, _, _ = load_model(folder, "bfloat16", device="cpu")
+    cost = model.cost()
+    c, f, L, v, d = cfg.n_embd, 4 * cfg.n_embd, cfg.n_layer, cfg.vocab_size, cfg.head_dim
+    matrices = L * (3 * c * c + c * c + 2 * f * c)
+    vectors = L * (2 * 2 * c + 3 * c + c + f + c) + 2 * c
+    assert cost.run_matrix_elements == matrices and cost.head_matrix_elements == v * c
+    assert cost.whole_tensor_bytes == (matrices + v * c) * 2 + vectors * 4
+    assert cost.table_row_bytes == c * 2                       # a position's row; the token's row is in the tied matrix
+    assert [(r.n_head, r.n_kv_head, r.head_dim, r.window) for r in cost.kv_runs] == [(cfg.n_head, cfg.n_head, d, 0)] * L
+    # a decode step of 3 requests that look at 10, 20 and 30 keys
+    kv = (10 + 20 + 30) * L * 2 * c * 2
+    assert cost.step_read_bytes(3, [10, 20, 30], 2) == cost.whole_tensor_bytes + 3 * c * 2 + kv
+    # two whole prompts of 7 and 4 tokens, logits at each one's last token
+    attention = sum(4 * (t * (t + 1) // 2) * c for t in (7, 4)) * L
+    assert cost.prompt_flops([7, 4], 2) == 2 * 11 * matrices + 2 * 2 * v * c + attention
