@@ -950,7 +950,18 @@ __global__ __launch_bounds__(256) void residual_settle_kernel(FusedResidual res,
   const long row = idx / V;
   const int c4 = (int)(idx - row * V);
   float4 s = reinterpret_cast<const float4*>(res.base)[row * V + c4];
-  for (int p = 0; p < res.n_parts; ++p) s = fd_add4(s, reinterpret_cast<const float4*>(res.partials + p * res.part_stride)[row * V + c4]);
+  // eight parts on their way at a time, added in the order of the parts (a part beyond the last reads the
+  // last one again and is dropped)
+  for (int p0 = 0; p0 < res.n_parts; p0 += 8) {
+    float4 t[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const int p = p0 + u < res.n_parts ? p0 + u : res.n_parts - 1;
+      t[u] = reinterpret_cast<const float4*>(res.partials + p * res.part_stride)[row * V + c4];
+    }
+#pragma unroll
+    for (int u = 0; u < 8; ++u) s = fd_add4(s, fd_keep4(p0 + u < res.n_parts, t[u]));
+  }
   reinterpret_cast<float4*>(res.settled)[row * V + c4] = s;
 }
 
