@@ -123,12 +123,20 @@ constexpr int MM_GROUP = 4;         // row tiles per block of tiles
 // (a 64 x 64 tile: 8 MFMAs a wave and step against a microsecond or more), and the product takes
 // a memory round trip every two steps; more steps in flight, each in registers of its own, take that
 // wait apart.
-template <int WTM, int WTN, int WVM, int WVN, int EPI, typename OT, int AHEAD = 1>
-__global__ __launch_bounds__(64 * WVM * WVN) void linear_mfma_kernel(
+// KG: wave groups that share a tile (1 or 2).  With 2, the workgroup has twice the waves: group 0
+// multiplies the first half (32) of every step along k and group 1 the second, each wave over the same
+// part of the tile as its twin in the other group, and the twins' sums meet in LDS once, after the last
+// step (float32 outputs only: the epilogue that stores them has no barrier, so group 1 is done then).
+// For few tiles of 64 x 64 under a long inner size: a compute unit that has one such tile has four
+// waves, too few to cover each other's waits for LDS and the barrier.
+template <int WTM, int WTN, int WVM, int WVN, int EPI, typename OT, int AHEAD = 1, int KG = 1>
+__global__ __launch_bounds__(64 * WVM * WVN * KG) void linear_mfma_kernel(
     const bf16_t* __restrict__ act, long lda, const bf16_t* __restrict__ w,
     const float* __restrict__ bias, OT* __restrict__ out, long ldo, int n_rows, int n_out, int k_dim,
     int k_parts, long part_stride, MfmaScatter sc) {
-  constexpr int T = 64 * WVM * WVN;
+  static_assert(KG == 1 || (KG == 2 && sizeof(OT) == 4 && AHEAD == 1), "two wave groups: float32 outputs");
+  constexpr int T = 64 * WVM * WVN * KG;
+  constexpr int HALVES = (MM_BK / 32) / KG;   // halves of a step along k that a wave multiplies
   constexpr int BM = WVM * WTM * 16, BN = WVN * WTN * 16;
   constexpr int TPR = MM_BK / 8;  // threads per staged row (16 bytes each)
   constexpr int RPP = T / TPR;      // rows per staging pass
@@ -138,7 +146,10 @@ __global__ __launch_bounds__(64 * WVM * WVN) void linear_mfma_kernel(
   bf16_t* const as_base = lds;                      // [2][BM * MM_LD]
   bf16_t* const ws_base = lds + 2 * BM * MM_LD;   // [2][BN * MM_LD]
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave_all = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int kg = KG == 1 ? 0 : wave_all / (WVM * WVN);     // this wave's group: which half of a step it multiplies
+  const int wave = KG == 1 ? wave_all : wave_all - kg * (WVM * WVN);
   const int row_tiles = (n_rows + BM - 1) / BM, col_tiles = (n_out + BN - 1) / BN;
   int row_tile, col_tile, part;
   {
@@ -217,15 +228,17 @@ __global__ __launch_bounds__(64 * WVM * WVN) void linear_mfma_kernel(
     const int buf = s & 1;
     const bf16_t* as = as_base + buf * (BM * MM_LD) + (wr + lrow) * MM_LD;
     const bf16_t* ws = ws_base + buf * (BN * MM_LD) + (wc + lrow) * MM_LD;
-    constexpr int GROUPS = (MM_BK / 32) * WTM;
-    bf16x8_t wf[MM_BK / 32][WTN], af[3];
+    constexpr int GROUPS = HALVES * WTM;
+    bf16x8_t wf[HALVES][WTN], af[3];
     // the second half's chunk is 4 further, which the swizzle turns into a flip of bit 5 of the offset
+    // (with two wave groups a wave has one half only: its group's)
+    const int h0 = kg * 32;
     auto read_a = [&](int g) {
-      return *reinterpret_cast<const bf16x8_t*>(as + (g % WTM) * 16 * MM_LD + (c0 ^ ((g / WTM) * 32)));
+      return *reinterpret_cast<const bf16x8_t*>(as + (g % WTM) * 16 * MM_LD + (c0 ^ (KG == 1 ? (g / WTM) * 32 : h0)));
     };
 #pragma unroll
-    for (int i = 0; i < WTN; ++i) wf[0][i] = *reinterpret_cast<const bf16x8_t*>(ws + i * 16 * MM_LD + c0);
-    if (WTM == 1) {  // the second half's groups start at once
+    for (int i = 0; i < WTN; ++i) wf[0][i] = *reinterpret_cast<const bf16x8_t*>(ws + i * 16 * MM_LD + (c0 ^ h0));
+    if (WTM == 1 && HALVES == 2) {  // the second half's groups start at once
 #pragma unroll
       for (int i = 0; i < WTN; ++i) wf[1][i] = *reinterpret_cast<const bf16x8_t*>(ws + i * 16 * MM_LD + (c0 ^ 32));
     }
@@ -234,7 +247,7 @@ __global__ __launch_bounds__(64 * WVM * WVN) void linear_mfma_kernel(
 #pragma unroll
     for (int g = 0; g < GROUPS; ++g) {
       if (g + 2 < GROUPS) af[(g + 2) % 3] = read_a(g + 2);
-      if (WTM >= 2 && g % WTM == WTM - 2 && g / WTM + 1 < MM_BK / 32) {
+      if (WTM >= 2 && g % WTM == WTM - 2 && g / WTM + 1 < HALVES) {
 #pragma unroll
         for (int i = 0; i < WTN; ++i)
           wf[g / WTM + 1][i] = *reinterpret_cast<const bf16x8_t*>(ws + i * 16 * MM_LD + (c0 ^ ((g / WTM + 1) * 32)));
@@ -295,6 +308,30 @@ __global__ __launch_bounds__(64 * WVM * WVN) void linear_mfma_kernel(
       else round(std::integral_constant<int, 0>{}, std::integral_constant<int, 1>{}, std::integral_constant<int, 2>{},
                  std::integral_constant<int, 3>{});
     }
+  }
+
+  if constexpr (KG == 2) {
+    // the two groups' sums of the same part of the tile meet: group 1 hands its over through LDS (the
+    // staged operands are done with) and is finished; group 0 adds them, first half of k first
+    static_assert(WVM * WVN * WTN * WTM * 64 * 16 <= 2 * (BM + BN) * MM_LD * (int)sizeof(bf16_t), "the sums fit the LDS");
+    f32x4_t* red = reinterpret_cast<f32x4_t*>(lds);
+    __syncthreads();
+    if (kg == 1) {
+#pragma unroll
+      for (int i = 0; i < WTN; ++i)
+#pragma unroll
+        for (int j = 0; j < WTM; ++j) red[((wave * WTN + i) * WTM + j) * 64 + lane] = acc[i][j];
+    }
+    __syncthreads();
+    if (kg == 1) return;
+#pragma unroll
+    for (int i = 0; i < WTN; ++i)
+#pragma unroll
+      for (int j = 0; j < WTM; ++j) {
+        const f32x4_t t = red[((wave * WTN + i) * WTM + j) * 64 + lane];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) acc[i][j][e] += t[e];
+      }
   }
 
   // lane holds out[row0 + wr + j*16 + (lane & 15)][col0 + wc + i*16 + (lane >> 4)*4 + e], e = 0..3
@@ -397,13 +434,13 @@ __global__ __launch_bounds__(64 * WVM * WVN) void linear_mfma_kernel(
   }
 }
 
-template <int WTM, int WTN, int WVM, int WVN, int EPI, typename OT, int AHEAD>
+template <int WTM, int WTN, int WVM, int WVN, int EPI, typename OT, int AHEAD, int KG = 1>
 int launch_one(const void* act, long lda, const void* w, const float* bias, void* out, long ldo, int n_rows,
                int n_out, int k_dim, int k_parts, long part_stride, const MfmaScatter& sc, hipStream_t stream) {
   static_assert(AHEAD >= 1 && AHEAD <= 4, "sets of staging registers");
   constexpr int BM = WVM * WTM * 16, BN = WVN * WTN * 16;
   constexpr size_t lds_bytes = 2ul * (BM + BN) * MM_LD * sizeof(bf16_t);
-  auto kernel = linear_mfma_kernel<WTM, WTN, WVM, WVN, EPI, OT, AHEAD>;
+  auto kernel = linear_mfma_kernel<WTM, WTN, WVM, WVN, EPI, OT, AHEAD, KG>;
   static bool allowed = false;  // more LDS than a kernel gets without asking
   if (!allowed) {
     const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
@@ -413,7 +450,7 @@ int launch_one(const void* act, long lda, const void* w, const float* bias, void
   }
   const long tiles = (long)((n_rows + BM - 1) / BM) * ((n_out + BN - 1) / BN) * k_parts;
   if (tiles > 0x7fffffffL) return MGPT_ERR_TOO_LARGE;
-  hipLaunchKernelGGL(kernel, dim3((unsigned int)tiles), dim3(64 * WVM * WVN), lds_bytes, stream,
+  hipLaunchKernelGGL(kernel, dim3((unsigned int)tiles), dim3(64 * WVM * WVN * KG), lds_bytes, stream,
                      (const bf16_t*)act, lda, (const bf16_t*)w, bias, (OT*)out, ldo, n_rows, n_out, k_dim, k_parts,
                      part_stride, sc);
   return mgpt_last_error();
@@ -432,6 +469,20 @@ int launch_shape(const void* act, long lda, const void* w, const float* bias, vo
   if (epilogue == MM_EPI_RESIDUAL && out_dtype == MGPT_F32) MM_LAUNCH(MM_EPI_RESIDUAL, float);
   if (epilogue == MM_EPI_QKV && out_dtype == MGPT_BF16) MM_LAUNCH(MM_EPI_QKV, bf16_t);
 #undef MM_LAUNCH
+  return MGPT_ERR_BAD_DTYPE;
+}
+
+// The 64 x 64 tile with two wave groups (float32 outputs: plain, or added into the residual stream).
+int launch_two_groups(const void* act, long lda, const void* w, const float* bias, void* out, int out_dtype, long ldo,
+                      int n_rows, int n_out, int k_dim, int epilogue, int k_parts, long part_stride,
+                      const MfmaScatter& sc, hipStream_t stream) {
+  if (out_dtype != MGPT_F32) return MGPT_ERR_BAD_DTYPE;
+  if (epilogue == MM_EPI_NONE)
+    return launch_one<2, 2, 2, 2, MM_EPI_NONE, float, 1, 2>(act, lda, w, bias, out, ldo, n_rows, n_out, k_dim, k_parts,
+                                                          part_stride, sc, stream);
+  if (epilogue == MM_EPI_RESIDUAL)
+    return launch_one<2, 2, 2, 2, MM_EPI_RESIDUAL, float, 1, 2>(act, lda, w, bias, out, ldo, n_rows, n_out, k_dim,
+                                                              k_parts, part_stride, sc, stream);
   return MGPT_ERR_BAD_DTYPE;
 }
 
@@ -581,7 +632,12 @@ int launch_any(int shape, int k_parts, const void* act, long lda, const void* w,
   if (!shapes_ok(act, lda, w, out, ldo, n_rows, n_out, k_dim)) return MGPT_ERR_BAD_SHAPE;
   // shapes MM_SHAPES and MM_SHAPES + 1: the two smallest tiles with more steps on their way from memory
   int ahead = 0;  // 0: chosen below
-  if (shape >= MM_SHAPES && shape < MM_SHAPES + 2) {
+  bool two_groups = false;  // the 64 x 64 tile with two wave groups (shape MM_SHAPES + 2)
+  if (shape == MM_SHAPES + 2) {
+    shape = 3;
+    ahead = 1;
+    two_groups = true;
+  } else if (shape >= MM_SHAPES && shape < MM_SHAPES + 2) {
     shape -= 2;
     ahead = MM_AHEAD;
   } else if (shape >= 0) {
@@ -615,6 +671,19 @@ int launch_any(int shape, int k_parts, const void* act, long lda, const void* w,
     }
   }
   const bool split = k_parts > 1;
+  if (two_groups) {
+    // forced: what this kernel stores must be float32, plain or added into the residual stream (the sums of
+    // a split product are)
+    const int dt_here = split ? MGPT_F32 : out_dtype, epi_here = split ? MM_EPI_NONE : epilogue;
+    if (dt_here != MGPT_F32 || (epi_here != MM_EPI_NONE && epi_here != MM_EPI_RESIDUAL)) return MGPT_ERR_BAD_SHAPE;
+  } else if (shape == 3 && ahead == 1) {
+    // 64 x 64 tiles under a long inner size (16 steps and more a workgroup), float32 out: two wave groups
+    // a tile.  [2048 x 2048 -> 512] 12.9 us against 14.4, [1024 x 2048 -> 512] 12.2 / 13.4, [2048 x 3072 ->
+    // 768] 24.2 / 25.5, [8192 x 2048 -> 512] 33.9 / 35.3; at 8 steps ([2048 x 512 -> 512]) nothing.
+    const int steps_here = ((k_dim + MM_BK - 1) / MM_BK + k_parts - 1) / k_parts;
+    const int dt_here = split ? MGPT_F32 : out_dtype, epi_here = split ? MM_EPI_NONE : epilogue;
+    two_groups = steps_here >= 16 && dt_here == MGPT_F32 && (epi_here == MM_EPI_NONE || epi_here == MM_EPI_RESIDUAL);
+  }
   if (leave_parts) {
     *leave_parts = split ? k_parts : 0;
     if (!split) return MGPT_OK;  // nothing launched: the caller takes another way
@@ -629,8 +698,9 @@ int launch_any(int shape, int k_parts, const void* act, long lda, const void* w,
     case 0: rc = launch_shape<8, 4, 2, 4>(MM_ARGS); break;  // 256 x 256, eight waves of 128 x 64
     case 1: rc = launch_shape<4, 4, 2, 4>(MM_ARGS); break;  // 128 x 256, eight waves of 64 x 64
     case 2: rc = launch_shape<4, 2, 2, 2>(MM_ARGS); break;  // 128 x 64, four waves of 64 x 32
-    case 3:  // 64 x 64, four waves of 32 x 32
-      rc = ahead > 1 ? launch_shape<2, 2, 2, 2, MM_AHEAD>(MM_ARGS) : launch_shape<2, 2, 2, 2>(MM_ARGS);
+    case 3:  // 64 x 64, four waves of 32 x 32 (or eight, in two groups)
+      rc = two_groups ? launch_two_groups(MM_ARGS)
+                      : ahead > 1 ? launch_shape<2, 2, 2, 2, MM_AHEAD>(MM_ARGS) : launch_shape<2, 2, 2, 2>(MM_ARGS);
       break;
     case 4:  // 32 x 32, four waves of 16 x 16
       rc = ahead > 1 ? launch_shape<1, 1, 2, 2, MM_AHEAD>(MM_ARGS) : launch_shape<1, 1, 2, 2>(MM_ARGS);
@@ -682,14 +752,14 @@ extern "C" int mgpt_linear_mfma(const void* act, long lda, const void* w, const 
 }
 
 // The same product with the tile shape given (0 = 256 x 256, 1 = 128 x 256, 2 = 128 x 64,
-// 3 = 64 x 64, 4 = 32 x 32, 5 and 6 = 64 x 64 and 32 x 32 with four steps on their way from memory;
-// negative: chosen) and the number of stretches of the inner size given
+// 3 = 64 x 64, 4 = 32 x 32, 5 and 6 = 64 x 64 and 32 x 32 with four steps on their way from memory,
+// 7 = 64 x 64 with two wave groups a tile (float32 outputs); negative: chosen) and the number of stretches of the inner size given
 // (k_parts as for launch_any above), instead of chosen by the size: for tests and measurements.
 extern "C" int mgpt_linear_mfma_shape(int shape, int k_parts, const void* act, long lda, const void* w,
                                       const float* bias, void* out, int out_dtype, long ldo, int n_rows,
                                       int n_out, int k_dim, int epilogue, float* partials, long partials_floats,
                                       hipStream_t stream) {
-  if (epilogue == MM_EPI_QKV || shape >= MM_SHAPES + 2 || k_parts < 0) return MGPT_ERR_BAD_SHAPE;
+  if (epilogue == MM_EPI_QKV || shape > MM_SHAPES + 2 || k_parts < 0) return MGPT_ERR_BAD_SHAPE;
   MfmaScatter sc = {};
   return launch_any(shape, k_parts, act, lda, w, bias, out, out_dtype, ldo, n_rows, n_out, k_dim, epilogue,
                     partials, partials_floats, sc, stream);

@@ -176,7 +176,7 @@ def test_linear_skinny(n, k, o, epi, o_dt, general):
 
 
 @pytest.mark.parametrize("n,k,o", [(65, 64, 257), (300, 512, 1536), (129, 96, 503), (2048, 80, 48), (128, 2048, 128),
-                                   (1000, 48, 130)])
+                                   (1000, 48, 130), (600, 1072, 136)])
 @pytest.mark.parametrize("epi,o_dt", [(kernels.EPI_NONE, "bfloat16"), (kernels.EPI_NONE, "float32"),
                                       (kernels.EPI_GELU, "bfloat16"), (kernels.EPI_RESIDUAL, "float32")])
 def test_linear_mfma(n, k, o, epi, o_dt):
@@ -197,12 +197,18 @@ def test_linear_mfma(n, k, o, epi, o_dt):
                                    (40, 1616, 272)])
 @pytest.mark.parametrize("epi,o_dt", [(kernels.EPI_NONE, "bfloat16"), (kernels.EPI_NONE, "float32"),
                                       (kernels.EPI_GELU, "bfloat16"), (kernels.EPI_RESIDUAL, "float32")])
-@pytest.mark.parametrize("shape", [0, 1, 2, 3, 4, 5, 6])
+@pytest.mark.parametrize("shape", [0, 1, 2, 3, 4, 5, 6, 7])
 def test_linear_mfma_each_tile_shape(n, k, o, epi, o_dt, shape):
     """Each tile shape forced at sizes that cut its tiles everywhere: rows and columns past the end, an
     inner size that ends inside a step, several tiles each way.  Shapes 5 and 6: the 64 x 64 and 32 x 32
     tiles with four steps on their way from memory, in whole rounds of four (inner sizes of 1, 2, 8, 26
-    and 32 steps: rounds that end beyond the last step)."""
+    and 32 steps: rounds that end beyond the last step).  Shape 7: the 64 x 64 tile with two wave groups,
+    each one half of every step along k (also a last step of which only the first half exists); float32
+    outputs only."""
+    if shape == 7 and o_dt != "float32":
+        a, w = torch.zeros(64, 64, dtype=torch.bfloat16, device=DEV), torch.zeros(64, 64, dtype=torch.bfloat16, device=DEV)
+        assert not kernels.linear_mfma(a, w, None, torch.zeros(64, 64, dtype=torch.bfloat16, device=DEV), 64, epi, shape=7)
+        return
     g = torch.Generator().manual_seed(16)
     a, w, bias = rnd(g, n, k, dtype="bfloat16"), rnd(g, o, k, dtype="bfloat16", scale=k ** -0.5), rnd(g, o)
     prev = rnd(g, n + 2, o, dtype=o_dt)
@@ -214,7 +220,7 @@ def test_linear_mfma_each_tile_shape(n, k, o, epi, o_dt, shape):
 
 @pytest.mark.parametrize("n,k,o,shape,parts", [(100, 2048, 96, 4, 4), (70, 1040, 132, 3, 2), (300, 6400, 64, 3, 8),
                                                 (33, 576, 40, 4, 3), (130, 1600, 260, 2, 4), (64, 1600, 528, 6, 2),
-                                                (50, 3200, 96, 5, 4), (48, 6400, 1600, None, 0)])
+                                                (50, 3200, 96, 5, 4), (48, 6400, 1600, None, 0), (90, 4128, 200, 7, 3)])
 @pytest.mark.parametrize("epi,o_dt", [(kernels.EPI_NONE, "bfloat16"), (kernels.EPI_NONE, "float32"),
                                       (kernels.EPI_GELU, "bfloat16"), (kernels.EPI_RESIDUAL, "float32")])
 def test_linear_mfma_split_along_the_inner_size(n, k, o, shape, parts, epi, o_dt):
