@@ -416,3 +416,61 @@ def test_records_are_kept_while_a_planned_burst_is_not_all_handed_in():
     s.commit_burst(tokens[2:], 2, last=True)
     s.forget_finished()
     assert s.num_records == 1 and s.info(ids[1]).status == RUNNING
+
+
+@pytest.mark.parametrize("seed", range(4))
+def test_random_load_with_forgetting_at_random_times(seed):
+    """Arrivals, steps, bursts, cancels and forget_finished in random order: ids are given out again,
+    and still every request gets its own outputs, each output index once and in order, nothing of a
+    forgotten request comes back, and the records follow the live requests."""
+    rng = random.Random(99 + seed)
+    cm, s = make(28, 4, max_batch=4, budget=24, chunk=6, mixed=True, max_positions=64)
+    live = {}            # id -> (serial number of the request, its output length so far, max_tokens)
+    serial = done = 0
+    for it in range(3000):
+        roll = rng.random()
+        if roll < 0.25 and serial < 120:
+            rid = s.add_request([rng.randrange(50) for _ in range(rng.randint(1, 20))], rng.randint(1, 10))
+            assert rid not in live, "an id in use was given out again"
+            live[rid] = [serial, 0, None]
+            serial += 1
+        elif roll < 0.30 and live:
+            rid = rng.choice(list(live))
+            if s.info(rid).status != FINISHED:
+                assert s.cancel(rid)
+        elif roll < 0.40:
+            before = s.num_records
+            s.forget_finished()
+            for rid in list(live):
+                try:
+                    s.info(rid)
+                except KeyError:
+                    del live[rid]
+                    done += 1
+            assert s.num_records == len(live) <= before
+        if not s.has_work():
+            continue
+        k = s.plan_burst(4) if rng.random() < 0.3 else 0
+        if k >= 2:
+            ents = s.entries()
+            toks = np.array([[live[e.request][0] * 100 + live[e.request][1] + j for e in ents] for j in range(k)],
+                            dtype=np.int32)
+            outs = s.commit_burst(toks, k)
+        else:
+            s.schedule()
+            ents = s.entries()
+            outs = s.commit(np.array([live[e.request][0] * 100 + live[e.request][1] for e in ents if e.sample],
+                                     dtype=np.int32))
+        for rid, tok, fin, why in outs:
+            rec = live[rid]
+            assert tok == rec[0] * 100 + rec[1], "a token of another request, or out of order"
+            rec[1] += 1
+        assert cm.check() == 0
+    while s.has_work():
+        s.schedule()
+        ents = s.entries()
+        for rid, tok, fin, why in s.commit(np.array([live[e.request][0] * 100 + live[e.request][1]
+                                                     for e in ents if e.sample], dtype=np.int32)):
+            live[rid][1] += 1
+    s.forget_finished()
+    assert s.num_records == 0 and serial > 50 and cm.num_free_pages() == 28 and cm.num_free_slots == 4
