@@ -741,10 +741,13 @@ __global__ __launch_bounds__(FUSED_THREADS) void fused_mlp_decode_kernel(FusedMl
   // ---- loads in the order in which their data is needed: this wave's share of a residual row,
   // then the weights of both products (the second product's behind the barrier that the rows'
   // sums need: a wave passes a barrier only when all others have issued what stands before it)
-  const int wpr = FUSED_WAVES / RW;           // waves of a row
-  const int lr = wave / wpr, sw = wave - lr * wpr;
+  // One row and few parts: the row's first wave sends for all of them itself and adds them in its
+  // registers; nothing of the row goes through LDS before the LayerNorm.
+  const bool alone = RW == 1 && a.res.n_parts <= FM_WAVE_PARTS;
+  const int wpr = alone ? 1 : FUSED_WAVES / RW;           // waves of a row
+  const int lr = alone ? 0 : wave / wpr, sw = alone ? 0 : wave - lr * wpr;
   const int row = r0 + lr;
-  const bool has_row = row < a.n_rows;        // the same in all lanes, like everything that decides a load here
+  const bool has_row = row < a.n_rows && (!alone || wave == 0);   // the same in all lanes, like everything that decides a load here
   float4 xs4[VU], gv[VU], bv[VU];
 #pragma unroll
   for (int u = 0; u < VU; ++u) xs4[u] = gv[u] = bv[u] = make_float4(0.f, 0.f, 0.f, 0.f);
