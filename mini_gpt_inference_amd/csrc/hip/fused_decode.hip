@@ -745,7 +745,7 @@ __global__ __launch_bounds__(FUSED_THREADS) void fused_mlp_decode_kernel(FusedMl
   // wave sends for all of them itself and adds them in its registers; nothing of the row goes through
   // LDS before the LayerNorm, no wave waits for another's loads, and the other waves have only their
   // weights to send for (a decode step of the 50.9M model: 0.146 -> 0.137 ms at batch 8).
-  const bool alone = a.res.n_parts <= FM_WAVE_PARTS;
+  const bool alone = a.res.n_parts <= FM_WAVE_PARTS && RW <= 4;   // (with two waves a row the shares stay: 0.256 against 0.258 ms at 64 rows)
   const int wpr = FUSED_WAVES / RW;           // waves of a row
   const int lr = wave / wpr, sw = wave - lr * wpr;
   const int row = r0 + lr;
