@@ -25,6 +25,10 @@
 //
 // Tiles are numbered so that the workgroups that run at the same time on an XCD (which has an L2
 // of its own) form a block of a few row tiles by a few column tiles, whose operands that L2 holds.
+//
+// Four further variants (DIRECT) send the slices from memory straight into LDS
+// (global_load_lds_dwordx4) instead of through registers: three or four stages for a long inner
+// size, and 128 x 192 tiles for wide outputs under many rows; see the kernel and choose_direct.
 #include "common.h"
 #include <type_traits>
 #include "launchers.h"
@@ -129,22 +133,25 @@ constexpr int MM_GROUP = 4;         // row tiles per block of tiles
 // step (float32 outputs only: the epilogue that stores them has no barrier, so group 1 is done then).
 // For few tiles of 64 x 64 under a long inner size: a compute unit that has one such tile has four
 // waves, too few to cover each other's waits for LDS and the barrier.
-template <int WTM, int WTN, int WVM, int WVN, int EPI, typename OT, int AHEAD = 1, int KG = 1>
+template <int WTM, int WTN, int WVM, int WVN, int EPI, typename OT, int AHEAD = 1, int KG = 1, int DIRECT = 0>
 __global__ __launch_bounds__(64 * WVM * WVN * KG) void linear_mfma_kernel(
     const bf16_t* __restrict__ act, long lda, const bf16_t* __restrict__ w,
     const float* __restrict__ bias, OT* __restrict__ out, long ldo, int n_rows, int n_out, int k_dim,
     int k_parts, long part_stride, MfmaScatter sc) {
   static_assert(KG == 1 || (KG == 2 && sizeof(OT) == 4 && AHEAD == 1), "two wave groups: float32 outputs");
+  static_assert(DIRECT == 0 || (DIRECT >= 2 && AHEAD == 1 && KG == 1), "slices straight into LDS: two stages or more");
   constexpr int T = 64 * WVM * WVN * KG;
+  constexpr int STAGES = DIRECT > 0 ? DIRECT : 2;   // slices of a step that LDS holds
   constexpr int HALVES = (MM_BK / 32) / KG;   // halves of a step along k that a wave multiplies
   constexpr int BM = WVM * WTM * 16, BN = WVN * WTN * 16;
   constexpr int TPR = MM_BK / 8;  // threads per staged row (16 bytes each)
   constexpr int RPP = T / TPR;      // rows per staging pass
   constexpr int PA = BM / RPP, PW = BN / RPP;
-  static_assert(BM % RPP == 0 && BN % RPP == 0 && RPP % 8 == 0 && MM_BK == 64, "tile rows must be whole staging passes");
+  static_assert(DIRECT > 0 || (BM % RPP == 0 && BN % RPP == 0), "tile rows must be whole staging passes");
+  static_assert(RPP % 8 == 0 && MM_BK == 64 && BM % 8 == 0 && BN % 8 == 0, "rows of eight chunks, swizzled in eights");
   extern __shared__ __align__(16) bf16_t lds[];
-  bf16_t* const as_base = lds;                      // [2][BM * MM_LD]
-  bf16_t* const ws_base = lds + 2 * BM * MM_LD;   // [2][BN * MM_LD]
+  bf16_t* const as_base = lds;                           // [STAGES][BM * MM_LD]
+  bf16_t* const ws_base = lds + STAGES * BM * MM_LD;   // [STAGES][BN * MM_LD]
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave_all = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -225,7 +232,7 @@ __global__ __launch_bounds__(64 * WVM * WVN * KG) void linear_mfma_kernel(
   // take step s + 1 + AHEAD
   auto k_step = [&](int s, auto store_next, auto load_after, auto set_c) {
     constexpr int set = decltype(set_c)::value;
-    const int buf = s & 1;
+    const int buf = DIRECT > 0 ? s % STAGES : s & 1;
     const bf16_t* as = as_base + buf * (BM * MM_LD) + (wr + lrow) * MM_LD;
     const bf16_t* ws = ws_base + buf * (BN * MM_LD) + (wc + lrow) * MM_LD;
     constexpr int GROUPS = HALVES * WTM;
@@ -270,43 +277,109 @@ __global__ __launch_bounds__(64 * WVM * WVN * KG) void linear_mfma_kernel(
   using no = std::integral_constant<bool, false>;
   using set0 = std::integral_constant<int, 0>;
 
-  // The first two steps' chunks are sent for together, the first step's into registers of their own
-  // (free before the loop needs them for MFMA operands): one trip to memory before the first MFMA
-  // instead of two, which is a fifth of the whole kernel when the inner size is a few steps long.
-  {
-    bf16x8_t first[ITEMS];
+  if constexpr (DIRECT > 0) {
+    // The slices go from memory straight into LDS (global_load_lds_dwordx4: a wave's load puts its 64 lanes'
+    // 16 bytes side by side, 1 KB, which is 8 rows of a slice).  The lane that fills position p of row r
+    // fetches the chunk that belongs there, p ^ (r & 7).  No registers hold operands on their way and no
+    // wave spends instructions on LDS stores; a compute unit also takes in more bytes a microsecond this
+    // way than through registers.  STAGES slices of a step in LDS, STAGES - 1 steps on their way; a
+    // step's loads are issued behind the barrier that says every wave has read the stage they overwrite.
+    // The inner size is whole steps here (the launcher sees to it): nothing can be zeroed on its way.
+    constexpr int WAVES = T / 64;
+    constexpr int GROUPS_A = BM / 8, GROUPS = (BM + BN) / 8;
+    // loads per wave and step: the same for every wave (each counts its own on their way); where the groups
+    // do not go round, the last waves fetch the last group once more
+    constexpr int LPW = (GROUPS + WAVES - 1) / WAVES;
+    constexpr int D = STAGES - 1;
+    static_assert((D - 1) * LPW < 64, "the counter of loads in flight");
+    typedef __attribute__((address_space(1))) const void* global_ptr_t;
+    typedef __attribute__((address_space(3))) void* lds_ptr_t;
+    const int lr = lane >> 3, lc = ((lane & 7) ^ lr) * 8;
+    const bf16_t* dp[LPW];
 #pragma unroll
-    for (int p = 0; p < ITEMS; ++p) first[p] = *reinterpret_cast<const bf16x8_t*>(gp[p] + (sk + 8 <= k_len ? 0 : -sk));
-    if (AHEAD > 1 || k_steps > 1) {
-#pragma unroll
-      for (int j = 1; j <= AHEAD; ++j)
-#pragma unroll
-        for (int p = 0; p < ITEMS; ++p) load_item(p, j, j - 1);
+    for (int i = 0; i < LPW; ++i) {
+      const int g = min(wave_all + i * WAVES, GROUPS - 1);   // 8 rows of the activations' slice, or of W's
+      if (g < GROUPS_A) {
+        const int r = row0 + g * 8 + lr;
+        dp[i] = act + (long)(r < n_rows ? r : n_rows - 1) * lda + k_begin + lc;
+      } else {
+        const int r = col0 + (g - GROUPS_A) * 8 + lr;
+        dp[i] = w + (long)(r < n_out ? r : n_out - 1) * k_dim + k_begin + lc;
+      }
     }
+    auto issue = [&](int step) {
+      const int st = step % STAGES;
 #pragma unroll
-    for (int p = 0; p < ITEMS; ++p) {
-      bf16_t* dst = p < PA ? as_base + p * RPP * MM_LD : ws_base + (p - PA) * RPP * MM_LD;
-      *reinterpret_cast<bf16x8_t*>(dst + s_lds) = sk + 8 <= k_len ? first[p] : zero8;
+      for (int i = 0; i < LPW; ++i) {
+        const int g = min(wave_all + i * WAVES, GROUPS - 1);
+        bf16_t* dst = g < GROUPS_A ? as_base + st * (BM * MM_LD) + g * (8 * MM_LD)
+                                   : ws_base + st * (BN * MM_LD) + (g - GROUPS_A) * (8 * MM_LD);
+        __builtin_amdgcn_global_load_lds((global_ptr_t)(dp[i] + step * MM_BK), (lds_ptr_t)dst, 16, 0, 0);
+      }
+    };
+    // waits until at most `steps_behind` steps' loads of this wave are still on their way, then for every wave
+    auto arrive = [&](int steps_behind) {
+      switch (steps_behind) {
+        case 0: asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); break;
+        case 1: asm volatile("s_waitcnt vmcnt(%0)" ::"n"(D >= 2 ? LPW : 0) : "memory"); break;
+        case 2: asm volatile("s_waitcnt vmcnt(%0)" ::"n"(D >= 3 ? 2 * LPW : 0) : "memory"); break;
+        default: asm volatile("s_waitcnt vmcnt(%0)" ::"n"(D >= 4 ? 3 * LPW : 0) : "memory"); break;
+      }
+      asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    };
+    static_assert(D <= 4, "arrive() knows up to three steps behind the one waited for");
+#pragma unroll
+    for (int j = 0; j < D; ++j)
+      if (j < k_steps) issue(j);
+    int s = 0;
+    for (; s + D < k_steps; ++s) {
+      arrive(D - 1);
+      issue(s + D);
+      k_step(s, no{}, no{}, set0{});
     }
-  }
-  __syncthreads();
-  int s = 0;
-  if constexpr (AHEAD == 1) {
-    for (; s + 2 < k_steps; ++s) k_step(s, yes{}, yes{}, set0{});
-    if (s + 1 < k_steps) k_step(s++, yes{}, no{}, set0{});
-    k_step(s, no{}, no{}, set0{});
+    for (; s < k_steps; ++s) {   // the last steps: nothing more to send for
+      arrive(k_steps - 1 - s);
+      k_step(s, no{}, no{}, set0{});
+    }
   } else {
-    // Step s + 1 lies in set s mod AHEAD: the sets take turns, AHEAD steps a round, in whole rounds
-    // and without a branch (where control flow joins the compiler waits for every load in flight):
-    // a step beyond the last multiplies the zeros that stand in for chunks beyond the stretch's
-    // end, and its loads read the stretch's start.
-    auto round = [&](auto... set_c) { ((k_step(s, yes{}, yes{}, set_c), ++s), ...); };
-    while (s < k_steps) {
-      if constexpr (AHEAD == 2) round(std::integral_constant<int, 0>{}, std::integral_constant<int, 1>{});
-      else if constexpr (AHEAD == 3) round(std::integral_constant<int, 0>{}, std::integral_constant<int, 1>{},
-                                           std::integral_constant<int, 2>{});
-      else round(std::integral_constant<int, 0>{}, std::integral_constant<int, 1>{}, std::integral_constant<int, 2>{},
-                 std::integral_constant<int, 3>{});
+    // The first two steps' chunks are sent for together, the first step's into registers of their own
+    // (free before the loop needs them for MFMA operands): one trip to memory before the first MFMA
+    // instead of two, which is a fifth of the whole kernel when the inner size is a few steps long.
+    {
+      bf16x8_t first[ITEMS];
+  #pragma unroll
+      for (int p = 0; p < ITEMS; ++p) first[p] = *reinterpret_cast<const bf16x8_t*>(gp[p] + (sk + 8 <= k_len ? 0 : -sk));
+      if (AHEAD > 1 || k_steps > 1) {
+  #pragma unroll
+        for (int j = 1; j <= AHEAD; ++j)
+  #pragma unroll
+          for (int p = 0; p < ITEMS; ++p) load_item(p, j, j - 1);
+      }
+  #pragma unroll
+      for (int p = 0; p < ITEMS; ++p) {
+        bf16_t* dst = p < PA ? as_base + p * RPP * MM_LD : ws_base + (p - PA) * RPP * MM_LD;
+        *reinterpret_cast<bf16x8_t*>(dst + s_lds) = sk + 8 <= k_len ? first[p] : zero8;
+      }
+    }
+    __syncthreads();
+    int s = 0;
+    if constexpr (AHEAD == 1) {
+      for (; s + 2 < k_steps; ++s) k_step(s, yes{}, yes{}, set0{});
+      if (s + 1 < k_steps) k_step(s++, yes{}, no{}, set0{});
+      k_step(s, no{}, no{}, set0{});
+    } else {
+      // Step s + 1 lies in set s mod AHEAD: the sets take turns, AHEAD steps a round, in whole rounds
+      // and without a branch (where control flow joins the compiler waits for every load in flight):
+      // a step beyond the last multiplies the zeros that stand in for chunks beyond the stretch's
+      // end, and its loads read the stretch's start.
+      auto round = [&](auto... set_c) { ((k_step(s, yes{}, yes{}, set_c), ++s), ...); };
+      while (s < k_steps) {
+        if constexpr (AHEAD == 2) round(std::integral_constant<int, 0>{}, std::integral_constant<int, 1>{});
+        else if constexpr (AHEAD == 3) round(std::integral_constant<int, 0>{}, std::integral_constant<int, 1>{},
+                                             std::integral_constant<int, 2>{});
+        else round(std::integral_constant<int, 0>{}, std::integral_constant<int, 1>{}, std::integral_constant<int, 2>{},
+                   std::integral_constant<int, 3>{});
+      }
     }
   }
 
@@ -341,7 +414,7 @@ __global__ __launch_bounds__(64 * WVM * WVN * KG) void linear_mfma_kernel(
   // bytes and a row's threads a whole stretch of the row, and a key's or value's eight channels
   // go to their cache page the same way.
   constexpr int LDT = BN + 8;   // row stride of the tile in LDS
-  constexpr int LDS_ELEMS = 2 * (BM + BN) * MM_LD;
+  constexpr int LDS_ELEMS = STAGES * (BM + BN) * MM_LD;
   // the whole tile at once if it fits, else the rows of one row of waves at a time
   constexpr int STAGE_ROWS = BM * LDT <= LDS_ELEMS ? BM : BM / WVM;
   constexpr bool CAN_STAGE = sizeof(OT) == 2 && STAGE_ROWS * LDT <= LDS_ELEMS;
@@ -434,13 +507,14 @@ __global__ __launch_bounds__(64 * WVM * WVN * KG) void linear_mfma_kernel(
   }
 }
 
-template <int WTM, int WTN, int WVM, int WVN, int EPI, typename OT, int AHEAD, int KG = 1>
+template <int WTM, int WTN, int WVM, int WVN, int EPI, typename OT, int AHEAD, int KG = 1, int DIRECT = 0>
 int launch_one(const void* act, long lda, const void* w, const float* bias, void* out, long ldo, int n_rows,
                int n_out, int k_dim, int k_parts, long part_stride, const MfmaScatter& sc, hipStream_t stream) {
   static_assert(AHEAD >= 1 && AHEAD <= 4, "sets of staging registers");
   constexpr int BM = WVM * WTM * 16, BN = WVN * WTN * 16;
-  constexpr size_t lds_bytes = 2ul * (BM + BN) * MM_LD * sizeof(bf16_t);
-  auto kernel = linear_mfma_kernel<WTM, WTN, WVM, WVN, EPI, OT, AHEAD, KG>;
+  constexpr size_t lds_bytes = (DIRECT > 0 ? DIRECT : 2ul) * (BM + BN) * MM_LD * sizeof(bf16_t);
+  static_assert(lds_bytes <= 160 * 1024, "a workgroup's LDS");
+  auto kernel = linear_mfma_kernel<WTM, WTN, WVM, WVN, EPI, OT, AHEAD, KG, DIRECT>;
   static bool allowed = false;  // more LDS than a kernel gets without asking
   if (!allowed) {
     const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
@@ -456,13 +530,13 @@ int launch_one(const void* act, long lda, const void* w, const float* bias, void
   return mgpt_last_error();
 }
 
-template <int WTM, int WTN, int WVM, int WVN, int AHEAD = 1>
+template <int WTM, int WTN, int WVM, int WVN, int AHEAD = 1, int DIRECT = 0>
 int launch_shape(const void* act, long lda, const void* w, const float* bias, void* out, int out_dtype, long ldo,
                  int n_rows, int n_out, int k_dim, int epilogue, int k_parts, long part_stride,
                  const MfmaScatter& sc, hipStream_t stream) {
 #define MM_LAUNCH(E, OT)                                                                                            \
-  return launch_one<WTM, WTN, WVM, WVN, E, OT, AHEAD>(act, lda, w, bias, out, ldo, n_rows, n_out, k_dim, k_parts, \
-                                                      part_stride, sc, stream)
+  return launch_one<WTM, WTN, WVM, WVN, E, OT, AHEAD, 1, DIRECT>(act, lda, w, bias, out, ldo, n_rows, n_out, k_dim, \
+                                                                 k_parts, part_stride, sc, stream)
   if (epilogue == MM_EPI_NONE && out_dtype == MGPT_BF16) MM_LAUNCH(MM_EPI_NONE, bf16_t);
   if (epilogue == MM_EPI_NONE && out_dtype == MGPT_F32) MM_LAUNCH(MM_EPI_NONE, float);
   if (epilogue == MM_EPI_GELU && out_dtype == MGPT_BF16) MM_LAUNCH(MM_EPI_GELU, bf16_t);
@@ -492,6 +566,14 @@ constexpr int MM_TILE_ROWS[MM_SHAPES] = {256, 128, 128, 64, 32};
 constexpr int MM_TILE_COLS[MM_SHAPES] = {256, 256, 64, 64, 32};
 constexpr int MM_MAX_PARTS = 8;
 constexpr int MM_AHEAD = 4;  // steps on their way from memory in the variant for few tiles over a large matrix
+// Shape ids from MM_DIRECT_FIRST on: the variants whose slices go from memory straight into LDS, by tile
+// (rows x columns), waves and stages: 32 x 32 (four waves of 16 x 16) and 64 x 64 (four of 32 x 32) with four
+// stages, 128 x 64 (eight of 32 x 32) with three, 128 x 192 (eight of 64 x 48) with two.
+constexpr int MM_DIRECT_FIRST = MM_SHAPES + 3;
+constexpr int MM_DIRECT_VARIANTS = 4;
+constexpr int MM_DIRECT_ROWS[MM_DIRECT_VARIANTS] = {32, 64, 128, 128};
+constexpr int MM_DIRECT_COLS[MM_DIRECT_VARIANTS] = {32, 64, 64, 192};
+constexpr int MM_SHAPE_IDS = MM_DIRECT_FIRST + MM_DIRECT_VARIANTS;
 
 long tiles_of(int shape, int n_rows, int n_out) {
   return (long)((n_rows + MM_TILE_ROWS[shape] - 1) / MM_TILE_ROWS[shape]) *
@@ -619,6 +701,44 @@ bool shapes_ok(const void* act, long lda, const void* w, const void* out, long l
          (lda % 8) == 0 && ldo >= n_out;
 }
 
+// whole steps along k, and operands aligned for 16-byte loads: what the variants that load straight into LDS need
+bool direct_ok(const void* act, const void* w, int k_dim) {
+  return (k_dim % MM_BK) == 0 && ((((size_t)act) | ((size_t)w)) & 15) == 0;
+}
+
+long direct_tiles(int variant, int n_rows, int n_out) {
+  return (long)((n_rows + MM_DIRECT_ROWS[variant] - 1) / MM_DIRECT_ROWS[variant]) *
+         ((n_out + MM_DIRECT_COLS[variant] - 1) / MM_DIRECT_COLS[variant]);
+}
+
+// The shape id for a product of a prompt portion (128 rows and more) whose slices can go straight into
+// LDS and that gains by it, or -1: the rules further down decide.  Which products gain was measured inside
+// the prefill step, one product of the layer changed at a time (alone in a graph of its own, with its
+// operands in the L2 from the launch before, every such variant is 10-20 % ahead of the register path, and
+// most of that is not there in the step):
+// - a long inner size (32 steps and more: the second feed-forward product).  Through registers two steps are
+//   on their way, or the inner size is split over workgroups and a second kernel adds the parts; here three
+//   or four stages hold as many steps, with no registers spent on them.  Prefill steps of 256 to 2,048
+//   tokens: width 512 -3 %, width 768 -1 to -10 %, width 1600 at 2,048 tokens -7 %.
+// - a wide output under many rows: tiles of 128 x 192 where a round of them costs less than a round of
+//   256 x 256 (qkv and first feed-forward product at 8,192 tokens, widths 512 to 1600: -2 to -5 % of the step).
+int choose_direct(int n_rows, int n_out, int k_dim) {
+  if (n_rows < 128 || (k_dim % MM_BK) != 0) return -1;
+  if (k_dim / MM_BK >= 32) {
+    const long t128 = direct_tiles(2, n_rows, n_out), t64 = direct_tiles(1, n_rows, n_out);
+    if (t128 > 520) return -1;
+    if (t128 >= 190) return MM_DIRECT_FIRST + 2;
+    return MM_DIRECT_FIRST + (t64 >= 190 ? 1 : 0);
+  }
+  const long wide = direct_tiles(3, n_rows, n_out), largest = tiles_of(0, n_rows, n_out);
+  if (wide < 190) return -1;
+  // a tile's cost: its outputs, times a factor that falls with its size, times the rounds of 256 tiles
+  const double cost_wide = (double)((wide + 255) / 256) * 128 * 192 * 0.78;
+  const double cost_largest = (double)((largest + 255) / 256) * 256 * 256 * 0.72;
+  if (largest >= 160 && cost_largest <= cost_wide) return -1;
+  return MM_DIRECT_FIRST + 3;
+}
+
 // shape < 0: chosen by the size.  k_parts: 0 = chosen by the size, together with the shape, if
 // `partials` holds enough floats (else unsplit; with a given shape unsplit too), 1 = unsplit,
 // more = that many stretches (refused if the buffer is too small).
@@ -633,7 +753,17 @@ int launch_any(int shape, int k_parts, const void* act, long lda, const void* w,
   // shapes MM_SHAPES and MM_SHAPES + 1: the two smallest tiles with more steps on their way from memory
   int ahead = 0;  // 0: chosen below
   bool two_groups = false;  // the 64 x 64 tile with two wave groups (shape MM_SHAPES + 2)
-  if (shape == MM_SHAPES + 2) {
+  int direct = -1;  // which of the variants whose slices go straight into LDS (-1: through registers)
+  if (shape < 0 && k_parts <= 1 && !leave_parts) {
+    const int chosen = direct_ok(act, w, k_dim) ? choose_direct(n_rows, n_out, k_dim) : -1;
+    if (chosen >= 0) shape = chosen, k_parts = 1;
+  }
+  if (shape >= MM_DIRECT_FIRST) {
+    if (shape >= MM_SHAPE_IDS || !direct_ok(act, w, k_dim)) return MGPT_ERR_BAD_SHAPE;
+    direct = shape - MM_DIRECT_FIRST;
+    shape = 3;   // (the rules below for the other variants do not apply)
+    ahead = 1;
+  } else if (shape == MM_SHAPES + 2) {
     shape = 3;
     ahead = 1;
     two_groups = true;
@@ -676,7 +806,7 @@ int launch_any(int shape, int k_parts, const void* act, long lda, const void* w,
     // a split product are)
     const int dt_here = split ? MGPT_F32 : out_dtype, epi_here = split ? MM_EPI_NONE : epilogue;
     if (dt_here != MGPT_F32 || (epi_here != MM_EPI_NONE && epi_here != MM_EPI_RESIDUAL)) return MGPT_ERR_BAD_SHAPE;
-  } else if (shape == 3 && ahead == 1) {
+  } else if (shape == 3 && ahead == 1 && direct < 0) {
     // 64 x 64 tiles under a long inner size (16 steps and more a workgroup), float32 out: two wave groups
     // a tile.  [2048 x 2048 -> 512] 12.9 us against 14.4, [1024 x 2048 -> 512] 12.2 / 13.4, [2048 x 3072 ->
     // 768] 24.2 / 25.5, [8192 x 2048 -> 512] 33.9 / 35.3; at 8 steps ([2048 x 512 -> 512]) nothing.
@@ -697,6 +827,15 @@ int launch_any(int shape, int k_parts, const void* act, long lda, const void* w,
   const long ld = split ? n_out : ldo, stride = split ? (long)n_rows * n_out : 0;
 #define MM_ARGS act, lda, w, b, dst, dt, ld, n_rows, n_out, k_dim, epi, k_parts, stride, sc, stream
   int rc = MGPT_ERR_BAD_SHAPE;
+  if (direct >= 0) {
+    switch (direct) {
+      case 0: rc = launch_shape<1, 1, 2, 2, 1, 4>(MM_ARGS); break;
+      case 1: rc = launch_shape<2, 2, 2, 2, 1, 4>(MM_ARGS); break;
+      case 2: rc = launch_shape<2, 2, 4, 2, 1, 3>(MM_ARGS); break;
+      case 3: rc = launch_shape<4, 3, 2, 4, 1, 2>(MM_ARGS); break;
+      default: break;
+    }
+  } else
   switch (shape) {
     case 0: rc = launch_shape<8, 4, 2, 4>(MM_ARGS); break;  // 256 x 256, eight waves of 128 x 64
     case 1: rc = launch_shape<4, 4, 2, 4>(MM_ARGS); break;  // 128 x 256, eight waves of 64 x 64
@@ -756,13 +895,15 @@ extern "C" int mgpt_linear_mfma(const void* act, long lda, const void* w, const 
 
 // The same product with the tile shape given (0 = 256 x 256, 1 = 128 x 256, 2 = 128 x 64,
 // 3 = 64 x 64, 4 = 32 x 32, 5 and 6 = 64 x 64 and 32 x 32 with four steps on their way from memory,
-// 7 = 64 x 64 with two wave groups a tile (float32 outputs); negative: chosen) and the number of stretches of the inner size given
+// 7 = 64 x 64 with two wave groups a tile (float32 outputs), 8 to 11 = the slices straight into LDS: 32 x 32 and
+// 64 x 64 with four stages, 128 x 64 with three, 128 x 192 with two (an inner size of whole steps of 64 and operands
+// aligned to 16 bytes, else refused); negative: chosen) and the number of stretches of the inner size given
 // (k_parts as for launch_any above), instead of chosen by the size: for tests and measurements.
 extern "C" int mgpt_linear_mfma_shape(int shape, int k_parts, const void* act, long lda, const void* w,
                                       const float* bias, void* out, int out_dtype, long ldo, int n_rows,
                                       int n_out, int k_dim, int epilogue, float* partials, long partials_floats,
                                       hipStream_t stream) {
-  if (epilogue == MM_EPI_QKV || shape > MM_SHAPES + 2 || k_parts < 0) return MGPT_ERR_BAD_SHAPE;
+  if (epilogue == MM_EPI_QKV || shape >= MM_SHAPE_IDS || k_parts < 0) return MGPT_ERR_BAD_SHAPE;
   MfmaScatter sc = {};
   return launch_any(shape, k_parts, act, lda, w, bias, out, out_dtype, ldo, n_rows, n_out, k_dim, epilogue,
                     partials, partials_floats, sc, stream);
@@ -780,7 +921,8 @@ extern "C" int mgpt_linear_mfma_qkv(const void* act, long lda, const void* w, co
   if (!kpool || !vpool || !slot_mapping) return MGPT_ERR_NULL;
   if (head_dim <= 0 || (head_dim % 4) != 0 || (q_width % 4) != 0 || q_width + 2 * kv_width != n_out ||
       kv_width != n_kv_head * head_dim || page_size <= 0 || (n_out % 4) != 0 || (ldo % 4) != 0 ||
-      (((size_t)out | (size_t)bias) & 15) != 0 || shape >= MM_SHAPES + 2)
+      (((size_t)out | (size_t)bias) & 15) != 0 || (shape >= MM_SHAPES + 2 && shape < MM_DIRECT_FIRST) ||
+      shape >= MM_SHAPE_IDS)
     return MGPT_ERR_BAD_SHAPE;
   MfmaScatter sc = {(bf16_t*)kpool, (bf16_t*)vpool, slot_mapping, q_width, kv_width, head_dim, n_kv_head, page_size};
   return launch_any(shape, 1, act, lda, w, bias, out, MGPT_BF16, ldo, n_rows, n_out, k_dim, MM_EPI_QKV, nullptr, 0, sc,

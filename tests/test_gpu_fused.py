@@ -330,9 +330,15 @@ def test_tiled_split_left_as_parts_of_a_pending_residual(rows, n_out, k_dim, bia
     helpers.assert_close(parts.sum(0), want, "bfloat16", "sum of the parts")
     joined = torch.zeros(rows, n_out, device=DEV)
     scratch = torch.zeros(need, device=DEV)
-    assert kernels.linear_mfma(dev(a), wd, dev(b), joined, rows, kernels.EPI_NONE, partials=scratch)
+    # (from 128 rows on the library, left to itself, does not split such a product: it sends the slices
+    # straight into LDS, four steps deep; the split is asked for then)
+    assert kernels.linear_mfma(dev(a), wd, dev(b), joined, rows, kernels.EPI_NONE, partials=scratch,
+                               k_parts=None if rows < 128 else n_parts)
     raw = scratch.view(n_parts, rows, n_out)
-    assert torch.equal(parts[1:], raw[1:])
+    if rows < 128:
+        assert torch.equal(parts[1:], raw[1:])
+    else:   # (the split that is asked for may take other tiles, whose waves add a step's halves in another order)
+        helpers.assert_close(parts[1:], raw[1:], "float32", "the parts of the split that was asked for")
     helpers.assert_close(parts[0], raw[0].double().cpu() + (0 if b is None else b.double()), "float32", "the first part")
     # read as a pending residual
     pending = PendingSums(dev(x), parts, n_parts)

@@ -218,9 +218,58 @@ def test_linear_mfma_each_tile_shape(n, k, o, epi, o_dt, shape):
     assert torch.equal(out[n:], prev[n:].to(DEV)), "rows beyond n_rows were written"
 
 
+@pytest.mark.parametrize("n,k,o", [(300, 64, 257), (513, 512, 520), (256, 2048, 256), (1000, 128, 130), (130, 192, 400),
+                                   (200, 320, 72), (40, 2112, 272)])
+@pytest.mark.parametrize("epi,o_dt", [(kernels.EPI_NONE, "bfloat16"), (kernels.EPI_NONE, "float32"),
+                                      (kernels.EPI_GELU, "bfloat16"), (kernels.EPI_RESIDUAL, "float32")])
+@pytest.mark.parametrize("shape", [8, 9, 10, 11])
+def test_linear_mfma_slices_straight_into_lds(n, k, o, epi, o_dt, shape):
+    """The variants whose operand slices go from memory straight into LDS (tiles of 32 x 32 and 64 x 64 with
+    four stages, 128 x 64 with three, 128 x 192 with two), forced at sizes that cut their tiles everywhere and
+    at inner sizes of 1, 2, 3, 5, 8, 32 and 33 steps: fewer steps than stages, as many, and more."""
+    g = torch.Generator().manual_seed(26)
+    a, w, bias = rnd(g, n, k, dtype="bfloat16"), rnd(g, o, k, dtype="bfloat16", scale=k ** -0.5), rnd(g, o)
+    prev = rnd(g, n + 2, o, dtype=o_dt)
+    out = prev.clone().to(DEV)
+    assert kernels.linear_mfma(a.to(DEV), w.to(DEV), bias.to(DEV), out, n, epi, shape=shape)
+    helpers.assert_close(out[:n], _linear_want(a, w, bias, epi, prev[:n]), "bfloat16", f"shape {shape} {n}x{k}x{o}")
+    assert torch.equal(out[n:], prev[n:].to(DEV)), "rows beyond n_rows were written"
+
+
+def test_linear_mfma_straight_into_lds_wants_whole_steps():
+    """An inner size that is no multiple of 64 is refused by those variants (nothing can be zeroed on its way
+    into LDS), and the library's own choice then goes through registers."""
+    g = torch.Generator().manual_seed(27)
+    n, k, o = 256, 2064, 512
+    a, w, bias = rnd(g, n, k, dtype="bfloat16"), rnd(g, o, k, dtype="bfloat16", scale=k ** -0.5), rnd(g, o)
+    out = torch.zeros(n, o, device=DEV)
+    for shape in (8, 9, 10, 11):
+        assert not kernels.linear_mfma(a.to(DEV), w.to(DEV), bias.to(DEV), out, n, kernels.EPI_NONE, shape=shape)
+    assert not kernels.linear_mfma(a.to(DEV), w.to(DEV), bias.to(DEV), out, n, kernels.EPI_NONE, shape=12)
+    assert kernels.linear_mfma(a.to(DEV), w.to(DEV), bias.to(DEV), out, n, kernels.EPI_NONE)
+    helpers.assert_close(out, _linear_want(a, w, bias, kernels.EPI_NONE, None), "bfloat16", "through registers")
+
+
+@pytest.mark.parametrize("n,k,o,shape", [(256, 2048, 512, 8), (2048, 2048, 512, 9), (2048, 3072, 768, 10), (8192, 512, 1536, 11),
+                                         (1024, 3072, 768, 9), (2048, 1600, 4800, 11)])
+def test_linear_mfma_chooses_the_variants_straight_into_lds(n, k, o, shape):
+    """A long inner size (32 steps and more) with few tiles, and a wide output under many rows: the library
+    takes those variants by itself, so its result equals the forced one bit by bit."""
+    g = torch.Generator().manual_seed(28)
+    a, w, bias = rnd(g, n, k, dtype="bfloat16"), rnd(g, o, k, dtype="bfloat16", scale=k ** -0.5), rnd(g, o)
+    prev = rnd(g, n, o)
+    out, out_f = prev.clone().to(DEV), prev.clone().to(DEV)
+    assert kernels.linear_mfma(a.to(DEV), w.to(DEV), bias.to(DEV), out, n, kernels.EPI_RESIDUAL)
+    assert kernels.linear_mfma(a.to(DEV), w.to(DEV), bias.to(DEV), out_f, n, kernels.EPI_RESIDUAL, shape=shape)
+    assert torch.equal(out, out_f)
+    helpers.assert_close(out, _linear_want(a, w, bias, kernels.EPI_RESIDUAL, prev), "bfloat16", "chosen")
+
+
 @pytest.mark.parametrize("n,k,o,shape,parts", [(100, 2048, 96, 4, 4), (70, 1040, 132, 3, 2), (300, 6400, 64, 3, 8),
                                                 (33, 576, 40, 4, 3), (130, 1600, 260, 2, 4), (64, 1600, 528, 6, 2),
-                                                (50, 3200, 96, 5, 4), (48, 6400, 1600, None, 0), (90, 4128, 200, 7, 3)])
+                                                (50, 3200, 96, 5, 4), (48, 6400, 1600, None, 0), (90, 4128, 200, 7, 3),
+                                                (100, 2048, 96, 8, 4), (300, 6400, 64, 9, 8), (130, 1600, 260, 10, 4),
+                                                (140, 1088, 400, 11, 3)])
 @pytest.mark.parametrize("epi,o_dt", [(kernels.EPI_NONE, "bfloat16"), (kernels.EPI_NONE, "float32"),
                                       (kernels.EPI_GELU, "bfloat16"), (kernels.EPI_RESIDUAL, "float32")])
 def test_linear_mfma_split_along_the_inner_size(n, k, o, shape, parts, epi, o_dt):
@@ -253,10 +302,12 @@ def test_linear_mfma_split_along_the_inner_size(n, k, o, shape, parts, epi, o_dt
 
 def test_linear_mfma_splits_by_itself_when_tiles_are_few_and_the_inner_size_long():
     g = torch.Generator().manual_seed(19)
-    n, k, o = 140, 6400, 1600
+    n, k, o = 140, 6416, 1600
     need = kernels.linear_mfma_partials(n, o, k, kernels.EPI_RESIDUAL)
     assert need > 0 and need % (n * o) == 0
     assert kernels.linear_mfma_partials(2048, 2048, 512, kernels.EPI_GELU) == 0
+    # (an inner size of whole steps under 128 rows and more is not split even with the buffer there: it goes
+    # straight into LDS, four steps deep; test_linear_mfma_chooses_the_variants_straight_into_lds)
     a, w, bias = rnd(g, n, k, dtype="bfloat16"), rnd(g, o, k, dtype="bfloat16", scale=k ** -0.5), rnd(g, o)
     prev = rnd(g, n, o)
     out, out1 = prev.clone().to(DEV), prev.clone().to(DEV)
@@ -456,7 +507,8 @@ def test_linear_skinny_few_rows_with_a_long_inner_size_split_over_workgroups(n, 
 
 
 @pytest.mark.parametrize("n,shape,k", [(70, None, 96), (300, 3, 96), (1100, 2, 96), (300, 1, 96), (520, 0, 96),
-                                       (40, None, 832), (60, 6, 96), (33, 5, 1024)])
+                                       (40, None, 832), (60, 6, 96), (33, 5, 1024), (200, 8, 256), (300, 9, 128),
+                                       (520, 10, 192), (1100, 11, 64)])
 def test_linear_mfma_stores_keys_and_values(n, shape, k):
     """The tiled kernel's fused QKV product: the tile shape chosen by the size and each larger one forced
     (at 40 rows over 13 steps the library takes the variant with four steps in flight by itself);
