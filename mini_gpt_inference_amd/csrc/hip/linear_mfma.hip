@@ -287,9 +287,9 @@ __global__ __launch_bounds__(64 * WVM * WVN * KG) void linear_mfma_kernel(
     // The inner size is whole steps here (the launcher sees to it): nothing can be zeroed on its way.
     constexpr int WAVES = T / 64;
     constexpr int GROUPS_A = BM / 8, GROUPS = (BM + BN) / 8;
-    // loads per wave and step: the same for every wave (each counts its own on their way); where the groups
-    // do not go round, the last waves fetch the last group once more
-    constexpr int LPW = (GROUPS + WAVES - 1) / WAVES;
+    // loads per wave and step: the same for every wave (each counts its own on their way)
+    static_assert(GROUPS % WAVES == 0, "the groups of eight rows go round among the waves");
+    constexpr int LPW = GROUPS / WAVES;
     constexpr int D = STAGES - 1;
     static_assert((D - 1) * LPW < 64, "the counter of loads in flight");
     typedef __attribute__((address_space(1))) const void* global_ptr_t;
@@ -298,7 +298,7 @@ __global__ __launch_bounds__(64 * WVM * WVN * KG) void linear_mfma_kernel(
     const bf16_t* dp[LPW];
 #pragma unroll
     for (int i = 0; i < LPW; ++i) {
-      const int g = min(wave_all + i * WAVES, GROUPS - 1);   // 8 rows of the activations' slice, or of W's
+      const int g = wave_all + i * WAVES;   // 8 rows of the activations' slice, or of W's
       if (g < GROUPS_A) {
         const int r = row0 + g * 8 + lr;
         dp[i] = act + (long)(r < n_rows ? r : n_rows - 1) * lda + k_begin + lc;
@@ -311,7 +311,7 @@ __global__ __launch_bounds__(64 * WVM * WVN * KG) void linear_mfma_kernel(
       const int st = step % STAGES;
 #pragma unroll
       for (int i = 0; i < LPW; ++i) {
-        const int g = min(wave_all + i * WAVES, GROUPS - 1);
+        const int g = wave_all + i * WAVES;
         bf16_t* dst = g < GROUPS_A ? as_base + st * (BM * MM_LD) + g * (8 * MM_LD)
                                    : ws_base + st * (BN * MM_LD) + (g - GROUPS_A) * (8 * MM_LD);
         __builtin_amdgcn_global_load_lds((global_ptr_t)(dp[i] + step * MM_BK), (lds_ptr_t)dst, 16, 0, 0);
@@ -319,15 +319,16 @@ __global__ __launch_bounds__(64 * WVM * WVN * KG) void linear_mfma_kernel(
     };
     // waits until at most `steps_behind` steps' loads of this wave are still on their way, then for every wave
     auto arrive = [&](int steps_behind) {
+#define MM_WAIT_CASE(N) \
+  case N: asm volatile("s_waitcnt vmcnt(%0)" ::"n"((N < D ? N : 0) * LPW) : "memory"); break;
       switch (steps_behind) {
-        case 0: asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); break;
-        case 1: asm volatile("s_waitcnt vmcnt(%0)" ::"n"(D >= 2 ? LPW : 0) : "memory"); break;
-        case 2: asm volatile("s_waitcnt vmcnt(%0)" ::"n"(D >= 3 ? 2 * LPW : 0) : "memory"); break;
-        default: asm volatile("s_waitcnt vmcnt(%0)" ::"n"(D >= 4 ? 3 * LPW : 0) : "memory"); break;
+        MM_WAIT_CASE(0) MM_WAIT_CASE(1) MM_WAIT_CASE(2) MM_WAIT_CASE(3) MM_WAIT_CASE(4) MM_WAIT_CASE(5) MM_WAIT_CASE(6)
+        default: asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); break;
       }
+#undef MM_WAIT_CASE
       asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
     };
-    static_assert(D <= 4, "arrive() knows up to three steps behind the one waited for");
+    static_assert(D <= 7, "arrive() knows up to six steps behind the one waited for");
 #pragma unroll
     for (int j = 0; j < D; ++j)
       if (j < k_steps) issue(j);
@@ -568,11 +569,11 @@ constexpr int MM_MAX_PARTS = 8;
 constexpr int MM_AHEAD = 4;  // steps on their way from memory in the variant for few tiles over a large matrix
 // Shape ids from MM_DIRECT_FIRST on: the variants whose slices go from memory straight into LDS, by tile
 // (rows x columns), waves and stages: 32 x 32 (four waves of 16 x 16) and 64 x 64 (four of 32 x 32) with four
-// stages, 128 x 64 (eight of 32 x 32) with three, 128 x 192 (eight of 64 x 48) with two.
+// stages, 128 x 64 (eight of 32 x 32) with three, 128 x 192 (eight of 64 x 48) with two, 32 x 32 with six.
 constexpr int MM_DIRECT_FIRST = MM_SHAPES + 3;
-constexpr int MM_DIRECT_VARIANTS = 4;
-constexpr int MM_DIRECT_ROWS[MM_DIRECT_VARIANTS] = {32, 64, 128, 128};
-constexpr int MM_DIRECT_COLS[MM_DIRECT_VARIANTS] = {32, 64, 64, 192};
+constexpr int MM_DIRECT_VARIANTS = 5;
+constexpr int MM_DIRECT_ROWS[MM_DIRECT_VARIANTS] = {32, 64, 128, 128, 32};
+constexpr int MM_DIRECT_COLS[MM_DIRECT_VARIANTS] = {32, 64, 64, 192, 32};
 constexpr int MM_SHAPE_IDS = MM_DIRECT_FIRST + MM_DIRECT_VARIANTS;
 
 long tiles_of(int shape, int n_rows, int n_out) {
@@ -791,6 +792,14 @@ int launch_any(int shape, int k_parts, const void* act, long lda, const void* w,
     // 12.8 against 11.7).
     const int steps = (k_dim + MM_BK - 1) / MM_BK;
     ahead = (shape == 4 && steps / k_parts >= 12 && tiles_of(4, n_rows, n_out) * k_parts <= 512) ? MM_AHEAD : 1;
+    // The same with the slices straight into LDS, where the operands allow it: the steps on their way need no
+    // registers, so there can be more of them (six stages while a compute unit has one such workgroup, four
+    // with more).  Decode steps of 12 layers of width 1600, in turns with the variant above on one box: 24 rows
+    // 0.774 -> 0.740 ms, 32 rows 0.795 -> 0.762, 64 rows 1.000 -> 0.949 (with six stages there 0.970).
+    if (ahead == MM_AHEAD && direct_ok(act, w, k_dim)) {
+      direct = tiles_of(4, n_rows, n_out) * k_parts <= 256 ? 4 : 0;
+      ahead = 1;
+    }
   }
   if (k_parts > 1) {
     k_parts = used_parts(k_dim, k_parts > MM_MAX_PARTS ? MM_MAX_PARTS : k_parts);
@@ -834,6 +843,7 @@ int launch_any(int shape, int k_parts, const void* act, long lda, const void* w,
       case 1: rc = launch_shape<2, 2, 2, 2, 1, 4>(MM_ARGS); break;
       case 2: rc = launch_shape<2, 2, 4, 2, 1, 3>(MM_ARGS); break;
       case 3: rc = launch_shape<4, 3, 2, 4, 1, 2>(MM_ARGS); break;
+      case 4: rc = launch_shape<1, 1, 2, 2, 1, 6>(MM_ARGS); break;
       default: break;
     }
   } else
@@ -896,8 +906,8 @@ extern "C" int mgpt_linear_mfma(const void* act, long lda, const void* w, const 
 
 // The same product with the tile shape given (0 = 256 x 256, 1 = 128 x 256, 2 = 128 x 64,
 // 3 = 64 x 64, 4 = 32 x 32, 5 and 6 = 64 x 64 and 32 x 32 with four steps on their way from memory,
-// 7 = 64 x 64 with two wave groups a tile (float32 outputs), 8 to 11 = the slices straight into LDS: 32 x 32 and
-// 64 x 64 with four stages, 128 x 64 with three, 128 x 192 with two (an inner size of whole steps of 64 and operands
+// 7 = 64 x 64 with two wave groups a tile (float32 outputs), 8 to 12 = the slices straight into LDS: 32 x 32 and
+// 64 x 64 with four stages, 128 x 64 with three, 128 x 192 with two, 32 x 32 with six (an inner size of whole steps of 64 and operands
 // aligned to 16 bytes, else refused); negative: chosen) and the number of stretches of the inner size given
 // (k_parts as for launch_any above), instead of chosen by the size: for tests and measurements.
 extern "C" int mgpt_linear_mfma_shape(int shape, int k_parts, const void* act, long lda, const void* w,

@@ -593,8 +593,9 @@ def linear_mfma(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], 
     epilogue).  `partials`: float32 scratch with which a long inner size over few tiles is split
     among workgroups (linear_mfma_partials says how much it takes).  `shape` (0 = 256 x 256 tiles,
     1 = 128 x 256, 2 = 128 x 64, 3 = 64 x 64, 4 = 32 x 32, 5 and 6 = 64 x 64 and 32 x 32 with four
-    steps on their way from memory, 7 = 64 x 64 with two wave groups that share a tile, float32 outputs, 8 to 11 = operand slices straight
-    into LDS with tiles of 32 x 32, 64 x 64, 128 x 64, 128 x 192: an inner size that is a multiple of 64) and
+    steps on their way from memory, 7 = 64 x 64 with two wave groups that share a tile, float32 outputs, 8 to 12 = operand slices straight
+    into LDS with tiles of 32 x 32, 64 x 64, 128 x 64, 128 x 192, 32 x 32 with six stages: an inner size that is a
+    multiple of 64) and
     `k_parts` fix what the library otherwise chooses by the size.  False when it does not take the shape."""
     if a.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
         return False

@@ -222,11 +222,11 @@ def test_linear_mfma_each_tile_shape(n, k, o, epi, o_dt, shape):
                                    (200, 320, 72), (40, 2112, 272)])
 @pytest.mark.parametrize("epi,o_dt", [(kernels.EPI_NONE, "bfloat16"), (kernels.EPI_NONE, "float32"),
                                       (kernels.EPI_GELU, "bfloat16"), (kernels.EPI_RESIDUAL, "float32")])
-@pytest.mark.parametrize("shape", [8, 9, 10, 11])
+@pytest.mark.parametrize("shape", [8, 9, 10, 11, 12])
 def test_linear_mfma_slices_straight_into_lds(n, k, o, epi, o_dt, shape):
     """The variants whose operand slices go from memory straight into LDS (tiles of 32 x 32 and 64 x 64 with
-    four stages, 128 x 64 with three, 128 x 192 with two), forced at sizes that cut their tiles everywhere and
-    at inner sizes of 1, 2, 3, 5, 8, 32 and 33 steps: fewer steps than stages, as many, and more."""
+    four stages, 128 x 64 with three, 128 x 192 with two, 32 x 32 with six), forced at sizes that cut their tiles
+    everywhere and at inner sizes of 1, 2, 3, 5, 8, 32 and 33 steps: fewer steps than stages, as many, and more."""
     g = torch.Generator().manual_seed(26)
     a, w, bias = rnd(g, n, k, dtype="bfloat16"), rnd(g, o, k, dtype="bfloat16", scale=k ** -0.5), rnd(g, o)
     prev = rnd(g, n + 2, o, dtype=o_dt)
@@ -243,18 +243,19 @@ def test_linear_mfma_straight_into_lds_wants_whole_steps():
     n, k, o = 256, 2064, 512
     a, w, bias = rnd(g, n, k, dtype="bfloat16"), rnd(g, o, k, dtype="bfloat16", scale=k ** -0.5), rnd(g, o)
     out = torch.zeros(n, o, device=DEV)
-    for shape in (8, 9, 10, 11):
+    for shape in (8, 9, 10, 11, 12):
         assert not kernels.linear_mfma(a.to(DEV), w.to(DEV), bias.to(DEV), out, n, kernels.EPI_NONE, shape=shape)
-    assert not kernels.linear_mfma(a.to(DEV), w.to(DEV), bias.to(DEV), out, n, kernels.EPI_NONE, shape=12)
+    assert not kernels.linear_mfma(a.to(DEV), w.to(DEV), bias.to(DEV), out, n, kernels.EPI_NONE, shape=13)
     assert kernels.linear_mfma(a.to(DEV), w.to(DEV), bias.to(DEV), out, n, kernels.EPI_NONE)
     helpers.assert_close(out, _linear_want(a, w, bias, kernels.EPI_NONE, None), "bfloat16", "through registers")
 
 
 @pytest.mark.parametrize("n,k,o,shape", [(256, 2048, 512, 8), (2048, 2048, 512, 9), (2048, 3072, 768, 10), (8192, 512, 1536, 11),
-                                         (1024, 3072, 768, 9), (2048, 1600, 4800, 11)])
+                                         (1024, 3072, 768, 9), (2048, 1600, 4800, 11), (32, 1600, 4800, 12), (64, 1600, 6400, 8)])
 def test_linear_mfma_chooses_the_variants_straight_into_lds(n, k, o, shape):
-    """A long inner size (32 steps and more) with few tiles, and a wide output under many rows: the library
-    takes those variants by itself, so its result equals the forced one bit by bit."""
+    """A long inner size (32 steps and more) with few tiles, a wide output under many rows, and few rows under
+    a large matrix (the rows of a decode step; six stages while the tiles are at most 256): the library takes
+    those variants by itself, so its result equals the forced one bit by bit."""
     g = torch.Generator().manual_seed(28)
     a, w, bias = rnd(g, n, k, dtype="bfloat16"), rnd(g, o, k, dtype="bfloat16", scale=k ** -0.5), rnd(g, o)
     prev = rnd(g, n, o)
@@ -269,7 +270,7 @@ def test_linear_mfma_chooses_the_variants_straight_into_lds(n, k, o, shape):
                                                 (33, 576, 40, 4, 3), (130, 1600, 260, 2, 4), (64, 1600, 528, 6, 2),
                                                 (50, 3200, 96, 5, 4), (48, 6400, 1600, None, 0), (90, 4128, 200, 7, 3),
                                                 (100, 2048, 96, 8, 4), (300, 6400, 64, 9, 8), (130, 1600, 260, 10, 4),
-                                                (140, 1088, 400, 11, 3)])
+                                                (140, 1088, 400, 11, 3), (64, 1600, 528, 12, 2)])
 @pytest.mark.parametrize("epi,o_dt", [(kernels.EPI_NONE, "bfloat16"), (kernels.EPI_NONE, "float32"),
                                       (kernels.EPI_GELU, "bfloat16"), (kernels.EPI_RESIDUAL, "float32")])
 def test_linear_mfma_split_along_the_inner_size(n, k, o, shape, parts, epi, o_dt):
@@ -508,7 +509,7 @@ def test_linear_skinny_few_rows_with_a_long_inner_size_split_over_workgroups(n, 
 
 @pytest.mark.parametrize("n,shape,k", [(70, None, 96), (300, 3, 96), (1100, 2, 96), (300, 1, 96), (520, 0, 96),
                                        (40, None, 832), (60, 6, 96), (33, 5, 1024), (200, 8, 256), (300, 9, 128),
-                                       (520, 10, 192), (1100, 11, 64)])
+                                       (520, 10, 192), (1100, 11, 64), (60, 12, 832)])
 def test_linear_mfma_stores_keys_and_values(n, shape, k):
     """The tiled kernel's fused QKV product: the tile shape chosen by the size and each larger one forced
     (at 40 rows over 13 steps the library takes the variant with four steps in flight by itself);
