@@ -397,7 +397,11 @@ def main(argv=None) -> int:
     spec = engine.model.spec
     raw = dict(arch.config_to_json(cfg))
     default_model = not args.model_config
-    config = {"model": "gpt2-mini-50.9M" if default_model else str(raw.get("architecture"))}
+    # the reference's 50.9M model: its widths (fewer layers are named beside the full count)
+    reference_sizes = default_model and (args.width, args.heads, args.vocab, args.positions) == (512, 8, 50304, 1024) \
+        and args.layers <= 8
+    config = {"model": "gpt2-mini-50.9M" if reference_sizes else
+              "gpt2-mini-other-sizes" if default_model else str(raw.get("architecture"))}
     # every size the architecture's config.json names, then what its code fixes (taken from the parts)
     config.update({k: v for k, v in raw.items() if k != "architecture" and isinstance(v, (int, float, str, bool))})
     config.pop("layer_norm_eps", None)
@@ -406,18 +410,21 @@ def main(argv=None) -> int:
         if role in layer0 and param in layer0[role][1].params:
             config[key] = layer0[role][1].params[param]
     if "n_layer" in config:
-        config["n_layer_full"] = 8 if default_model else config["n_layer"]
+        config["n_layer_full"] = 8 if reference_sizes else config["n_layer"]
     config.update({"global_batch": args.batch, "seq_len": spec.max_positions, "prompt_len": args.prompt,
                    "generated": run["generate"], "mean_context": round(mean_ctx, 1), "kv_block": args.kv_block,
                    "weights": "random", "hip_graph": bool(stats["graph_steps"]), "decode_burst": args.burst,
                    "parallelism": "single-gpu"})
-    name = "50.9M GPT-2-style" if default_model else config["model"]
+    name = ("50.9M GPT-2-style" if reference_sizes and args.layers == 8 else
+            f"50.9M GPT-2-style, {args.layers} of 8 layers" if reference_sizes else
+            f"GPT-2-style, {args.layers} layers of width {args.width}" if default_model else config["model"])
     record = {
         "metric": f"decode tokens/s ({name}, batch {args.batch}, {args.prompt}-token prompts, "
                   f"{run['generate']} generated tokens)",
         "value": round(value, 1), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(step_s * 1e3, 4), "higher_is_better": True, "scaling": "weak",
-        "vs_baseline": round(value / REFERENCE_DECODE_B8, 2) if args.batch == 8 and default_model else None,
+        "vs_baseline": round(value / REFERENCE_DECODE_B8, 2) if args.batch == 8 and reference_sizes and args.layers == 8
+        else None,
         "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "data": "synthetic",
         "config": config,
         # the timing rule: `value` is from the median block of `steps` decode steps; the quartiles' distance per step
