@@ -456,6 +456,29 @@ def test_the_benchmarked_prefill_step(tmp_path_factory, dtype, cut):
     assert rep.cache.num_free_pages() == 0, "the pool was meant to be exactly the two prompts"
 
 
+def test_the_benchmarked_prefill_step_replayed_from_its_graph(tmp_path_factory):
+    """The same step six times with other prompts each time, the requests ended in between so that the
+    pages come back: the first comings run eagerly and from the recorded plan, the third is captured, the
+    later ones are replays of that graph (whose products include the variants that load straight into
+    LDS: the second feed-forward product's inner size is 32 steps).  Every coming is compared with the
+    plain implementation."""
+    folder, cfg, pcfg, w = _family_model(tmp_path_factory, "50M")
+    rng = np.random.default_rng(78)
+    rep = TraceReplayer(folder, "bfloat16", 2048, poison=True)
+    assert rep.runner.graph_steps
+    rows = [0, 700, 1023]
+    for i in range(6):
+        prompts = [helpers.random_ids(rng, cfg.vocab_size, 1024) for _ in range(2)]
+        out = rep.run_step({"step": i, "entries": [{"id": f"r{i}p{j}", "tokens": t, "want": rows}
+                                                   for j, t in enumerate(prompts)],
+                            "end": [f"r{i}p0", f"r{i}p1"]})
+        got = out.clone().view(2, len(rows), -1)
+        for j, prompt in enumerate(prompts):
+            helpers.assert_close(got[j], P.plain_forward(w, pcfg, prompt, rows=rows), "bfloat16", f"coming {i}, prompt {j}")
+    assert rep.runner.num_replayed_steps >= 3
+    assert rep.cache.check() == 0 and rep.cache.num_free_pages() == rep.num_pages
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("n_req", [8, 17, 40, 64, 100, 128, 200, 256])
 @pytest.mark.parametrize("shape", ["small", "xl", "50M"])
