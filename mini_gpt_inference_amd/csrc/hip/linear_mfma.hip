@@ -26,9 +26,10 @@
 // Tiles are numbered so that the workgroups that run at the same time on an XCD (which has an L2
 // of its own) form a block of a few row tiles by a few column tiles, whose operands that L2 holds.
 //
-// Four further variants (DIRECT) send the slices from memory straight into LDS
+// Five further variants (DIRECT) send the slices from memory straight into LDS
 // (global_load_lds_dwordx4) instead of through registers: three or four stages for a long inner
-// size, and 128 x 192 tiles for wide outputs under many rows; see the kernel and choose_direct.
+// size, 128 x 192 tiles for wide outputs under many rows, and four or six stages of 32 x 32 tiles for
+// the rows of a decode step under a large matrix; see the kernel, choose_direct and launch_any.
 #include "common.h"
 #include <type_traits>
 #include "launchers.h"
